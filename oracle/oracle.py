@@ -1,0 +1,182 @@
+"""numpy/ctypes front end of the CPU oracle (test infrastructure only).
+
+Only tests, ``__graft_entry__.smoke`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module.  The product package never does.
+
+Every matrix is ``rows x N`` C-contiguous float32 (element (r, i) at r*N + i).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libneus2_oracle.so")
+_lib = None
+
+_f = C.POINTER(C.c_float)
+_u = C.POINTER(C.c_uint32)
+
+
+def build(force=False):
+    """Compile the oracle with its Makefile (g++ -O3 -fopenmp)."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "-B"], stdout=subprocess.DEVNULL)
+    else:
+        subprocess.check_call(["make", "-C", _HERE], stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_num_threads.restype = C.c_int
+        _lib.orc_mlp_n_params.restype = C.c_uint32
+    return _lib
+
+
+def num_threads():
+    return int(lib().orc_num_threads())
+
+
+def _fp(a):
+    if a is None:
+        return None
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"], (a.dtype, a.flags)
+    return a.ctypes.data_as(_f)
+
+
+def _up(a):
+    if a is None:
+        return None
+    assert a.dtype == np.uint32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_u)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class Grid:
+    """Level table + the grid functions of the oracle."""
+
+    def __init__(self, n_levels=16, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447):
+        self.n_levels = n_levels
+        self.n_features = 2
+        self.scale = np.zeros(n_levels, np.float32)
+        self.resolution = np.zeros(n_levels, np.uint32)
+        self.entries = np.zeros(n_levels, np.uint32)
+        self.offset = np.zeros(n_levels + 1, np.uint32)
+        lib().orc_grid_make_levels(C.c_uint32(n_levels), C.c_uint32(log2_hashmap_size), C.c_uint32(base_resolution),
+                                   C.c_float(per_level_scale), _fp(self.scale), _up(self.resolution),
+                                   _up(self.entries), _up(self.offset))
+        self.n_params = int(self.offset[-1]) * 2
+        self.n_out = n_levels * 2
+
+    def _tab(self):
+        return (C.c_uint32(self.n_levels), _fp(self.scale), _up(self.resolution), _up(self.entries))
+
+    def indices(self, xyz):
+        xyz = _f32(xyz)
+        n = xyz.shape[1]
+        idx = np.zeros((self.n_levels, 8, n), np.uint32)
+        w = np.zeros((self.n_levels, 3, n), np.float32)
+        lib().orc_grid_indices(*self._tab(), _fp(xyz), C.c_uint32(n), _up(idx), _fp(w))
+        return idx, w
+
+    def forward(self, params, xyz, want_dy_dx=False):
+        params, xyz = _f32(params), _f32(xyz)
+        n = xyz.shape[1]
+        y = np.zeros((self.n_out, n), np.float32)
+        j = np.zeros((self.n_out, n, 3), np.float32) if want_dy_dx else None
+        lib().orc_grid_forward(*self._tab(), _up(self.offset), _fp(params), _fp(xyz), C.c_uint32(n), _fp(y), _fp(j))
+        return (y, j) if want_dy_dx else y
+
+    def backward(self, params, xyz, dL_dy, want_grad=True, want_dx=True):
+        params, xyz, dL_dy = _f32(params), _f32(xyz), _f32(dL_dy)
+        n = xyz.shape[1]
+        grad = np.zeros(self.n_params, np.float32) if want_grad else None
+        dx = np.zeros((3, n), np.float32) if want_dx else None
+        lib().orc_grid_backward(*self._tab(), _up(self.offset), _fp(params), _fp(xyz), C.c_uint32(n), _fp(dL_dy),
+                                _fp(grad), _fp(dx))
+        return grad, dx
+
+    def backward_backward_input(self, params, xyz, v, g, grad=None, want_dinput=True):
+        """Returns (grad, dL_ddLdoutput, dL_dinput); ``grad`` is accumulated into when given."""
+        params, xyz, v, g = _f32(params), _f32(xyz), _f32(v), _f32(g)
+        n = xyz.shape[1]
+        if grad is None:
+            grad = np.zeros(self.n_params, np.float32)
+        out = np.zeros((self.n_out, n), np.float32)
+        din = np.zeros((3, n), np.float32) if want_dinput else None
+        lib().orc_grid_backward_backward_input(*self._tab(), _up(self.offset), _fp(params), _fp(xyz), C.c_uint32(n),
+                                               _fp(v), _fp(g), _fp(grad), _fp(out), _fp(din))
+        return grad, out, din
+
+
+class Mlp:
+    def __init__(self, in_width, width, n_hidden, out_width):
+        self.in_w, self.width, self.n_hidden, self.out_w = in_width, width, n_hidden, out_width
+        self.n_params = int(lib().orc_mlp_n_params(in_width, width, n_hidden, out_width))
+
+    def _d(self):
+        return (C.c_uint32(self.in_w), C.c_uint32(self.width), C.c_uint32(self.n_hidden), C.c_uint32(self.out_w))
+
+    def layer_shapes(self):
+        s = [(self.width, self.in_w)] + [(self.width, self.width)] * (self.n_hidden - 1) + [(self.out_w, self.width)]
+        return s
+
+    def split(self, W):
+        out, o = [], 0
+        for r, c in self.layer_shapes():
+            out.append(np.asarray(W[o:o + r * c]).reshape(r, c))
+            o += r * c
+        return out
+
+    def forward(self, W, x):
+        W, x = _f32(W), _f32(x)
+        n = x.shape[1]
+        y = np.zeros((self.out_w, n), np.float32)
+        h = np.zeros((self.n_hidden, self.width, n), np.float32)
+        lib().orc_mlp_forward(*self._d(), _fp(W), _fp(x), C.c_uint32(n), _fp(y), _fp(h))
+        return y, h
+
+    def backward(self, W, x, hidden, dL_dy, want_dx=True, want_dW=True):
+        W, x, hidden, dL_dy = _f32(W), _f32(x), _f32(hidden), _f32(dL_dy)
+        n = x.shape[1]
+        dx = np.zeros((self.in_w, n), np.float32) if want_dx else None
+        dW = np.zeros(self.n_params, np.float32) if want_dW else None
+        lib().orc_mlp_backward(*self._d(), _fp(W), _fp(x), _fp(hidden), _fp(dL_dy), C.c_uint32(n), _fp(dx), _fp(dW))
+        return dx, dW
+
+    def backward_backward_input(self, W, hidden, v, g, dW=None):
+        W, hidden, v, g = _f32(W), _f32(hidden), _f32(v), _f32(g)
+        n = v.shape[1]
+        if dW is None:
+            dW = np.zeros(self.n_params, np.float32)
+        out = np.zeros((self.out_w, n), np.float32)
+        lib().orc_mlp_backward_backward_input(*self._d(), _fp(W), _fp(hidden), _fp(v), _fp(g), C.c_uint32(n),
+                                              _fp(dW), _fp(out))
+        return dW, out
+
+
+def sh4(dirs):
+    dirs = _f32(dirs)
+    n = dirs.shape[1]
+    out = np.zeros((16, n), np.float32)
+    lib().orc_sh4(_fp(dirs), C.c_uint32(n), _fp(out))
+    return out
+
+
+def adam_step(w, grad, m1, m2, steps, n_matrix_params, loss_scale=128.0, lr=1e-3, beta1=0.9, beta2=0.99,
+              eps=1e-15, l2_reg=1e-6):
+    """In place on w, m1, m2 (float32) and steps (uint32)."""
+    grad = _f32(grad)
+    for a in (w, m1, m2):
+        assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    lib().orc_adam_step(C.c_uint32(w.size), C.c_uint32(n_matrix_params), C.c_float(loss_scale), C.c_float(lr),
+                        C.c_float(beta1), C.c_float(beta2), C.c_float(eps), C.c_float(l2_reg), _fp(w), _fp(grad),
+                        _fp(m1), _fp(m2), _up(steps))
