@@ -1,0 +1,192 @@
+/*
+ * neus2_amd.h - C ABI of the MI355X (gfx950) implementation of NeuS2's SDF-field hot path.
+ *
+ * The reference reaches this path through C++ virtual classes of its tcnn
+ * submodule (tcnn::Encoding<T>, tcnn::Network<float,T>); the entry points
+ * below are the flat C equivalents a binding for that interface would call.
+ * Each declaration cites the reference call site it replaces
+ * (paths relative to the reference checkout).
+ *
+ * Conventions
+ *  - Every pointer named d_* is DEVICE memory owned by the caller.  The library
+ *    allocates no device memory in any of these calls.
+ *  - "SoA rows x N": element (r, i) at r*N + i  (tcnn RM / SoA layout,
+ *    nerf_network.h:121-122).  fp16 buffers are IEEE binary16 (uint16_t here).
+ *  - stream is a hipStream_t passed as void* (NULL = the default stream).
+ *    Calls only enqueue work; they never synchronise.
+ *  - Every function returning int returns N2_OK (0) or an n2_status error;
+ *    n2_last_error() gives the message for the calling thread.
+ *  - Not re-entrant per object: one host thread, one stream per object, like
+ *    the reference (src/testbed.cu:2620-2621).
+ */
+#ifndef NEUS2_AMD_H
+#define NEUS2_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum n2_status {
+	N2_OK = 0,
+	N2_ERR_INVALID_ARGUMENT = 1, /* shape / alignment / null-pointer checks failed; nothing was launched */
+	N2_ERR_HIP = 2,              /* a HIP runtime call failed */
+	N2_ERR_UNSUPPORTED = 3       /* configuration outside what the kernels implement */
+} n2_status;
+
+/* tcnn::EGradientMode as used at nerf_network.h:229,340,402,429,543,570 */
+typedef enum n2_grad_mode {
+	N2_GRAD_IGNORE = 0,    /* do not touch parameter gradients */
+	N2_GRAD_OVERWRITE = 1, /* zero the gradient buffer, then accumulate this call */
+	N2_GRAD_ACCUMULATE = 2 /* add to what the gradient buffer holds */
+} n2_grad_mode;
+
+typedef void* n2_stream_t;
+typedef uint16_t n2_half;
+
+const char* n2_last_error(void);
+/* Library version string, e.g. "neus2_amd 0.1 gfx950". */
+const char* n2_version(void);
+
+/* ------------------------------------------------------------------------
+ * Multi-resolution hash grid encoding: tcnn::GridEncoding<__half, 3, 2>
+ * created by tcnn::create_encoding at nerf_network.h:46 from
+ * configs/nerf/base.json:29-39.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_grid n2_grid_t;
+
+/* create_encoding<T>(3, {otype HashGrid, n_levels, n_features_per_level = 2,
+ * log2_hashmap_size, base_resolution, per_level_scale}); nerf_network.h:46.
+ * The per-level table (scale, resolution, entries, offset) is computed once
+ * on the host in fp32 and handed to every kernel. */
+int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint32_t log2_hashmap_size,
+                   uint32_t base_resolution, float per_level_scale, n2_grid_t** out);
+void n2_grid_destroy(n2_grid_t* grid);
+
+/* Encoding::n_params / output_width (takikawa_encoding.cuh:424-447 shows the in-tree form). */
+uint32_t n2_grid_n_params(const n2_grid_t* grid);
+uint32_t n2_grid_output_width(const n2_grid_t* grid);
+uint32_t n2_grid_n_levels(const n2_grid_t* grid);
+
+/* Host copy of the level table; arrays of n_levels (offset: n_levels + 1) entries.
+ * Counterpart of GridEncoding::level_params_offset / level_n_params used at
+ * src/testbed.cu:3070-3091. */
+int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolution, uint32_t* entries,
+                        uint32_t* offset);
+
+/* Encoding::set_params(params, inference_params, backward_params, gradients),
+ * nerf_network.h:746-753.  One fp16 parameter buffer (n_params) and one fp16
+ * gradient buffer (n_params, may be NULL until a backward needs it). */
+int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients);
+
+/* Encoding::forward(stream, input, &output, use_inference_params, prepare_input_gradients),
+ * nerf_network.h:184-190 and inference at :671-676.
+ *  d_xyz      positions in [0,1]^3; coordinate d of point i at d_xyz[i*point_stride + d*dim_stride]
+ *             (the 7 x N column-major NerfCoordinate batch is point_stride = 7, dim_stride = 1;
+ *              a 3 x N SoA matrix is point_stride = 1, dim_stride = N)
+ *  d_out      fp16, SoA output_width x N
+ *  d_dy_dx    NULL, or fp32 [output_width][N][3]: the saved forward context the
+ *             input-gradient passes read (prepare_input_gradients = true) */
+int n2_grid_forward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                    uint32_t dim_stride, uint32_t n_points, n2_half* d_out, float* d_dy_dx);
+
+/* Encoding::backward(stream, ctx, input, output, dL_doutput, &dL_dinput, use_inference_params, mode),
+ * nerf_network.h:234 (normals, Ignore) and :419-429 (training, Overwrite).
+ *  d_dL_dy    fp16 SoA output_width x N
+ *  d_dy_dx    context saved by the forward (needed only when d_dL_dx != NULL)
+ *  d_dL_dx    NULL or fp32 SoA 3 x N
+ *  mode       what to do with the parameter gradients set by n2_grid_set_params */
+int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                     uint32_t dim_stride, uint32_t n_points, const n2_half* d_dL_dy, const float* d_dy_dx,
+                     float* d_dL_dx, n2_grad_mode mode);
+
+/* Encoding::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
+ * &dL_ddLdoutput, &dL_dinput, use_inference_params, mode), nerf_network.h:534-544.
+ *  d_dL_ddLdx       fp32 SoA 3 x N: gradient w.r.t. the first backward's dL_dx
+ *  d_dL_dy          fp16 SoA output_width x N: the dL_doutput the first backward was run with
+ *  d_dL_ddLdy       NULL or fp16 SoA output_width x N
+ *  d_dL_dx          NULL or fp32 SoA 3 x N (cross second derivatives; the reference
+ *                   computes and then drops it, nerf_network.h:529-541) */
+int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz,
+                                    uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
+                                    const float* d_dL_ddLdx, const n2_half* d_dL_dy, n2_half* d_dL_ddLdy,
+                                    float* d_dL_dx, n2_grad_mode mode);
+
+/* Test hook for the bit-exact contract: entry index (without the level offset)
+ * of the 8 trilinear corners, uint32 [n_levels][8][N], corner c uses +1 on
+ * dimension d iff bit d of c is set (takikawa_encoding.cuh:82-92). */
+int n2_grid_corner_indices(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                           uint32_t dim_stride, uint32_t n_points, uint32_t* d_indices);
+
+/* ------------------------------------------------------------------------
+ * Fully fused 64-wide MLP: tcnn::FullyFusedMLP<__half, 64>, ReLU hidden
+ * activations, linear output, no bias; created by tcnn::create_network at
+ * nerf_network.h:57 (SDF net, configs/nerf/base.json:40-47) and :65 (colour
+ * net, base.json:63-69).
+ * Weights: fp16, layers concatenated, each row-major [out][in]:
+ *   W_0 [64][in_width], W_1 .. W_{H-1} [64][64], W_H [16][64]
+ * (the order utils/mlp_weights.txt is stored in, nerf_network.h:774-803).
+ * Batch sizes must be multiples of 8 (the reference demands multiples of
+ * 128, src/testbed_nerf.cu:3429,3768).
+ * ---------------------------------------------------------------------- */
+typedef struct n2_mlp n2_mlp_t;
+
+/* Matrix layout of the 16-row network output / its gradient.  Inputs and
+ * input gradients are always SoA (the layout both encodings prefer). */
+typedef enum n2_layout {
+	N2_LAYOUT_SOA = 0, /* rows x N, element (r,i) at r*N + i                                   */
+	N2_LAYOUT_AOS = 1  /* N x 16, element (r,i) at i*16 + r: the testbed's column-major 16 x N
+	                      network output, src/testbed_nerf.cu:3771-3777                        */
+} n2_layout;
+
+/* create_network<T>({otype FullyFusedMLP, activation ReLU, output_activation None,
+ * n_neurons 64, n_hidden_layers, n_input_dims, n_output_dims 16}); nerf_network.h:53-57,63-65.
+ * in_width must be a multiple of 16 in [16, 64]; n_hidden_layers 1 or 2. */
+int n2_mlp_create(uint32_t in_width, uint32_t n_hidden_layers, n2_mlp_t** out);
+void n2_mlp_destroy(n2_mlp_t* mlp);
+uint32_t n2_mlp_n_params(const n2_mlp_t* mlp);
+uint32_t n2_mlp_input_width(const n2_mlp_t* mlp);
+uint32_t n2_mlp_output_width(const n2_mlp_t* mlp); /* padded_output_width() = 16 */
+
+/* Network::set_params(params, inference_params, backward_params, gradients), nerf_network.h:730-743. */
+int n2_mlp_set_params(n2_mlp_t* mlp, const n2_half* d_params, n2_half* d_gradients);
+
+/* Scratch for the batch reduction of weight gradients: fp32 partial sums, one
+ * slab per workgroup.  Needed by n2_mlp_backward with mode != IGNORE and by
+ * n2_mlp_backward_backward_input.  The reference takes this from tcnn's
+ * stream-ordered arena (src/testbed_nerf.cu:3723-3749); here the caller owns it. */
+uint64_t n2_mlp_workspace_bytes(const n2_mlp_t* mlp);
+int n2_mlp_set_workspace(n2_mlp_t* mlp, void* d_workspace, uint64_t n_bytes);
+
+/* Network::forward / inference_mixed_precision, nerf_network.h:212, 271, 686.
+ *  d_input   fp16 SoA in_width x N
+ *  d_output  fp16 16 x N in out_layout
+ *  d_hidden  NULL, or fp16 SoA (64*n_hidden_layers) x N: post-activation values of
+ *            every hidden layer (the forward context; Network::forward_activations).
+ *            The backward passes recompute them from d_input and never need it. */
+int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n, n2_half* d_output,
+                   n2_layout out_layout, n2_half* d_hidden);
+
+/* Network::backward(stream, ctx, input, output, dL_doutput, &dL_dinput, use_inference_params, mode),
+ * nerf_network.h:229 (normals, Ignore), :340, :402 (training), :509.
+ *  d_dL_doutput  fp16 16 x N in dL_layout
+ *  d_dL_dinput   NULL or fp16 SoA in_width x N */
+int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                    const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode);
+
+/* Network::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
+ * dL_ddLdoutput, dL_dinput, use_inference_params, mode): the second-order pass the
+ * reference fork adds for the eikonal loss, nerf_network.h:560-571.  One hidden
+ * layer only (the SDF net); dL_dinput is identically zero for ReLU and is not produced.
+ *  d_dL_ddLdinput  fp16 SoA in_width x N
+ *  d_dL_doutput    fp16 SoA 16 x N (the reference passes e_0)
+ *  d_dL_ddLdoutput NULL or fp16 SoA 16 x N */
+int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                                   const n2_half* d_dL_ddLdinput, const n2_half* d_dL_doutput,
+                                   n2_half* d_dL_ddLdoutput, n2_grad_mode mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NEUS2_AMD_H */

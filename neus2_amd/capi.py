@@ -1,0 +1,50 @@
+"""ctypes binding of libneus2_amd.so (the C ABI declared in include/neus2_amd.h).
+
+The library must have been built (``python -m neus2_amd.build``); there is no
+fallback implementation: a missing library is an ImportError-class failure.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libneus2_amd.so")
+
+N2_OK = 0
+GRAD_IGNORE, GRAD_OVERWRITE, GRAD_ACCUMULATE = 0, 1, 2
+
+_lib = None
+
+
+class N2Error(RuntimeError):
+    """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise N2Error(f"{LIB_PATH} is missing: build it with `python -m neus2_amd.build` "
+                          "(there is no CPU or eager fallback)")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.n2_last_error.restype = C.c_char_p
+        _lib.n2_version.restype = C.c_char_p
+        for name in ("n2_grid_n_params", "n2_grid_output_width", "n2_grid_n_levels"):
+            getattr(_lib, name).restype = C.c_uint32
+            getattr(_lib, name).argtypes = [C.c_void_p]
+        _lib.n2_grid_destroy.restype = None
+        _lib.n2_grid_destroy.argtypes = [C.c_void_p]
+    return _lib
+
+
+def check(rc, what=""):
+    if rc != N2_OK:
+        raise N2Error(f"{what} failed with status {rc}: {lib().n2_last_error().decode()}")
+
+
+def ptr(t):
+    """Device (or host) address of a torch tensor / numpy array, or NULL for None."""
+    if t is None:
+        return C.c_void_p(0)
+    if hasattr(t, "data_ptr"):
+        return C.c_void_p(t.data_ptr())
+    return C.c_void_p(t.ctypes.data)

@@ -1,0 +1,37 @@
+// Error reporting, version string and small utility kernels.
+#include "n2_common.h"
+
+static thread_local char g_err[512] = "";
+
+void n2_set_error(const char* fmt, ...) {
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_err, sizeof(g_err), fmt, ap);
+	va_end(ap);
+}
+
+N2_API const char* n2_last_error(void) { return g_err; }
+N2_API const char* n2_version(void) { return "neus2_amd 0.1 gfx950"; }
+
+__global__ void __launch_bounds__(256) n2_fill_zero_kernel(uint4* __restrict__ p16, size_t n16, uint8_t* __restrict__ tail, uint32_t n_tail) {
+	const size_t stride = (size_t)gridDim.x * blockDim.x;
+	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) p16[i] = make_uint4(0, 0, 0, 0);
+	if (blockIdx.x == 0 && threadIdx.x < n_tail) tail[threadIdx.x] = 0;
+}
+
+int n2_fill_zero_u32(hipStream_t stream, void* d_ptr, size_t n_bytes) {
+	if (n_bytes == 0) return N2_OK;
+	if (reinterpret_cast<uintptr_t>(d_ptr) % 16 != 0) {
+		n2_set_error("zero fill needs a 16-byte aligned buffer");
+		return N2_ERR_INVALID_ARGUMENT;
+	}
+	const size_t n16 = n_bytes / 16;
+	const uint32_t n_tail = (uint32_t)(n_bytes % 16);
+	size_t blocks = (n16 + 255) / 256;
+	if (blocks > 4096) blocks = 4096;
+	if (blocks == 0) blocks = 1;
+	n2_fill_zero_kernel<<<dim3((uint32_t)blocks), dim3(256), 0, stream>>>(
+		reinterpret_cast<uint4*>(d_ptr), n16, reinterpret_cast<uint8_t*>(d_ptr) + n16 * 16, n_tail);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

@@ -1,0 +1,480 @@
+// Multi-resolution hash grid encoding for gfx950: forward, backward
+// (parameter scatter + input gradient) and the second-order
+// backward_backward_input, behind the n2_grid_* C ABI.
+//
+// Work decomposition: one workgroup handles a tile of points for ONE level.
+// Workgroup ids are level-major (all tiles of level 0, then level 1, ...).
+// The hardware deals consecutive workgroup ids round-robin over the 8 XCDs,
+// so at any moment every XCD works on the same level and its private 4 MiB
+// L2 only has to hold that level's table (<= 2 MiB at T = 2^19) while the
+// points stream through.
+#include "n2_common.h"
+
+#include <cmath>
+#include <new>
+
+struct n2_grid {
+	N2LevelTable tab;
+	uint32_t n_features;
+	uint32_t n_params;
+	const __half2* params;
+	__half2* grads;
+};
+
+// ----------------------------------------------------------------------------
+// device helpers
+// ----------------------------------------------------------------------------
+
+// pos = x*scale + 0.5 as one fused multiply-add, then floor: the integer cell
+// and the fractional weight.  The fused form is part of the bit-exact contract
+// with the CPU oracle.
+__device__ __forceinline__ void n2_locate(float x, float scale, float& w, uint32_t& cell) {
+	const float p = __fmaf_rn(x, scale, 0.5f);
+	const float f = floorf(p);
+	cell = (uint32_t)(int32_t)f;
+	w = p - f;
+}
+
+template <uint32_t MODE>
+__device__ __forceinline__ uint32_t n2_entry(uint32_t entries, uint32_t res, uint32_t gx, uint32_t gy, uint32_t gz) {
+	if (MODE == N2_LEVEL_DENSE) {
+		uint32_t i = gx + gy * res + gz * res * res;
+		// the host has checked res^3 + res^2 + res < 2*entries
+		return i >= entries ? i - entries : i;
+	} else if (MODE == N2_LEVEL_HASH) {
+		return (gx ^ (gy * 2654435761u) ^ (gz * 805459861u)) & (entries - 1u);
+	} else if (MODE == N2_LEVEL_DENSE_MOD) {
+		return (gx + gy * res + gz * res * res) % entries;
+	} else {
+		return (gx ^ (gy * 2654435761u) ^ (gz * 805459861u)) % entries;
+	}
+}
+
+struct N2Point {
+	float w[3];
+	uint32_t c[3];
+};
+
+__device__ __forceinline__ N2Point n2_load_point(const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                 uint32_t i, float scale) {
+	N2Point p;
+	const float* q = xyz + (size_t)i * point_stride;
+#pragma unroll
+	for (int d = 0; d < 3; ++d) n2_locate(q[(size_t)d * dim_stride], scale, p.w[d], p.c[d]);
+	return p;
+}
+
+template <uint32_t MODE>
+__device__ __forceinline__ void n2_corner_entries(const N2Point& p, uint32_t entries, uint32_t res, uint32_t e[8]) {
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		e[k] = n2_entry<MODE>(entries, res, p.c[0] + (k & 1u), p.c[1] + ((k >> 1) & 1u), p.c[2] + ((k >> 2) & 1u));
+	}
+}
+
+__device__ __forceinline__ float n2_corner_weight(const N2Point& p, uint32_t k) {
+	float wt = (k & 1u) ? p.w[0] : 1.f - p.w[0];
+	wt *= (k & 2u) ? p.w[1] : 1.f - p.w[1];
+	wt *= (k & 4u) ? p.w[2] : 1.f - p.w[2];
+	return wt;
+}
+
+#define N2_DISPATCH_MODE(mode, CALL)                        \
+	switch (mode) {                                         \
+		case N2_LEVEL_DENSE: { CALL(N2_LEVEL_DENSE); } break;       \
+		case N2_LEVEL_HASH: { CALL(N2_LEVEL_HASH); } break;         \
+		case N2_LEVEL_DENSE_MOD: { CALL(N2_LEVEL_DENSE_MOD); } break; \
+		default: { CALL(N2_LEVEL_HASH_MOD); } break;                \
+	}
+
+constexpr uint32_t GRID_BLOCK = 256;
+
+// ----------------------------------------------------------------------------
+// forward
+// ----------------------------------------------------------------------------
+template <uint32_t MODE, bool WANT_DYDX>
+__device__ __forceinline__ void grid_forward_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
+                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                   const __half2* __restrict__ params, __half* __restrict__ out,
+                                                   float* __restrict__ dy_dx) {
+	const float scale = tab.scale[level];
+	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
+	const __half2* P = params + tab.offset[level];
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	uint32_t e[8];
+	n2_corner_entries<MODE>(p, entries, res, e);
+	float2 v[8];
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) v[k] = __half22float2(P[e[k]]);
+	float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		const float wt = n2_corner_weight(p, k);
+		a0 = fmaf(wt, v[k].x, a0);
+		a1 = fmaf(wt, v[k].y, a1);
+	}
+	const size_t row = (size_t)level * 2;
+	out[row * N + i] = __float2half_rn(a0);
+	out[(row + 1) * N + i] = __float2half_rn(a1);
+	if (WANT_DYDX) {
+		float g0[3], g1[3];
+#pragma unroll
+		for (int gd = 0; gd < 3; ++gd) {
+			const int d1 = (gd + 1) % 3, d2 = (gd + 2) % 3;
+			float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+			for (uint32_t k = 0; k < 8; ++k) {
+				if ((k >> gd) & 1u) continue;
+				float wt = ((k >> d1) & 1u) ? p.w[d1] : 1.f - p.w[d1];
+				wt *= ((k >> d2) & 1u) ? p.w[d2] : 1.f - p.w[d2];
+				const uint32_t kr = k | (1u << gd);
+				s0 = fmaf(wt, v[kr].x - v[k].x, s0);
+				s1 = fmaf(wt, v[kr].y - v[k].y, s1);
+			}
+			g0[gd] = s0 * scale;
+			g1[gd] = s1 * scale;
+		}
+		float* j0 = dy_dx + (row * N + i) * 3;
+		float* j1 = dy_dx + ((row + 1) * N + i) * 3;
+		j0[0] = g0[0]; j0[1] = g0[1]; j0[2] = g0[2];
+		j1[0] = g1[0]; j1[1] = g1[1]; j1[2] = g1[2];
+	}
+}
+
+template <bool WANT_DYDX>
+__global__ void __launch_bounds__(GRID_BLOCK) grid_forward_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                                  const float* __restrict__ xyz, uint32_t point_stride,
+                                                                  uint32_t dim_stride, const __half2* __restrict__ params,
+                                                                  __half* __restrict__ out, float* __restrict__ dy_dx) {
+	const uint32_t level = blockIdx.x / tiles;
+	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+#define CALL(M) grid_forward_point<M, WANT_DYDX>(tab, level, i, N, xyz, point_stride, dim_stride, params, out, dy_dx)
+	N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+}
+
+// ----------------------------------------------------------------------------
+// corner indices (test hook of the bit-exact contract)
+// ----------------------------------------------------------------------------
+__global__ void __launch_bounds__(GRID_BLOCK) grid_indices_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                                  const float* __restrict__ xyz, uint32_t point_stride,
+                                                                  uint32_t dim_stride, uint32_t* __restrict__ idx) {
+	const uint32_t level = blockIdx.x / tiles;
+	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, tab.scale[level]);
+	uint32_t e[8];
+#define CALL(M) n2_corner_entries<M>(p, tab.entries[level], tab.resolution[level], e)
+	N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) idx[((size_t)level * 8 + k) * N + i] = e[k];
+}
+
+// ----------------------------------------------------------------------------
+// backward: parameter scatter (packed fp16 atomics) ...
+// ----------------------------------------------------------------------------
+template <uint32_t MODE>
+__device__ __forceinline__ void grid_scatter_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
+                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                   const __half* __restrict__ dL_dy, __half2* __restrict__ grads) {
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, tab.scale[level]);
+	uint32_t e[8];
+	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
+	const size_t row = (size_t)level * 2;
+	const float g0 = __half2float(dL_dy[row * N + i]);
+	const float g1 = __half2float(dL_dy[(row + 1) * N + i]);
+	if (g0 == 0.f && g1 == 0.f) return;
+	__half2* G = grads + tab.offset[level];
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		const float wt = n2_corner_weight(p, k);
+		unsafeAtomicAdd(&G[e[k]], __floats2half2_rn(g0 * wt, g1 * wt));
+	}
+}
+
+__global__ void __launch_bounds__(GRID_BLOCK) grid_backward_params_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                                          const float* __restrict__ xyz, uint32_t point_stride,
+                                                                          uint32_t dim_stride, const __half* __restrict__ dL_dy,
+                                                                          __half2* __restrict__ grads) {
+	const uint32_t level = blockIdx.x / tiles;
+	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+#define CALL(M) grid_scatter_point<M>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, grads)
+	N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+}
+
+// ... and input gradient dL_dx[d][i] = sum_k dL_dy[k][i] * dy_dx[k][i][d]
+__global__ void __launch_bounds__(GRID_BLOCK) grid_backward_input_kernel(uint32_t N, uint32_t n_out,
+                                                                         const __half* __restrict__ dL_dy,
+                                                                         const float* __restrict__ dy_dx,
+                                                                         float* __restrict__ dL_dx) {
+	const uint32_t i = blockIdx.x * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+	float r0 = 0.f, r1 = 0.f, r2 = 0.f;
+	for (uint32_t k = 0; k < n_out; ++k) {
+		const float g = __half2float(dL_dy[(size_t)k * N + i]);
+		const float* j = dy_dx + ((size_t)k * N + i) * 3;
+		r0 = fmaf(g, j[0], r0);
+		r1 = fmaf(g, j[1], r1);
+		r2 = fmaf(g, j[2], r2);
+	}
+	dL_dx[i] = r0;
+	dL_dx[(size_t)N + i] = r1;
+	dL_dx[(size_t)2 * N + i] = r2;
+}
+
+// ----------------------------------------------------------------------------
+// second order: gradient of <v, dL_dx> w.r.t. the table, dL_dy and x
+// ----------------------------------------------------------------------------
+template <uint32_t MODE>
+__device__ __forceinline__ void grid_bbi_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
+                                               const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                               const float* __restrict__ v, const __half* __restrict__ dL_dy,
+                                               const __half2* __restrict__ params, __half2* __restrict__ grads,
+                                               __half* __restrict__ dL_ddLdy, float* __restrict__ dL_dx) {
+	const float scale = tab.scale[level];
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	uint32_t e[8];
+	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
+	const size_t row = (size_t)level * 2;
+	const float v0 = v[i] * scale, v1 = v[(size_t)N + i] * scale, v2 = v[(size_t)2 * N + i] * scale;
+	const float g0 = __half2float(dL_dy[row * N + i]);
+	const float g1 = __half2float(dL_dy[(row + 1) * N + i]);
+	const bool need_vals = dL_ddLdy != nullptr || dL_dx != nullptr;
+	const __half2* P = params + tab.offset[level];
+	__half2* G = grads ? grads + tab.offset[level] : nullptr;
+	float o0 = 0.f, o1 = 0.f, dx0 = 0.f, dx1 = 0.f, dx2 = 0.f;
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		const float w0 = (k & 1u) ? p.w[0] : 1.f - p.w[0];
+		const float w1 = (k & 2u) ? p.w[1] : 1.f - p.w[1];
+		const float w2 = (k & 4u) ? p.w[2] : 1.f - p.w[2];
+		const float s0 = (k & 1u) ? 1.f : -1.f, s1 = (k & 2u) ? 1.f : -1.f, s2 = (k & 4u) ? 1.f : -1.f;
+		// sum_d v_d * d(weight_k)/dx_d   (v already carries one factor of scale)
+		const float coef = v0 * s0 * w1 * w2 + v1 * s1 * w0 * w2 + v2 * s2 * w0 * w1;
+		if (G) unsafeAtomicAdd(&G[e[k]], __floats2half2_rn(g0 * coef, g1 * coef));
+		if (need_vals) {
+			const float2 val = __half22float2(P[e[k]]);
+			o0 = fmaf(coef, val.x, o0);
+			o1 = fmaf(coef, val.y, o1);
+			if (dL_dx) {
+				const float gp = (g0 * val.x + g1 * val.y) * scale;  // second factor of scale
+				const float h01 = s0 * s1 * w2, h02 = s0 * s2 * w1, h12 = s1 * s2 * w0;
+				dx0 = fmaf(gp, v1 * h01 + v2 * h02, dx0);
+				dx1 = fmaf(gp, v0 * h01 + v2 * h12, dx1);
+				dx2 = fmaf(gp, v0 * h02 + v1 * h12, dx2);
+			}
+		}
+	}
+	if (dL_ddLdy) {
+		dL_ddLdy[row * N + i] = __float2half_rn(o0);
+		dL_ddLdy[(row + 1) * N + i] = __float2half_rn(o1);
+	}
+	if (dL_dx) {
+		unsafeAtomicAdd(&dL_dx[i], dx0);
+		unsafeAtomicAdd(&dL_dx[(size_t)N + i], dx1);
+		unsafeAtomicAdd(&dL_dx[(size_t)2 * N + i], dx2);
+	}
+}
+
+__global__ void __launch_bounds__(GRID_BLOCK) grid_bbi_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                              const float* __restrict__ xyz, uint32_t point_stride,
+                                                              uint32_t dim_stride, const float* __restrict__ v,
+                                                              const __half* __restrict__ dL_dy, const __half2* __restrict__ params,
+                                                              __half2* __restrict__ grads, __half* __restrict__ dL_ddLdy,
+                                                              float* __restrict__ dL_dx) {
+	const uint32_t level = blockIdx.x / tiles;
+	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+#define CALL(M) grid_bbi_point<M>(tab, level, i, N, xyz, point_stride, dim_stride, v, dL_dy, params, grads, dL_ddLdy, dL_dx)
+	N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+}
+
+// ----------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------
+static uint32_t level_mode(uint32_t res, uint32_t entries) {
+	// Mirror of the reference index rule: add dimensions while the running
+	// stride still fits into the level; hashed iff the final stride exceeds it.
+	uint64_t stride = 1;
+	for (int d = 0; d < 3 && stride <= entries; ++d) stride *= res;
+	const bool hashed = entries < stride;
+	const bool pow2 = (entries & (entries - 1u)) == 0;
+	if (hashed) return pow2 ? N2_LEVEL_HASH : N2_LEVEL_HASH_MOD;
+	const uint64_t r = res;
+	const uint64_t max_index = r + r * r + r * r * r;  // every coordinate at most res
+	return (max_index < 2ull * entries) ? N2_LEVEL_DENSE : N2_LEVEL_DENSE_MOD;
+}
+
+N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint32_t log2_hashmap_size,
+                          uint32_t base_resolution, float per_level_scale, n2_grid_t** out) {
+	N2_REQUIRE(out != nullptr, "n2_grid_create: out is null");
+	*out = nullptr;
+	N2_REQUIRE(n_levels >= 1 && n_levels <= N2_MAX_LEVELS, "n2_grid_create: n_levels %u outside [1, %u]", n_levels, N2_MAX_LEVELS);
+	if (n_features_per_level != 2) {
+		n2_set_error("n2_grid_create: only n_features_per_level = 2 is implemented (got %u)", n_features_per_level);
+		return N2_ERR_UNSUPPORTED;
+	}
+	N2_REQUIRE(log2_hashmap_size >= 3 && log2_hashmap_size <= 28, "n2_grid_create: log2_hashmap_size %u outside [3, 28]", log2_hashmap_size);
+	N2_REQUIRE(base_resolution >= 1 && per_level_scale >= 1.0f, "n2_grid_create: base_resolution >= 1 and per_level_scale >= 1 required");
+	n2_grid* g = new (std::nothrow) n2_grid();
+	N2_REQUIRE(g != nullptr, "n2_grid_create: out of host memory");
+	g->n_features = n_features_per_level;
+	g->tab.n_levels = n_levels;
+	uint64_t off = 0;
+	const float log2_b = std::log2(per_level_scale);
+	for (uint32_t l = 0; l < n_levels; ++l) {
+		const float s = exp2f((float)l * log2_b) * (float)base_resolution - 1.0f;
+		const uint32_t res = (uint32_t)ceilf(s) + 1u;
+		const uint32_t max_params = 0xFFFFFFFFu / 2u;
+		const double cube = (double)res * (double)res * (double)res;
+		uint32_t n = cube > (double)max_params ? max_params : res * res * res;
+		n = (n + 7u) / 8u * 8u;
+		const uint32_t cap = 1u << log2_hashmap_size;
+		if (n > cap) n = cap;
+		g->tab.scale[l] = s;
+		g->tab.resolution[l] = res;
+		g->tab.entries[l] = n;
+		g->tab.offset[l] = (uint32_t)off;
+		g->tab.mode[l] = level_mode(res, n);
+		off += n;
+	}
+	if (off * n_features_per_level > 0x7FFFFFFFull) {
+		delete g;
+		n2_set_error("n2_grid_create: %llu parameters exceed the 2^31 limit", (unsigned long long)(off * n_features_per_level));
+		return N2_ERR_UNSUPPORTED;
+	}
+	g->tab.offset[n_levels] = (uint32_t)off;
+	g->n_params = (uint32_t)off * n_features_per_level;
+	g->params = nullptr;
+	g->grads = nullptr;
+	*out = g;
+	return N2_OK;
+}
+
+N2_API void n2_grid_destroy(n2_grid_t* grid) { delete grid; }
+N2_API uint32_t n2_grid_n_params(const n2_grid_t* grid) { return grid ? grid->n_params : 0; }
+N2_API uint32_t n2_grid_output_width(const n2_grid_t* grid) { return grid ? grid->tab.n_levels * grid->n_features : 0; }
+N2_API uint32_t n2_grid_n_levels(const n2_grid_t* grid) { return grid ? grid->tab.n_levels : 0; }
+
+N2_API int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolution, uint32_t* entries, uint32_t* offset) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_level_table: grid is null");
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
+		if (scale) scale[l] = grid->tab.scale[l];
+		if (resolution) resolution[l] = grid->tab.resolution[l];
+		if (entries) entries[l] = grid->tab.entries[l];
+		if (offset) offset[l] = grid->tab.offset[l];
+	}
+	if (offset) offset[grid->tab.n_levels] = grid->tab.offset[grid->tab.n_levels];
+	return N2_OK;
+}
+
+N2_API int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_params: grid is null");
+	N2_REQUIRE(d_params != nullptr, "n2_grid_set_params: d_params is null");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 16 == 0, "n2_grid_set_params: d_params must be 16-byte aligned");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_gradients) % 16 == 0, "n2_grid_set_params: d_gradients must be 16-byte aligned");
+	grid->params = reinterpret_cast<const __half2*>(d_params);
+	grid->grads = reinterpret_cast<__half2*>(d_gradients);
+	return N2_OK;
+}
+
+// Shared argument checks.  Row offsets are computed in 64 bits on the device;
+// the point index itself is 32 bits.
+static int check_batch(const n2_grid_t* grid, const char* fn, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride,
+                       uint32_t n_points) {
+	N2_REQUIRE(grid != nullptr, "%s: grid is null", fn);
+	N2_REQUIRE(grid->params != nullptr, "%s: n2_grid_set_params has not been called", fn);
+	N2_REQUIRE(d_xyz != nullptr || n_points == 0, "%s: d_xyz is null", fn);
+	N2_REQUIRE(point_stride >= 1 && dim_stride >= 1, "%s: strides must be >= 1", fn);
+	N2_REQUIRE(n_points <= (1u << 30), "%s: n_points %u exceeds 2^30", fn, n_points);
+	return N2_OK;
+}
+
+static inline uint32_t n_tiles(uint32_t n_points) { return (n_points + GRID_BLOCK - 1) / GRID_BLOCK; }
+
+N2_API int n2_grid_forward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                           uint32_t dim_stride, uint32_t n_points, n2_half* d_out, float* d_dy_dx) {
+	if (int rc = check_batch(grid, "n2_grid_forward", d_xyz, point_stride, dim_stride, n_points)) return rc;
+	if (n_points == 0) return N2_OK;
+	N2_REQUIRE(d_out != nullptr, "n2_grid_forward: d_out is null");
+	const uint32_t tiles = n_tiles(n_points);
+	const dim3 grid_dim(tiles * grid->tab.n_levels), block(GRID_BLOCK);
+	if (d_dy_dx) {
+		grid_forward_kernel<true><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride,
+			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), d_dy_dx);
+	} else {
+		grid_forward_kernel<false><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride,
+			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), nullptr);
+	}
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API int n2_grid_corner_indices(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                                  uint32_t dim_stride, uint32_t n_points, uint32_t* d_indices) {
+	if (int rc = check_batch(grid, "n2_grid_corner_indices", d_xyz, point_stride, dim_stride, n_points)) return rc;
+	if (n_points == 0) return N2_OK;
+	N2_REQUIRE(d_indices != nullptr, "n2_grid_corner_indices: d_indices is null");
+	const uint32_t tiles = n_tiles(n_points);
+	grid_indices_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, n2_stream(stream)>>>(
+		grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, d_indices);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2_grad_mode mode) {
+	N2_REQUIRE(mode == N2_GRAD_IGNORE || mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "%s: bad gradient mode %d", fn, (int)mode);
+	if (mode == N2_GRAD_IGNORE) return N2_OK;
+	N2_REQUIRE(grid->grads != nullptr, "%s: gradient mode %d needs a gradient buffer (n2_grid_set_params)", fn, (int)mode);
+	if (mode == N2_GRAD_OVERWRITE) return n2_fill_zero_u32(stream, grid->grads, (size_t)grid->n_params * sizeof(__half));
+	return N2_OK;
+}
+
+N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                            uint32_t dim_stride, uint32_t n_points, const n2_half* d_dL_dy, const float* d_dy_dx,
+                            float* d_dL_dx, n2_grad_mode mode) {
+	if (int rc = check_batch(grid, "n2_grid_backward", d_xyz, point_stride, dim_stride, n_points)) return rc;
+	N2_REQUIRE(d_dL_dy != nullptr || n_points == 0, "n2_grid_backward: d_dL_dy is null");
+	N2_REQUIRE(d_dL_dx == nullptr || d_dy_dx != nullptr, "n2_grid_backward: d_dL_dx needs the d_dy_dx context of the forward");
+	hipStream_t s = n2_stream(stream);
+	if (int rc = prepare_grads(grid, "n2_grid_backward", s, mode)) return rc;
+	if (n_points == 0) return N2_OK;
+	const uint32_t tiles = n_tiles(n_points);
+	if (mode != N2_GRAD_IGNORE) {
+		grid_backward_params_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
+			grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, reinterpret_cast<const __half*>(d_dL_dy), grid->grads);
+		N2_LAUNCH_CHECK();
+	}
+	if (d_dL_dx) {
+		grid_backward_input_kernel<<<dim3(tiles), dim3(GRID_BLOCK), 0, s>>>(
+			n_points, grid->tab.n_levels * grid->n_features, reinterpret_cast<const __half*>(d_dL_dy), d_dy_dx, d_dL_dx);
+		N2_LAUNCH_CHECK();
+	}
+	return N2_OK;
+}
+
+N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz,
+                                           uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
+                                           const float* d_dL_ddLdx, const n2_half* d_dL_dy, n2_half* d_dL_ddLdy,
+                                           float* d_dL_dx, n2_grad_mode mode) {
+	if (int rc = check_batch(grid, "n2_grid_backward_backward_input", d_xyz, point_stride, dim_stride, n_points)) return rc;
+	N2_REQUIRE((d_dL_ddLdx != nullptr && d_dL_dy != nullptr) || n_points == 0, "n2_grid_backward_backward_input: d_dL_ddLdx and d_dL_dy are required");
+	hipStream_t s = n2_stream(stream);
+	if (int rc = prepare_grads(grid, "n2_grid_backward_backward_input", s, mode)) return rc;
+	if (n_points == 0) return N2_OK;
+	if (mode == N2_GRAD_IGNORE && !d_dL_ddLdy && !d_dL_dx) return N2_OK;
+	if (d_dL_dx) {
+		if (int rc = n2_fill_zero_u32(s, d_dL_dx, sizeof(float) * 3 * (size_t)n_points)) return rc;
+	}
+	const uint32_t tiles = n_tiles(n_points);
+	grid_bbi_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
+		grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, d_dL_ddLdx, reinterpret_cast<const __half*>(d_dL_dy),
+		grid->params, mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy), d_dL_dx);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

@@ -1,0 +1,59 @@
+// Internal helpers shared by the HIP sources of libneus2_amd (not installed).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "neus2_amd.h"
+
+#define N2_API extern "C" __attribute__((visibility("default")))
+
+void n2_set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define N2_REQUIRE(cond, ...)                      \
+	do {                                           \
+		if (!(cond)) {                             \
+			n2_set_error(__VA_ARGS__);             \
+			return N2_ERR_INVALID_ARGUMENT;        \
+		}                                          \
+	} while (0)
+
+#define N2_HIP(call)                                                                         \
+	do {                                                                                     \
+		hipError_t e_ = (call);                                                              \
+		if (e_ != hipSuccess) {                                                              \
+			n2_set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+			return N2_ERR_HIP;                                                               \
+		}                                                                                    \
+	} while (0)
+
+// After a kernel launch: launch-configuration errors surface here.
+#define N2_LAUNCH_CHECK() N2_HIP(hipGetLastError())
+
+constexpr uint32_t N2_MAX_LEVELS = 32;
+
+// How a level turns integer grid coordinates into an entry index.
+enum : uint32_t {
+	N2_LEVEL_DENSE = 0,  // x + y*res + z*res^2, one conditional subtract stands in for the modulo
+	N2_LEVEL_HASH = 1,   // spatial hash, entries is a power of two -> mask
+	N2_LEVEL_DENSE_MOD = 2,  // dense index with a true modulo (tables too small for the subtract trick)
+	N2_LEVEL_HASH_MOD = 3    // spatial hash with a true modulo
+};
+
+// Host-computed per-level constants, passed to kernels by value so that host
+// and device can never disagree on exp2f/ceilf rounding.
+struct N2LevelTable {
+	float scale[N2_MAX_LEVELS];
+	uint32_t resolution[N2_MAX_LEVELS];
+	uint32_t entries[N2_MAX_LEVELS];
+	uint32_t offset[N2_MAX_LEVELS + 1];
+	uint32_t mode[N2_MAX_LEVELS];
+	uint32_t n_levels;
+};
+
+static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Zero-fill with a kernel (safe to record into HIP graphs, unlike memset nodes).
+int n2_fill_zero_u32(hipStream_t stream, void* d_ptr, size_t n_bytes);

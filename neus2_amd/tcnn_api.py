@@ -1,0 +1,120 @@
+"""Python mirror of the reference's tcnn-style objects on top of the C ABI.
+
+torch is used for device memory and streams only; every computation is a call
+into libneus2_amd.so.  Method names and argument meaning follow the interface
+the reference drives (``tcnn::Encoding`` / ``tcnn::Network``; call sites in
+include/neural-graphics-primitives/nerf_network.h).
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE, N2Error, check, ptr  # noqa: F401
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _positions(xyz):
+    """Accepts a 3 x N SoA float32 tensor or an N x C (C >= 3) row-per-point tensor
+    (the 7-float NerfCoordinate batch, nerf.h:76-102).  Returns (tensor, point_stride, dim_stride, N)."""
+    if xyz.dtype != torch.float32 or not xyz.is_cuda:
+        raise N2Error("positions must be a float32 CUDA tensor")
+    if not xyz.is_contiguous():
+        raise N2Error("positions must be contiguous")
+    if xyz.dim() == 2 and xyz.shape[0] == 3:
+        return xyz, 1, xyz.shape[1], xyz.shape[1]
+    if xyz.dim() == 2 and xyz.shape[1] >= 3:
+        return xyz, xyz.shape[1], 1, xyz.shape[0]
+    raise N2Error(f"positions must be 3 x N or N x C, got {tuple(xyz.shape)}")
+
+
+class GridEncoding:
+    """tcnn::GridEncoding<__half, 3, 2> (created at nerf_network.h:46)."""
+
+    def __init__(self, n_levels=16, n_features_per_level=2, log2_hashmap_size=19, base_resolution=16,
+                 per_level_scale=1.447):
+        self._h = C.c_void_p()
+        check(capi.lib().n2_grid_create(C.c_uint32(n_levels), C.c_uint32(n_features_per_level),
+                                        C.c_uint32(log2_hashmap_size), C.c_uint32(base_resolution),
+                                        C.c_float(per_level_scale), C.byref(self._h)), "n2_grid_create")
+        self.n_levels = n_levels
+        self._params = self._grads = None
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) is not None and self._h.value:
+                capi.lib().n2_grid_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:  # interpreter shutdown: the module globals may already be gone
+            pass
+
+    def n_params(self):
+        return int(capi.lib().n2_grid_n_params(self._h))
+
+    def output_width(self):
+        return int(capi.lib().n2_grid_output_width(self._h))
+
+    padded_output_width = output_width
+
+    def input_width(self):
+        return 3
+
+    def level_table(self):
+        L = self.n_levels
+        scale = np.zeros(L, np.float32)
+        res, ent, off = np.zeros(L, np.uint32), np.zeros(L, np.uint32), np.zeros(L + 1, np.uint32)
+        check(capi.lib().n2_grid_level_table(self._h, ptr(scale), ptr(res), ptr(ent), ptr(off)), "n2_grid_level_table")
+        return scale, res, ent, off
+
+    def set_params(self, params, gradients=None):
+        """params / gradients: fp16 CUDA tensors of n_params elements (kept alive by this object)."""
+        for t in (params, gradients):
+            if t is not None and (t.dtype != torch.float16 or not t.is_cuda or t.numel() != self.n_params()
+                                  or not t.is_contiguous()):
+                raise N2Error("grid params/gradients must be contiguous fp16 CUDA tensors of n_params elements")
+        check(capi.lib().n2_grid_set_params(self._h, ptr(params), ptr(gradients)), "n2_grid_set_params")
+        self._params, self._grads = params, gradients
+
+    def forward(self, xyz, prepare_input_gradients=False):
+        """Returns (out fp16 [width, N], ctx) where ctx holds dy_dx when requested."""
+        x, ps, ds, n = _positions(xyz)
+        out = torch.empty((self.output_width(), n), dtype=torch.float16, device=x.device)
+        dy_dx = torch.empty((self.output_width(), n, 3), dtype=torch.float32, device=x.device) \
+            if prepare_input_gradients else None
+        check(capi.lib().n2_grid_forward(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds), C.c_uint32(n),
+                                         ptr(out), ptr(dy_dx)), "n2_grid_forward")
+        return out, dy_dx
+
+    def backward(self, ctx, xyz, dL_dy, want_input_grad=False, mode=GRAD_OVERWRITE):
+        x, ps, ds, n = _positions(xyz)
+        if dL_dy.dtype != torch.float16 or tuple(dL_dy.shape) != (self.output_width(), n) or not dL_dy.is_contiguous():
+            raise N2Error("dL_dy must be a contiguous fp16 [output_width, N] tensor")
+        dx = torch.empty((3, n), dtype=torch.float32, device=x.device) if want_input_grad else None
+        check(capi.lib().n2_grid_backward(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds), C.c_uint32(n),
+                                          ptr(dL_dy), ptr(ctx), ptr(dx), C.c_int(mode)), "n2_grid_backward")
+        return dx
+
+    def backward_backward_input(self, xyz, dL_ddLdx, dL_dy, want_dL_ddLdy=True, want_dL_dx=False,
+                                mode=GRAD_ACCUMULATE):
+        x, ps, ds, n = _positions(xyz)
+        if dL_ddLdx.dtype != torch.float32 or tuple(dL_ddLdx.shape) != (3, n) or not dL_ddLdx.is_contiguous():
+            raise N2Error("dL_ddLdx must be a contiguous fp32 [3, N] tensor")
+        if dL_dy.dtype != torch.float16 or tuple(dL_dy.shape) != (self.output_width(), n) or not dL_dy.is_contiguous():
+            raise N2Error("dL_dy must be a contiguous fp16 [output_width, N] tensor")
+        o = torch.empty((self.output_width(), n), dtype=torch.float16, device=x.device) if want_dL_ddLdy else None
+        dx = torch.empty((3, n), dtype=torch.float32, device=x.device) if want_dL_dx else None
+        check(capi.lib().n2_grid_backward_backward_input(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds),
+                                                         C.c_uint32(n), ptr(dL_ddLdx), ptr(dL_dy), ptr(o), ptr(dx),
+                                                         C.c_int(mode)), "n2_grid_backward_backward_input")
+        return o, dx
+
+    def corner_indices(self, xyz):
+        x, ps, ds, n = _positions(xyz)
+        idx = torch.empty((self.n_levels, 8, n), dtype=torch.int32, device=x.device)
+        check(capi.lib().n2_grid_corner_indices(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds),
+                                                C.c_uint32(n), ptr(idx)), "n2_grid_corner_indices")
+        return idx

@@ -1,0 +1,193 @@
+"""GPU parity of the hash-grid kernels against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import RTOL, assert_close, dev, host, q16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(n_levels=16, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447)
+
+
+@pytest.fixture(scope="module")
+def setup(oracle):
+    from neus2_amd.tcnn_api import GridEncoding
+    og = oracle.Grid(CFG["n_levels"], CFG["log2_hashmap_size"], CFG["base_resolution"], CFG["per_level_scale"])
+    gg = GridEncoding(**CFG)
+    assert gg.n_params() == og.n_params
+    rng = np.random.default_rng(0)
+    params = q16(rng.uniform(-1, 1, og.n_params))
+    d_params = dev(params, torch.float16)
+    d_grads = torch.zeros_like(d_params)
+    gg.set_params(d_params, d_grads)
+    return og, gg, params, d_params, d_grads
+
+
+def test_config1_indices_bit_exact(setup):
+    """BASELINE config 1: 2^14 points U[0,1)^3, seed 0: every corner index of every level identical."""
+    og, gg, *_ = setup
+    xyz = np.random.default_rng(0).random((3, 1 << 14), dtype=np.float32)
+    ref, _ = og.indices(xyz)
+    got = host(gg.corner_indices(dev(xyz))).view(np.uint32)
+    assert np.array_equal(got, ref)
+
+
+def test_indices_bit_exact_edge_positions(setup):
+    og, gg, *_ = setup
+    edge = np.array([0.0, 1.0, np.nextafter(np.float32(1), np.float32(0)), 0.5, 1e-8, 0.25, 0.999999, 1.0 / 3], np.float32)
+    xyz = np.stack(np.meshgrid(edge, edge, edge, indexing="ij")).reshape(3, -1).astype(np.float32)
+    # plus vertices of several levels, where floor() sits on a knife edge
+    extra = [((np.arange(40, dtype=np.float32) - 0.5) / s) for s in og.scale[[0, 3, 9, 15]]]
+    e = np.clip(np.concatenate(extra), 0, 1).astype(np.float32)
+    xyz = np.concatenate([xyz, np.stack([e, e[::-1], e])], axis=1)
+    ref, _ = og.indices(xyz)
+    got = host(gg.corner_indices(dev(xyz))).view(np.uint32)
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 5000])
+def test_forward_values_and_ragged_sizes(setup, n):
+    og, gg, params, *_ = setup
+    xyz = np.random.default_rng(n).random((3, n), dtype=np.float32)
+    ref, ref_j = og.forward(params, xyz, want_dy_dx=True)
+    out, dy_dx = gg.forward(dev(xyz), prepare_input_gradients=True)
+    assert_close(host(out), ref, what="grid forward")
+    # dy_dx is fp32 on both sides; differences of fp16 table values times scale
+    assert_close(host(dy_dx), ref_j, rtol=1e-4, what="dy_dx")
+    out2, none = gg.forward(dev(xyz))
+    # the two instantiations may round a tie differently: at most one fp16 ulp apart
+    assert none is None
+    assert_close(host(out2), host(out), rtol=1e-3, what="forward without dy_dx")
+
+
+def test_forward_accepts_nerf_coordinate_rows(setup):
+    """7 floats per point (xyz, dt, dir), the column-major batch the reference feeds (nerf.h:76-102)."""
+    og, gg, params, *_ = setup
+    n = 3000
+    rng = np.random.default_rng(7)
+    coords = rng.random((n, 7), dtype=np.float32)
+    out_rows, _ = gg.forward(dev(coords))
+    out_soa, _ = gg.forward(dev(np.ascontiguousarray(coords[:, :3].T)))
+    assert torch.equal(out_rows, out_soa)
+
+
+def test_forward_empty_batch(setup):
+    _, gg, *_ = setup
+    out, _ = gg.forward(torch.zeros((3, 0), dtype=torch.float32, device="cuda"))
+    assert out.shape == (32, 0)
+
+
+def test_forward_small_uniform_params_config1(setup, oracle):
+    """Config 1's parameter distribution U(-1e-4, 1e-4), seed 0."""
+    og, gg, _, d_params, d_grads = setup
+    rng = np.random.default_rng(0)
+    p = q16(rng.uniform(-1e-4, 1e-4, og.n_params))
+    from neus2_amd.tcnn_api import GridEncoding
+    g2 = GridEncoding(**CFG)
+    dp = dev(p, torch.float16)
+    g2.set_params(dp, None)
+    xyz = rng.random((3, 1 << 14), dtype=np.float32)
+    out, _ = g2.forward(dev(xyz))
+    # fp16 subnormal spacing (6e-8) dominates at this magnitude: absolute floor of one subnormal ulp
+    ref = og.forward(p, xyz)
+    assert np.abs(host(out) - ref).max() <= 6e-8 + RTOL * np.abs(ref).max()
+
+
+def test_backward_param_scatter_and_input_grad(setup):
+    og, gg, params, d_params, d_grads = setup
+    n = 1 << 14
+    rng = np.random.default_rng(11)
+    xyz = rng.random((3, n), dtype=np.float32)
+    dy = q16(rng.standard_normal((32, n)))
+    ref_grad, ref_dx = og.backward(params, xyz, dy)
+    d_xyz = dev(xyz)
+    _, ctx = gg.forward(d_xyz, prepare_input_gradients=True)
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE
+    d_grads.fill_(7.0)  # Overwrite must discard this
+    dx = gg.backward(ctx, d_xyz, dev(dy, torch.float16), want_input_grad=True, mode=GRAD_OVERWRITE)
+    got = host(d_grads)
+    assert_close(host(dx), ref_dx, rtol=1e-4, what="dL_dx")
+    # fp16 atomics round after every addition: the error of an entry that received
+    # k contributions grows like sqrt(k) half-ulps, so coarse levels get a wider band
+    for l in range(16):
+        a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+        k = 8.0 * n / max(1, int(og.entries[l]))
+        tol = RTOL * max(1.0, np.sqrt(k))
+        assert rel_l2(got[a:b], ref_grad[a:b]) < tol, (l, rel_l2(got[a:b], ref_grad[a:b]), tol)
+    # Accumulate adds a second copy; Ignore leaves the buffer alone
+    gg.backward(ctx, d_xyz, dev(dy, torch.float16), mode=GRAD_ACCUMULATE)
+    got2 = host(d_grads)
+    assert rel_l2(got2, 2 * ref_grad) < 2e-2
+    before = d_grads.clone()
+    dx2 = gg.backward(ctx, d_xyz, dev(dy, torch.float16), want_input_grad=True, mode=GRAD_IGNORE)
+    assert torch.equal(before, d_grads) and torch.equal(dx, dx2)
+
+
+def test_backward_backward_input(setup):
+    og, gg, params, d_params, d_grads = setup
+    n = 1 << 13
+    rng = np.random.default_rng(13)
+    xyz = rng.random((3, n), dtype=np.float32)
+    g = q16(rng.standard_normal((32, n)) * 0.1)
+    v = (rng.standard_normal((3, n)) * 1e-3).astype(np.float32)
+    ref_grad, ref_out, ref_din = og.backward_backward_input(params, xyz, v, g)
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE
+    d_xyz, d_v, d_g = dev(xyz), dev(v), dev(g, torch.float16)
+    out, din = gg.backward_backward_input(d_xyz, d_v, d_g, want_dL_ddLdy=True, want_dL_dx=True, mode=GRAD_OVERWRITE)
+    assert_close(host(out), ref_out, what="dL_ddLdy")
+    assert_close(host(din), ref_din, rtol=1e-3, what="second-order dL_dx")
+    got = host(d_grads)
+    for l in range(16):
+        a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+        k = 8.0 * n / max(1, int(og.entries[l]))
+        tol = RTOL * max(1.0, np.sqrt(k))
+        assert rel_l2(got[a:b], ref_grad[a:b]) < tol, (l, rel_l2(got[a:b], ref_grad[a:b]), tol)
+    # the reference's call: Accumulate on top of the first-order gradients, outputs optional
+    base = q16(rng.standard_normal(og.n_params) * 1e-3)
+    d_grads.copy_(dev(base, torch.float16))
+    out2, none = gg.backward_backward_input(d_xyz, d_v, d_g, want_dL_ddLdy=True, want_dL_dx=False, mode=GRAD_ACCUMULATE)
+    assert none is None and torch.equal(out, out2)
+    assert rel_l2(host(d_grads), base + ref_grad) < 1e-2
+    before = d_grads.clone()
+    gg.backward_backward_input(d_xyz, d_v, d_g, mode=GRAD_IGNORE)
+    assert torch.equal(before, d_grads)
+
+
+@pytest.mark.parametrize("cfg", [(6, 12, 4, 1.6), (5, 4, 2, 1.5), (8, 14, 4, 2.0), (14, 19, 16, 1.4472692012786865)])
+def test_other_table_shapes(oracle, cfg):
+    """Small tables exercise the true-modulo index paths; 14 levels is the reference's shipped config."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding
+    og = oracle.Grid(*cfg)
+    gg = GridEncoding(n_levels=cfg[0], log2_hashmap_size=cfg[1], base_resolution=cfg[2], per_level_scale=cfg[3])
+    rng = np.random.default_rng(17)
+    params = q16(rng.uniform(-1, 1, og.n_params))
+    dp = dev(params, torch.float16)
+    dg = torch.zeros_like(dp)
+    gg.set_params(dp, dg)
+    n = 2049
+    xyz = rng.random((3, n), dtype=np.float32)
+    ref_idx, _ = og.indices(xyz)
+    assert np.array_equal(host(gg.corner_indices(dev(xyz))).view(np.uint32), ref_idx)
+    out, ctx = gg.forward(dev(xyz), prepare_input_gradients=True)
+    assert_close(host(out), og.forward(params, xyz), what="forward")
+    dy = q16(rng.standard_normal((og.n_out, n)))
+    ref_grad, ref_dx = og.backward(params, xyz, dy)
+    dx = gg.backward(ctx, dev(xyz), dev(dy, torch.float16), want_input_grad=True, mode=GRAD_OVERWRITE)
+    assert_close(host(dx), ref_dx, rtol=1e-4, what="dL_dx")
+    assert rel_l2(host(dg), ref_grad) < 2e-2
+
+
+def test_errors_are_reported_not_launched():
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding, N2Error
+    gg = GridEncoding(**CFG)
+    x = torch.rand((3, 16), device="cuda")
+    with pytest.raises(N2Error, match="set_params"):
+        gg.forward(x)
+    p = torch.zeros(gg.n_params(), dtype=torch.float16, device="cuda")
+    gg.set_params(p, None)
+    out, ctx = gg.forward(x, prepare_input_gradients=True)
+    with pytest.raises(N2Error, match="gradient buffer"):
+        gg.backward(ctx, x, torch.zeros((32, 16), dtype=torch.float16, device="cuda"), mode=GRAD_OVERWRITE)
+    with pytest.raises(N2Error):
+        gg.forward(x.double())
