@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_PKG, "libneus2_amd.so")
 
 N2_OK = 0
 GRAD_IGNORE, GRAD_OVERWRITE, GRAD_ACCUMULATE = 0, 1, 2
+LAYOUT_SOA, LAYOUT_AOS = 0, 1
 
 _lib = None
 
@@ -33,6 +34,13 @@ def lib():
             getattr(_lib, name).argtypes = [C.c_void_p]
         _lib.n2_grid_destroy.restype = None
         _lib.n2_grid_destroy.argtypes = [C.c_void_p]
+        for name in ("n2_mlp_n_params", "n2_mlp_input_width", "n2_mlp_output_width"):
+            getattr(_lib, name).restype = C.c_uint32
+            getattr(_lib, name).argtypes = [C.c_void_p]
+        _lib.n2_mlp_workspace_bytes.restype = C.c_uint64
+        _lib.n2_mlp_workspace_bytes.argtypes = [C.c_void_p]
+        _lib.n2_mlp_destroy.restype = None
+        _lib.n2_mlp_destroy.argtypes = [C.c_void_p]
     return _lib
 
 

@@ -11,7 +11,8 @@ import numpy as np
 import torch
 
 from . import capi
-from .capi import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE, N2Error, check, ptr  # noqa: F401
+from .capi import (GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE, LAYOUT_AOS, LAYOUT_SOA, N2Error, check,  # noqa: F401
+                   ptr)
 
 
 def _stream():
@@ -118,3 +119,88 @@ class GridEncoding:
         check(capi.lib().n2_grid_corner_indices(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds),
                                                 C.c_uint32(n), ptr(idx)), "n2_grid_corner_indices")
         return idx
+
+
+def _check_half(t, shape, what):
+    if t.dtype != torch.float16 or not t.is_cuda or not t.is_contiguous() or tuple(t.shape) != tuple(shape):
+        raise N2Error(f"{what} must be a contiguous fp16 CUDA tensor of shape {tuple(shape)}, got {t.dtype} {tuple(t.shape)}")
+
+
+class FullyFusedMLP:
+    """tcnn::FullyFusedMLP<__half, 64>: ReLU hidden layers, linear 16-wide output, no bias
+    (created at nerf_network.h:57 and :65)."""
+
+    def __init__(self, n_input_dims, n_hidden_layers, n_neurons=64, n_output_dims=16):
+        if n_neurons != 64 or n_output_dims != 16:
+            raise N2Error("only n_neurons = 64 and n_output_dims = 16 are implemented")
+        self._h = C.c_void_p()
+        check(capi.lib().n2_mlp_create(C.c_uint32(n_input_dims), C.c_uint32(n_hidden_layers), C.byref(self._h)),
+              "n2_mlp_create")
+        self.n_hidden_layers = n_hidden_layers
+        self._params = self._grads = self._ws = None
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) is not None and self._h.value:
+                capi.lib().n2_mlp_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+    def n_params(self):
+        return int(capi.lib().n2_mlp_n_params(self._h))
+
+    def input_width(self):
+        return int(capi.lib().n2_mlp_input_width(self._h))
+
+    def padded_output_width(self):
+        return int(capi.lib().n2_mlp_output_width(self._h))
+
+    output_width = padded_output_width
+
+    def set_params(self, params, gradients=None):
+        for t in (params, gradients):
+            if t is not None:
+                _check_half(t, (self.n_params(),), "mlp params/gradients")
+        check(capi.lib().n2_mlp_set_params(self._h, ptr(params), ptr(gradients)), "n2_mlp_set_params")
+        self._params, self._grads = params, gradients
+        if gradients is not None and self._ws is None:
+            nbytes = int(capi.lib().n2_mlp_workspace_bytes(self._h))
+            self._ws = torch.empty(nbytes, dtype=torch.uint8, device=params.device)
+            check(capi.lib().n2_mlp_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes)), "n2_mlp_set_workspace")
+
+    def _out(self, n, layout, device):
+        shape = (n, 16) if layout == LAYOUT_AOS else (16, n)
+        return torch.empty(shape, dtype=torch.float16, device=device)
+
+    def forward(self, x, out_layout=LAYOUT_SOA, want_hidden=False, out=None):
+        """x: fp16 [in_width, N].  Returns (y, hidden): y is [16, N] (SoA) or [N, 16] (AoS)."""
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        y = self._out(n, out_layout, x.device) if out is None else out
+        hid = torch.empty((64 * self.n_hidden_layers, n), dtype=torch.float16, device=x.device) if want_hidden else None
+        check(capi.lib().n2_mlp_forward(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(y), C.c_int(out_layout),
+                                        ptr(hid)), "n2_mlp_forward")
+        return y, hid
+
+    inference_mixed_precision = forward
+
+    def backward(self, x, dL_dy, dL_layout=LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE):
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        _check_half(dL_dy, (n, 16) if dL_layout == LAYOUT_AOS else (16, n), "dL_doutput")
+        dx = torch.empty((self.input_width(), n), dtype=torch.float16, device=x.device) if want_input_grad else None
+        check(capi.lib().n2_mlp_backward(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(dL_dy), C.c_int(dL_layout),
+                                         ptr(dx), C.c_int(mode)), "n2_mlp_backward")
+        return dx
+
+    def backward_backward_input(self, x, dL_ddLdinput, dL_doutput, want_dL_ddLdoutput=False, mode=GRAD_ACCUMULATE):
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        _check_half(dL_ddLdinput, (self.input_width(), n), "dL_ddLdinput")
+        _check_half(dL_doutput, (16, n), "dL_doutput")
+        o = torch.empty((16, n), dtype=torch.float16, device=x.device) if want_dL_ddLdoutput else None
+        check(capi.lib().n2_mlp_backward_backward_input(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(dL_ddLdinput),
+                                                        ptr(dL_doutput), ptr(o), C.c_int(mode)),
+              "n2_mlp_backward_backward_input")
+        return o

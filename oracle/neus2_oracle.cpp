@@ -298,13 +298,48 @@ static inline size_t mlp_layer_off(const MlpDesc& m, uint32_t k) {
 	return off;
 }
 
+// Round an fp32 value to the nearest fp16 (ties to even) and back: the storage
+// precision of activations between layers in the reference (T = __half).
+static inline float round_fp16(float f) {
+	uint32_t x;
+	std::memcpy(&x, &f, 4);
+	const uint32_t sign = x & 0x80000000u;
+	x &= 0x7FFFFFFFu;
+	float out;
+	if (x >= 0x7F800000u) {  // inf / nan
+		out = f;
+		return out;
+	}
+	if (x >= 0x477FF000u) {  // rounds to >= 65520 -> inf
+		x = 0x7F800000u;
+	} else if (x < 0x38800000u) {  // below the smallest normal half: fixed-point rounding to multiples of 2^-24
+		float a;
+		std::memcpy(&a, &x, 4);
+		const float magic = 0.5f;  // adding 0.5 aligns the mantissa so that the ulp is 2^-24
+		a = (a + magic) - magic;
+		std::memcpy(&x, &a, 4);
+	} else {
+		const uint32_t lsb = (x >> 13) & 1u;
+		x += 0xFFFu + lsb;
+		x &= ~0x1FFFu;
+	}
+	x |= sign;
+	std::memcpy(&out, &x, 4);
+	return out;
+}
+ORC_API void orc_round_fp16(const float* in, float* out, uint32_t n) {
+	for (uint32_t i = 0; i < n; ++i) out[i] = round_fp16(in[i]);
+}
+
 ORC_API uint32_t orc_mlp_n_params(uint32_t in_w, uint32_t width, uint32_t n_hidden, uint32_t out_w) {
 	return width * in_w + (n_hidden - 1) * width * width + out_w * width;
 }
 
 // y = W_H relu(... relu(W_0 x)); hidden may be null (inference).
+// round_hidden != 0 rounds every hidden activation to fp16 before it feeds the
+// next layer, as the reference's fp16 activation storage does.
 ORC_API void orc_mlp_forward(uint32_t in_w, uint32_t width, uint32_t n_hidden, uint32_t out_w, const float* W,
-                             const float* x, uint32_t N, float* y, float* hidden) {
+                             const float* x, uint32_t N, float* y, float* hidden, int round_hidden) {
 	const MlpDesc m{in_w, width, n_hidden, out_w};
 	#pragma omp parallel
 	{
@@ -319,6 +354,7 @@ ORC_API void orc_mlp_forward(uint32_t in_w, uint32_t width, uint32_t n_hidden, u
 					float s = 0.f;
 					for (uint32_t c = 0; c < cols; ++c) s += Wk[(size_t)r * cols + c] * a[c];
 					b[r] = (k < n_hidden) ? std::max(s, 0.f) : s;
+					if (k < n_hidden && round_hidden) b[r] = round_fp16(b[r]);
 				}
 				if (k < n_hidden) {
 					if (hidden) for (uint32_t r = 0; r < rows; ++r) hidden[((size_t)k * width + r) * N + i] = b[r];

@@ -136,12 +136,13 @@ class Mlp:
             o += r * c
         return out
 
-    def forward(self, W, x):
+    def forward(self, W, x, round_hidden=False):
+        """round_hidden: keep hidden activations at fp16 precision between layers (reference storage type)."""
         W, x = _f32(W), _f32(x)
         n = x.shape[1]
         y = np.zeros((self.out_w, n), np.float32)
         h = np.zeros((self.n_hidden, self.width, n), np.float32)
-        lib().orc_mlp_forward(*self._d(), _fp(W), _fp(x), C.c_uint32(n), _fp(y), _fp(h))
+        lib().orc_mlp_forward(*self._d(), _fp(W), _fp(x), C.c_uint32(n), _fp(y), _fp(h), C.c_int(int(round_hidden)))
         return y, h
 
     def backward(self, W, x, hidden, dL_dy, want_dx=True, want_dW=True):
@@ -161,6 +162,13 @@ class Mlp:
         lib().orc_mlp_backward_backward_input(*self._d(), _fp(W), _fp(hidden), _fp(v), _fp(g), C.c_uint32(n),
                                               _fp(dW), _fp(out))
         return dW, out
+
+
+def round_fp16(a):
+    a = _f32(a)
+    out = np.empty_like(a)
+    lib().orc_round_fp16(_fp(a), _fp(out), C.c_uint32(a.size))
+    return out
 
 
 def sh4(dirs):

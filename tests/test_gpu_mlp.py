@@ -1,0 +1,147 @@
+"""GPU parity of the fully fused MLP kernels against the CPU oracle, through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import RTOL, assert_close, assert_grad_close, dev, host, q16, rel_l2
+
+pytestmark = pytest.mark.gpu
+# A hidden pre-activation within fp32 summation-order error of zero can land on
+# either side of the ReLU; allow that for at most one entry in 10^4.
+FLIP = 1e-4
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def make(oracle, in_w, n_hidden, seed, scale=0.3):
+    from neus2_amd.tcnn_api import FullyFusedMLP
+    om = oracle.Mlp(in_w, 64, n_hidden, 16)
+    gm = FullyFusedMLP(in_w, n_hidden)
+    assert gm.n_params() == om.n_params
+    rng = np.random.default_rng(seed)
+    W = q16(rng.standard_normal(om.n_params) * scale)
+    dW = dev(W, torch.float16)
+    dG = torch.zeros_like(dW)
+    gm.set_params(dW, dG)
+    return om, gm, W, dW, dG, rng
+
+
+SHAPES = [(48, 1), (48, 2), (32, 1), (16, 1), (64, 2), (64, 1), (32, 2), (16, 2)]
+
+
+@pytest.mark.parametrize("in_w,n_hidden", SHAPES)
+@pytest.mark.parametrize("n", [8, 64, 200, 4096 + 72])
+def test_forward(oracle, in_w, n_hidden, n):
+    from neus2_amd.tcnn_api import LAYOUT_AOS, LAYOUT_SOA
+    om, gm, W, *_ , rng = make(oracle, in_w, n_hidden, 1)
+    x = q16(rng.standard_normal((in_w, n)))
+    ref_y, ref_h = om.forward(W, x, round_hidden=True)
+    y, hid = gm.forward(dev(x, torch.float16), LAYOUT_SOA, want_hidden=True)
+    assert_close(host(y), ref_y, what="mlp forward SoA", outlier_frac=FLIP)
+    assert_close(host(hid), ref_h.reshape(-1, n), what="hidden activations", outlier_frac=FLIP)
+    y2, _ = gm.forward(dev(x, torch.float16), LAYOUT_AOS)
+    assert torch.equal(y2.t().contiguous(), y)
+
+
+@pytest.mark.parametrize("in_w,n_hidden", SHAPES)
+def test_backward_all_modes(oracle, in_w, n_hidden):
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE, LAYOUT_AOS, LAYOUT_SOA
+    om, gm, W, dW, dG, rng = make(oracle, in_w, n_hidden, 2)
+    n = 10000
+    x = q16(rng.standard_normal((in_w, n)))
+    dy = q16(rng.standard_normal((16, n)))
+    _, h = om.forward(W, x, round_hidden=True)
+    ref_dx, ref_dW = om.backward(W, x, h, dy)
+    dx_, ddy = dev(x, torch.float16), dev(dy, torch.float16)
+    dG.fill_(3.0)
+    dx = gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE)
+    assert_close(host(dx), ref_dx, what="dL_dinput", outlier_frac=FLIP)
+    # fp32 accumulation over the batch, one rounding to fp16 at the end
+    assert_grad_close(host(dG), ref_dW, what="weight gradients")
+    # AoS gradient layout gives the same result
+    dG.zero_()
+    dx2 = gm.backward(dx_, ddy.t().contiguous(), LAYOUT_AOS, want_input_grad=True, mode=GRAD_OVERWRITE)
+    assert torch.equal(dx, dx2)
+    assert_grad_close(host(dG), ref_dW, what="weight gradients (AoS dL_dy)")
+    # Ignore: gradient buffer untouched
+    before = dG.clone()
+    dx3 = gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=True, mode=GRAD_IGNORE)
+    assert torch.equal(before, dG) and torch.equal(dx3, dx)
+    # Accumulate, without input gradient
+    none = gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=False, mode=GRAD_ACCUMULATE)
+    assert none is None
+    assert_grad_close(host(dG), 2 * ref_dW, what="accumulated weight gradients")
+
+
+@pytest.mark.parametrize("in_w", [48, 32, 16, 64])
+def test_backward_backward_input(oracle, in_w):
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE
+    om, gm, W, dW, dG, rng = make(oracle, in_w, 1, 3)
+    n = 8192 + 40
+    x = q16(rng.standard_normal((in_w, n)))
+    v = q16(rng.standard_normal((in_w, n)))
+    g = q16(rng.standard_normal((16, n)))
+    _, h = om.forward(W, x, round_hidden=True)
+    ref_dW, ref_out = om.backward_backward_input(W, h, v, g)
+    out = gm.backward_backward_input(dev(x, torch.float16), dev(v, torch.float16), dev(g, torch.float16),
+                                     want_dL_ddLdoutput=True, mode=GRAD_OVERWRITE)
+    assert_close(host(out), ref_out, what="dL_ddLdoutput", outlier_frac=FLIP)
+    assert_grad_close(host(dG), ref_dW, what="second-order weight gradients")
+    # the reference's call: g = e_0, Accumulate on top of first-order gradients, no outputs
+    e0 = np.zeros((16, n), np.float32)
+    e0[0] = 1
+    ref2, _ = om.backward_backward_input(W, h, v, e0)
+    base = q16(rng.standard_normal(om.n_params))
+    dG.copy_(dev(base, torch.float16))
+    none = gm.backward_backward_input(dev(x, torch.float16), dev(v, torch.float16), dev(e0, torch.float16),
+                                      want_dL_ddLdoutput=False, mode=GRAD_ACCUMULATE)
+    assert none is None
+    assert_grad_close(host(dG), base + ref2, what="accumulated second-order gradients")
+    before = dG.clone()
+    gm.backward_backward_input(dev(x, torch.float16), dev(v, torch.float16), dev(e0, torch.float16), mode=GRAD_IGNORE)
+    assert torch.equal(before, dG)
+
+
+def test_geometric_init_sphere_on_gpu(oracle):
+    """The reference's utils/mlp_weights.txt through the GPU path: identical to the oracle's sphere."""
+    from neus2_amd.tcnn_api import GRAD_IGNORE, FullyFusedMLP
+    W = q16(np.load(os.path.join(GOLD, "sdf_mlp_weights_48.npy")))
+    om = oracle.Mlp(48, 64, 1, 16)
+    gm = FullyFusedMLP(48, 1)
+    gm.set_params(dev(W, torch.float16), None)
+    rng = np.random.default_rng(0)
+    n = 1 << 14
+    x = np.zeros((48, n), np.float32)
+    x[:3] = q16(rng.random((3, n)) - 0.5)
+    ref_y, h = om.forward(W, x, round_hidden=True)
+    y, _ = gm.forward(dev(x, torch.float16))
+    assert_close(host(y), ref_y, what="sdf of the geometric init")
+    e0 = np.zeros((16, n), np.float32)
+    e0[0] = 1
+    ref_dx, _ = om.backward(W, x, h, e0, want_dW=False)
+    dx = gm.backward(dev(x, torch.float16), dev(e0, torch.float16), want_input_grad=True, mode=GRAD_IGNORE)
+    assert_close(host(dx), ref_dx, what="normals of the geometric init")
+
+
+def test_mlp_errors(oracle):
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, FullyFusedMLP, N2Error
+    with pytest.raises(N2Error, match="in_width"):
+        FullyFusedMLP(40, 1)
+    with pytest.raises(N2Error, match="n_hidden_layers"):
+        FullyFusedMLP(48, 3)
+    m = FullyFusedMLP(48, 2)
+    x = torch.zeros((48, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(N2Error, match="set_params"):
+        m.forward(x)
+    m.set_params(torch.zeros(m.n_params(), dtype=torch.float16, device="cuda"), None)
+    with pytest.raises(N2Error, match="multiple of 8"):
+        m.forward(torch.zeros((48, 12), dtype=torch.float16, device="cuda"))
+    with pytest.raises(N2Error, match="gradient buffer"):
+        m.backward(x, torch.zeros((16, 64), dtype=torch.float16, device="cuda"), mode=GRAD_OVERWRITE)
+    with pytest.raises(N2Error, match="one hidden layer"):
+        m.set_params(torch.zeros(m.n_params(), dtype=torch.float16, device="cuda"),
+                     torch.zeros(m.n_params(), dtype=torch.float16, device="cuda"))
+        m.backward_backward_input(x, x, torch.zeros((16, 64), dtype=torch.float16, device="cuda"))
+    y, _ = m.forward(torch.zeros((48, 0), dtype=torch.float16, device="cuda"))
+    assert y.shape == (16, 0)

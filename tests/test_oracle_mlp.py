@@ -145,3 +145,22 @@ def test_adam_non_matrix_rules(oracle):
     oracle.adam_step(w, np.full(n, 128, np.float32), m1, m2, steps, n_matrix_params=4)
     assert steps.tolist() == [2, 2, 2, 2, 1, 2, 1, 2]
     np.testing.assert_allclose(1 - w[4], 1e-3, rtol=1e-3)
+
+
+def test_round_fp16_matches_numpy(oracle):
+    rng = np.random.default_rng(9)
+    a = np.concatenate([rng.standard_normal(20000) * 10.0 ** rng.integers(-9, 5, 20000),
+                        [0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 6.1e-5, 6.0e-5, 5.96e-8, 2.9e-8, 3.0e-8,
+                         1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, np.inf, -np.inf]]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        ref = a.astype(np.float16).astype(np.float32)
+    got = oracle.round_fp16(a)
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_mlp_forward_fp16_hidden_option(oracle):
+    m, W, x, _ = _setup(oracle, 48, 64, 2, 16, n=64, seed=5)
+    y0, h0 = m.forward(W, x)
+    y1, h1 = m.forward(W, x, round_hidden=True)
+    np.testing.assert_array_equal(h1[0], h0[0].astype(np.float16).astype(np.float32))
+    assert np.abs(y1 - y0).max() < 2e-2 and not np.array_equal(y1, y0)
