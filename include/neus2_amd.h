@@ -175,16 +175,96 @@ int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, ui
 int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                     const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode);
 
+/* DifferentiableObject::input_gradient(stream, dim, input, d_dinput): gradient of output
+ * row `dim` w.r.t. the input, i.e. backward with dL_doutput = e_dim and no parameter
+ * gradients.  The reference builds e_0 by hand and calls backward with Ignore to get the
+ * SDF normal (nerf_network.h:215-229, 497-512); this entry point reads no dL_doutput.
+ *  d_dinput  fp16 SoA in_width x N */
+int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
+                          n2_half* d_dinput);
+
 /* Network::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
  * dL_ddLdoutput, dL_dinput, use_inference_params, mode): the second-order pass the
  * reference fork adds for the eikonal loss, nerf_network.h:560-571.  One hidden
  * layer only (the SDF net); dL_dinput is identically zero for ReLU and is not produced.
  *  d_dL_ddLdinput  fp16 SoA in_width x N
- *  d_dL_doutput    fp16 SoA 16 x N (the reference passes e_0)
+ *  d_dL_doutput    fp16 SoA 16 x N, or NULL for the constant e_0 (unit gradient on output
+ *                  row 0), the only value the reference passes (nerf_network.h:499-504, 565)
  *  d_dL_ddLdoutput NULL or fp16 SoA 16 x N */
 int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                                    const n2_half* d_dL_ddLdinput, const n2_half* d_dL_doutput,
                                    n2_half* d_dL_ddLdoutput, n2_grad_mode mode);
+
+/* ------------------------------------------------------------------------
+ * The NeuS field: NerfNetwork<__half> (include/neural-graphics-primitives/nerf_network.h),
+ * static scene (delta network off, src/testbed.cu:2695-2697).  Composes the hash grid, the
+ * SDF MLP (3 centred coordinates + encoding, padded to a multiple of 16 -> 64 -> 16), the
+ * degree-4 spherical-harmonics direction encoding, the colour MLP (16 SDF features + 16 SH +
+ * xyz + normal, padded to 48 -> 64 -> 64 -> 16) and the learnable variance scalar.
+ *
+ * One parameter vector in the trainer's order (nerf_network.h:728-772):
+ *   [SDF MLP | colour MLP | grid | variance (4 slots, slot 0 used)]
+ * ---------------------------------------------------------------------- */
+typedef struct n2_field n2_field_t;
+
+typedef struct n2_field_config {
+	uint32_t n_levels;             /* configs/nerf/base.json:31 */
+	uint32_t n_features_per_level; /* 2 */
+	uint32_t log2_hashmap_size;    /* 19 */
+	uint32_t base_resolution;      /* 16 */
+	float per_level_scale;         /* derived from top_resolution at src/testbed.cu:2165-2177 */
+	uint32_t sdf_hidden_layers;    /* 1, base.json:45 */
+	uint32_t rgb_hidden_layers;    /* 2, base.json:68 */
+	float sdf_bias;                /* -0.1, base.json:46, nerf_network.h:74 */
+} n2_field_config;
+
+/* NerfNetwork<T>::NerfNetwork(...), nerf_network.h:40-83 */
+int n2_field_create(const n2_field_config* config, n2_field_t** out);
+void n2_field_destroy(n2_field_t* field);
+
+uint32_t n2_field_n_params(const n2_field_t* field);
+/* Offsets of the five segments [sdf mlp, colour mlp, grid, variance, end] in the parameter
+ * vector; everything before offsets[2] is a matrix parameter for the optimiser
+ * (NerfNetwork::layer_sizes, nerf_network.h:902-990). */
+int n2_field_param_offsets(const n2_field_t* field, uint32_t offsets[5]);
+
+/* NerfNetwork::set_params, nerf_network.h:728-772 (fp16 params and gradients, n_params each). */
+int n2_field_set_params(n2_field_t* field, const n2_half* d_params, n2_half* d_gradients);
+
+/* Scratch the reference takes from tcnn's arena inside forward_impl/backward_impl
+ * (every GPUMatrixDynamic temporary, nerf_network.h:137-267, 332-557): network inputs,
+ * the grid's dy_dx context, input gradients and the MLP weight-gradient slabs. */
+uint64_t n2_field_workspace_bytes(const n2_field_t* field, uint32_t max_batch);
+int n2_field_set_workspace(n2_field_t* field, void* d_workspace, uint64_t n_bytes, uint32_t max_batch);
+
+/* NerfNetwork::forward_impl / inference_mixed_precision_impl (which the reference routes
+ * to forward_impl), nerf_network.h:87-90, 132-315.
+ *  d_coords  fp32, N rows of 7: x y z dt dx dy dz (NerfCoordinate, nerf.h:76-102), positions
+ *            in [0,1]^3, directions warped to [0,1]^3
+ *  d_output  fp16 N x 16 (N2_LAYOUT_AOS): [r g b raw | sdf + bias | normal xyz | variance |
+ *            direction xyz | 5 unused colour-net rows]
+ * The forward context stays in the workspace until the next forward. */
+int n2_field_forward(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, n2_half* d_output);
+
+/* NerfNetwork::backward_impl, nerf_network.h:317-588, for the batch of the last forward.
+ *  d_dL_doutput   fp16 N x 16 (AoS): rows 0..2 colour, 3 sdf, 4..6 eikonal (divided here by
+ *                 ek_batch_size), 7 variance, 8..10 gradient w.r.t. the normal through cos
+ *  ek_batch_size  NerfNetwork::indeed_batch_size (src/testbed_nerf.cu:3927)
+ *  mode           OVERWRITE as the reference calls it; ACCUMULATE adds to existing gradients
+ * Includes the second-order passes through grid and SDF MLP. */
+int n2_field_backward(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n,
+                      const n2_half* d_dL_doutput, uint32_t ek_batch_size, n2_grad_mode mode);
+
+/* NerfNetwork::sdf, nerf_network.h:643-709: encoding + SDF MLP, bias added on row 0.
+ *  d_xyz     positions with the strides of n2_grid_forward
+ *  d_output  fp16 SoA 16 x N */
+int n2_field_sdf(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                 uint32_t dim_stride, uint32_t n, n2_half* d_output);
+
+/* NerfNetwork::density, nerf_network.h:711-726: sdf, then row 0 becomes the logistic density
+ * s*sigmoid(s*sdf)*(1 - sigmoid(s*sdf)) with s = exp(10*variance) (common_operation.cuh:310-328). */
+int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                     uint32_t dim_stride, uint32_t n, n2_half* d_output);
 
 #ifdef __cplusplus
 }

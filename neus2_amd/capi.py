@@ -16,6 +16,13 @@ LAYOUT_SOA, LAYOUT_AOS = 0, 1
 _lib = None
 
 
+class FieldConfig(C.Structure):
+    """struct n2_field_config"""
+    _fields_ = [("n_levels", C.c_uint32), ("n_features_per_level", C.c_uint32), ("log2_hashmap_size", C.c_uint32),
+                ("base_resolution", C.c_uint32), ("per_level_scale", C.c_float), ("sdf_hidden_layers", C.c_uint32),
+                ("rgb_hidden_layers", C.c_uint32), ("sdf_bias", C.c_float)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 
@@ -41,6 +48,12 @@ def lib():
         _lib.n2_mlp_workspace_bytes.argtypes = [C.c_void_p]
         _lib.n2_mlp_destroy.restype = None
         _lib.n2_mlp_destroy.argtypes = [C.c_void_p]
+        _lib.n2_field_n_params.restype = C.c_uint32
+        _lib.n2_field_n_params.argtypes = [C.c_void_p]
+        _lib.n2_field_workspace_bytes.restype = C.c_uint64
+        _lib.n2_field_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
+        _lib.n2_field_destroy.restype = None
+        _lib.n2_field_destroy.argtypes = [C.c_void_p]
     return _lib
 
 

@@ -1,0 +1,417 @@
+// The NeuS field: host-side composition of grid, SDF MLP, direction encoding,
+// colour MLP and variance (counterpart of NerfNetwork<T>::forward_impl /
+// backward_impl / sdf / density) plus the few element-wise kernels it needs.
+//
+// Where the reference moves rows between temporaries with ~25 tiny launches,
+// the buffers here are laid out so that producers write straight into their
+// consumer's rows (the grid writes rows 3..34 of the SDF net's input, the SDF
+// net writes rows 0..15 of the colour net's input, the second-order grid pass
+// writes rows 3..34 of the MLP's second-order input), which leaves three glue
+// kernels in the forward and three in the backward.
+#include "n2_common.h"
+
+#include <new>
+
+typedef _Float16 hf;
+
+struct n2_field {
+	n2_grid_t* grid;
+	n2_mlp_t* sdf;
+	n2_mlp_t* rgb;
+	uint32_t enc_w, sdf_in_w, rgb_in_w;
+	float sdf_bias;
+	uint32_t off_sdf, off_rgb, off_grid, off_var, n_params;
+	const hf* params;
+	hf* grads;
+	unsigned char* ws;
+	uint64_t ws_bytes;
+	uint32_t max_batch;
+	// carved from the workspace
+	hf* sdf_in;        // [sdf_in_w][N]
+	hf* rgb_in;        // [48][N]
+	float* dy_dx;      // [enc_w][N][3]
+	hf* dsdf_din;      // [sdf_in_w][N]  d sdf / d (SDF net input)
+	float* normal;     // [3][N]
+	hf* d_rgb_in;      // [48][N]
+	hf* d_sdf_in;      // [sdf_in_w][N]
+	float* v;          // [3][N]  dL / d normal
+	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
+	hf* dL_drgb;       // [N][16]
+	float* var_acc;    // [4]
+	void* ws_sdf;
+	void* ws_rgb;
+};
+
+constexpr uint32_t FB = 256;
+
+// ----------------------------------------------------------------------------
+// glue kernels
+// ----------------------------------------------------------------------------
+// rows 0..2 = half(x) - half(0.5) (computed in half precision like the reference's
+// (T)pos - (T)0.5f), rows [3 + enc_w, sdf_in_w) = 0.
+__global__ void __launch_bounds__(FB) field_pack_sdf_input_kernel(const float* __restrict__ xyz, uint32_t ps, uint32_t ds, uint32_t N,
+                                                                  hf* __restrict__ sdf_in, uint32_t enc_w, uint32_t sdf_in_w) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	const float* q = xyz + (size_t)i * ps;
+#pragma unroll
+	for (int d = 0; d < 3; ++d) sdf_in[(size_t)d * N + i] = (hf)q[(size_t)d * ds] - (hf)0.5f;
+	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) sdf_in[(size_t)r * N + i] = (hf)0;
+}
+
+__device__ __forceinline__ void sh4_eval(float x, float y, float z, float* o) {
+	const float xy = x * y, xz = x * z, yz = y * z, x2 = x * x, y2 = y * y, z2 = z * z;
+	o[0] = 0.28209479177387814f;
+	o[1] = -0.48860251190291987f * y;
+	o[2] = 0.48860251190291987f * z;
+	o[3] = -0.48860251190291987f * x;
+	o[4] = 1.0925484305920792f * xy;
+	o[5] = -1.0925484305920792f * yz;
+	o[6] = 0.94617469575755997f * z2 - 0.31539156525251999f;
+	o[7] = -1.0925484305920792f * xz;
+	o[8] = 0.54627421529603959f * x2 - 0.54627421529603959f * y2;
+	o[9] = 0.59004358992664352f * y * (-3.0f * x2 + y2);
+	o[10] = 2.8906114426405538f * xy * z;
+	o[11] = 0.45704579946446572f * y * (1.0f - 5.0f * z2);
+	o[12] = 0.3731763325901154f * z * (5.0f * z2 - 3.0f);
+	o[13] = 0.45704579946446572f * x * (1.0f - 5.0f * z2);
+	o[14] = 1.4453057213202769f * z * (x2 - y2);
+	o[15] = 0.59004358992664352f * x * (-x2 + 3.0f * y2);
+}
+
+// normal = dy_dx^T dsdf_din[3..3+enc_w) + dsdf_din[0..3); then the colour net's input rows
+// 16..31 (SH of the direction), 32..34 (xyz), 35..37 (normal), 38..47 (zero).
+__global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float* __restrict__ coords, uint32_t N, uint32_t enc_w,
+                                                                     const hf* __restrict__ dsdf_din, const float* __restrict__ dy_dx,
+                                                                     float* __restrict__ normal, hf* __restrict__ rgb_in) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	float n0 = 0.f, n1 = 0.f, n2 = 0.f;
+	for (uint32_t k = 0; k < enc_w; ++k) {
+		const float g = (float)dsdf_din[(size_t)(3 + k) * N + i];
+		const float* j = dy_dx + ((size_t)k * N + i) * 3;
+		n0 = fmaf(g, j[0], n0);
+		n1 = fmaf(g, j[1], n1);
+		n2 = fmaf(g, j[2], n2);
+	}
+	n0 += (float)dsdf_din[i];
+	n1 += (float)dsdf_din[(size_t)N + i];
+	n2 += (float)dsdf_din[(size_t)2 * N + i];
+	normal[i] = n0;
+	normal[(size_t)N + i] = n1;
+	normal[(size_t)2 * N + i] = n2;
+	const float* c = coords + (size_t)i * 7;
+	float sh[16];
+	sh4_eval(c[4] * 2.f - 1.f, c[5] * 2.f - 1.f, c[6] * 2.f - 1.f, sh);
+#pragma unroll
+	for (int k = 0; k < 16; ++k) rgb_in[(size_t)(16 + k) * N + i] = (hf)sh[k];
+	rgb_in[(size_t)32 * N + i] = (hf)c[0];
+	rgb_in[(size_t)33 * N + i] = (hf)c[1];
+	rgb_in[(size_t)34 * N + i] = (hf)c[2];
+	rgb_in[(size_t)35 * N + i] = (hf)n0;
+	rgb_in[(size_t)36 * N + i] = (hf)n1;
+	rgb_in[(size_t)37 * N + i] = (hf)n2;
+#pragma unroll
+	for (int k = 38; k < 48; ++k) rgb_in[(size_t)k * N + i] = (hf)0;
+}
+
+// output rows 3 (sdf + bias), 4..6 (normal), 7 (variance), 8..10 (direction); rows 0..2 and
+// 11..15 keep what the colour net wrote.
+__global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __restrict__ coords, uint32_t N, const hf* __restrict__ sdf_out,
+                                                                 hf bias, const float* __restrict__ normal, const hf* __restrict__ variance,
+                                                                 hf* __restrict__ output) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	hf* o = output + (size_t)i * 16;
+	const float* c = coords + (size_t)i * 7;
+	o[3] = sdf_out[i] + bias;
+	o[4] = (hf)normal[i];
+	o[5] = (hf)normal[(size_t)N + i];
+	o[6] = (hf)normal[(size_t)2 * N + i];
+	o[7] = variance[0];
+	o[8] = (hf)c[4];
+	o[9] = (hf)c[5];
+	o[10] = (hf)c[6];
+}
+
+// dL_drgb = rows 0..2 of dL_doutput (rest zero); variance gradient = sum of row 7.
+__global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ dL_drgb,
+                                                                 float* __restrict__ var_acc) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	float s = 0.f;
+	if (i < N) {
+		const hf* src = dL_dout + (size_t)i * 16;
+		typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+		half8 lo = {src[0], src[1], src[2], (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
+		half8 hi = {(hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
+		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16) = lo;
+		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16 + 8) = hi;
+		s = (float)src[7];
+	}
+	// wave reduction, then one atomic per wave
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+	if ((threadIdx.x & 63) == 0 && s != 0.f) atomicAdd(var_acc, s);
+}
+
+__global__ void __launch_bounds__(FB) field_add_density_gradient_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ d_sdf_out_row0) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	d_sdf_out_row0[i] = d_sdf_out_row0[i] + dL_dout[(size_t)i * 16 + 3];
+}
+
+// v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
+// second-order MLP input rows 0..2 = half(v), rows [3 + enc_w, sdf_in_w) = 0; variance gradient written.
+__global__ void __launch_bounds__(FB) field_second_order_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, const hf* __restrict__ d_rgb_in,
+                                                                     const hf* __restrict__ dL_dout, float ek_batch, float* __restrict__ v,
+                                                                     hf* __restrict__ d_density_in, const float* __restrict__ var_acc,
+                                                                     hf* __restrict__ var_grad, int accumulate) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + var_acc[0]) : (hf)var_acc[0];
+	if (i >= N) return;
+	const hf* g = dL_dout + (size_t)i * 16;
+#pragma unroll
+	for (int d = 0; d < 3; ++d) {
+		float x = (float)d_rgb_in[(size_t)(35 + d) * N + i];
+		x += (float)g[4 + d] / ek_batch;
+		x += (float)g[8 + d];
+		v[(size_t)d * N + i] = x;
+		d_density_in[(size_t)d * N + i] = (hf)x;
+	}
+	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
+}
+
+__global__ void __launch_bounds__(FB) field_add_bias_kernel(uint32_t N, hf bias, hf* __restrict__ row0) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	row0[i] = row0[i] + bias;
+}
+
+// sdf -> logistic density, computed in half precision like the reference kernel
+__global__ void __launch_bounds__(FB) field_sdf_to_density_kernel(uint32_t N, const hf* __restrict__ variance, hf* __restrict__ row0) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	const hf s = (hf)__expf((float)(variance[0] * (hf)10.0f));
+	const hf x = row0[i] * s;
+	const hf sig = (hf)(1.0f / (1.0f + __expf(-(float)x)));
+	row0[i] = s * sig * ((hf)1.0f - sig);
+}
+
+// ----------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------
+static inline uint64_t align256(uint64_t x) { return (x + 255) / 256 * 256; }
+
+N2_API int n2_field_create(const n2_field_config* cfg, n2_field_t** out) {
+	N2_REQUIRE(out != nullptr && cfg != nullptr, "n2_field_create: null argument");
+	*out = nullptr;
+	n2_field* f = new (std::nothrow) n2_field();
+	N2_REQUIRE(f != nullptr, "n2_field_create: out of host memory");
+	*f = n2_field{};
+	int rc = n2_grid_create(cfg->n_levels, cfg->n_features_per_level, cfg->log2_hashmap_size, cfg->base_resolution,
+	                        cfg->per_level_scale, &f->grid);
+	if (rc == N2_OK) {
+		f->enc_w = n2_grid_output_width(f->grid);
+		f->sdf_in_w = (3 + f->enc_w + 15) / 16 * 16;  // next_multiple(3 + encoding, 16)
+		f->rgb_in_w = 48;                             // next_multiple(3 + 3 + 16 + 16, 16)
+		rc = n2_mlp_create(f->sdf_in_w, cfg->sdf_hidden_layers, &f->sdf);
+	}
+	if (rc == N2_OK) rc = n2_mlp_create(f->rgb_in_w, cfg->rgb_hidden_layers, &f->rgb);
+	if (rc != N2_OK) {
+		n2_field_destroy(f);
+		return rc;
+	}
+	f->sdf_bias = cfg->sdf_bias;
+	f->off_sdf = 0;
+	f->off_rgb = n2_mlp_n_params(f->sdf);
+	f->off_grid = f->off_rgb + n2_mlp_n_params(f->rgb);
+	f->off_var = f->off_grid + n2_grid_n_params(f->grid);
+	f->n_params = f->off_var + 4;
+	*out = f;
+	return N2_OK;
+}
+
+N2_API void n2_field_destroy(n2_field_t* f) {
+	if (!f) return;
+	n2_grid_destroy(f->grid);
+	n2_mlp_destroy(f->sdf);
+	n2_mlp_destroy(f->rgb);
+	delete f;
+}
+
+N2_API uint32_t n2_field_n_params(const n2_field_t* f) { return f ? f->n_params : 0; }
+
+N2_API int n2_field_param_offsets(const n2_field_t* f, uint32_t offsets[5]) {
+	N2_REQUIRE(f != nullptr && offsets != nullptr, "n2_field_param_offsets: null argument");
+	offsets[0] = f->off_sdf; offsets[1] = f->off_rgb; offsets[2] = f->off_grid; offsets[3] = f->off_var; offsets[4] = f->n_params;
+	return N2_OK;
+}
+
+N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* d_gradients) {
+	N2_REQUIRE(f != nullptr && d_params != nullptr, "n2_field_set_params: null argument");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 16 == 0 && reinterpret_cast<uintptr_t>(d_gradients) % 16 == 0,
+	           "n2_field_set_params: buffers must be 16-byte aligned");
+	f->params = reinterpret_cast<const hf*>(d_params);
+	f->grads = reinterpret_cast<hf*>(d_gradients);
+	auto g = [&](uint32_t off) { return d_gradients ? d_gradients + off : nullptr; };
+	if (int rc = n2_mlp_set_params(f->sdf, d_params + f->off_sdf, g(f->off_sdf))) return rc;
+	if (int rc = n2_mlp_set_params(f->rgb, d_params + f->off_rgb, g(f->off_rgb))) return rc;
+	return n2_grid_set_params(f->grid, d_params + f->off_grid, g(f->off_grid));
+}
+
+struct FieldCarve {
+	uint64_t sdf_in, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, total;
+};
+
+static FieldCarve carve(const n2_field_t* f, uint32_t nb) {
+	FieldCarve c{};
+	uint64_t o = 0;
+	const uint64_t n = nb;
+	auto take = [&](uint64_t bytes) { const uint64_t at = o; o = align256(o + bytes); return at; };
+	c.sdf_in = take(2ull * f->sdf_in_w * n);
+	c.rgb_in = take(2ull * f->rgb_in_w * n);
+	c.dy_dx = take(12ull * f->enc_w * n);
+	c.dsdf_din = take(2ull * f->sdf_in_w * n);
+	c.normal = take(12ull * n);
+	c.d_rgb_in = take(2ull * f->rgb_in_w * n);
+	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
+	c.v = take(12ull * n);
+	c.d_density_in = take(2ull * f->sdf_in_w * n);
+	c.dL_drgb = take(32ull * n);
+	c.var_acc = take(16);
+	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
+	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
+	c.total = o;
+	return c;
+}
+
+N2_API uint64_t n2_field_workspace_bytes(const n2_field_t* f, uint32_t max_batch) { return f ? carve(f, max_batch).total : 0; }
+
+N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_bytes, uint32_t max_batch) {
+	N2_REQUIRE(f != nullptr, "n2_field_set_workspace: field is null");
+	N2_REQUIRE(d_workspace != nullptr, "n2_field_set_workspace: workspace is null");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256 == 0, "n2_field_set_workspace: workspace must be 256-byte aligned");
+	N2_REQUIRE(max_batch % 8 == 0, "n2_field_set_workspace: max_batch %u must be a multiple of 8", max_batch);
+	const FieldCarve c = carve(f, max_batch);
+	N2_REQUIRE(n_bytes >= c.total, "n2_field_set_workspace: %llu bytes given, %llu needed for batch %u", (unsigned long long)n_bytes,
+	           (unsigned long long)c.total, max_batch);
+	unsigned char* b = reinterpret_cast<unsigned char*>(d_workspace);
+	f->ws = b; f->ws_bytes = n_bytes; f->max_batch = max_batch;
+	f->sdf_in = reinterpret_cast<hf*>(b + c.sdf_in);
+	f->rgb_in = reinterpret_cast<hf*>(b + c.rgb_in);
+	f->dy_dx = reinterpret_cast<float*>(b + c.dy_dx);
+	f->dsdf_din = reinterpret_cast<hf*>(b + c.dsdf_din);
+	f->normal = reinterpret_cast<float*>(b + c.normal);
+	f->d_rgb_in = reinterpret_cast<hf*>(b + c.d_rgb_in);
+	f->d_sdf_in = reinterpret_cast<hf*>(b + c.d_sdf_in);
+	f->v = reinterpret_cast<float*>(b + c.v);
+	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
+	f->dL_drgb = reinterpret_cast<hf*>(b + c.dL_drgb);
+	f->var_acc = reinterpret_cast<float*>(b + c.var_acc);
+	f->ws_sdf = b + c.ws_sdf;
+	f->ws_rgb = b + c.ws_rgb;
+	if (int rc = n2_mlp_set_workspace(f->sdf, f->ws_sdf, n2_mlp_workspace_bytes(f->sdf))) return rc;
+	return n2_mlp_set_workspace(f->rgb, f->ws_rgb, n2_mlp_workspace_bytes(f->rgb));
+}
+
+static int check_field(const n2_field_t* f, const char* fn, uint32_t n) {
+	N2_REQUIRE(f != nullptr, "%s: field is null", fn);
+	N2_REQUIRE(f->params != nullptr, "%s: n2_field_set_params has not been called", fn);
+	N2_REQUIRE(f->ws != nullptr, "%s: n2_field_set_workspace has not been called", fn);
+	N2_REQUIRE(n <= f->max_batch, "%s: batch %u exceeds the workspace's max_batch %u", fn, n, f->max_batch);
+	N2_REQUIRE(n % 8 == 0, "%s: batch size %u is not a multiple of 8", fn, n);
+	return N2_OK;
+}
+
+static inline dim3 fgrid(uint32_t n) { return dim3((n + FB - 1) / FB); }
+
+N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, n2_half* d_output) {
+	if (int rc = check_field(f, "n2_field_forward", n)) return rc;
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_coords != nullptr && d_output != nullptr, "n2_field_forward: null buffer");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "n2_field_forward: d_output must be 16-byte aligned");
+	hipStream_t s = n2_stream(stream);
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w);
+	N2_LAUNCH_CHECK();
+	if (int rc = n2_grid_forward(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
+	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<n2_half*>(f->rgb_in),
+	                            N2_LAYOUT_SOA, nullptr)) return rc;
+	if (int rc = n2_mlp_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
+	                                   reinterpret_cast<n2_half*>(f->dsdf_din))) return rc;
+	field_normals_rgb_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->enc_w, f->dsdf_din, f->dy_dx, f->normal, f->rgb_in);
+	N2_LAUNCH_CHECK();
+	if (int rc = n2_mlp_forward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_output, N2_LAYOUT_AOS, nullptr)) return rc;
+	field_finish_output_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->rgb_in, (hf)f->sdf_bias, f->normal, f->params + f->off_var,
+	                                                         reinterpret_cast<hf*>(d_output));
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n,
+                             const n2_half* d_dL_doutput, uint32_t ek_batch_size, n2_grad_mode mode) {
+	if (int rc = check_field(f, "n2_field_backward", n)) return rc;
+	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_field_backward: mode must be OVERWRITE or ACCUMULATE");
+	N2_REQUIRE(f->grads != nullptr, "n2_field_backward: no gradient buffer (n2_field_set_params)");
+	N2_REQUIRE(ek_batch_size > 0, "n2_field_backward: ek_batch_size must be positive");
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_coords != nullptr && d_dL_doutput != nullptr, "n2_field_backward: null buffer");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0, "n2_field_backward: d_dL_doutput must be 16-byte aligned");
+	hipStream_t s = n2_stream(stream);
+	const hf* dL = reinterpret_cast<const hf*>(d_dL_doutput);
+	if (int rc = n2_fill_zero_u32(s, f->var_acc, 16)) return rc;
+	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, dL, f->dL_drgb, f->var_acc);
+	N2_LAUNCH_CHECK();
+	// colour net
+	if (int rc = n2_mlp_backward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, reinterpret_cast<const n2_half*>(f->dL_drgb),
+	                             N2_LAYOUT_AOS, reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
+	field_add_density_gradient_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, dL, f->d_rgb_in);
+	N2_LAUNCH_CHECK();
+	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient
+	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
+	                             N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), mode)) return rc;
+	// grid, first order
+	if (int rc = n2_grid_backward(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), nullptr,
+	                              nullptr, mode)) return rc;
+	// dL/dnormal and the variance gradient
+	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->v,
+	                                                             f->d_density_in, f->var_acc, f->grads + f->off_var,
+	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+	N2_LAUNCH_CHECK();
+	// second order: grid (its dL_ddLdy lands in rows 3.. of the MLP's second-order input), then the SDF net
+	if (int rc = n2_grid_backward_backward_input(f->grid, stream, d_coords, 7, 1, n, f->v,
+	                                             reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n),
+	                                             reinterpret_cast<n2_half*>(f->d_density_in + (size_t)3 * n), nullptr, N2_GRAD_ACCUMULATE)) return rc;
+	return n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
+	                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE);
+}
+
+static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n,
+                          n2_half* d_output, bool density) {
+	if (int rc = check_field(f, fn, n)) return rc;
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_xyz != nullptr && d_output != nullptr, "%s: null buffer", fn);
+	N2_REQUIRE(ps >= 1 && ds >= 1, "%s: strides must be >= 1", fn);
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "%s: d_output must be 16-byte aligned", fn);
+	hipStream_t s = n2_stream(stream);
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->enc_w, f->sdf_in_w);
+	N2_LAUNCH_CHECK();
+	if (int rc = n2_grid_forward(f->grid, stream, d_xyz, ps, ds, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), nullptr)) return rc;
+	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, d_output, N2_LAYOUT_SOA, nullptr)) return rc;
+	field_add_bias_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, (hf)f->sdf_bias, reinterpret_cast<hf*>(d_output));
+	N2_LAUNCH_CHECK();
+	if (density) {
+		field_sdf_to_density_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->params + f->off_var, reinterpret_cast<hf*>(d_output));
+		N2_LAUNCH_CHECK();
+	}
+	return N2_OK;
+}
+
+N2_API int n2_field_sdf(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n,
+                        n2_half* d_output) {
+	return field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, point_stride, dim_stride, n, d_output, false);
+}
+
+N2_API int n2_field_density(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n,
+                            n2_half* d_output) {
+	return field_sdf_impl(f, "n2_field_density", stream, d_xyz, point_stride, dim_stride, n, d_output, true);
+}

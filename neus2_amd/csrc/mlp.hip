@@ -152,6 +152,14 @@ __device__ __forceinline__ half8 batch_frag_soa(const hf* __restrict__ M, size_t
 	if (row < n_rows && col < N) z = *reinterpret_cast<const half8*>(M + (size_t)row * N + col);
 	return z;
 }
+// the constant matrix e_{unit_row} 1^T restricted to valid samples
+__device__ __forceinline__ half8 batch_frag_unit(size_t N, uint32_t b0, int row, int unit_row, int c, int g) {
+	const uint32_t col = b0 + 16 * c + 8 * g;
+	half8 z;
+#pragma unroll
+	for (int e = 0; e < 8; ++e) z[e] = (row == unit_row && col < N) ? (hf)1 : (hf)0;
+	return z;
+}
 __device__ __forceinline__ half8 batch_frag_aos16(const hf* __restrict__ M, size_t N, uint32_t b0, int row, int c, int g) {
 	half8 z;
 #pragma unroll
@@ -163,8 +171,12 @@ __device__ __forceinline__ half8 batch_frag_aos16(const hf* __restrict__ M, size
 }
 
 // 16-row operand (network output gradient) as B operand of both tiles, K = 16
-__device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N, uint32_t col, int g, bool aos, half8& t0, half8& t1) {
-	if (aos) {
+__device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N, uint32_t col, int g, bool aos, int unit_row, half8& t0, half8& t1) {
+	if (unit_row >= 0) {
+		// dL_dy = e_{unit_row} for every sample: nothing is read
+#pragma unroll
+		for (int e = 0; e < 8; ++e) t0[e] = t1[e] = (8 * g + e == unit_row) ? (hf)1 : (hf)0;
+	} else if (aos) {
 		t0 = *reinterpret_cast<const half8*>(dY + (size_t)col * MLP_OUT + 8 * g);
 		t1 = *reinterpret_cast<const half8*>(dY + (size_t)(col + 1) * MLP_OUT + 8 * g);
 	} else {
@@ -333,7 +345,7 @@ __device__ __forceinline__ void outer_staged(float16v (&acc)[2][NT], const hf* S
 // B comes straight from an SoA global matrix with n_rows valid rows.
 template <int NT>
 __device__ __forceinline__ void outer_global(float16v (&acc)[2][NT], const hf* SA, const hf* __restrict__ M, size_t N, uint32_t b0,
-                                             int n_rows, bool aos16, int n, int g) {
+                                             int n_rows, bool aos16, int unit_row, int n, int g) {
 	stage_sync();
 #pragma unroll
 	for (int c = 0; c < 4; ++c) {
@@ -342,7 +354,8 @@ __device__ __forceinline__ void outer_global(float16v (&acc)[2][NT], const hf* S
 		for (int mt = 0; mt < 2; ++mt) a[mt] = stage_frag(SA, 32 * mt + n, c, g);
 #pragma unroll
 		for (int nt = 0; nt < NT; ++nt)
-			b[nt] = aos16 ? batch_frag_aos16(M, N, b0, 32 * nt + n, c, g) : batch_frag_soa(M, N, b0, 32 * nt + n, n_rows, c, g);
+			b[nt] = unit_row >= 0 ? batch_frag_unit(N, b0, 32 * nt + n, unit_row, c, g)
+			      : aos16 ? batch_frag_aos16(M, N, b0, 32 * nt + n, c, g) : batch_frag_soa(M, N, b0, 32 * nt + n, n_rows, c, g);
 #pragma unroll
 		for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -379,8 +392,8 @@ __device__ __forceinline__ void flush_acc(float* Wl, int ld, bool transposed, in
 // ----------------------------------------------------------------------------
 template <int IN_CHUNKS, int N_HIDDEN, bool WANT_DX, bool WANT_DW>
 __global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
-                                                                 const hf* __restrict__ dY, int dy_aos, hf* __restrict__ dX,
-                                                                 float* __restrict__ partials) {
+                                                                 const hf* __restrict__ dY, int dy_aos, int unit_row,
+                                                                 hf* __restrict__ dX, float* __restrict__ partials) {
 	constexpr int IN_W = 16 * IN_CHUNKS;
 	constexpr int IN_MT = (IN_W + 31) / 32;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (N_HIDDEN - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
@@ -439,7 +452,7 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __res
 		half8 h[N_HIDDEN][2][4];
 		forward_hidden<IN_CHUNKS, N_HIDDEN>(w, x, h);
 		half8 dy[2];
-		outgrad_frag(dY, N, col, g, dy_aos != 0, dy[0], dy[1]);
+		outgrad_frag(dY, N, col, g, dy_aos != 0, unit_row, dy[0], dy[1]);
 		if (!valid) {
 #pragma unroll
 			for (int e = 0; e < 8; ++e) { dy[0][e] = (hf)0; dy[1][e] = (hf)0; }
@@ -456,7 +469,7 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __res
 		if (WANT_DW) {
 			// dW_out^T [neuron][o] += h_last dY^T
 			stage_store(SA, h[N_HIDDEN - 1], n, g);
-			outer_global<1>(gWo, SA, dY, N, b0, MLP_OUT, dy_aos != 0, n, g);
+			outer_global<1>(gWo, SA, dY, N, b0, MLP_OUT, dy_aos != 0, unit_row, n, g);
 		}
 #pragma unroll
 		for (int k = N_HIDDEN - 1; k >= 1; --k) {
@@ -484,7 +497,7 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __res
 		if (WANT_DW) {
 			// dW_0 [neuron][input] += dh_0 x^T
 			stage_store(SA, dh, n, g);
-			outer_global<IN_MT>(gW0, SA, X, N, b0, IN_W, false, n, g);
+			outer_global<IN_MT>(gW0, SA, X, N, b0, IN_W, false, -1, n, g);
 		}
 		if (WANT_DX) {
 			float16v dx[2][IN_MT];
@@ -522,7 +535,7 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __res
 // ----------------------------------------------------------------------------
 template <int IN_CHUNKS>
 __global__ void __launch_bounds__(MLP_BLOCK) mlp_bbi_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
-                                                            const hf* __restrict__ V, const hf* __restrict__ G,
+                                                            const hf* __restrict__ V, const hf* __restrict__ G, int unit_row,
                                                             hf* __restrict__ dLddY, float* __restrict__ partials) {
 	constexpr int IN_W = 16 * IN_CHUNKS;
 	constexpr int IN_MT = (IN_W + 31) / 32;
@@ -553,7 +566,7 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_bbi_kernel(const hf* __restrict
 		half8 x[2][IN_CHUNKS], v[2][IN_CHUNKS], gg[2];
 		load_input<IN_CHUNKS>(X, N, col, g, x);
 		load_input<IN_CHUNKS>(V, N, col, g, v);
-		bfrag_soa(G, N, col, 0, g, MLP_OUT, gg[0], gg[1]);
+		outgrad_frag(G, N, col, g, false, unit_row, gg[0], gg[1]);
 		if (!valid) {
 #pragma unroll
 			for (int e = 0; e < 8; ++e) {
@@ -578,9 +591,9 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_bbi_kernel(const hf* __restrict
 			}
 		if (partials) {
 			stage_store(SA, b, n, g);
-			outer_global<IN_MT>(gW0, SA, V, N, b0, IN_W, false, n, g);
+			outer_global<IN_MT>(gW0, SA, V, N, b0, IN_W, false, -1, n, g);
 			stage_store(SA, a, n, g);
-			outer_global<1>(gWo, SA, G, N, b0, MLP_OUT, false, n, g);
+			outer_global<1>(gWo, SA, G, N, b0, MLP_OUT, false, unit_row, n, g);
 		}
 		if (dLddY) {
 			float16v out[2][1];
@@ -743,12 +756,13 @@ static int allow_lds(K kernel, size_t bytes) {
 	return N2_OK;
 }
 
-N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
-                           const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode) {
+// unit_row >= 0: dL_doutput is the constant e_{unit_row} and d_dL_doutput is not read
+static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                             const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
-	N2_REQUIRE(d_dL_doutput != nullptr || n == 0, "n2_mlp_backward: d_dL_doutput is null");
+	N2_REQUIRE(d_dL_doutput != nullptr || n == 0 || unit_row >= 0, "n2_mlp_backward: d_dL_doutput is null");
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0 && reinterpret_cast<uintptr_t>(d_dL_dinput) % 16 == 0,
 	           "n2_mlp_backward: buffers must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
@@ -768,7 +782,7 @@ N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_i
 #define LAUNCH(IC, NH, DX, DW)                                                                                      \
 	do {                                                                                                            \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
-		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, dX, mlp->workspace); \
+		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, mlp->workspace); \
 	} while (0)
 #define CALL(IC, NH)                                   \
 	do {                                               \
@@ -784,6 +798,18 @@ N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_i
 	return N2_OK;
 }
 
+N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                           const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode) {
+	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode);
+}
+
+N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
+                                 n2_half* d_dinput) {
+	N2_REQUIRE(dim < (uint32_t)MLP_OUT, "n2_mlp_input_gradient: output dimension %u out of range", dim);
+	N2_REQUIRE(d_dinput != nullptr || n == 0, "n2_mlp_input_gradient: d_dinput is null");
+	return mlp_backward_impl(mlp, stream, d_input, n, nullptr, N2_LAYOUT_SOA, (int)dim, d_dinput, N2_GRAD_IGNORE);
+}
+
 N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                                           const n2_half* d_dL_ddLdinput, const n2_half* d_dL_doutput,
                                           n2_half* d_dL_ddLdoutput, n2_grad_mode mode) {
@@ -793,7 +819,8 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 		n2_set_error("n2_mlp_backward_backward_input: implemented for one hidden layer (got %u)", mlp->n_hidden);
 		return N2_ERR_UNSUPPORTED;
 	}
-	N2_REQUIRE((d_dL_ddLdinput != nullptr && d_dL_doutput != nullptr) || n == 0, "n2_mlp_backward_backward_input: d_dL_ddLdinput and d_dL_doutput are required");
+	N2_REQUIRE(d_dL_ddLdinput != nullptr || n == 0, "n2_mlp_backward_backward_input: d_dL_ddLdinput is required");
+	const int unit_row = d_dL_doutput == nullptr ? 0 : -1;
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_ddLdinput) % 16 == 0 && reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0 &&
 	           reinterpret_cast<uintptr_t>(d_dL_ddLdoutput) % 16 == 0, "n2_mlp_backward_backward_input: buffers must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
@@ -810,7 +837,7 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 	case IC:                                                                                                               \
 		if (int rc = allow_lds(mlp_bbi_kernel<IC>, lds)) return rc;                                                        \
 		mlp_bbi_kernel<IC><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
-			reinterpret_cast<const hf*>(d_dL_ddLdinput), reinterpret_cast<const hf*>(d_dL_doutput),                        \
+			reinterpret_cast<const hf*>(d_dL_ddLdinput), reinterpret_cast<const hf*>(d_dL_doutput), unit_row,              \
 			reinterpret_cast<hf*>(d_dL_ddLdoutput), want_dw ? mlp->workspace : nullptr);                                   \
 		break;
 		CASE(1) CASE(2) CASE(3) CASE(4)

@@ -204,3 +204,91 @@ class FullyFusedMLP:
                                                         ptr(dL_doutput), ptr(o), C.c_int(mode)),
               "n2_mlp_backward_backward_input")
         return o
+
+
+class NerfNetwork:
+    """NerfNetwork<__half> of the reference (nerf_network.h), static scene: grid + SDF MLP +
+    SH direction encoding + colour MLP + variance, with normals computed inside the forward and
+    the second-order passes inside the backward."""
+
+    def __init__(self, n_levels=16, log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447,
+                 sdf_hidden_layers=1, rgb_hidden_layers=2, sdf_bias=-0.1):
+        cfg = capi.FieldConfig(n_levels, 2, log2_hashmap_size, base_resolution, per_level_scale, sdf_hidden_layers,
+                               rgb_hidden_layers, sdf_bias)
+        self._h = C.c_void_p()
+        check(capi.lib().n2_field_create(C.byref(cfg), C.byref(self._h)), "n2_field_create")
+        self._params = self._grads = self._ws = None
+        self.max_batch = 0
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) is not None and self._h.value:
+                capi.lib().n2_field_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+    def n_params(self):
+        return int(capi.lib().n2_field_n_params(self._h))
+
+    def param_offsets(self):
+        o = (C.c_uint32 * 5)()
+        check(capi.lib().n2_field_param_offsets(self._h, o), "n2_field_param_offsets")
+        return list(o)
+
+    def padded_output_width(self):
+        return 16
+
+    def set_params(self, params, gradients=None):
+        for t in (params, gradients):
+            if t is not None:
+                _check_half(t, (self.n_params(),), "field params/gradients")
+        check(capi.lib().n2_field_set_params(self._h, ptr(params), ptr(gradients)), "n2_field_set_params")
+        self._params, self._grads = params, gradients
+
+    def reserve(self, max_batch):
+        """Allocates the workspace (the reference's arena temporaries) for batches up to max_batch."""
+        if max_batch <= self.max_batch:
+            return
+        nbytes = int(capi.lib().n2_field_workspace_bytes(self._h, C.c_uint32(max_batch)))
+        self._ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        check(capi.lib().n2_field_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes), C.c_uint32(max_batch)),
+              "n2_field_set_workspace")
+        self.max_batch = max_batch
+
+    @staticmethod
+    def _coords(coords):
+        if coords.dtype != torch.float32 or not coords.is_cuda or not coords.is_contiguous() or coords.dim() != 2 \
+                or coords.shape[1] != 7:
+            raise N2Error("coords must be a contiguous float32 CUDA tensor [N, 7]")
+        return coords.shape[0]
+
+    def forward(self, coords, out=None):
+        n = self._coords(coords)
+        self.reserve(n)
+        y = torch.empty((n, 16), dtype=torch.float16, device=coords.device) if out is None else out
+        check(capi.lib().n2_field_forward(self._h, _stream(), ptr(coords), C.c_uint32(n), ptr(y)), "n2_field_forward")
+        return y
+
+    inference_mixed_precision = forward
+
+    def backward(self, coords, dL_doutput, ek_batch_size=None, mode=GRAD_OVERWRITE):
+        n = self._coords(coords)
+        _check_half(dL_doutput, (n, 16), "dL_doutput")
+        check(capi.lib().n2_field_backward(self._h, _stream(), ptr(coords), C.c_uint32(n), ptr(dL_doutput),
+                                           C.c_uint32(n if ek_batch_size is None else ek_batch_size), C.c_int(mode)),
+              "n2_field_backward")
+
+    def _sdf(self, fn, xyz):
+        x, ps, ds, n = _positions(xyz)
+        self.reserve(n)
+        out = torch.empty((16, n), dtype=torch.float16, device=x.device)
+        check(getattr(capi.lib(), fn)(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds), C.c_uint32(n),
+                                      ptr(out)), fn)
+        return out
+
+    def sdf(self, xyz):
+        return self._sdf("n2_field_sdf", xyz)
+
+    def density(self, xyz):
+        return self._sdf("n2_field_density", xyz)
