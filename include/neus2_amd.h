@@ -266,6 +266,30 @@ int n2_field_sdf(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint
 int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
                      uint32_t dim_stride, uint32_t n, n2_half* d_output);
 
+/* ------------------------------------------------------------------------
+ * Adam on fp32 master weights with an fp16 working copy: tcnn's Adam as the
+ * trainer runs it, Trainer::optimizer_step(stream, LOSS_SCALE) at
+ * src/testbed_nerf.cu:3498, hyper-parameters from configs/nerf/base.json:13-26
+ * (the Ema and ExponentialDecay wrappers around it are not part of this path).
+ * Per parameter i:  g = grad/loss_scale;  i >= n_matrix_params and g == 0: skipped entirely;
+ * i < n_matrix_params: g += l2_reg*w;  moments with beta1/beta2;  per-parameter step counter t;
+ * w -= lr*sqrt(1-beta2^t)/(1-beta1^t) * m/(sqrt(v)+epsilon);  fp16 copy refreshed.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_adam_config {
+	float learning_rate; /* 1e-3 */
+	float beta1;         /* 0.9 */
+	float beta2;         /* 0.99 */
+	float epsilon;       /* 1e-15 */
+	float l2_reg;        /* 1e-6 */
+} n2_adam_config;
+
+/* All buffers hold n_params elements and are caller-owned device memory:
+ *  d_master fp32 weights, d_params fp16 copy (written), d_gradients fp16 (read),
+ *  d_m1 / d_m2 fp32 moments, d_steps uint32 per-parameter step counters. */
+int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
+                 float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
+                 float* d_m2, uint32_t* d_steps);
+
 #ifdef __cplusplus
 }
 #endif

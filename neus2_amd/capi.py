@@ -23,6 +23,12 @@ class FieldConfig(C.Structure):
                 ("rgb_hidden_layers", C.c_uint32), ("sdf_bias", C.c_float)]
 
 
+class AdamConfig(C.Structure):
+    """struct n2_adam_config (defaults: configs/nerf/base.json:13-26)"""
+    _fields_ = [("learning_rate", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("epsilon", C.c_float),
+                ("l2_reg", C.c_float)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 

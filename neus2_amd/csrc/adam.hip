@@ -1,0 +1,81 @@
+// Adam step over the whole parameter vector: a pure streaming kernel.
+// Four parameters per lane so that every buffer is moved with 8- or 16-byte
+// accesses; parameters whose gradient is zero (most of the hash table in any
+// one step) cost only the 2-byte gradient read.
+#include "n2_common.h"
+
+typedef _Float16 hf;
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float loss_scale, const n2_adam_config& c, float g16,
+                                         float& w, float& m1, float& m2, uint32_t& t) {
+	float g = g16 / loss_scale;
+	if (i >= n_matrix) {
+		if (g == 0.f) return false;
+	} else {
+		g += c.l2_reg * w;
+	}
+	const float gs = g * g;
+	m1 = c.beta1 * m1 + (1.f - c.beta1) * g;
+	m2 = c.beta2 * m2 + (1.f - c.beta2) * gs;
+	t += 1u;
+	const float lr = c.learning_rate * sqrtf(1.f - powf(c.beta2, (float)t)) / (1.f - powf(c.beta1, (float)t));
+	w -= lr * m1 / (sqrtf(m2) + c.epsilon);
+	return true;
+}
+
+__global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale,
+                                                        float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
+                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps) {
+	const uint32_t q = blockIdx.x * 256 + threadIdx.x;
+	const uint32_t i0 = q * 4;
+	if (i0 >= n) return;
+	if (i0 + 4 <= n) {
+		const half4 g = *reinterpret_cast<const half4*>(grads + i0);
+		const bool all_zero = g[0] == (hf)0 && g[1] == (hf)0 && g[2] == (hf)0 && g[3] == (hf)0;
+		if (all_zero && i0 >= n_matrix) return;  // nothing but the gradient is touched
+		float4 w = *reinterpret_cast<float4*>(master + i0);
+		float4 a = *reinterpret_cast<float4*>(m1 + i0);
+		float4 b = *reinterpret_cast<float4*>(m2 + i0);
+		uint4 t = *reinterpret_cast<uint4*>(steps + i0);
+		bool any = false;
+		any |= adam_one(i0 + 0, n_matrix, loss_scale, c, (float)g[0], w.x, a.x, b.x, t.x);
+		any |= adam_one(i0 + 1, n_matrix, loss_scale, c, (float)g[1], w.y, a.y, b.y, t.y);
+		any |= adam_one(i0 + 2, n_matrix, loss_scale, c, (float)g[2], w.z, a.z, b.z, t.z);
+		any |= adam_one(i0 + 3, n_matrix, loss_scale, c, (float)g[3], w.w, a.w, b.w, t.w);
+		if (!any) return;
+		*reinterpret_cast<float4*>(master + i0) = w;
+		*reinterpret_cast<float4*>(m1 + i0) = a;
+		*reinterpret_cast<float4*>(m2 + i0) = b;
+		*reinterpret_cast<uint4*>(steps + i0) = t;
+		*reinterpret_cast<half4*>(params + i0) = half4{(hf)w.x, (hf)w.y, (hf)w.z, (hf)w.w};
+	} else {
+		for (uint32_t i = i0; i < n; ++i) {
+			float w = master[i], a = m1[i], b = m2[i];
+			uint32_t t = steps[i];
+			if (adam_one(i, n_matrix, loss_scale, c, (float)grads[i], w, a, b, t)) {
+				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+			}
+		}
+	}
+}
+
+N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
+                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
+                        float* d_m2, uint32_t* d_steps) {
+	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
+	if (n_params == 0) return N2_OK;
+	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
+	N2_REQUIRE(loss_scale > 0.f, "n2_adam_step: loss_scale must be positive");
+	N2_REQUIRE(n_matrix_params <= n_params, "n2_adam_step: n_matrix_params %u > n_params %u", n_matrix_params, n_params);
+	const uintptr_t a = reinterpret_cast<uintptr_t>(d_master) | reinterpret_cast<uintptr_t>(d_m1) | reinterpret_cast<uintptr_t>(d_m2) |
+	                    reinterpret_cast<uintptr_t>(d_steps);
+	N2_REQUIRE(a % 16 == 0, "n2_adam_step: fp32/uint32 buffers must be 16-byte aligned");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 8 == 0 && reinterpret_cast<uintptr_t>(d_gradients) % 8 == 0,
+	           "n2_adam_step: fp16 buffers must be 8-byte aligned");
+	const uint32_t quads = (n_params + 3) / 4;
+	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(*config, n_params, n_matrix_params, loss_scale,
+		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

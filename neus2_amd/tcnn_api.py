@@ -292,3 +292,27 @@ class NerfNetwork:
 
     def density(self, xyz):
         return self._sdf("n2_field_density", xyz)
+
+
+class Adam:
+    """tcnn Adam as Trainer::optimizer_step runs it (src/testbed_nerf.cu:3498): fp32 master weights,
+    fp16 working copy, per-parameter step counters, l2_reg on matrix parameters only and a skip
+    for non-matrix parameters whose gradient is exactly zero."""
+
+    def __init__(self, master, n_matrix_params, learning_rate=1e-3, beta1=0.9, beta2=0.99, epsilon=1e-15, l2_reg=1e-6):
+        if master.dtype != torch.float32 or not master.is_cuda or not master.is_contiguous():
+            raise N2Error("master weights must be a contiguous float32 CUDA tensor")
+        self.cfg = capi.AdamConfig(learning_rate, beta1, beta2, epsilon, l2_reg)
+        self.master = master
+        self.n_matrix_params = n_matrix_params
+        self.m1 = torch.zeros_like(master)
+        self.m2 = torch.zeros_like(master)
+        self.steps = torch.zeros(master.numel(), dtype=torch.int32, device=master.device)
+
+    def step(self, params, gradients, loss_scale=128.0):
+        n = self.master.numel()
+        _check_half(params, (n,), "params")
+        _check_half(gradients, (n,), "gradients")
+        check(capi.lib().n2_adam_step(_stream(), C.byref(self.cfg), C.c_uint32(n), C.c_uint32(self.n_matrix_params),
+                                      C.c_float(loss_scale), ptr(self.master), ptr(params), ptr(gradients),
+                                      ptr(self.m1), ptr(self.m2), ptr(self.steps)), "n2_adam_step")
