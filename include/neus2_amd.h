@@ -290,6 +290,51 @@ int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_pa
                  float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
                  float* d_m2, uint32_t* d_steps);
 
+/* ------------------------------------------------------------------------
+ * NeuS logistic-density alpha compositing, Huber(0.1)/5 colour loss and the hand-derived
+ * backward to the 16 network outputs, with compaction of the samples that survive early
+ * termination: compute_loss_kernel_train_nerf_with_global_movement,
+ * src/testbed_nerf.cu:1465-1996 (static scene: no global movement, envmap, exposure,
+ * depth or mask supervision; Logistic colour activation; BENT_DIR 1).
+ *
+ * The reference runs one thread per ray with two serial loops; here one wavefront owns a ray
+ * and transmittance / colour prefixes are wave-level scans over 64 samples at a time.
+ * The reference hands out compacted ranges with atomicAdd (ray order is a race); here they are
+ * an exclusive scan in ray order, i.e. deterministic.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_composite_config {
+	float loss_scale;       /* LOSS_SCALE = 128, testbed.h:237 */
+	float ek_loss_weight;   /* hyperparams.ek_loss_weight, configs/nerf/base.json:80 */
+	float cos_anneal_ratio; /* NerfNetwork::cos_anneal_ratio, nerf_network.h:1109-1118 (1 when anneal_end = 0) */
+	float background[3];    /* m_background_color, added as T*background to rays that are not cut short */
+	uint32_t n_rays_norm;   /* n_rays_per_batch: loss and gradients are divided by it (:1717, :1756) */
+} n2_composite_config;
+
+uint64_t n2_composite_workspace_bytes(uint32_t max_rays);
+
+/*  n_rays                upper bound of rays; d_ray_counter (may be NULL) holds the live count (rays_counter)
+ *  d_numsteps            uint32 [n_rays][2] in: (samples, first sample) per ray; out: (kept samples, compacted first)
+ *  d_network_output      fp16 [S][16] (AoS) field output of every marched sample
+ *  d_coords              fp32 [S][7] NerfCoordinate of every marched sample
+ *  d_rgb_target          fp32 [n_rays][3] target colour of each ray's pixel (the dataset side of :1619-1662)
+ *  max_samples_compacted target batch size (2^18)
+ *  d_compacted_counter   uint32 out: total samples the rays wanted to keep (numsteps_counter; may exceed the maximum)
+ *  d_coords_compacted    fp32 [max][7] out
+ *  d_dloss_doutput       fp16 [max][16] out (rows 11..15, which the reference leaves unset, are zero)
+ *  d_loss                NULL or fp32 [n_rays] out: per-ray mean loss / n_rays_norm */
+int n2_composite_loss(n2_stream_t stream, const n2_composite_config* config, uint32_t n_rays,
+                      const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                      const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                      uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                      float* d_loss, void* d_workspace, uint64_t workspace_bytes);
+
+/* tcnn fill_rollover / fill_rollover_and_rescale, src/testbed_nerf.cu:3908-3916: pad a compacted
+ * batch of *d_n_in rows to n_total rows by wrapping around; the fp16 variant scales the wrapped
+ * copies by n_in/n_total.  No-op when *d_n_in is 0 or >= n_total. */
+int n2_fill_rollover_f32(n2_stream_t stream, uint32_t n_total, uint32_t stride, const uint32_t* d_n_in, float* d_inout);
+int n2_fill_rollover_and_rescale_f16(n2_stream_t stream, uint32_t n_total, uint32_t stride, const uint32_t* d_n_in,
+                                     n2_half* d_inout);
+
 #ifdef __cplusplus
 }
 #endif

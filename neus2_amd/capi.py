@@ -29,6 +29,12 @@ class AdamConfig(C.Structure):
                 ("l2_reg", C.c_float)]
 
 
+class CompositeConfig(C.Structure):
+    """struct n2_composite_config"""
+    _fields_ = [("loss_scale", C.c_float), ("ek_loss_weight", C.c_float), ("cos_anneal_ratio", C.c_float),
+                ("background", C.c_float * 3), ("n_rays_norm", C.c_uint32)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 
@@ -58,6 +64,8 @@ def lib():
         _lib.n2_field_n_params.argtypes = [C.c_void_p]
         _lib.n2_field_workspace_bytes.restype = C.c_uint64
         _lib.n2_field_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
+        _lib.n2_composite_workspace_bytes.restype = C.c_uint64
+        _lib.n2_composite_workspace_bytes.argtypes = [C.c_uint32]
         _lib.n2_field_destroy.restype = None
         _lib.n2_field_destroy.argtypes = [C.c_void_p]
     return _lib

@@ -35,3 +35,11 @@ int n2_fill_zero_u32(hipStream_t stream, void* d_ptr, size_t n_bytes) {
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
+
+__global__ void n2_set_u32_kernel(uint32_t* p, uint32_t v) { *p = v; }
+
+int n2_set_u32(hipStream_t stream, uint32_t* d_ptr, uint32_t value) {
+	n2_set_u32_kernel<<<dim3(1), dim3(1), 0, stream>>>(d_ptr, value);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

@@ -1,0 +1,339 @@
+// NeuS alpha compositing, colour loss and backward to the network outputs.
+//
+// One wavefront owns one ray and walks it 64 samples at a time: each lane loads
+// one sample's 16 fp16 outputs (32 contiguous bytes), the transmittance before
+// every sample is an exclusive product scan of (1 - alpha) across the wave,
+// composited colour and the prefix the backward needs are wave reductions /
+// inclusive scans.  Three kernels: forward (how many samples each ray keeps and
+// its colour), an exclusive scan over rays that hands out compacted ranges in
+// ray order, backward (gradients and compacted coordinates).
+#include "n2_common.h"
+
+typedef _Float16 hf;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+struct CompParams {
+	float loss_scale, ek_loss_weight, anneal;
+	float bg[3];
+	float inv_n_rays;
+	float min_step, max_step;
+};
+
+struct Sample {
+	float alpha, p_div_c, iter_cos, true_cos, inv_s, dt, next_sdf;
+	float rgb[3], n[3], raw[3];
+};
+
+__device__ __forceinline__ float logistic(float x) { return 1.f / (1.f + __expf(-x)); }
+
+__device__ __forceinline__ void load_out(const hf* __restrict__ net_out, size_t s, float* o) {
+	const half8 a = *reinterpret_cast<const half8*>(net_out + s * 16);
+	const half8 b = *reinterpret_cast<const half8*>(net_out + s * 16 + 8);
+#pragma unroll
+	for (int k = 0; k < 8; ++k) { o[k] = (float)a[k]; o[8 + k] = (float)b[k]; }
+}
+
+__device__ __forceinline__ Sample eval_sample(const float* o, hf var_h, float warped_dt, const float* dir, const CompParams& c) {
+	Sample s;
+	s.dt = warped_dt * (c.max_step - c.min_step) + c.min_step;
+#pragma unroll
+	for (int k = 0; k < 3; ++k) { s.raw[k] = o[k]; s.rgb[k] = logistic(o[k]); s.n[k] = o[4 + k]; }
+	s.inv_s = __expf((float)((hf)10.0f * var_h));  // product formed in half precision
+	const float sdf = o[3];
+	s.true_cos = dir[0] * s.n[0] + dir[1] * s.n[1] + dir[2] * s.n[2];
+	const float a = fmaxf(-s.true_cos * 0.5f + 0.5f, 0.f), b = fmaxf(-s.true_cos, 0.f);
+	s.iter_cos = -(a * (1.f - c.anneal) + b * c.anneal);
+	s.next_sdf = sdf + s.iter_cos * s.dt * 0.5f;
+	const float prev_sdf = sdf - s.iter_cos * s.dt * 0.5f;
+	const float next_cdf = logistic(s.next_sdf * s.inv_s), prev_cdf = logistic(prev_sdf * s.inv_s);
+	s.p_div_c = (prev_cdf - next_cdf + 1e-5f) / (prev_cdf + 1e-5f);
+	s.alpha = fminf(fmaxf(s.p_div_c, 0.f), 1.f);
+	return s;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+	return v;
+}
+// exclusive product scan over the 64 lanes
+__device__ __forceinline__ float wave_excl_prod(float v, int lane) {
+#pragma unroll
+	for (int o = 1; o < 64; o <<= 1) {
+		const float u = __shfl_up(v, o);
+		if (lane >= o) v *= u;
+	}
+	const float e = __shfl_up(v, 1);
+	return lane == 0 ? 1.f : e;
+}
+__device__ __forceinline__ float wave_incl_sum(float v, int lane) {
+#pragma unroll
+	for (int o = 1; o < 64; o <<= 1) {
+		const float u = __shfl_up(v, o);
+		if (lane >= o) v += u;
+	}
+	return v;
+}
+
+// direction of the ray: rows 8..10 of its first sample, unwarped and normalised
+__device__ __forceinline__ void ray_dir(const hf* __restrict__ net_out, size_t base, float* dir) {
+	const hf* o = net_out + base * 16;
+	const float x = (float)o[8] * 2.f - 1.f, y = (float)o[9] * 2.f - 1.f, z = (float)o[10] * 2.f - 1.f;
+	const float len = sqrtf(x * x + y * y + z * z);
+	dir[0] = x / len; dir[1] = y / len; dir[2] = z / len;
+}
+
+struct RayScratch {
+	float rgb[3];
+	uint32_t kept;
+};
+
+constexpr float T_EPS = 1e-4f;
+constexpr int CB = 256;  // 4 rays per workgroup
+
+__global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uint32_t n_rays, const uint32_t* __restrict__ ray_counter,
+                                                               const uint32_t* __restrict__ numsteps, const hf* __restrict__ net_out,
+                                                               const float* __restrict__ coords, RayScratch* __restrict__ scratch) {
+	const int lane = threadIdx.x & 63;
+	const uint32_t ray = blockIdx.x * (CB / 64) + (threadIdx.x >> 6);
+	if (ray >= n_rays) return;
+	const uint32_t live = ray_counter ? min(*ray_counter, n_rays) : n_rays;
+	if (ray >= live) {
+		if (lane == 0) scratch[ray] = RayScratch{{0.f, 0.f, 0.f}, 0u};
+		return;
+	}
+	const uint32_t n = numsteps[2 * ray], base = numsteps[2 * ray + 1];
+	float dir[3] = {0.f, 0.f, 0.f};
+	if (n > 0) ray_dir(net_out, base, dir);
+	float T = 1.f, r0 = 0.f, r1 = 0.f, r2 = 0.f;
+	uint32_t kept = 0;
+	for (uint32_t c0 = 0; c0 < n; c0 += 64) {
+		const uint32_t s = c0 + lane;
+		const bool valid = s < n;
+		float alpha = 0.f, rgb[3] = {0.f, 0.f, 0.f};
+		if (valid) {
+			float o[16];
+			load_out(net_out, (size_t)base + s, o);
+			const Sample sm = eval_sample(o, net_out[((size_t)base + s) * 16 + 7], coords[((size_t)base + s) * 7 + 3], dir, c);
+			alpha = sm.alpha; rgb[0] = sm.rgb[0]; rgb[1] = sm.rgb[1]; rgb[2] = sm.rgb[2];
+		}
+		const float Tb = T * wave_excl_prod(1.f - alpha, lane);
+		// samples are consumed while the transmittance before them is >= 1e-4
+		const unsigned long long stop = __ballot(!valid || Tb < T_EPS);
+		const int n_proc = stop ? (int)__ffsll((long long)stop) - 1 : 64;
+		const float w = lane < n_proc ? alpha * Tb : 0.f;
+		r0 += wave_sum(w * rgb[0]);
+		r1 += wave_sum(w * rgb[1]);
+		r2 += wave_sum(w * rgb[2]);
+		kept += n_proc;
+		if (n_proc > 0) T = __shfl(Tb * (1.f - alpha), n_proc - 1);
+		if (n_proc < 64) break;
+	}
+	if (kept == n) { r0 += T * c.bg[0]; r1 += T * c.bg[1]; r2 += T * c.bg[2]; }
+	if (lane == 0) scratch[ray] = RayScratch{{r0, r1, r2}, kept};
+}
+
+// exclusive scan of kept counts in ray order, one workgroup; also applies the budget clamp
+__global__ void __launch_bounds__(1024) composite_scan_kernel(uint32_t n_rays, uint32_t max_compacted, const RayScratch* __restrict__ scratch,
+                                                              uint32_t* __restrict__ cbase, uint32_t* __restrict__ ckept,
+                                                              uint32_t* __restrict__ counter) {
+	__shared__ uint32_t wave_tot[16];
+	__shared__ uint32_t carry_s;
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	if (threadIdx.x == 0) carry_s = 0;
+	__syncthreads();
+	for (uint32_t r0 = 0; r0 < n_rays; r0 += 1024) {
+		const uint32_t r = r0 + threadIdx.x;
+		const uint32_t k = r < n_rays ? scratch[r].kept : 0u;
+		uint32_t v = k;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) {
+			const uint32_t u = __shfl_up(v, o);
+			if (lane >= o) v += u;
+		}
+		if (lane == 63) wave_tot[wave] = v;
+		__syncthreads();
+		uint32_t before = carry_s;
+		for (int w = 0; w < wave; ++w) before += wave_tot[w];
+		const uint32_t excl = before + v - k;
+		if (r < n_rays) {
+			cbase[r] = excl;
+			ckept[r] = min(max_compacted - min(max_compacted, excl), k);
+		}
+		__syncthreads();
+		if (threadIdx.x == 1023) carry_s = excl + k;
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) *counter = carry_s;
+}
+
+__global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, uint32_t n_rays, uint32_t* __restrict__ numsteps,
+                                                                const hf* __restrict__ net_out, const float* __restrict__ coords,
+                                                                const float* __restrict__ rgb_target, const RayScratch* __restrict__ scratch,
+                                                                const uint32_t* __restrict__ cbase, const uint32_t* __restrict__ ckept,
+                                                                float* __restrict__ coords_out, hf* __restrict__ dloss, float* __restrict__ loss) {
+	const int lane = threadIdx.x & 63;
+	const uint32_t ray = blockIdx.x * (CB / 64) + (threadIdx.x >> 6);
+	if (ray >= n_rays) return;
+	const uint32_t base = numsteps[2 * ray + 1];
+	const uint32_t m = ckept[ray], cb = cbase[ray];
+	const RayScratch rs = scratch[ray];
+	// Huber(0.1)/5 per channel
+	float grad[3], lsum = 0.f;
+#pragma unroll
+	for (int k = 0; k < 3; ++k) {
+		const float d = rs.rgb[k] - rgb_target[(size_t)ray * 3 + k], ad = fabsf(d);
+		lsum += (ad > 0.1f ? ad - 0.05f : 5.f * d * d) / 5.f;
+		grad[k] = (ad > 0.1f ? (d > 0.f ? 1.f : -1.f) : d / 0.1f) / 5.f;
+	}
+	__builtin_amdgcn_wave_barrier();
+	if (lane == 0) {
+		numsteps[2 * ray] = m;
+		numsteps[2 * ray + 1] = cb;
+		if (loss) loss[ray] = m == 0 ? 0.f : lsum / 3.f * c.inv_n_rays;
+	}
+	if (m == 0) return;
+	const float loss_scale = c.loss_scale * c.inv_n_rays;
+	float dir[3];
+	ray_dir(net_out, base, dir);
+	float T = 1.f, p0 = 0.f, p1 = 0.f, p2 = 0.f;  // transmittance and colour prefix carried between chunks
+	for (uint32_t c0 = 0; c0 < m; c0 += 64) {
+		const uint32_t s = c0 + lane;
+		const bool valid = s < m;
+		Sample sm;
+		sm.alpha = 0.f;
+		hf var_h = (hf)0;
+		if (valid) {
+			float o[16];
+			load_out(net_out, (size_t)base + s, o);
+			var_h = net_out[((size_t)base + s) * 16 + 7];
+			sm = eval_sample(o, var_h, coords[((size_t)base + s) * 7 + 3], dir, c);
+		}
+		const float alpha = valid ? sm.alpha : 0.f;
+		const float Tb = T * wave_excl_prod(1.f - alpha, lane);
+		const float w = valid ? alpha * Tb : 0.f;
+		const float Ta = Tb * (1.f - alpha);
+		const float q0 = p0 + wave_incl_sum(valid ? w * sm.rgb[0] : 0.f, lane);
+		const float q1 = p1 + wave_incl_sum(valid ? w * sm.rgb[1] : 0.f, lane);
+		const float q2 = p2 + wave_incl_sum(valid ? w * sm.rgb[2] : 0.f, lane);
+		if (valid) {
+			const float dot = grad[0] * (Ta * sm.rgb[0] - (rs.rgb[0] - q0)) + grad[1] * (Ta * sm.rgb[1] - (rs.rgb[1] - q1)) +
+			                  grad[2] * (Ta * sm.rgb[2] - (rs.rgb[2] - q2));
+			const float dloss_dalpha = dot / (1.f - alpha + 1e-5f);
+			float da_dE = 0.f, dE_dsdf = 0.f, dE_dinvs = 0.f, da_dP = 0.f, dP_dinvs = 0.f, dP_dcos = 0.f, dE_dcos = 0.f;
+			if (!(sm.p_div_c <= 0.f || sm.p_div_c >= 1.f)) {
+				const float P = __expf(sm.inv_s * sm.iter_cos * sm.dt);
+				const float E = __expf(-sm.next_sdf * sm.inv_s);
+				const float a = 1.f + E, b = 1.f + P * E, cc = 1e-5f + 1.f / (1.f + P * E);
+				const float delta = a * (b * b) * (cc * cc);
+				da_dE = -(P / delta - 1.f / (a * a * cc));
+				da_dP = -E / delta;
+				dE_dsdf = -sm.inv_s * E;
+				dE_dinvs = -sm.next_sdf * E;
+				dP_dinvs = P * sm.iter_cos * sm.dt;
+				dP_dcos = P * sm.inv_s * sm.dt;
+				dE_dcos = -sm.inv_s * E * sm.dt * 0.5f;
+			}
+			const float dloss_dinvs = dloss_dalpha * (da_dE * dE_dinvs + da_dP * dP_dinvs);
+			const float dloss_dvar = dloss_dinvs * sm.inv_s * 10.f;
+			const float dcos = sm.true_cos >= 0.f ? 0.f : 1.f;
+			const float gnorm = sqrtf(sm.n[0] * sm.n[0] + sm.n[1] * sm.n[1] + sm.n[2] * sm.n[2] + 1e-6f);
+			const float ek = c.ek_loss_weight * 2.f * c.loss_scale * (1.f - 1.f / gnorm);
+			const float dnorm = loss_scale * dloss_dalpha * (da_dE * dE_dcos + dP_dcos * da_dP) * dcos;
+			half8 lo, hi;
+#pragma unroll
+			for (int k = 0; k < 3; ++k) lo[k] = (hf)(loss_scale * (w * grad[k] * sm.rgb[k] * (1.f - sm.rgb[k])));
+			lo[3] = (hf)(loss_scale * dloss_dalpha * da_dE * dE_dsdf);
+			lo[4] = (hf)(ek * sm.n[0]); lo[5] = (hf)(ek * sm.n[1]); lo[6] = (hf)(ek * sm.n[2]);
+			lo[7] = (hf)(loss_scale * dloss_dvar);
+			hi[0] = (hf)(dnorm * dir[0]); hi[1] = (hf)(dnorm * dir[1]); hi[2] = (hf)(dnorm * dir[2]);
+#pragma unroll
+			for (int k = 3; k < 8; ++k) hi[k] = (hf)0;
+			hf* g = dloss + ((size_t)cb + s) * 16;
+			*reinterpret_cast<half8*>(g) = lo;
+			*reinterpret_cast<half8*>(g + 8) = hi;
+			const float* ci = coords + ((size_t)base + s) * 7;
+			float* co = coords_out + ((size_t)cb + s) * 7;
+#pragma unroll
+			for (int k = 0; k < 7; ++k) co[k] = ci[k];
+		}
+		T = __shfl(Ta, 63);
+		p0 = __shfl(q0, 63); p1 = __shfl(q1, 63); p2 = __shfl(q2, 63);
+	}
+}
+
+template <typename T, bool RESCALE>
+__global__ void __launch_bounds__(256) fill_rollover_kernel(uint32_t n_total, uint32_t stride, const uint32_t* __restrict__ n_in_ptr,
+                                                            T* __restrict__ inout) {
+	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+	const uint32_t n_in = *n_in_ptr;
+	const size_t lim = (size_t)n_in * stride;
+	if (n_in == 0 || i < lim || i >= (size_t)n_total * stride) return;
+	T r = inout[i % lim];
+	if (RESCALE) r = (T)((float)r * (float)n_in / (float)n_total);
+	inout[i] = r;
+}
+
+// ----------------------------------------------------------------------------
+static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
+
+N2_API uint64_t n2_composite_workspace_bytes(uint32_t max_rays) {
+	return up256(sizeof(RayScratch) * (uint64_t)max_rays) + 2 * up256(4ull * max_rays);
+}
+
+N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
+                             const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                             const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                             uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                             float* d_loss, void* d_workspace, uint64_t workspace_bytes) {
+	N2_REQUIRE(cfg != nullptr, "n2_composite_loss: config is null");
+	N2_REQUIRE(d_compacted_counter != nullptr, "n2_composite_loss: d_compacted_counter is null");
+	hipStream_t s = n2_stream(stream);
+	if (n_rays == 0) return n2_set_u32(s, d_compacted_counter, 0u);
+	N2_REQUIRE(d_numsteps && d_network_output && d_coords && d_rgb_target && d_coords_compacted && d_dloss_doutput && d_workspace,
+	           "n2_composite_loss: null buffer");
+	N2_REQUIRE(cfg->n_rays_norm > 0 && cfg->loss_scale > 0.f, "n2_composite_loss: n_rays_norm and loss_scale must be positive");
+	N2_REQUIRE(workspace_bytes >= n2_composite_workspace_bytes(n_rays), "n2_composite_loss: workspace of %llu bytes, %llu needed",
+	           (unsigned long long)workspace_bytes, (unsigned long long)n2_composite_workspace_bytes(n_rays));
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_network_output) % 16 == 0 && reinterpret_cast<uintptr_t>(d_dloss_doutput) % 16 == 0 &&
+	           reinterpret_cast<uintptr_t>(d_workspace) % 16 == 0, "n2_composite_loss: fp16 buffers and workspace must be 16-byte aligned");
+	CompParams c;
+	c.loss_scale = cfg->loss_scale; c.ek_loss_weight = cfg->ek_loss_weight; c.anneal = cfg->cos_anneal_ratio;
+	c.bg[0] = cfg->background[0]; c.bg[1] = cfg->background[1]; c.bg[2] = cfg->background[2];
+	c.inv_n_rays = 1.f / (float)cfg->n_rays_norm;
+	c.min_step = 1.73205080757f / 1024.f;  // STEPSIZE(), src/testbed_nerf.cu:51-53
+	c.max_step = c.min_step * 128.f;       // * 2^(NERF_CASCADES-1), unwarp_dt :617-620
+	unsigned char* w = reinterpret_cast<unsigned char*>(d_workspace);
+	RayScratch* scratch = reinterpret_cast<RayScratch*>(w);
+	uint32_t* cbase = reinterpret_cast<uint32_t*>(w + up256(sizeof(RayScratch) * (uint64_t)n_rays));
+	uint32_t* ckept = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(cbase) + up256(4ull * n_rays));
+	const dim3 grid((n_rays + CB / 64 - 1) / (CB / 64)), block(CB);
+	const hf* out = reinterpret_cast<const hf*>(d_network_output);
+	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch);
+	N2_LAUNCH_CHECK();
+	composite_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples_compacted, scratch, cbase, ckept, d_compacted_counter);
+	N2_LAUNCH_CHECK();
+	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, cbase, ckept,
+	                                                 d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API int n2_fill_rollover_f32(n2_stream_t stream, uint32_t n_total, uint32_t stride, const uint32_t* d_n_in, float* d_inout) {
+	N2_REQUIRE(d_n_in && d_inout, "n2_fill_rollover_f32: null buffer");
+	const size_t n = (size_t)n_total * stride;
+	if (n == 0) return N2_OK;
+	fill_rollover_kernel<float, false><<<dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, n2_stream(stream)>>>(n_total, stride, d_n_in, d_inout);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API int n2_fill_rollover_and_rescale_f16(n2_stream_t stream, uint32_t n_total, uint32_t stride, const uint32_t* d_n_in, n2_half* d_inout) {
+	N2_REQUIRE(d_n_in && d_inout, "n2_fill_rollover_and_rescale_f16: null buffer");
+	const size_t n = (size_t)n_total * stride;
+	if (n == 0) return N2_OK;
+	fill_rollover_kernel<hf, true><<<dim3((uint32_t)((n + 255) / 256)), dim3(256), 0, n2_stream(stream)>>>(n_total, stride, d_n_in,
+		reinterpret_cast<hf*>(d_inout));
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

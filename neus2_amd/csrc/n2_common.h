@@ -57,3 +57,5 @@ static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hip
 
 // Zero-fill with a kernel (safe to record into HIP graphs, unlike memset nodes).
 int n2_fill_zero_u32(hipStream_t stream, void* d_ptr, size_t n_bytes);
+// Store one 32-bit value with a one-thread kernel.
+int n2_set_u32(hipStream_t stream, uint32_t* d_ptr, uint32_t value);

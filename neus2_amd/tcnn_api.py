@@ -316,3 +316,48 @@ class Adam:
         check(capi.lib().n2_adam_step(_stream(), C.byref(self.cfg), C.c_uint32(n), C.c_uint32(self.n_matrix_params),
                                       C.c_float(loss_scale), ptr(self.master), ptr(params), ptr(gradients),
                                       ptr(self.m1), ptr(self.m2), ptr(self.steps)), "n2_adam_step")
+
+
+def composite_loss(numsteps, network_output, coords, rgb_target, max_samples_compacted, n_rays_norm=None,
+                   loss_scale=128.0, ek_loss_weight=0.01, cos_anneal_ratio=1.0, background=(0.0, 0.0, 0.0),
+                   ray_counter=None, want_loss=True):
+    """compute_loss_kernel_train_nerf_with_global_movement (src/testbed_nerf.cu:1465-1996), static path.
+    numsteps: int32/uint32 [n_rays, 2] (updated in place); network_output fp16 [S, 16]; coords fp32 [S, 7];
+    rgb_target fp32 [n_rays, 3].  Returns dict(counter, coords, dloss, loss)."""
+    n_rays = numsteps.shape[0]
+    dev_ = network_output.device
+    _check_half(network_output, (network_output.shape[0], 16), "network_output")
+    if coords.dtype != torch.float32 or tuple(coords.shape) != (network_output.shape[0], 7) or not coords.is_contiguous():
+        raise N2Error("coords must be contiguous fp32 [S, 7]")
+    if rgb_target.dtype != torch.float32 or tuple(rgb_target.shape) != (n_rays, 3) or not rgb_target.is_contiguous():
+        raise N2Error("rgb_target must be contiguous fp32 [n_rays, 3]")
+    if numsteps.dtype != torch.int32 or not numsteps.is_contiguous() or tuple(numsteps.shape) != (n_rays, 2):
+        raise N2Error("numsteps must be contiguous int32 [n_rays, 2]")
+    cfg = capi.CompositeConfig(loss_scale, ek_loss_weight, cos_anneal_ratio, (C.c_float * 3)(*background),
+                               n_rays if n_rays_norm is None else n_rays_norm)
+    nbytes = int(capi.lib().n2_composite_workspace_bytes(C.c_uint32(max(n_rays, 1))))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev_)
+    counter = torch.zeros(1, dtype=torch.int32, device=dev_)
+    cout = torch.zeros((max_samples_compacted, 7), dtype=torch.float32, device=dev_)
+    dloss = torch.zeros((max_samples_compacted, 16), dtype=torch.float16, device=dev_)
+    loss = torch.zeros(n_rays, dtype=torch.float32, device=dev_) if want_loss else None
+    check(capi.lib().n2_composite_loss(_stream(), C.byref(cfg), C.c_uint32(n_rays), ptr(ray_counter), ptr(numsteps),
+                                       ptr(network_output), ptr(coords), ptr(rgb_target),
+                                       C.c_uint32(max_samples_compacted), ptr(counter), ptr(cout), ptr(dloss), ptr(loss),
+                                       ptr(ws), C.c_uint64(nbytes)), "n2_composite_loss")
+    return dict(counter=counter, coords=cout, dloss=dloss, loss=loss)
+
+
+def fill_rollover(inout, n_in):
+    """tcnn fill_rollover (fp32) / fill_rollover_and_rescale (fp16) on a [n_total, stride] tensor, in place;
+    n_in is a device int32 scalar tensor (the compacted counter)."""
+    n_total, stride = inout.shape[0], (inout.shape[1] if inout.dim() > 1 else 1)
+    if inout.dtype == torch.float32:
+        check(capi.lib().n2_fill_rollover_f32(_stream(), C.c_uint32(n_total), C.c_uint32(stride), ptr(n_in), ptr(inout)),
+              "n2_fill_rollover_f32")
+    elif inout.dtype == torch.float16:
+        check(capi.lib().n2_fill_rollover_and_rescale_f16(_stream(), C.c_uint32(n_total), C.c_uint32(stride), ptr(n_in),
+                                                          ptr(inout)), "n2_fill_rollover_and_rescale_f16")
+    else:
+        raise N2Error("fill_rollover supports float32 and float16")
+    return inout

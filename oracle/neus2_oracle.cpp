@@ -557,3 +557,180 @@ ORC_API void orc_adam_step(uint32_t n, uint32_t n_matrix_params, float loss_scal
 		w[i] -= lr_eff * a / (sqrtf(b) + eps);
 	}
 }
+
+// ---------------------------------------------------------------------------
+// NeuS alpha compositing + loss + hand-derived backward, one ray at a time:
+// compute_loss_kernel_train_nerf_with_global_movement, src/testbed_nerf.cu:1465-1996,
+// restricted to the static path (no global movement, no envmap, no exposure /
+// depth / mask supervision, Logistic colour activation, Huber(0.1)/5 loss,
+// BENT_DIR 1, NORMAL_VECTORS_NORMALIZED 0).
+//
+// The reference allocates the compacted range of a ray with atomicAdd, so the
+// order of rays in the compacted batch is a race; here the ranges are handed
+// out in ray order (one of the orders the reference can produce).
+//
+//  numsteps   [n_rays][2] in: (samples, first sample); out: (compacted samples, compacted first)
+//  net_out    [*][16]  network output per marched sample (values as stored in fp16)
+//  coords     [*][7]   NerfCoordinate per marched sample
+//  rgb_target [n_rays][3]
+//  dloss      [max_compacted][16] out (rows 11..15 are left unset by the reference; zero here)
+//  coords_out [max_compacted][7] out
+//  loss       [n_rays] out: mean over channels / n_rays_norm        (testbed_nerf.cu:1717-1719)
+//  counter    out: total number of samples the rays wanted to keep (may exceed max_compacted)
+// ---------------------------------------------------------------------------
+struct CompositeCfg {
+	float loss_scale;        // LOSS_SCALE = 128, testbed.h:237
+	float ek_loss_weight;    // hyperparams.ek_loss_weight
+	float cos_anneal_ratio;  // nerf_network.h:1109-1118 (1 when anneal_end = 0)
+	float background[3];
+	uint32_t n_rays_norm;    // n_rays_per_batch: what loss and gradients are divided by (:1756)
+	float min_step;          // MIN_CONE_STEPSIZE = sqrt(3)/1024 (:52-53)
+	float max_step;          // MIN_CONE_STEPSIZE * 2^(NERF_CASCADES-1): unwarp_dt (:617-620)
+	int exact_inv_s;         // 0: 10*variance is formed in fp16 as in the reference (:1581); 1: in fp32 (smooth, for finite differences)
+};
+
+static inline float logistic(float x) { return 1.f / (1.f + expf(-x)); }
+
+struct SampleAlpha {
+	float alpha, p_div_c, iter_cos, true_cos, inv_s, sdf, dt, next_sdf;
+	float rgb[3], n[3];
+};
+
+static inline SampleAlpha sample_alpha(const float* o, float warped_dt, const float* dir, const CompositeCfg& c) {
+	SampleAlpha s;
+	s.dt = warped_dt * (c.max_step - c.min_step) + c.min_step;  // unwarp_dt
+	for (int k = 0; k < 3; ++k) { s.rgb[k] = logistic(o[k]); s.n[k] = o[4 + k]; }
+	s.inv_s = expf(c.exact_inv_s ? 10.f * o[7] : round_fp16(10.f * o[7]));  // the product is formed in fp16 (:1581)
+	s.sdf = o[3];
+	s.true_cos = dir[0] * s.n[0] + dir[1] * s.n[1] + dir[2] * s.n[2];
+	const float a = std::max(-s.true_cos * 0.5f + 0.5f, 0.f), b = std::max(-s.true_cos, 0.f);
+	s.iter_cos = -(a * (1.f - c.cos_anneal_ratio) + b * c.cos_anneal_ratio);
+	s.next_sdf = s.sdf + s.iter_cos * s.dt * 0.5f;
+	const float prev_sdf = s.sdf - s.iter_cos * s.dt * 0.5f;
+	const float next_cdf = logistic(s.next_sdf * s.inv_s), prev_cdf = logistic(prev_sdf * s.inv_s);
+	s.p_div_c = (prev_cdf - next_cdf + 1e-5f) / (prev_cdf + 1e-5f);
+	s.alpha = std::min(std::max(s.p_div_c, 0.f), 1.f);
+	return s;
+}
+
+ORC_API void orc_composite_loss(const CompositeCfg* cfg, uint32_t n_rays, uint32_t* numsteps, const float* net_out, const float* coords,
+                                const float* rgb_target, uint32_t max_compacted, float* dloss, float* coords_out, float* loss,
+                                uint32_t* counter, float* rgb_ray_out /* optional [n_rays][3] */) {
+	const CompositeCfg c = *cfg;
+	const float EPSILON = 1e-4f;
+	std::vector<uint32_t> kept(n_rays);
+	std::vector<float> rgb_ray_all((size_t)n_rays * 3);
+	// first pass (:1562-1617): composite until the transmittance drops below 1e-4
+	#pragma omp parallel for schedule(dynamic, 16)
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		const uint32_t n = numsteps[2 * i], base = numsteps[2 * i + 1];
+		float T = 1.f, rgb_ray[3] = {0, 0, 0}, dir[3] = {0, 0, 0};
+		uint32_t j = 0;
+		for (; j < n; ++j) {
+			if (T < EPSILON) break;
+			const float* o = net_out + (size_t)(base + j) * 16;
+			if (j == 0) {  // BENT_DIR: direction carried by the first sample's output rows 8..10 (:1574-1579)
+				float d[3] = {o[8] * 2.f - 1.f, o[9] * 2.f - 1.f, o[10] * 2.f - 1.f};
+				const float len = sqrtf(d[0] * d[0] + d[1] * d[1] + d[2] * d[2]);
+				for (int k = 0; k < 3; ++k) dir[k] = d[k] / len;
+			}
+			const SampleAlpha s = sample_alpha(o, coords[(size_t)(base + j) * 7 + 3], dir, c);
+			const float w = s.alpha * T;
+			for (int k = 0; k < 3; ++k) rgb_ray[k] += w * s.rgb[k];
+			T *= (1.f - s.alpha);
+		}
+		if (j == n) for (int k = 0; k < 3; ++k) rgb_ray[k] += T * c.background[k];  // (:1664-1667)
+		kept[i] = j;
+		for (int k = 0; k < 3; ++k) rgb_ray_all[(size_t)i * 3 + k] = rgb_ray[k];
+		if (rgb_ray_out) for (int k = 0; k < 3; ++k) rgb_ray_out[(size_t)i * 3 + k] = rgb_ray[k];
+	}
+	// compaction ranges in ray order (:1673-1679)
+	std::vector<uint32_t> cbase(n_rays);
+	uint64_t run = 0;
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		cbase[i] = (uint32_t)std::min<uint64_t>(run, 0xFFFFFFFFull);
+		run += kept[i];
+	}
+	*counter = (uint32_t)std::min<uint64_t>(run, 0xFFFFFFFFull);
+	// second pass (:1767-1952)
+	#pragma omp parallel for schedule(dynamic, 16)
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		const uint32_t base = numsteps[2 * i + 1];
+		const uint32_t cb = cbase[i];
+		const uint32_t m = std::min(max_compacted - std::min(max_compacted, cb), kept[i]);
+		numsteps[2 * i] = m;
+		numsteps[2 * i + 1] = cb;
+		const float* rgb_ray = &rgb_ray_all[(size_t)i * 3];
+		// Huber(0.1)/5 per channel (:301-317, 1459)
+		float grad[3], lsum = 0.f;
+		for (int k = 0; k < 3; ++k) {
+			const float d = rgb_ray[k] - rgb_target[(size_t)i * 3 + k], ad = fabsf(d), al = 0.1f;
+			lsum += (ad > al ? ad - 0.5f * al : 0.5f / al * d * d) / 5.f;
+			grad[k] = (ad > al ? (d > 0 ? 1.f : -1.f) : d / al) / 5.f;
+		}
+		if (loss) loss[i] = m == 0 ? 0.f : lsum / 3.f / (float)c.n_rays_norm;
+		if (m == 0) continue;
+		const float loss_scale = c.loss_scale / (float)c.n_rays_norm;
+		float T = 1.f, rgb_ray2[3] = {0, 0, 0}, dir[3] = {0, 0, 0};
+		for (uint32_t j = 0; j < m; ++j) {
+			const float* o = net_out + (size_t)(base + j) * 16;
+			if (j == 0) {
+				float d[3] = {o[8] * 2.f - 1.f, o[9] * 2.f - 1.f, o[10] * 2.f - 1.f};
+				const float len = sqrtf(d[0] * d[0] + d[1] * d[1] + d[2] * d[2]);
+				for (int k = 0; k < 3; ++k) dir[k] = d[k] / len;
+			}
+			for (int k = 0; k < 7; ++k) coords_out[(size_t)(cb + j) * 7 + k] = coords[(size_t)(base + j) * 7 + k];
+			const SampleAlpha s = sample_alpha(o, coords[(size_t)(base + j) * 7 + 3], dir, c);
+			const float w = s.alpha * T;
+			for (int k = 0; k < 3; ++k) rgb_ray2[k] += w * s.rgb[k];
+			T *= (1.f - s.alpha);
+			float dot = 0.f;
+			for (int k = 0; k < 3; ++k) dot += grad[k] * (T * s.rgb[k] - (rgb_ray[k] - rgb_ray2[k]));
+			const float dloss_dalpha = dot / (1.f - s.alpha + 1e-5f);  // mask term is zero at mask_loss_weight = 0
+			float da_dE = 0, dE_dsdf = 0, dE_dinvs = 0, da_dP = 0, dP_dinvs = 0, dP_dcos = 0, dE_dcos = 0;
+			if (!(s.p_div_c <= 0.f || s.p_div_c >= 1.f)) {  // (:1843-1873)
+				const float P = expf(s.inv_s * s.iter_cos * s.dt);
+				const float E = expf(-s.next_sdf * s.inv_s);
+				const float a = 1.f + E, b = 1.f + P * E, cc = 1e-5f + 1.f / (1.f + P * E);
+				const float delta = a * (b * b) * (cc * cc);
+				da_dE = -(P / delta - 1.f / (a * a * cc));
+				da_dP = -E / delta;
+				dE_dsdf = -s.inv_s * E;
+				dE_dinvs = -s.next_sdf * E;
+				dP_dinvs = P * s.iter_cos * s.dt;
+				dP_dcos = P * s.inv_s * s.dt;
+				dE_dcos = -s.inv_s * E * s.dt * 0.5f;
+			}
+			const float dloss_dinvs = dloss_dalpha * (da_dE * dE_dinvs + da_dP * dP_dinvs);
+			const float dloss_dvariance = dloss_dinvs * s.inv_s * 10.f;
+			const float dcos_dtrue = s.true_cos >= 0.f ? 0.f : 1.f;  // the anneal ratio is ignored here (:1881-1887)
+			const float gnorm = sqrtf(s.n[0] * s.n[0] + s.n[1] * s.n[1] + s.n[2] * s.n[2] + 1e-6f);
+			const float ek = 1.f - 1.f / gnorm;
+			const float dloss_dnormal = dloss_dalpha * (da_dE * dE_dcos + dP_dcos * da_dP) * dcos_dtrue;
+			const float dloss_dsdf = dloss_dalpha * da_dE * dE_dsdf;
+			float* g = dloss + (size_t)(cb + j) * 16;
+			for (int k = 0; k < 3; ++k) {
+				const float sg = logistic(o[k]);
+				g[k] = loss_scale * (w * grad[k] * sg * (1.f - sg));
+			}
+			g[3] = loss_scale * dloss_dsdf;
+			for (int k = 0; k < 3; ++k) g[4 + k] = c.ek_loss_weight * 2.f * c.loss_scale * ek * s.n[k];
+			g[7] = loss_scale * dloss_dvariance;
+			for (int k = 0; k < 3; ++k) g[8 + k] = loss_scale * dloss_dnormal * dir[k];
+			for (int k = 11; k < 16; ++k) g[k] = 0.f;
+		}
+	}
+}
+
+// fill_rollover / fill_rollover_and_rescale (tcnn; call sites src/testbed_nerf.cu:3908-3916): pad a
+// compacted batch of n_in rows (stride floats each) to n_total rows by wrapping around; the
+// wrapped copies are scaled by n_in/n_total when rescale != 0.
+ORC_API void orc_fill_rollover(uint32_t n_total, uint32_t stride, uint32_t n_in, float* inout, int rescale) {
+	if (n_in == 0 || n_in >= n_total) return;
+	const size_t lim = (size_t)n_in * stride;
+	for (size_t i = lim; i < (size_t)n_total * stride; ++i) {
+		float r = inout[i % lim];
+		if (rescale) r = r * (float)n_in / (float)n_total;
+		inout[i] = r;
+	}
+}

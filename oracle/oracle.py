@@ -188,3 +188,40 @@ def adam_step(w, grad, m1, m2, steps, n_matrix_params, loss_scale=128.0, lr=1e-3
     lib().orc_adam_step(C.c_uint32(w.size), C.c_uint32(n_matrix_params), C.c_float(loss_scale), C.c_float(lr),
                         C.c_float(beta1), C.c_float(beta2), C.c_float(eps), C.c_float(l2_reg), _fp(w), _fp(grad),
                         _fp(m1), _fp(m2), _up(steps))
+
+
+class CompositeCfg(C.Structure):
+    _fields_ = [("loss_scale", C.c_float), ("ek_loss_weight", C.c_float), ("cos_anneal_ratio", C.c_float),
+                ("background", C.c_float * 3), ("n_rays_norm", C.c_uint32), ("min_step", C.c_float),
+                ("max_step", C.c_float), ("exact_inv_s", C.c_int)]
+
+
+MIN_STEP = float(np.float32(1.73205080757) / np.float32(1024))  # STEPSIZE(), src/testbed_nerf.cu:51-53
+MAX_STEP = float(np.float32(MIN_STEP) * np.float32(128))        # * 2^(NERF_CASCADES-1)
+
+
+def composite_loss(numsteps, net_out, coords, rgb_target, max_compacted, n_rays_norm=None, loss_scale=128.0,
+                   ek_loss_weight=0.01, cos_anneal_ratio=1.0, background=(0.0, 0.0, 0.0), exact_inv_s=False):
+    """numsteps [n_rays, 2] uint32 (count, base); net_out [S, 16]; coords [S, 7]; rgb_target [n_rays, 3].
+    Returns dict(numsteps, dloss [max_compacted,16], coords [max_compacted,7], loss [n_rays], counter, rgb_ray)."""
+    numsteps = np.ascontiguousarray(numsteps, np.uint32).copy()
+    n_rays = numsteps.shape[0]
+    net_out, coords, rgb_target = _f32(net_out), _f32(coords), _f32(rgb_target)
+    cfg = CompositeCfg(loss_scale, ek_loss_weight, cos_anneal_ratio, (C.c_float * 3)(*background),
+                       n_rays if n_rays_norm is None else n_rays_norm, MIN_STEP, MAX_STEP, int(exact_inv_s))
+    dloss = np.zeros((max_compacted, 16), np.float32)
+    cout = np.zeros((max_compacted, 7), np.float32)
+    loss = np.zeros(n_rays, np.float32)
+    rgb_ray = np.zeros((n_rays, 3), np.float32)
+    counter = C.c_uint32(0)
+    lib().orc_composite_loss(C.byref(cfg), C.c_uint32(n_rays), _up(numsteps), _fp(net_out), _fp(coords), _fp(rgb_target),
+                             C.c_uint32(max_compacted), _fp(dloss), _fp(cout), _fp(loss), C.byref(counter), _fp(rgb_ray))
+    return dict(numsteps=numsteps, dloss=dloss, coords=cout, loss=loss, counter=int(counter.value), rgb_ray=rgb_ray)
+
+
+def fill_rollover(a, n_in, rescale=False):
+    """a: [n_total, stride] float32, in place."""
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    lib().orc_fill_rollover(C.c_uint32(a.shape[0]), C.c_uint32(a.shape[1] if a.ndim > 1 else 1), C.c_uint32(n_in), _fp(a),
+                            C.c_int(int(rescale)))
+    return a
