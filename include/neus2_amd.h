@@ -335,6 +335,43 @@ int n2_fill_rollover_f32(n2_stream_t stream, uint32_t n_total, uint32_t stride, 
 int n2_fill_rollover_and_rescale_f16(n2_stream_t stream, uint32_t n_total, uint32_t stride, const uint32_t* d_n_in,
                                      n2_half* d_inout);
 
+/* ------------------------------------------------------------------------
+ * Training-sample generator: one pixel per ray, ray/unit-cube intersection, march through the
+ * 128^3 morton-ordered occupancy bitfield with the fixed step sqrt(3)/1024, one NerfCoordinate per
+ * occupied step: generate_training_samples_nerf_with_global_movement,
+ * src/testbed_nerf.cu:1253-1446 (static path, cone_angle_constant = 0, unit aabb).
+ * Random draws come from a counter-based hash (tcnn's pcg32 is not part of the reference
+ * checkout); sample ranges and ray slots are handed out in ray order, not by atomicAdd.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_camera {
+	float xform[12];          /* row-major 3x4 camera-to-world [R | origin] (TrainingXForm::start) */
+	float focal_length[2];    /* pixels (TrainingImageMetadata::focal_length) */
+	float principal_point[2]; /* fraction of the image (0.5 = centre) */
+	uint32_t resolution[2];
+	uint32_t pixel_offset_lo; /* index of the image's first pixel in the RGBA array, low / high word */
+	uint32_t pixel_offset_hi;
+} n2_camera;
+
+uint64_t n2_sampler_workspace_bytes(uint32_t max_rays);
+
+/*  n_rays            rays to try (n_rays_per_batch);  n_rays_total: rays drawn in earlier steps (image rotation)
+ *  d_cameras         n_images cameras;  d_rgba fp32 [pixels][4] premultiplied-alpha training images
+ *  background        colour behind transparent pixels (host array of 3)
+ *  d_bitfield        occupancy bits of mip 0: 128^3/8 bytes, bit (idx%8) of byte idx/8, idx = morton3D(x,y,z)
+ *                    (grid_to_bitfield, src/testbed_nerf.cu:738-759)
+ *  max_samples       capacity of d_coords; rays from the first one that does not fit are dropped
+ *  d_ray_counter     out: live rays;  d_sample_counter out: samples all rays with >= 1 step asked for
+ *  d_ray_indices     out uint32 [n_rays]: original ray id per live slot
+ *  d_numsteps        out uint32 [n_rays][2]: (samples, first sample) per live slot
+ *  d_rgb_target      out fp32 [n_rays][3]: pixel colour composited over the background
+ *  d_coords          out fp32 [max_samples][7] */
+int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
+                                 const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
+                                 const float background[3], const uint8_t* d_bitfield, uint32_t max_samples,
+                                 uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices,
+                                 uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
+                                 uint64_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

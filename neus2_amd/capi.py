@@ -35,6 +35,12 @@ class CompositeConfig(C.Structure):
                 ("background", C.c_float * 3), ("n_rays_norm", C.c_uint32)]
 
 
+class Camera(C.Structure):
+    """struct n2_camera"""
+    _fields_ = [("xform", C.c_float * 12), ("focal_length", C.c_float * 2), ("principal_point", C.c_float * 2),
+                ("resolution", C.c_uint32 * 2), ("pixel_offset_lo", C.c_uint32), ("pixel_offset_hi", C.c_uint32)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 
@@ -66,6 +72,8 @@ def lib():
         _lib.n2_field_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
         _lib.n2_composite_workspace_bytes.restype = C.c_uint64
         _lib.n2_composite_workspace_bytes.argtypes = [C.c_uint32]
+        _lib.n2_sampler_workspace_bytes.restype = C.c_uint64
+        _lib.n2_sampler_workspace_bytes.argtypes = [C.c_uint32]
         _lib.n2_field_destroy.restype = None
         _lib.n2_field_destroy.argtypes = [C.c_void_p]
     return _lib

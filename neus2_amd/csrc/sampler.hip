@@ -1,0 +1,243 @@
+// Training-sample generator: pixel pick, ray / unit-cube intersection and the
+// march through the occupancy bitfield.  One thread per ray (a ray is a serial,
+// data-dependent walk); three kernels: count steps, exclusive scan in ray order,
+// emit coordinates.
+//
+// Sample positions are part of the bit-exact contract with the CPU oracle, so
+// floating-point contraction is switched off for this file and every fused
+// operation is spelled out.
+#include "n2_common.h"
+
+#pragma clang fp contract(off)
+
+constexpr float STEP = 1.73205080757f / 1024.f;  // STEPSIZE(), src/testbed_nerf.cu:51-53
+constexpr uint32_t GRIDSIZE = 128, MARCH_STEPS = 1024;
+
+__device__ __forceinline__ uint32_t hash_u32(uint32_t seed, uint32_t ctr) {
+	uint32_t x = ctr * 747796405u + seed * 2891336453u + 1u;
+	x = ((x >> ((x >> 28) + 4u)) ^ x) * 277803737u;
+	x = (x >> 22) ^ x;
+	x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+	return x;
+}
+__device__ __forceinline__ float rand01(uint32_t seed, uint32_t ray, uint32_t k) {
+	return (float)(hash_u32(seed, ray * 8u + k) >> 8) * (1.0f / 16777216.0f);
+}
+__device__ __forceinline__ uint32_t expand_bits(uint32_t v) {
+	v = (v * 0x00010001u) & 0xFF0000FFu;
+	v = (v * 0x00000101u) & 0x0F00F00Fu;
+	v = (v * 0x00000011u) & 0xC30C30C3u;
+	v = (v * 0x00000005u) & 0x49249249u;
+	return v;
+}
+__device__ __forceinline__ bool occupied(const uint8_t* __restrict__ bitfield, const float* pos) {
+	int c[3];
+#pragma unroll
+	for (int d = 0; d < 3; ++d) {
+		float p = pos[d] - 0.5f;
+		p = p * 1.0f;
+		p = p + 0.5f;
+		const int i = (int)(p * (float)GRIDSIZE);
+		c[d] = min(max(i, 0), (int)GRIDSIZE - 1);
+	}
+	const uint32_t idx = expand_bits((uint32_t)c[0]) | (expand_bits((uint32_t)c[1]) << 1) | (expand_bits((uint32_t)c[2]) << 2);
+	return (bitfield[idx / 8] >> (idx % 8)) & 1;
+}
+__device__ __forceinline__ float to_next_voxel(const float* pos, const float* dir, const float* idir) {
+	float t = 3.4e38f;
+#pragma unroll
+	for (int d = 0; d < 3; ++d) {
+		const float p = (float)GRIDSIZE * pos[d];
+		const float sgn = copysignf(1.0f, dir[d]);
+		const float td = (floorf(p + 0.5f + 0.5f * sgn) - p) * idir[d];
+		t = fminf(t, td);
+	}
+	return fmaxf(__fdiv_rn(t, (float)GRIDSIZE), 0.0f);
+}
+
+struct RaySetup {
+	bool alive;
+	float o[3], dir[3], idir[3], startt, target[3];
+};
+
+__device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
+                                              const n2_camera* __restrict__ cams, uint32_t n_images, const float* __restrict__ rgba,
+                                              float bg0, float bg1, float bg2) {
+	RaySetup r;
+	const uint32_t img = (((i + n_rays_total) * n_images) / n_rays) % n_images;
+	const n2_camera c = cams[img];
+	const float u0 = rand01(seed, i, 0), u1 = rand01(seed, i, 1);
+	const int px = min(max((int)(u0 * (float)c.resolution[0]), 0), (int)c.resolution[0] - 1);
+	const int py = min(max((int)(u1 * (float)c.resolution[1]), 0), (int)c.resolution[1] - 1);
+	const float x = __fdiv_rn((float)px + 0.5f, (float)c.resolution[0]), y = __fdiv_rn((float)py + 0.5f, (float)c.resolution[1]);
+	const uint64_t off = ((uint64_t)c.pixel_offset_hi << 32) | c.pixel_offset_lo;
+	const float4 pix = *reinterpret_cast<const float4*>(rgba + (off + (uint64_t)px + (uint64_t)py * c.resolution[0]) * 4);
+	if (pix.x <= 0.0f && rand01(seed, i, 2) >= 0.9f) {
+		r.alive = false;
+		return r;
+	}
+	const float bg[3] = {bg0, bg1, bg2};
+	const float pc[3] = {pix.x, pix.y, pix.z};
+#pragma unroll
+	for (int k = 0; k < 3; ++k) r.target[k] = pc[k] + (1.0f - pix.w) * bg[k];
+	const float d[3] = {__fdiv_rn((x - c.principal_point[0]) * (float)c.resolution[0], c.focal_length[0]),
+	                    __fdiv_rn((y - c.principal_point[1]) * (float)c.resolution[1], c.focal_length[1]), 1.0f};
+	float w[3];
+#pragma unroll
+	for (int k = 0; k < 3; ++k) {
+		w[k] = __fmaf_rn(c.xform[k * 4 + 2], d[2], __fmaf_rn(c.xform[k * 4 + 1], d[1], c.xform[k * 4 + 0] * d[0]));
+		r.o[k] = c.xform[k * 4 + 3];
+	}
+	const float len = sqrtf(__fmaf_rn(w[2], w[2], __fmaf_rn(w[1], w[1], w[0] * w[0])));
+#pragma unroll
+	for (int k = 0; k < 3; ++k) { r.dir[k] = __fdiv_rn(w[k], len); r.idir[k] = __fdiv_rn(1.0f, r.dir[k]); }
+	float tmin = __fdiv_rn(0.f - r.o[0], r.dir[0]), tmax = __fdiv_rn(1.f - r.o[0], r.dir[0]);
+	if (tmin > tmax) { const float t = tmin; tmin = tmax; tmax = t; }
+	bool hit = true;
+	for (int k = 1; k < 3 && hit; ++k) {
+		float a = __fdiv_rn(0.f - r.o[k], r.dir[k]), b = __fdiv_rn(1.f - r.o[k], r.dir[k]);
+		if (a > b) { const float t = a; a = b; b = t; }
+		if (tmin > b || a > tmax) { hit = false; break; }
+		if (a > tmin) tmin = a;
+		if (b < tmax) tmax = b;
+	}
+	if (!hit) tmin = 3.402823466e38f;
+	tmin = fmaxf(tmin, 0.0f);
+	r.startt = __fmaf_rn(STEP, rand01(seed, i, 3), tmin);
+	r.alive = true;
+	return r;
+}
+
+template <bool EMIT>
+__device__ __forceinline__ uint32_t march(const RaySetup& r, const uint8_t* __restrict__ bitfield, float* __restrict__ coords, uint32_t max_emit) {
+	uint32_t j = 0;
+	float t = r.startt;
+	const uint32_t limit = EMIT ? max_emit : MARCH_STEPS;
+	while (j < limit) {
+		float pos[3];
+#pragma unroll
+		for (int k = 0; k < 3; ++k) pos[k] = __fmaf_rn(t, r.dir[k], r.o[k]);
+		if (!(pos[0] >= 0.f && pos[0] <= 1.f && pos[1] >= 0.f && pos[1] <= 1.f && pos[2] >= 0.f && pos[2] <= 1.f)) break;
+		if (occupied(bitfield, pos)) {
+			if (EMIT) {
+				float* c = coords + (size_t)j * 7;
+				c[0] = pos[0]; c[1] = pos[1]; c[2] = pos[2];
+				c[3] = 0.0f;
+#pragma unroll
+				for (int k = 0; k < 3; ++k) c[4 + k] = (r.dir[k] + 1.0f) * 0.5f;
+			}
+			++j;
+			t += STEP;
+		} else {
+			const float t_target = t + to_next_voxel(pos, r.dir, r.idir);
+			do { t += STEP; } while (t < t_target);
+		}
+	}
+	return j;
+}
+
+__global__ void __launch_bounds__(128) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+                                                            uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
+                                                            const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts) {
+	const uint32_t i = blockIdx.x * 128 + threadIdx.x;
+	if (i >= n_rays) return;
+	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
+	counts[i] = r.alive ? march<false>(r, bitfield, nullptr, 0) : 0u;
+}
+
+// base[i] = exclusive sum of counts; slot[i] = rank among rays that have samples and fit the budget
+__global__ void __launch_bounds__(1024) sampler_scan_kernel(uint32_t n_rays, uint32_t max_samples, const uint32_t* __restrict__ counts,
+                                                            uint32_t* __restrict__ base, uint32_t* __restrict__ slot,
+                                                            uint32_t* __restrict__ ray_counter, uint32_t* __restrict__ sample_counter) {
+	__shared__ uint32_t wt_a[16], wt_b[16];
+	__shared__ uint32_t carry_a, carry_b;
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	if (threadIdx.x == 0) { carry_a = 0; carry_b = 0; }
+	__syncthreads();
+	for (uint32_t r0 = 0; r0 < n_rays; r0 += 1024) {
+		const uint32_t r = r0 + threadIdx.x;
+		const uint32_t k = r < n_rays ? counts[r] : 0u;
+		uint32_t v = k;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(v, o); if (lane >= o) v += u; }
+		if (lane == 63) wt_a[wave] = v;
+		__syncthreads();
+		uint32_t before = carry_a;
+		for (int w = 0; w < wave; ++w) before += wt_a[w];
+		const uint32_t excl = before + v - k;
+		const uint32_t keep = (k > 0 && (uint64_t)excl + k <= max_samples) ? 1u : 0u;
+		uint32_t f = keep;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(f, o); if (lane >= o) f += u; }
+		if (lane == 63) wt_b[wave] = f;
+		__syncthreads();
+		uint32_t before_b = carry_b;
+		for (int w = 0; w < wave; ++w) before_b += wt_b[w];
+		if (r < n_rays) {
+			base[r] = excl;
+			slot[r] = keep ? before_b + f - 1u : 0xFFFFFFFFu;
+		}
+		__syncthreads();
+		if (threadIdx.x == 1023) { carry_a = excl + k; carry_b = before_b + f; }
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) { *ray_counter = carry_b; *sample_counter = carry_a; }
+}
+
+__global__ void __launch_bounds__(128) sampler_emit_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+                                                           uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
+                                                           const uint8_t* __restrict__ bitfield, const uint32_t* __restrict__ counts,
+                                                           const uint32_t* __restrict__ base, const uint32_t* __restrict__ slot,
+                                                           uint32_t* __restrict__ ray_indices, uint32_t* __restrict__ numsteps,
+                                                           float* __restrict__ rgb_target, float* __restrict__ coords) {
+	const uint32_t i = blockIdx.x * 128 + threadIdx.x;
+	if (i >= n_rays) return;
+	const uint32_t s = slot[i];
+	if (s == 0xFFFFFFFFu) return;
+	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
+	ray_indices[s] = i;
+	numsteps[2 * s] = counts[i];
+	numsteps[2 * s + 1] = base[i];
+	rgb_target[(size_t)s * 3 + 0] = r.target[0];
+	rgb_target[(size_t)s * 3 + 1] = r.target[1];
+	rgb_target[(size_t)s * 3 + 2] = r.target[2];
+	march<true>(r, bitfield, coords + (size_t)base[i] * 7, counts[i]);
+}
+
+static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
+
+N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays); }
+
+N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
+                                        const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
+                                        const float background[3], const uint8_t* d_bitfield, uint32_t max_samples,
+                                        uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices,
+                                        uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
+                                        uint64_t workspace_bytes) {
+	N2_REQUIRE(d_ray_counter && d_sample_counter, "n2_generate_training_samples: counters are null");
+	hipStream_t s = n2_stream(stream);
+	if (n_rays == 0) {
+		if (int rc = n2_set_u32(s, d_ray_counter, 0u)) return rc;
+		return n2_set_u32(s, d_sample_counter, 0u);
+	}
+	N2_REQUIRE(d_cameras && d_rgba && background && d_bitfield && d_ray_indices && d_numsteps && d_rgb_target && d_coords && d_workspace,
+	           "n2_generate_training_samples: null buffer");
+	N2_REQUIRE(n_images > 0, "n2_generate_training_samples: n_images must be positive");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_rgba) % 16 == 0, "n2_generate_training_samples: d_rgba must be 16-byte aligned");
+	N2_REQUIRE(workspace_bytes >= n2_sampler_workspace_bytes(n_rays), "n2_generate_training_samples: workspace of %llu bytes, %llu needed",
+	           (unsigned long long)workspace_bytes, (unsigned long long)n2_sampler_workspace_bytes(n_rays));
+	unsigned char* w = reinterpret_cast<unsigned char*>(d_workspace);
+	uint32_t* counts = reinterpret_cast<uint32_t*>(w);
+	uint32_t* base = reinterpret_cast<uint32_t*>(w + up256(4ull * n_rays));
+	uint32_t* slot = reinterpret_cast<uint32_t*>(w + 2 * up256(4ull * n_rays));
+	const dim3 grid((n_rays + 127) / 128), block(128);
+	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
+	                                            background[2], d_bitfield, counts);
+	N2_LAUNCH_CHECK();
+	sampler_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples, counts, base, slot, d_ray_counter, d_sample_counter);
+	N2_LAUNCH_CHECK();
+	sampler_emit_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
+	                                           background[2], d_bitfield, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}

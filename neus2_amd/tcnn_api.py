@@ -361,3 +361,39 @@ def fill_rollover(inout, n_in):
     else:
         raise N2Error("fill_rollover supports float32 and float16")
     return inout
+
+
+def pack_cameras(cams, device="cuda"):
+    """List of dicts (xform[12], focal[2], principal[2], res[2], pixel_offset) -> device byte tensor of n2_camera."""
+    arr = (capi.Camera * len(cams))()
+    for a, c in zip(arr, cams):
+        po = int(c["pixel_offset"])
+        a.xform[:] = [float(v) for v in c["xform"]]
+        a.focal_length[:] = [float(v) for v in c["focal"]]
+        a.principal_point[:] = [float(v) for v in c["principal"]]
+        a.resolution[:] = [int(v) for v in c["res"]]
+        a.pixel_offset_lo, a.pixel_offset_hi = po & 0xFFFFFFFF, po >> 32
+    raw = np.frombuffer(bytes(arr), dtype=np.uint8).copy()
+    return torch.from_numpy(raw).to(device)
+
+
+def generate_training_samples(n_rays, n_rays_total, seed, cameras, n_images, rgba, background, bitfield, max_samples):
+    """generate_training_samples_nerf_with_global_movement (src/testbed_nerf.cu:1253-1446), static path.
+    cameras: device byte tensor from pack_cameras; rgba fp32 [pixels, 4]; bitfield uint8 device tensor."""
+    dev_ = rgba.device
+    nbytes = int(capi.lib().n2_sampler_workspace_bytes(C.c_uint32(max(n_rays, 1))))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev_)
+    out = dict(ray_counter=torch.zeros(1, dtype=torch.int32, device=dev_),
+               sample_counter=torch.zeros(1, dtype=torch.int32, device=dev_),
+               ray_indices=torch.zeros(n_rays, dtype=torch.int32, device=dev_),
+               numsteps=torch.zeros((n_rays, 2), dtype=torch.int32, device=dev_),
+               rgb_target=torch.zeros((n_rays, 3), dtype=torch.float32, device=dev_),
+               coords=torch.zeros((max_samples, 7), dtype=torch.float32, device=dev_))
+    bg = (C.c_float * 3)(*background)
+    check(capi.lib().n2_generate_training_samples(_stream(), C.c_uint32(n_rays), C.c_uint32(n_rays_total), C.c_uint32(seed),
+                                                  ptr(cameras), C.c_uint32(n_images), ptr(rgba), bg, ptr(bitfield),
+                                                  C.c_uint32(max_samples), ptr(out["ray_counter"]),
+                                                  ptr(out["sample_counter"]), ptr(out["ray_indices"]), ptr(out["numsteps"]),
+                                                  ptr(out["rgb_target"]), ptr(out["coords"]), ptr(ws), C.c_uint64(nbytes)),
+          "n2_generate_training_samples")
+    return out

@@ -734,3 +734,197 @@ ORC_API void orc_fill_rollover(uint32_t n_total, uint32_t stride, uint32_t n_in,
 		inout[i] = r;
 	}
 }
+
+// ---------------------------------------------------------------------------
+// Training-sample generator: pick a pixel per ray, march the ray through the
+// 128^3 morton-ordered occupancy bitfield with the fixed step sqrt(3)/1024 and
+// emit one NerfCoordinate per occupied step:
+// generate_training_samples_nerf_with_global_movement, src/testbed_nerf.cu:1253-1446,
+// with its helpers (:139-154, 346-368, 484-510, 614-628) and BoundingBox::ray_intersect /
+// contains (bounding_box.cuh:163-221); static path (no global movement, no
+// distortion, no extra dims, no error-map CDFs, cone_angle_constant = 0 as load_nerf
+// sets it for aabb_scale <= 1, src/testbed_nerf.cu:3084; unit aabb).
+//
+// Two deliberate differences, both inside what the reference leaves open:
+//  * the random numbers come from a counter-based hash instead of tcnn's pcg32
+//    (absent source); draw k of ray i is hash(seed, 8*i + k);
+//  * sample ranges and compact ray slots are handed out in ray order instead of
+//    by atomicAdd (the reference's order is a race).
+// Every floating-point step is written so that a GPU and a CPU evaluate it
+// identically (explicit fmaf, no contraction): sample positions are bit-exact.
+// ---------------------------------------------------------------------------
+struct Camera {
+	float xform[12];  // row-major 3x4 camera-to-world: [R | o]
+	float focal[2], principal[2];
+	uint32_t res[2];
+	uint32_t pixel_offset_lo, pixel_offset_hi;  // first pixel of this image in the RGBA array
+};
+
+static inline uint32_t hash_u32(uint32_t seed, uint32_t ctr) {
+	// pcg-style output permutation of a Weyl-mixed counter
+	uint32_t x = ctr * 747796405u + seed * 2891336453u + 1u;
+	x = ((x >> ((x >> 28) + 4u)) ^ x) * 277803737u;
+	x = (x >> 22) ^ x;
+	x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+	return x;
+}
+static inline float rand01(uint32_t seed, uint32_t ray, uint32_t k) { return (float)(hash_u32(seed, ray * 8u + k) >> 8) * (1.0f / 16777216.0f); }
+
+static inline uint32_t expand_bits(uint32_t v) {
+	v = (v * 0x00010001u) & 0xFF0000FFu;
+	v = (v * 0x00000101u) & 0x0F00F00Fu;
+	v = (v * 0x00000011u) & 0xC30C30C3u;
+	v = (v * 0x00000005u) & 0x49249249u;
+	return v;
+}
+ORC_API uint32_t orc_morton3d(uint32_t x, uint32_t y, uint32_t z) { return expand_bits(x) | (expand_bits(y) << 1) | (expand_bits(z) << 2); }
+ORC_API void orc_morton3d_invert(uint32_t m, uint32_t* xyz) {
+	for (int d = 0; d < 3; ++d) {
+		uint32_t x = (m >> d) & 0x49249249u;
+		x = (x | (x >> 2)) & 0xc30c30c3u;
+		x = (x | (x >> 4)) & 0x0f00f00fu;
+		x = (x | (x >> 8)) & 0xff0000ffu;
+		x = (x | (x >> 16)) & 0x0000ffffu;
+		xyz[d] = x;
+	}
+}
+
+static const float STEP = 1.73205080757f / 1024.f;  // STEPSIZE()
+static const uint32_t GRIDSIZE = 128, MARCH_STEPS = 1024;
+
+static inline bool occupied(const uint8_t* bitfield, const float* pos) {
+	// cascaded_grid_idx_at(pos, mip = 0) + density_grid_occupied_at (:484-510)
+	int c[3];
+	for (int d = 0; d < 3; ++d) {
+		float p = pos[d] - 0.5f;
+		p = p * 1.0f;
+		p = p + 0.5f;
+		int i = (int)(p * (float)GRIDSIZE);
+		c[d] = std::min(std::max(i, 0), (int)GRIDSIZE - 1);
+	}
+	const uint32_t idx = orc_morton3d((uint32_t)c[0], (uint32_t)c[1], (uint32_t)c[2]);
+	return (bitfield[idx / 8] >> (idx % 8)) & 1;
+}
+
+static inline float to_next_voxel(const float* pos, const float* dir, const float* idir) {
+	// distance_to_next_voxel at res = 128 (:346-354)
+	float t = 3.4e38f;
+	for (int d = 0; d < 3; ++d) {
+		const float p = (float)GRIDSIZE * pos[d];
+		const float sgn = copysignf(1.0f, dir[d]);
+		const float td = (floorf(p + 0.5f + 0.5f * sgn) - p) * idir[d];
+		t = std::min(t, td);
+	}
+	return std::max(t / (float)GRIDSIZE, 0.0f);
+}
+
+struct RaySetup {
+	bool alive;
+	float o[3], dir[3], idir[3], startt;
+	float target[3];
+};
+
+static RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const Camera* cams, uint32_t n_images,
+                          const float* rgba, const float* background) {
+	RaySetup r{};
+	const uint32_t img = (((i + n_rays_total) * n_images) / n_rays) % n_images;  // image_idx (:1243-1250)
+	const Camera& c = cams[img];
+	// nerf_random_image_pos_training with snap_to_pixel_centers (:1216-1228)
+	const float u0 = rand01(seed, i, 0), u1 = rand01(seed, i, 1);
+	const int px = std::min(std::max((int)(u0 * (float)c.res[0]), 0), (int)c.res[0] - 1);
+	const int py = std::min(std::max((int)(u1 * (float)c.res[1]), 0), (int)c.res[1] - 1);
+	const float x = ((float)px + 0.5f) / (float)c.res[0], y = ((float)py + 0.5f) / (float)c.res[1];
+	const uint64_t off = ((uint64_t)c.pixel_offset_hi << 32) | c.pixel_offset_lo;
+	const float* pix = rgba + (off + (uint64_t)px + (uint64_t)py * c.res[0]) * 4;
+	// masked-away pixels are mostly skipped (:1300-1302)
+	if (pix[0] <= 0.0f && rand01(seed, i, 2) >= 0.9f) { r.alive = false; return r; }
+	for (int k = 0; k < 3; ++k) r.target[k] = pix[k] + (1.0f - pix[3]) * background[k];
+	const float d[3] = {(x - c.principal[0]) * (float)c.res[0] / c.focal[0], (y - c.principal[1]) * (float)c.res[1] / c.focal[1], 1.0f};
+	float w[3];
+	for (int k = 0; k < 3; ++k) {
+		w[k] = fmaf(c.xform[k * 4 + 2], d[2], fmaf(c.xform[k * 4 + 1], d[1], c.xform[k * 4 + 0] * d[0]));
+		r.o[k] = c.xform[k * 4 + 3];
+	}
+	const float len = sqrtf(fmaf(w[2], w[2], fmaf(w[1], w[1], w[0] * w[0])));
+	for (int k = 0; k < 3; ++k) { r.dir[k] = w[k] / len; r.idir[k] = 1.0f / r.dir[k]; }
+	// BoundingBox::ray_intersect against the unit cube (bounding_box.cuh:163-210)
+	float tmin = (0.f - r.o[0]) / r.dir[0], tmax = (1.f - r.o[0]) / r.dir[0];
+	if (tmin > tmax) std::swap(tmin, tmax);
+	bool hit = true;
+	for (int k = 1; k < 3 && hit; ++k) {
+		float a = (0.f - r.o[k]) / r.dir[k], b = (1.f - r.o[k]) / r.dir[k];
+		if (a > b) std::swap(a, b);
+		if (tmin > b || a > tmax) { hit = false; break; }
+		if (a > tmin) tmin = a;
+		if (b < tmax) tmax = b;
+	}
+	if (!hit) tmin = 3.402823466e38f;
+	tmin = std::max(tmin, 0.0f);
+	r.startt = fmaf(STEP, rand01(seed, i, 3), tmin);
+	r.alive = true;
+	return r;
+}
+
+// March; when coords != null emits up to max_emit coordinates.  Returns the number of occupied steps.
+static uint32_t march(const RaySetup& r, const uint8_t* bitfield, float* coords, uint32_t max_emit) {
+	uint32_t j = 0;
+	float t = r.startt;
+	const uint32_t limit = coords ? max_emit : MARCH_STEPS;
+	while (j < limit) {
+		float pos[3];
+		for (int k = 0; k < 3; ++k) pos[k] = fmaf(t, r.dir[k], r.o[k]);
+		if (!(pos[0] >= 0.f && pos[0] <= 1.f && pos[1] >= 0.f && pos[1] <= 1.f && pos[2] >= 0.f && pos[2] <= 1.f)) break;
+		if (occupied(bitfield, pos)) {
+			if (coords) {
+				float* c = coords + (size_t)j * 7;
+				c[0] = pos[0]; c[1] = pos[1]; c[2] = pos[2];
+				c[3] = 0.0f;  // warp_dt(MIN_CONE_STEPSIZE) = 0
+				for (int k = 0; k < 3; ++k) c[4 + k] = (r.dir[k] + 1.0f) * 0.5f;  // warp_direction
+			}
+			++j;
+			t += STEP;
+		} else {
+			const float t_target = t + to_next_voxel(pos, r.dir, r.idir);
+			do { t += STEP; } while (t < t_target);
+		}
+	}
+	return j;
+}
+
+//  cams [n_images]; rgba fp32 [pixels][4]; bitfield 128^3/8 bytes (mip 0)
+//  outputs: ray_counter, sample_counter, ray_indices [n_rays], numsteps [n_rays][2], rgb_target [n_rays][3],
+//           coords [max_samples][7]
+ORC_API void orc_generate_training_samples(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const Camera* cams, uint32_t n_images,
+                                           const float* rgba, const float* background, const uint8_t* bitfield, uint32_t max_samples,
+                                           uint32_t* ray_counter, uint32_t* sample_counter, uint32_t* ray_indices, uint32_t* numsteps,
+                                           float* rgb_target, float* coords) {
+	std::vector<uint32_t> cnt(n_rays, 0);
+	#pragma omp parallel for schedule(dynamic, 64)
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, background);
+		cnt[i] = r.alive ? march(r, bitfield, nullptr, 0) : 0;
+	}
+	std::vector<uint32_t> base(n_rays), slot(n_rays, 0xFFFFFFFFu);
+	uint64_t run = 0;
+	uint32_t rays = 0;
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		if (cnt[i] == 0) continue;  // (:1406-1408)
+		base[i] = (uint32_t)std::min<uint64_t>(run, 0xFFFFFFFFull);
+		run += cnt[i];
+		if ((uint64_t)base[i] + cnt[i] > max_samples) continue;  // (:1411-1414)
+		slot[i] = rays++;
+	}
+	*ray_counter = rays;
+	*sample_counter = (uint32_t)std::min<uint64_t>(run, 0xFFFFFFFFull);
+	#pragma omp parallel for schedule(dynamic, 64)
+	for (uint32_t i = 0; i < n_rays; ++i) {
+		if (slot[i] == 0xFFFFFFFFu) continue;
+		const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, background);
+		const uint32_t s = slot[i];
+		ray_indices[s] = i;
+		numsteps[2 * s] = cnt[i];
+		numsteps[2 * s + 1] = base[i];
+		for (int k = 0; k < 3; ++k) rgb_target[(size_t)s * 3 + k] = r.target[k];
+		march(r, bitfield, coords + (size_t)base[i] * 7, cnt[i]);
+	}
+}

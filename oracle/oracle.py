@@ -225,3 +225,41 @@ def fill_rollover(a, n_in, rescale=False):
     lib().orc_fill_rollover(C.c_uint32(a.shape[0]), C.c_uint32(a.shape[1] if a.ndim > 1 else 1), C.c_uint32(n_in), _fp(a),
                             C.c_int(int(rescale)))
     return a
+
+
+class Camera(C.Structure):
+    """Matches struct n2_camera of the product ABI."""
+    _fields_ = [("xform", C.c_float * 12), ("focal", C.c_float * 2), ("principal", C.c_float * 2),
+                ("res", C.c_uint32 * 2), ("pixel_offset_lo", C.c_uint32), ("pixel_offset_hi", C.c_uint32)]
+
+
+def morton3d(x, y, z):
+    lib().orc_morton3d.restype = C.c_uint32
+    return int(lib().orc_morton3d(C.c_uint32(x), C.c_uint32(y), C.c_uint32(z)))
+
+
+def morton3d_invert(m):
+    out = (C.c_uint32 * 3)()
+    lib().orc_morton3d_invert(C.c_uint32(m), out)
+    return tuple(out)
+
+
+def generate_training_samples(n_rays, n_rays_total, seed, cameras, rgba, background, bitfield, max_samples):
+    """cameras: numpy structured bytes (n_images * sizeof(Camera)) or list of Camera; rgba [pixels, 4] float32;
+    bitfield uint8 [128^3/8].  Returns dict(ray_counter, sample_counter, ray_indices, numsteps, rgb_target, coords)."""
+    cams = (Camera * len(cameras))(*cameras)
+    rgba = _f32(rgba)
+    bg = (C.c_float * 3)(*background)
+    bitfield = np.ascontiguousarray(bitfield, np.uint8)
+    ray_counter, sample_counter = C.c_uint32(0), C.c_uint32(0)
+    ray_indices = np.zeros(n_rays, np.uint32)
+    numsteps = np.zeros((n_rays, 2), np.uint32)
+    target = np.zeros((n_rays, 3), np.float32)
+    coords = np.zeros((max_samples, 7), np.float32)
+    lib().orc_generate_training_samples(C.c_uint32(n_rays), C.c_uint32(n_rays_total), C.c_uint32(seed), cams,
+                                        C.c_uint32(len(cameras)), _fp(rgba), bg,
+                                        bitfield.ctypes.data_as(C.POINTER(C.c_uint8)), C.c_uint32(max_samples),
+                                        C.byref(ray_counter), C.byref(sample_counter), _up(ray_indices), _up(numsteps),
+                                        _fp(target), _fp(coords))
+    return dict(ray_counter=int(ray_counter.value), sample_counter=int(sample_counter.value), ray_indices=ray_indices,
+                numsteps=numsteps, rgb_target=target, coords=coords)
