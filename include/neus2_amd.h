@@ -233,9 +233,13 @@ int n2_field_set_params(n2_field_t* field, const n2_half* d_params, n2_half* d_g
 
 /* Scratch the reference takes from tcnn's arena inside forward_impl/backward_impl
  * (every GPUMatrixDynamic temporary, nerf_network.h:137-267, 332-557): network inputs,
- * the grid's dy_dx context, input gradients and the MLP weight-gradient slabs. */
-uint64_t n2_field_workspace_bytes(const n2_field_t* field, uint32_t max_batch);
-int n2_field_set_workspace(n2_field_t* field, void* d_workspace, uint64_t n_bytes, uint32_t max_batch);
+ * the grid's dy_dx context, input gradients and the MLP weight-gradient slabs.
+ * max_batch bounds forward / sdf / density calls, max_batch_backward (<= max_batch) the batches
+ * that are also run backward: the training step runs the forward over every marched sample
+ * (up to 16 x 2^18) but the backward only over the compacted 2^18 (src/testbed_nerf.cu:3840, 3931-3932). */
+uint64_t n2_field_workspace_bytes(const n2_field_t* field, uint32_t max_batch, uint32_t max_batch_backward);
+int n2_field_set_workspace(n2_field_t* field, void* d_workspace, uint64_t n_bytes, uint32_t max_batch,
+                           uint32_t max_batch_backward);
 
 /* NerfNetwork::forward_impl / inference_mixed_precision_impl (which the reference routes
  * to forward_impl), nerf_network.h:87-90, 132-315.
@@ -371,6 +375,80 @@ int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n
                                  uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices,
                                  uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
                                  uint64_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * One training step: counterpart of Testbed::train_nerf_step followed by
+ * Trainer::optimizer_step (src/testbed_nerf.cu:3717-3987, 3498):
+ *   generate samples -> field forward over every marched sample -> compositing / loss /
+ *   compaction -> roll the compacted batch over to exactly target_batch_size -> field forward
+ *   and backward on it -> Adam.
+ * Nothing in a step synchronises with the host; counters are read on request.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_trainer n2_trainer_t;
+
+typedef struct n2_trainer_config {
+	n2_field_config field;
+	n2_adam_config adam;
+	n2_composite_config composite;  /* n_rays_norm is overwritten per step with the step's n_rays */
+	uint32_t target_batch_size;     /* 2^18, src/testbed.cu:2110 */
+	uint32_t max_rays_per_batch;    /* upper bound of n_rays in a step */
+	uint32_t max_samples;           /* capacity for marched samples; the reference uses 16 x target (src/testbed_nerf.cu:3719) */
+	float loss_scale;               /* 128, testbed.h:237 */
+} n2_trainer_config;
+
+/* All device memory a trainer uses (parameters, optimiser state, every temporary) lives in one
+ * caller-owned workspace, counterpart of the Trainer's parameter buffer plus the arena allocation
+ * of src/testbed_nerf.cu:3723-3749. */
+uint64_t n2_trainer_workspace_bytes(const n2_trainer_config* config);
+int n2_trainer_create(const n2_trainer_config* config, void* d_workspace, uint64_t workspace_bytes, n2_trainer_t** out);
+void n2_trainer_destroy(n2_trainer_t* trainer);
+
+/* Parameter buffers inside the workspace ([fp32 master | fp16 params | fp16 gradients], the Trainer's
+ * layout mirrored at nerf_network.h:1010-1016).  The caller initialises d_master (NerfNetwork::
+ * initialize_params, nerf_network.h:805-876) and calls n2_trainer_sync_params to refresh the fp16 copy. */
+int n2_trainer_buffers(n2_trainer_t* trainer, float** d_master, n2_half** d_params, n2_half** d_gradients, uint32_t* n_params);
+int n2_trainer_sync_params(n2_trainer_t* trainer, n2_stream_t stream);
+n2_field_t* n2_trainer_field(n2_trainer_t* trainer);
+
+/* Training images, cameras and the occupancy bitfield (see n2_generate_training_samples). */
+int n2_trainer_set_scene(n2_trainer_t* trainer, const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
+                         const uint8_t* d_bitfield);
+
+/*  n_rays       rays to draw this step (<= max_rays_per_batch)
+ *  n_inference  how many marched samples the first forward covers (a multiple of 8, <= max_samples); the
+ *               reference uses the sample count measured in earlier steps, rounded up to 128
+ *               (src/testbed_nerf.cu:3751-3756)
+ *  seed         seed of this step's random draws */
+int n2_trainer_step(n2_trainer_t* trainer, n2_stream_t stream, uint32_t n_rays, uint32_t n_inference, uint32_t seed);
+
+/* Waits for the stream, then returns the last step's counters: live rays, marched samples, samples the
+ * rays wanted to keep (before the clamp to target_batch_size), and the summed loss
+ * (counters.update_after_training, src/testbed_nerf.cu:3406-3429). */
+int n2_trainer_read_counters(n2_trainer_t* trainer, n2_stream_t stream, uint32_t* rays, uint32_t* samples,
+                             uint32_t* compacted, float* loss);
+
+/* ------------------------------------------------------------------------
+ * Optional event timing of the dominant kernels (off by default; the reference has only
+ * wall-clock timers, src/testbed.cu:2707-2710).  When enabled, every launch of a listed kernel is
+ * bracketed by a pair of events on its own stream.
+ * ---------------------------------------------------------------------- */
+typedef enum n2_prof_id {
+	N2_PROF_GRID_FORWARD = 0,
+	N2_PROF_GRID_BACKWARD_PARAMS = 1,
+	N2_PROF_GRID_SECOND_ORDER = 2,
+	N2_PROF_MLP_FORWARD = 3,
+	N2_PROF_MLP_BACKWARD = 4,
+	N2_PROF_MLP_SECOND_ORDER = 5,
+	N2_PROF_COMPOSITE = 6,
+	N2_PROF_SAMPLER = 7,
+	N2_PROF_ADAM = 8,
+	N2_PROF_COUNT = 9
+} n2_prof_id;
+
+int n2_profile_enable(int enable);
+/* Waits for all recorded events; total milliseconds and launch count per id since the last reset. */
+int n2_profile_read(n2_prof_id id, float* total_ms, uint32_t* launches);
+int n2_profile_reset(void);
 
 #ifdef __cplusplus
 }

@@ -41,6 +41,13 @@ class Camera(C.Structure):
                 ("resolution", C.c_uint32 * 2), ("pixel_offset_lo", C.c_uint32), ("pixel_offset_hi", C.c_uint32)]
 
 
+class TrainerConfig(C.Structure):
+    """struct n2_trainer_config"""
+    _fields_ = [("field", FieldConfig), ("adam", AdamConfig), ("composite", CompositeConfig),
+                ("target_batch_size", C.c_uint32), ("max_rays_per_batch", C.c_uint32), ("max_samples", C.c_uint32),
+                ("loss_scale", C.c_float)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 
@@ -69,11 +76,17 @@ def lib():
         _lib.n2_field_n_params.restype = C.c_uint32
         _lib.n2_field_n_params.argtypes = [C.c_void_p]
         _lib.n2_field_workspace_bytes.restype = C.c_uint64
-        _lib.n2_field_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
+        _lib.n2_field_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32]
         _lib.n2_composite_workspace_bytes.restype = C.c_uint64
         _lib.n2_composite_workspace_bytes.argtypes = [C.c_uint32]
         _lib.n2_sampler_workspace_bytes.restype = C.c_uint64
         _lib.n2_sampler_workspace_bytes.argtypes = [C.c_uint32]
+        _lib.n2_trainer_workspace_bytes.restype = C.c_uint64
+        _lib.n2_trainer_workspace_bytes.argtypes = [C.c_void_p]
+        _lib.n2_trainer_destroy.restype = None
+        _lib.n2_trainer_destroy.argtypes = [C.c_void_p]
+        _lib.n2_trainer_field.restype = C.c_void_p
+        _lib.n2_trainer_field.argtypes = [C.c_void_p]
         _lib.n2_field_destroy.restype = None
         _lib.n2_field_destroy.argtypes = [C.c_void_p]
     return _lib

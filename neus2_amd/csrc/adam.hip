@@ -74,6 +74,7 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 8 == 0 && reinterpret_cast<uintptr_t>(d_gradients) % 8 == 0,
 	           "n2_adam_step: fp16 buffers must be 8-byte aligned");
 	const uint32_t quads = (n_params + 3) / 4;
+	N2ProfScope prof(N2_PROF_ADAM, n2_stream(stream));
 	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(*config, n_params, n_matrix_params, loss_scale,
 		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
 	N2_LAUNCH_CHECK();

@@ -43,3 +43,86 @@ int n2_set_u32(hipStream_t stream, uint32_t* d_ptr, uint32_t value) {
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
+
+// ---------------------------------------------------------------------------
+// event timing
+// ---------------------------------------------------------------------------
+#include <vector>
+
+namespace {
+struct ProfState {
+	bool enabled = false;
+	std::vector<hipEvent_t> pool;                 // recycled events
+	std::vector<hipEvent_t> pending[N2_PROF_COUNT];  // begin/end pairs, not yet read
+	float total_ms[N2_PROF_COUNT] = {};
+	uint32_t launches[N2_PROF_COUNT] = {};
+	hipEvent_t open_begin[N2_PROF_COUNT] = {};
+};
+ProfState g_prof;
+
+hipEvent_t prof_take() {
+	if (!g_prof.pool.empty()) {
+		hipEvent_t e = g_prof.pool.back();
+		g_prof.pool.pop_back();
+		return e;
+	}
+	hipEvent_t e = nullptr;
+	if (hipEventCreate(&e) != hipSuccess) return nullptr;
+	return e;
+}
+
+void prof_collect(int id) {
+	auto& v = g_prof.pending[id];
+	for (size_t i = 0; i + 1 < v.size(); i += 2) {
+		float ms = 0.f;
+		if (hipEventSynchronize(v[i + 1]) == hipSuccess && hipEventElapsedTime(&ms, v[i], v[i + 1]) == hipSuccess) {
+			g_prof.total_ms[id] += ms;
+			g_prof.launches[id] += 1;
+		}
+		g_prof.pool.push_back(v[i]);
+		g_prof.pool.push_back(v[i + 1]);
+	}
+	v.clear();
+}
+}  // namespace
+
+void n2_prof_begin(int id, hipStream_t stream) {
+	if (!g_prof.enabled) return;
+	hipEvent_t e = prof_take();
+	if (!e) return;
+	(void)hipEventRecord(e, stream);
+	g_prof.open_begin[id] = e;
+}
+
+void n2_prof_end(int id, hipStream_t stream) {
+	if (!g_prof.enabled || !g_prof.open_begin[id]) return;
+	hipEvent_t e = prof_take();
+	if (!e) return;
+	(void)hipEventRecord(e, stream);
+	g_prof.pending[id].push_back(g_prof.open_begin[id]);
+	g_prof.pending[id].push_back(e);
+	g_prof.open_begin[id] = nullptr;
+	if (g_prof.pending[id].size() >= 8192) prof_collect(id);  // bound the number of live events
+}
+
+N2_API int n2_profile_enable(int enable) {
+	g_prof.enabled = enable != 0;
+	return N2_OK;
+}
+
+N2_API int n2_profile_read(n2_prof_id id, float* total_ms, uint32_t* launches) {
+	N2_REQUIRE((int)id >= 0 && (int)id < N2_PROF_COUNT, "n2_profile_read: bad id %d", (int)id);
+	prof_collect((int)id);
+	if (total_ms) *total_ms = g_prof.total_ms[id];
+	if (launches) *launches = g_prof.launches[id];
+	return N2_OK;
+}
+
+N2_API int n2_profile_reset(void) {
+	for (int id = 0; id < N2_PROF_COUNT; ++id) {
+		prof_collect(id);
+		g_prof.total_ms[id] = 0.f;
+		g_prof.launches[id] = 0;
+	}
+	return N2_OK;
+}

@@ -309,6 +309,7 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
 	uint32_t* ckept = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(cbase) + up256(4ull * n_rays));
 	const dim3 grid((n_rays + CB / 64 - 1) / (CB / 64)), block(CB);
 	const hf* out = reinterpret_cast<const hf*>(d_network_output);
+	N2ProfScope prof(N2_PROF_COMPOSITE, s);
 	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch);
 	N2_LAUNCH_CHECK();
 	composite_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples_compacted, scratch, cbase, ckept, d_compacted_counter);

@@ -25,7 +25,7 @@ struct n2_field {
 	hf* grads;
 	unsigned char* ws;
 	uint64_t ws_bytes;
-	uint32_t max_batch;
+	uint32_t max_batch, max_batch_bwd;
 	// carved from the workspace
 	hf* sdf_in;        // [sdf_in_w][N]
 	hf* rgb_in;        // [48][N]
@@ -263,16 +263,18 @@ struct FieldCarve {
 	uint64_t sdf_in, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, total;
 };
 
-static FieldCarve carve(const n2_field_t* f, uint32_t nb) {
+// nf: largest forward batch, nbw: largest batch that is also run backward
+static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	FieldCarve c{};
 	uint64_t o = 0;
-	const uint64_t n = nb;
+	uint64_t n = nf;
 	auto take = [&](uint64_t bytes) { const uint64_t at = o; o = align256(o + bytes); return at; };
 	c.sdf_in = take(2ull * f->sdf_in_w * n);
 	c.rgb_in = take(2ull * f->rgb_in_w * n);
 	c.dy_dx = take(12ull * f->enc_w * n);
 	c.dsdf_din = take(2ull * f->sdf_in_w * n);
 	c.normal = take(12ull * n);
+	n = nbw;
 	c.d_rgb_in = take(2ull * f->rgb_in_w * n);
 	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
 	c.v = take(12ull * n);
@@ -285,18 +287,21 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nb) {
 	return c;
 }
 
-N2_API uint64_t n2_field_workspace_bytes(const n2_field_t* f, uint32_t max_batch) { return f ? carve(f, max_batch).total : 0; }
+N2_API uint64_t n2_field_workspace_bytes(const n2_field_t* f, uint32_t max_batch, uint32_t max_batch_backward) {
+	return f ? carve(f, max_batch, max_batch_backward < max_batch ? max_batch_backward : max_batch).total : 0;
+}
 
-N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_bytes, uint32_t max_batch) {
+N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_bytes, uint32_t max_batch, uint32_t max_batch_backward) {
 	N2_REQUIRE(f != nullptr, "n2_field_set_workspace: field is null");
 	N2_REQUIRE(d_workspace != nullptr, "n2_field_set_workspace: workspace is null");
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256 == 0, "n2_field_set_workspace: workspace must be 256-byte aligned");
 	N2_REQUIRE(max_batch % 8 == 0, "n2_field_set_workspace: max_batch %u must be a multiple of 8", max_batch);
-	const FieldCarve c = carve(f, max_batch);
+	if (max_batch_backward > max_batch) max_batch_backward = max_batch;
+	const FieldCarve c = carve(f, max_batch, max_batch_backward);
 	N2_REQUIRE(n_bytes >= c.total, "n2_field_set_workspace: %llu bytes given, %llu needed for batch %u", (unsigned long long)n_bytes,
 	           (unsigned long long)c.total, max_batch);
 	unsigned char* b = reinterpret_cast<unsigned char*>(d_workspace);
-	f->ws = b; f->ws_bytes = n_bytes; f->max_batch = max_batch;
+	f->ws = b; f->ws_bytes = n_bytes; f->max_batch = max_batch; f->max_batch_bwd = max_batch_backward;
 	f->sdf_in = reinterpret_cast<hf*>(b + c.sdf_in);
 	f->rgb_in = reinterpret_cast<hf*>(b + c.rgb_in);
 	f->dy_dx = reinterpret_cast<float*>(b + c.dy_dx);
@@ -350,6 +355,7 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n,
                              const n2_half* d_dL_doutput, uint32_t ek_batch_size, n2_grad_mode mode) {
 	if (int rc = check_field(f, "n2_field_backward", n)) return rc;
+	N2_REQUIRE(n <= f->max_batch_bwd, "n2_field_backward: batch %u exceeds the workspace's backward capacity %u", n, f->max_batch_bwd);
 	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_field_backward: mode must be OVERWRITE or ACCUMULATE");
 	N2_REQUIRE(f->grads != nullptr, "n2_field_backward: no gradient buffer (n2_field_set_params)");
 	N2_REQUIRE(ek_batch_size > 0, "n2_field_backward: ek_batch_size must be positive");

@@ -38,8 +38,11 @@ __device__ __forceinline__ void n2_locate(float x, float scale, float& w, uint32
 template <uint32_t MODE>
 __device__ __forceinline__ uint32_t n2_entry(uint32_t entries, uint32_t res, uint32_t gx, uint32_t gy, uint32_t gz) {
 	if (MODE == N2_LEVEL_DENSE) {
+		// Positions inside [0,1]^3 never give a coordinate above res; the clamp only keeps
+		// stray inputs (padding rows of a batch) inside the table.  The host has checked
+		// res^3 + res^2 + res < 2*entries, so one subtraction is the modulo.
+		gx = min(gx, res); gy = min(gy, res); gz = min(gz, res);
 		uint32_t i = gx + gy * res + gz * res * res;
-		// the host has checked res^3 + res^2 + res < 2*entries
 		return i >= entries ? i - entries : i;
 	} else if (MODE == N2_LEVEL_HASH) {
 		return (gx ^ (gy * 2654435761u) ^ (gz * 805459861u)) & (entries - 1u);
@@ -404,6 +407,7 @@ N2_API int n2_grid_forward(n2_grid_t* grid, n2_stream_t stream, const float* d_x
 	N2_REQUIRE(d_out != nullptr, "n2_grid_forward: d_out is null");
 	const uint32_t tiles = n_tiles(n_points);
 	const dim3 grid_dim(tiles * grid->tab.n_levels), block(GRID_BLOCK);
+	N2ProfScope prof(N2_PROF_GRID_FORWARD, n2_stream(stream));
 	if (d_dy_dx) {
 		grid_forward_kernel<true><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride,
 			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), d_dy_dx);
@@ -446,6 +450,7 @@ N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_
 	if (n_points == 0) return N2_OK;
 	const uint32_t tiles = n_tiles(n_points);
 	if (mode != N2_GRAD_IGNORE) {
+		N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
 		grid_backward_params_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
 			grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, reinterpret_cast<const __half*>(d_dL_dy), grid->grads);
 		N2_LAUNCH_CHECK();
@@ -472,6 +477,7 @@ N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, 
 		if (int rc = n2_fill_zero_u32(s, d_dL_dx, sizeof(float) * 3 * (size_t)n_points)) return rc;
 	}
 	const uint32_t tiles = n_tiles(n_points);
+	N2ProfScope prof(N2_PROF_GRID_SECOND_ORDER, s);
 	grid_bbi_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
 		grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, d_dL_ddLdx, reinterpret_cast<const __half*>(d_dL_dy),
 		grid->params, mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy), d_dL_dx);

@@ -723,6 +723,7 @@ N2_API int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_in
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0 && reinterpret_cast<uintptr_t>(d_hidden) % 16 == 0,
 	           "n2_mlp_forward: outputs must be 16-byte aligned");
 	const dim3 grid(stream_grid(n, 2048)), block(MLP_BLOCK);
+	N2ProfScope prof(N2_PROF_MLP_FORWARD, n2_stream(stream));
 #define CALL(IC, NH)                                                                                                     \
 	mlp_forward_kernel<IC, NH><<<grid, block, 0, n2_stream(stream)>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
 		reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0, reinterpret_cast<hf*>(d_hidden))
@@ -779,6 +780,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
 	const int aos = dL_layout == N2_LAYOUT_AOS ? 1 : 0;
+	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 #define LAUNCH(IC, NH, DX, DW)                                                                                      \
 	do {                                                                                                            \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
@@ -832,6 +834,7 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 	if (!want_dw && !d_dL_ddLdoutput) return N2_OK;
 	const uint32_t blocks = stream_grid(n, MLP_MAX_SLABS);
 	const size_t lds = STAGE_BYTES > mlp->n_params * sizeof(float) ? STAGE_BYTES : mlp->n_params * sizeof(float);
+	N2ProfScope prof(N2_PROF_MLP_SECOND_ORDER, s);
 	switch (mlp->in_w / 16) {
 #define CASE(IC)                                                                                                           \
 	case IC:                                                                                                               \

@@ -59,3 +59,13 @@ static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hip
 int n2_fill_zero_u32(hipStream_t stream, void* d_ptr, size_t n_bytes);
 // Store one 32-bit value with a one-thread kernel.
 int n2_set_u32(hipStream_t stream, uint32_t* d_ptr, uint32_t value);
+
+// Event timing of a kernel launch; a no-op unless n2_profile_enable(1) was called.
+void n2_prof_begin(int id, hipStream_t stream);
+void n2_prof_end(int id, hipStream_t stream);
+struct N2ProfScope {
+	int id;
+	hipStream_t s;
+	N2ProfScope(int id_, hipStream_t s_) : id(id_), s(s_) { n2_prof_begin(id, s); }
+	~N2ProfScope() { n2_prof_end(id, s); }
+};

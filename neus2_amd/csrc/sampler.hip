@@ -231,6 +231,7 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	uint32_t* base = reinterpret_cast<uint32_t*>(w + up256(4ull * n_rays));
 	uint32_t* slot = reinterpret_cast<uint32_t*>(w + 2 * up256(4ull * n_rays));
 	const dim3 grid((n_rays + 127) / 128), block(128);
+	N2ProfScope prof(N2_PROF_SAMPLER, s);
 	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
 	                                            background[2], d_bitfield, counts);
 	N2_LAUNCH_CHECK();

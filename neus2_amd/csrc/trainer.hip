@@ -1,0 +1,264 @@
+// One training step on one GPU: sample generation, field forward over all
+// marched samples, compositing / loss / compaction, roll-over to the target
+// batch size, field forward + backward (first and second order), Adam.
+// Everything is enqueued on the caller's stream; no host synchronisation.
+#include "n2_common.h"
+
+#include <cstring>
+#include <new>
+
+typedef _Float16 hf;
+
+struct n2_trainer {
+	n2_trainer_config cfg;
+	n2_field_t* field;
+	uint32_t n_params, n_matrix_params;
+	unsigned char* ws;
+	// parameters and optimiser state
+	float* master;
+	hf* params;
+	hf* grads;
+	float* m1;
+	float* m2;
+	uint32_t* steps;
+	// per-step buffers
+	float* coords;            // [max_samples][7]
+	hf* mlp_out;              // [max(max_samples, target)][16]
+	hf* dloss;                // [target][16]
+	float* coords_compacted;  // [target][7]
+	uint32_t* numsteps;       // [max_rays][2]
+	uint32_t* ray_indices;    // [max_rays]
+	float* rgb_target;        // [max_rays][3]
+	float* ray_loss;          // [max_rays]
+	uint32_t* counters;       // [0] live rays, [1] marched samples, [2] compacted samples (+ [4] as float: loss)
+	void* ws_sampler;
+	void* ws_composite;
+	uint64_t ws_sampler_bytes, ws_composite_bytes;
+	void* ws_field;
+	// scene
+	const n2_camera* cameras;
+	uint32_t n_images;
+	const float* rgba;
+	const uint8_t* bitfield;
+	uint32_t n_rays_total;
+};
+
+struct TrainerCarve {
+	uint64_t master, params, grads, m1, m2, steps, coords, mlp_out, dloss, coords_compacted, numsteps, ray_indices, rgb_target, ray_loss,
+		counters, ws_sampler, ws_composite, ws_field, total;
+};
+
+static inline uint64_t a256(uint64_t x) { return (x + 255) / 256 * 256; }
+
+static int make_field(const n2_trainer_config* cfg, n2_field_t** f) { return n2_field_create(&cfg->field, f); }
+
+static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t* f) {
+	TrainerCarve c{};
+	uint64_t o = 0;
+	auto take = [&](uint64_t bytes) { const uint64_t at = o; o = a256(o + bytes); return at; };
+	const uint64_t np = n2_field_n_params(f), T = cfg->target_batch_size, S = cfg->max_samples, R = cfg->max_rays_per_batch;
+	c.master = take(4 * np);
+	c.params = take(2 * np);
+	c.grads = take(2 * np);
+	c.m1 = take(4 * np);
+	c.m2 = take(4 * np);
+	c.steps = take(4 * np);
+	c.coords = take(28 * S);
+	c.mlp_out = take(32 * (S > T ? S : T));
+	c.dloss = take(32 * T);
+	c.coords_compacted = take(28 * T);
+	c.numsteps = take(8 * R);
+	c.ray_indices = take(4 * R);
+	c.rgb_target = take(12 * R);
+	c.ray_loss = take(4 * R);
+	c.counters = take(64);
+	c.ws_sampler = take(n2_sampler_workspace_bytes((uint32_t)R));
+	c.ws_composite = take(n2_composite_workspace_bytes((uint32_t)R));
+	c.ws_field = take(n2_field_workspace_bytes(f, (uint32_t)(S > T ? S : T), (uint32_t)T));
+	c.total = o;
+	return c;
+}
+
+static int check_cfg(const n2_trainer_config* cfg, const char* fn) {
+	N2_REQUIRE(cfg != nullptr, "%s: config is null", fn);
+	N2_REQUIRE(cfg->target_batch_size >= 8 && cfg->target_batch_size % 8 == 0, "%s: target_batch_size %u must be a positive multiple of 8", fn,
+	           cfg->target_batch_size);
+	N2_REQUIRE(cfg->max_samples >= cfg->target_batch_size && cfg->max_samples % 8 == 0, "%s: max_samples %u must be a multiple of 8 and >= target_batch_size", fn,
+	           cfg->max_samples);
+	N2_REQUIRE(cfg->max_rays_per_batch >= 1, "%s: max_rays_per_batch must be positive", fn);
+	N2_REQUIRE(cfg->loss_scale > 0.f, "%s: loss_scale must be positive", fn);
+	return N2_OK;
+}
+
+N2_API uint64_t n2_trainer_workspace_bytes(const n2_trainer_config* cfg) {
+	if (check_cfg(cfg, "n2_trainer_workspace_bytes") != N2_OK) return 0;
+	n2_field_t* f = nullptr;
+	if (make_field(cfg, &f) != N2_OK) return 0;
+	const uint64_t total = trainer_carve(cfg, f).total;
+	n2_field_destroy(f);
+	return total;
+}
+
+__global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, const float* __restrict__ master, hf* __restrict__ params) {
+	const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+	if (i < n) params[i] = (hf)master[i];
+}
+
+// sum of the per-ray losses of the live rays (one workgroup)
+__global__ void __launch_bounds__(1024) trainer_loss_sum_kernel(const uint32_t* __restrict__ ray_counter, uint32_t max_rays,
+                                                                const float* __restrict__ ray_loss, float* __restrict__ out) {
+	__shared__ float part[16];
+	const uint32_t n = min(*ray_counter, max_rays);
+	float s = 0.f;
+	for (uint32_t i = threadIdx.x; i < n; i += 1024) s += ray_loss[i];
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		float t = 0.f;
+		for (int w = 0; w < 16; ++w) t += part[w];
+		*out = t;
+	}
+}
+
+N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, uint64_t workspace_bytes, n2_trainer_t** out) {
+	N2_REQUIRE(out != nullptr, "n2_trainer_create: out is null");
+	*out = nullptr;
+	if (int rc = check_cfg(cfg, "n2_trainer_create")) return rc;
+	N2_REQUIRE(d_workspace != nullptr && reinterpret_cast<uintptr_t>(d_workspace) % 256 == 0, "n2_trainer_create: workspace must be non-null and 256-byte aligned");
+	n2_trainer* t = new (std::nothrow) n2_trainer();
+	N2_REQUIRE(t != nullptr, "n2_trainer_create: out of host memory");
+	*t = n2_trainer{};
+	t->cfg = *cfg;
+	int rc = make_field(cfg, &t->field);
+	if (rc != N2_OK) { delete t; return rc; }
+	const TrainerCarve c = trainer_carve(cfg, t->field);
+	if (workspace_bytes < c.total) {
+		n2_set_error("n2_trainer_create: %llu bytes given, %llu needed", (unsigned long long)workspace_bytes, (unsigned long long)c.total);
+		n2_field_destroy(t->field);
+		delete t;
+		return N2_ERR_INVALID_ARGUMENT;
+	}
+	unsigned char* b = reinterpret_cast<unsigned char*>(d_workspace);
+	t->ws = b;
+	t->n_params = n2_field_n_params(t->field);
+	uint32_t offs[5];
+	n2_field_param_offsets(t->field, offs);
+	t->n_matrix_params = offs[2];
+	t->master = reinterpret_cast<float*>(b + c.master);
+	t->params = reinterpret_cast<hf*>(b + c.params);
+	t->grads = reinterpret_cast<hf*>(b + c.grads);
+	t->m1 = reinterpret_cast<float*>(b + c.m1);
+	t->m2 = reinterpret_cast<float*>(b + c.m2);
+	t->steps = reinterpret_cast<uint32_t*>(b + c.steps);
+	t->coords = reinterpret_cast<float*>(b + c.coords);
+	t->mlp_out = reinterpret_cast<hf*>(b + c.mlp_out);
+	t->dloss = reinterpret_cast<hf*>(b + c.dloss);
+	t->coords_compacted = reinterpret_cast<float*>(b + c.coords_compacted);
+	t->numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps);
+	t->ray_indices = reinterpret_cast<uint32_t*>(b + c.ray_indices);
+	t->rgb_target = reinterpret_cast<float*>(b + c.rgb_target);
+	t->ray_loss = reinterpret_cast<float*>(b + c.ray_loss);
+	t->counters = reinterpret_cast<uint32_t*>(b + c.counters);
+	t->ws_sampler = b + c.ws_sampler;
+	t->ws_sampler_bytes = c.ws_composite - c.ws_sampler;
+	t->ws_composite = b + c.ws_composite;
+	t->ws_composite_bytes = c.ws_field - c.ws_composite;
+	t->ws_field = b + c.ws_field;
+	const uint32_t S = cfg->max_samples > cfg->target_batch_size ? cfg->max_samples : cfg->target_batch_size;
+	rc = n2_field_set_params(t->field, reinterpret_cast<const n2_half*>(t->params), reinterpret_cast<n2_half*>(t->grads));
+	if (rc == N2_OK) rc = n2_field_set_workspace(t->field, t->ws_field, c.total - c.ws_field, S, cfg->target_batch_size);
+	// optimiser state, gradients, counters and every per-step buffer start at zero (padding rows of a
+	// batch are then valid positions with zero gradient)
+	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.grads, c.coords - c.grads);
+	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.coords, c.ws_sampler - c.coords);
+	if (rc == N2_OK && hipStreamSynchronize(nullptr) != hipSuccess) { n2_set_error("n2_trainer_create: workspace initialisation failed"); rc = N2_ERR_HIP; }
+	if (rc != N2_OK) {
+		n2_field_destroy(t->field);
+		delete t;
+		return rc;
+	}
+	*out = t;
+	return N2_OK;
+}
+
+N2_API void n2_trainer_destroy(n2_trainer_t* t) {
+	if (!t) return;
+	n2_field_destroy(t->field);
+	delete t;
+}
+
+N2_API int n2_trainer_buffers(n2_trainer_t* t, float** d_master, n2_half** d_params, n2_half** d_gradients, uint32_t* n_params) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_buffers: trainer is null");
+	if (d_master) *d_master = t->master;
+	if (d_params) *d_params = reinterpret_cast<n2_half*>(t->params);
+	if (d_gradients) *d_gradients = reinterpret_cast<n2_half*>(t->grads);
+	if (n_params) *n_params = t->n_params;
+	return N2_OK;
+}
+
+N2_API int n2_trainer_sync_params(n2_trainer_t* t, n2_stream_t stream) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_sync_params: trainer is null");
+	trainer_cast_params_kernel<<<dim3((t->n_params + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(t->n_params, t->master, t->params);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API n2_field_t* n2_trainer_field(n2_trainer_t* t) { return t ? t->field : nullptr; }
+
+N2_API int n2_trainer_set_scene(n2_trainer_t* t, const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba, const uint8_t* d_bitfield) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_set_scene: trainer is null");
+	N2_REQUIRE(d_cameras && d_rgba && d_bitfield && n_images > 0, "n2_trainer_set_scene: null scene buffer or no images");
+	t->cameras = d_cameras; t->n_images = n_images; t->rgba = d_rgba; t->bitfield = d_bitfield;
+	return N2_OK;
+}
+
+N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays, uint32_t n_inference, uint32_t seed) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_step: trainer is null");
+	N2_REQUIRE(t->cameras != nullptr, "n2_trainer_step: n2_trainer_set_scene has not been called");
+	N2_REQUIRE(n_rays >= 1 && n_rays <= t->cfg.max_rays_per_batch, "n2_trainer_step: n_rays %u outside [1, %u]", n_rays, t->cfg.max_rays_per_batch);
+	N2_REQUIRE(n_inference % 8 == 0 && n_inference <= t->cfg.max_samples, "n2_trainer_step: n_inference %u must be a multiple of 8 and <= %u",
+	           n_inference, t->cfg.max_samples);
+	hipStream_t s = n2_stream(stream);
+	const uint32_t T = t->cfg.target_batch_size;
+	uint32_t* ray_counter = t->counters;
+	uint32_t* sample_counter = t->counters + 1;
+	uint32_t* compacted_counter = t->counters + 2;
+	// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
+	if (int rc = n2_generate_training_samples(stream, n_rays, t->n_rays_total, seed, t->cameras, t->n_images, t->rgba, t->cfg.composite.background,
+	                                          t->bitfield, n_inference, ray_counter, sample_counter, t->ray_indices, t->numsteps, t->rgb_target,
+	                                          t->coords, t->ws_sampler, t->ws_sampler_bytes)) return rc;
+	t->n_rays_total += n_rays;
+	// field over every marched sample
+	if (int rc = n2_field_forward(t->field, stream, t->coords, n_inference, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	// compositing, loss, gradients w.r.t. the outputs, compaction
+	n2_composite_config cc = t->cfg.composite;
+	cc.n_rays_norm = n_rays;
+	cc.loss_scale = t->cfg.loss_scale;
+	if (int rc = n2_composite_loss(stream, &cc, n_rays, ray_counter, t->numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), t->coords,
+	                               t->rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
+	                               t->ws_composite, t->ws_composite_bytes)) return rc;
+	trainer_loss_sum_kernel<<<dim3(1), dim3(1024), 0, s>>>(ray_counter, n_rays, t->ray_loss, reinterpret_cast<float*>(t->counters + 4));
+	N2_LAUNCH_CHECK();
+	// pad the compacted batch to exactly T samples
+	if (int rc = n2_fill_rollover_and_rescale_f16(stream, T, 16, compacted_counter, reinterpret_cast<n2_half*>(t->dloss))) return rc;
+	if (int rc = n2_fill_rollover_f32(stream, T, 7, compacted_counter, t->coords_compacted)) return rc;
+	// forward + backward on the compacted batch, then the optimiser
+	if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
+	return n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
+	                    reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps);
+}
+
+N2_API int n2_trainer_read_counters(n2_trainer_t* t, n2_stream_t stream, uint32_t* rays, uint32_t* samples, uint32_t* compacted, float* loss) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_read_counters: trainer is null");
+	uint32_t host[8] = {};
+	N2_HIP(hipMemcpyAsync(host, t->counters, sizeof(host), hipMemcpyDeviceToHost, n2_stream(stream)));
+	N2_HIP(hipStreamSynchronize(n2_stream(stream)));
+	if (rays) *rays = host[0];
+	if (samples) *samples = host[1];
+	if (compacted) *compacted = host[2];
+	if (loss) { float f; memcpy(&f, &host[4], 4); *loss = f; }
+	return N2_OK;
+}

@@ -250,10 +250,10 @@ class NerfNetwork:
         """Allocates the workspace (the reference's arena temporaries) for batches up to max_batch."""
         if max_batch <= self.max_batch:
             return
-        nbytes = int(capi.lib().n2_field_workspace_bytes(self._h, C.c_uint32(max_batch)))
+        nbytes = int(capi.lib().n2_field_workspace_bytes(self._h, C.c_uint32(max_batch), C.c_uint32(max_batch)))
         self._ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-        check(capi.lib().n2_field_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes), C.c_uint32(max_batch)),
-              "n2_field_set_workspace")
+        check(capi.lib().n2_field_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes), C.c_uint32(max_batch),
+                                                C.c_uint32(max_batch)), "n2_field_set_workspace")
         self.max_batch = max_batch
 
     @staticmethod

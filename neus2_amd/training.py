@@ -1,0 +1,161 @@
+"""Host side of the training loop: the trainer object over the C ABI, parameter
+initialisation and the ray-count feedback of the reference's train_nerf
+(src/testbed_nerf.cu:3393-3498).  torch supplies device memory and the stream."""
+import ctypes as C
+import math
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import N2Error, check, ptr
+
+BATCH_SIZE_GRANULARITY = 128  # tcnn::batch_size_granularity, src/testbed_nerf.cu:3429, 3768
+
+
+def next_multiple(x, m):
+    return (int(x) + m - 1) // m * m
+
+
+def default_config(target_batch_size=1 << 18, max_rays_per_batch=1 << 16, max_samples=None, n_levels=16,
+                   log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447, ek_loss_weight=0.01,
+                   background=(1.0, 1.0, 1.0), learning_rate=1e-3):
+    """configs/nerf/base.json, with the level count / growth factor BASELINE's configs fix."""
+    if max_samples is None:
+        max_samples = 16 * target_batch_size  # src/testbed_nerf.cu:3719
+    cfg = capi.TrainerConfig()
+    cfg.field = capi.FieldConfig(n_levels, 2, log2_hashmap_size, base_resolution, per_level_scale, 1, 2, -0.1)
+    cfg.adam = capi.AdamConfig(learning_rate, 0.9, 0.99, 1e-15, 1e-6)
+    cfg.composite = capi.CompositeConfig(128.0, ek_loss_weight, 1.0, (C.c_float * 3)(*background), 1)
+    cfg.target_batch_size = target_batch_size
+    cfg.max_rays_per_batch = max_rays_per_batch
+    cfg.max_samples = max_samples
+    cfg.loss_scale = 128.0
+    return cfg
+
+
+def initial_parameters(offsets, sdf_in_width, seed=1337, sdf_mlp_weights=None):
+    """NerfNetwork::initialize_params (nerf_network.h:805-876): Xavier-uniform MLPs, the SDF MLP overwritten with
+    the geometric-init weights when given (utils/mlp_weights*.txt), grid U(-1e-4, 1e-4), variance 0.3.
+    The reference draws from tcnn's pcg32, which is not reproducible here: numpy's generator stands in."""
+    off_sdf, off_rgb, off_grid, off_var, n = offsets
+    rng = np.random.default_rng(seed)
+    p = np.zeros(n, np.float32)
+
+    def xavier(rows, cols):
+        s = math.sqrt(6.0 / (rows + cols))
+        return rng.uniform(-s, s, rows * cols).astype(np.float32)
+
+    p[off_sdf:off_rgb] = np.concatenate([xavier(64, sdf_in_width), xavier(16, 64)])
+    if sdf_mlp_weights is not None:
+        w = np.asarray(sdf_mlp_weights, np.float32)
+        if w.size != off_rgb - off_sdf:
+            raise N2Error(f"SDF MLP weight file has {w.size} values, the network needs {off_rgb - off_sdf}")
+        p[off_sdf:off_rgb] = w
+    p[off_rgb:off_grid] = np.concatenate([xavier(64, 48), xavier(64, 64), xavier(16, 64)])
+    p[off_grid:off_var] = rng.uniform(-1e-4, 1e-4, off_var - off_grid).astype(np.float32)
+    p[off_var:] = 0.3
+    return p
+
+
+class RayBudget:
+    """Feedback that keeps the compacted batch near the target (src/testbed_nerf.cu:3406-3429, 3751-3756):
+    after reading the counters, rays_per_batch is rescaled by target / measured compacted samples, and the
+    next steps' inference window is the measured number of marched samples rounded up to 128."""
+
+    def __init__(self, target_batch_size, max_rays, max_samples, rays_per_batch=1 << 12):
+        self.target, self.max_rays, self.max_samples = target_batch_size, max_rays, max_samples
+        self.rays_per_batch = min(rays_per_batch, max_rays)
+        self.measured_before_compaction = 0
+
+    def n_inference(self):
+        if self.measured_before_compaction == 0:
+            return self.max_samples
+        return next_multiple(min(self.measured_before_compaction, self.max_samples), BATCH_SIZE_GRANULARITY)
+
+    def update(self, rays, samples, compacted):
+        if compacted == 0 or samples == 0:
+            return False  # the reference warns and stops training (src/testbed_nerf.cu:3536-3542)
+        self.measured_before_compaction = min(int(samples), self.max_samples)
+        r = next_multiple(self.rays_per_batch * self.target / compacted, BATCH_SIZE_GRANULARITY)
+        self.rays_per_batch = int(min(max(r, BATCH_SIZE_GRANULARITY), self.max_rays))
+        return True
+
+
+class Trainer:
+    def __init__(self, cfg=None, device="cuda"):
+        self.cfg = cfg if cfg is not None else default_config()
+        L = capi.lib()
+        nbytes = int(L.n2_trainer_workspace_bytes(C.byref(self.cfg)))
+        if nbytes == 0:
+            raise N2Error("invalid trainer configuration: " + L.n2_last_error().decode())
+        self.workspace_bytes = nbytes
+        self._ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self._h = C.c_void_p()
+        check(L.n2_trainer_create(C.byref(self.cfg), ptr(self._ws), C.c_uint64(nbytes), C.byref(self._h)), "n2_trainer_create")
+        m, p, g, n = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_uint32()
+        check(L.n2_trainer_buffers(self._h, C.byref(m), C.byref(p), C.byref(g), C.byref(n)), "n2_trainer_buffers")
+        self.n_params = int(n.value)
+        base = self._ws.data_ptr()
+        self.master = self._ws[m.value - base:m.value - base + 4 * self.n_params].view(torch.float32)
+        self.params = self._ws[p.value - base:p.value - base + 2 * self.n_params].view(torch.float16)
+        self.grads = self._ws[g.value - base:g.value - base + 2 * self.n_params].view(torch.float16)
+        self._field = C.c_void_p(L.n2_trainer_field(self._h))
+        o = (C.c_uint32 * 5)()
+        check(L.n2_field_param_offsets(self._field, o), "n2_field_param_offsets")
+        self.offsets = list(o)
+        self.sdf_in_width = (3 + 2 * self.cfg.field.n_levels + 15) // 16 * 16
+        self._scene = None
+        self.budget = RayBudget(self.cfg.target_batch_size, self.cfg.max_rays_per_batch, self.cfg.max_samples)
+        self.step_index = 0
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) is not None and self._h.value:
+                capi.lib().n2_trainer_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+    def _stream(self):
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def set_parameters(self, master_np):
+        self.master.copy_(torch.from_numpy(np.ascontiguousarray(master_np, np.float32)).to(self.master.device))
+        check(capi.lib().n2_trainer_sync_params(self._h, self._stream()), "n2_trainer_sync_params")
+
+    def initialize_params(self, seed=1337, sdf_mlp_weights=None):
+        self.set_parameters(initial_parameters(self.offsets, self.sdf_in_width, seed, sdf_mlp_weights))
+
+    def set_scene(self, cameras, n_images, rgba, bitfield):
+        """cameras: device byte tensor (tcnn_api.pack_cameras); rgba fp32 [pixels, 4]; bitfield uint8."""
+        self._scene = (cameras, rgba, bitfield)  # keep alive
+        check(capi.lib().n2_trainer_set_scene(self._h, ptr(cameras), C.c_uint32(n_images), ptr(rgba), ptr(bitfield)),
+              "n2_trainer_set_scene")
+
+    def step(self, n_rays=None, n_inference=None, seed=None):
+        n_rays = self.budget.rays_per_batch if n_rays is None else n_rays
+        n_inference = self.budget.n_inference() if n_inference is None else n_inference
+        seed = self.step_index if seed is None else seed
+        check(capi.lib().n2_trainer_step(self._h, self._stream(), C.c_uint32(n_rays), C.c_uint32(n_inference),
+                                         C.c_uint32(seed)), "n2_trainer_step")
+        self.step_index += 1
+
+    def read_counters(self):
+        r, s, c, l = C.c_uint32(), C.c_uint32(), C.c_uint32(), C.c_float()
+        check(capi.lib().n2_trainer_read_counters(self._h, self._stream(), C.byref(r), C.byref(s), C.byref(c), C.byref(l)),
+              "n2_trainer_read_counters")
+        return dict(rays=int(r.value), samples=int(s.value), compacted=int(c.value), loss=float(l.value))
+
+    def update_budget(self):
+        c = self.read_counters()
+        ok = self.budget.update(c["rays"], c["samples"], c["compacted"])
+        return c, ok
+
+    def sdf(self, xyz):
+        """NerfNetwork::sdf on a [3, N] tensor (N <= max_samples, multiple of 8): fp16 [16, N]."""
+        n = xyz.shape[1]
+        out = torch.empty((16, n), dtype=torch.float16, device=xyz.device)
+        check(capi.lib().n2_field_sdf(self._field, self._stream(), ptr(xyz), C.c_uint32(1), C.c_uint32(n), C.c_uint32(n),
+                                      ptr(out)), "n2_field_sdf")
+        return out

@@ -1,0 +1,65 @@
+"""Host-side logic that needs no GPU: ray budget feedback, parameter initialisation, scene helpers."""
+import os
+
+import numpy as np
+import pytest
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_ray_budget_feedback():
+    from neus2_amd.training import RayBudget
+    b = RayBudget(1 << 18, 1 << 16, 16 << 18, rays_per_batch=4096)
+    assert b.n_inference() == 16 << 18  # nothing measured yet: worst case (src/testbed_nerf.cu:3751-3753)
+    assert b.update(4000, 500000, 131072)
+    assert b.rays_per_batch == 8192 and b.n_inference() == 500096  # 2x rays, samples rounded up to 128
+    assert b.update(8000, 10 ** 9, 262144)
+    assert b.n_inference() == 16 << 18 and b.rays_per_batch == 8192
+    assert not b.update(0, 0, 0)  # nothing generated: the reference stops training here
+    b.update(8000, 1000, 10)
+    assert b.rays_per_batch == 1 << 16  # clamped to the maximum
+
+
+def test_initial_parameters_layout():
+    from neus2_amd.training import initial_parameters
+    W = np.load(os.path.join(GOLD, "sdf_mlp_weights_48.npy"))
+    offs = [0, 4096, 12288, 12288 + 12599920, 12288 + 12599920 + 4]
+    p = initial_parameters(offs, 48, seed=1, sdf_mlp_weights=W)
+    assert p.dtype == np.float32 and p.size == offs[4]
+    np.testing.assert_array_equal(p[:4096], W)
+    assert np.abs(p[4096:12288]).max() <= np.sqrt(6 / (16 + 64)) + 1e-6 and p[4096:12288].std() > 0.05  # widest: the 16x64 layer
+    g = p[12288:offs[3]]
+    assert np.abs(g).max() <= 1e-4 and abs(g.mean()) < 1e-6
+    np.testing.assert_array_equal(p[offs[3]:], np.float32(0.3))
+    from neus2_amd.capi import N2Error
+    with pytest.raises(N2Error):
+        initial_parameters(offs, 48, sdf_mlp_weights=W[:100])
+
+
+def test_scene_cameras_look_at_the_centre():
+    from neus2_amd import scene
+    cams = scene.cameras_on_sphere(16, 32)
+    for c in cams:
+        X = c["xform"].reshape(3, 4)
+        R, o = X[:, :3], X[:, 3]
+        np.testing.assert_allclose(R.T @ R, np.eye(3), atol=1e-5)
+        np.testing.assert_allclose(np.linalg.norm(o - 0.5), 2.0, rtol=1e-5)
+        np.testing.assert_allclose(R[:, 2], (0.5 - o) / 2.0, atol=1e-5)
+    img = scene.render_sphere_images(cams[:2])
+    a = img[:, 3].reshape(2, 32, 32)
+    assert a[:, 16, 16].all() and not a[:, 0, 0].any()  # sphere in the middle, empty corners
+
+
+def test_trainer_config_struct_matches_header():
+    """ctypes mirror vs the C declaration: same field count and 4-byte packing."""
+    import ctypes
+    from neus2_amd import capi
+    assert ctypes.sizeof(capi.FieldConfig) == 32 and ctypes.sizeof(capi.AdamConfig) == 20
+    assert ctypes.sizeof(capi.CompositeConfig) == 28 and ctypes.sizeof(capi.Camera) == 80
+    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 16
+    L = capi.lib()
+    cfg = capi.TrainerConfig()
+    assert L.n2_trainer_workspace_bytes(ctypes.byref(cfg)) == 0  # all-zero config is rejected on the host
+    from neus2_amd.training import default_config
+    n = L.n2_trainer_workspace_bytes(ctypes.byref(default_config()))
+    assert 3 * 2 ** 30 < n < 6 * 2 ** 30
