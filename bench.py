@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the NeuS2 SDF-field hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid] [--no-cpu-baseline]
+
+A step is one full static NeuS2 training step (BASELINE config 4) on a synthetic scene: an analytic sphere of
+radius 0.3, Lambertian-textured, seen by 64 cameras at 512x512 on a sphere of radius 2; rays are marched through a
+128^3 occupancy bitfield and compacted to 2^18 samples; hash grid + SDF MLP + colour MLP forward, first- and
+second-order backward, compositing and Adam, all on the GPU.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+TARGET = 1 << 18
+HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
+# algorithmic bytes per sample of the kernels a roofline is reported for:
+#   grid backward (parameter scatter): 12 (xyz) + 64 (dL_dy, 32 fp16) + 128 x 4 (packed fp16 atomics) = 588
+#   grid forward:                      12 (xyz) + 128 x 4 (gathers) + 64 (32 fp16 out)             = 588
+#   grid second order:                 12 + 12 (v) + 64 (dL_dy) + 64 (dL_ddLdy) + 128 x 4           = 664
+ALGO_BYTES = {"grid_backward_params": 588, "grid_forward": 588, "grid_second_order": 664}
+PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
+        "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8}
+
+
+def build_scene(n_cameras=64, resolution=512):
+    from neus2_amd import scene
+    cams = scene.cameras_on_sphere(n_cameras, resolution)
+    rgba = scene.render_sphere_images(cams)
+    bits = scene.sphere_bitfield(radius=0.3, band=0.03)
+    return cams, rgba, bits
+
+
+def profile_read(lib, name):
+    import ctypes as C
+    ms, n = C.c_float(), C.c_uint32()
+    lib.n2_profile_read(C.c_int(PROF[name]), C.byref(ms), C.byref(n))
+    return float(ms.value), int(n.value)
+
+
+def cpu_baseline(cams, rgba, bits, sdf_weights, budget_s=20.0):
+    """The oracle's full training step on the host cores, on a bounded sample of the same workload."""
+    import numpy as np
+    from oracle import oracle as orc
+    from oracle.field import Field
+    from oracle.step import StepState, training_step
+    from neus2_amd.training import initial_parameters
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    f = Field(fp16=True)
+    offs = [f.off_sdf, f.off_rgb, f.off_grid, f.off_var, f.n_params]
+    st = StepState(f, initial_parameters(offs, f.sdf_in_w, seed=1337, sdf_mlp_weights=sdf_weights))
+    ocams = []
+    for c in cams:
+        po = int(c["pixel_offset"])
+        ocams.append(orc.Camera((orc.C.c_float * 12)(*c["xform"]), (orc.C.c_float * 2)(*c["focal"]),
+                                (orc.C.c_float * 2)(*c["principal"]), (orc.C.c_uint32 * 2)(*c["res"]), po & 0xFFFFFFFF, po >> 32))
+    T = 1 << 15
+    n_rays = 768  # about 45% of the rays hit the shell, ~115 marched samples each -> a little over T samples
+    best, done, t_all = None, 0, time.time()
+    while done < 3 or (time.time() - t_all < budget_s and done < 8):
+        t0 = time.time()
+        r = training_step(st, ocams, rgba, bits, n_rays, 16 * T, seed=done, target_batch_size=T)
+        dt = time.time() - t0
+        best = dt if best is None else min(best, dt)
+        done += 1
+    return {"value": T / best, "unit": "samples/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": f"one full training step at a 2^15-sample batch ({r['rays']} rays, {r['samples']} marched samples, "
+                      f"same scene and initialisation), best of {done} runs, {best * 1e3:.0f} ms"}
+
+
+def run_step_workload(args):
+    import ctypes as C
+    import numpy as np
+    import torch
+    from neus2_amd import capi
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    lib = capi.lib()
+    cams, rgba, bits = build_scene()
+    sdf_w = np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy"))
+    tr = Trainer(default_config(target_batch_size=TARGET, max_rays_per_batch=1 << 16, max_samples=16 * TARGET))
+    d_cams, d_rgba, d_bits = pack_cameras(cams), torch.from_numpy(rgba).cuda(), torch.from_numpy(bits).cuda()
+    tr.set_scene(d_cams, len(cams), d_rgba, d_bits)
+    tr.initialize_params(seed=1337, sdf_mlp_weights=sdf_w)
+    # untimed: let the ray-count feedback settle so that the compacted batch fills the 2^18 target
+    tr.budget.rays_per_batch = 4096
+    for _ in range(6):
+        tr.step()
+        counters, ok = tr.update_budget()
+        if not ok:
+            raise SystemExit(f"no samples generated: {counters}")
+    n_rays, n_inf = tr.budget.rays_per_batch, tr.budget.n_inference()
+    for _ in range(args.warmup):
+        tr.step(n_rays=n_rays, n_inference=n_inf)
+    torch.cuda.synchronize()
+    lib.n2_profile_reset()
+    lib.n2_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        tr.step(n_rays=n_rays, n_inference=n_inf)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.n2_profile_enable(0)
+    counters = tr.read_counters()
+    kernels = {}
+    for name in PROF:
+        ms, n = profile_read(lib, name)
+        if n:
+            kernels[name] = {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_us": ms / n * 1e3}
+    dom = max((k for k in ALGO_BYTES if k in kernels), key=lambda k: kernels[k]["ms_per_step"])
+    # per-launch batch of the dominant kernel: the backward kernels always see the 2^18 compacted batch; the forward
+    # also runs over the marched samples, so use the average batch per launch
+    per_launch = TARGET if dom != "grid_forward" else (TARGET + n_inf) / 2
+    achieved = ALGO_BYTES[dom] * per_launch / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    result = {
+        "metric": "SDF train samples/sec @2^18 batch (1 GPU)",
+        "value": args.steps * TARGET / elapsed,
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "full NeuS2 static training step (BASELINE configs[3]): analytic sphere r=0.3, 64 cameras 512x512 "
+                               "on a radius-2 sphere, 128^3 occupancy bitfield, rays compacted to 2^18 samples; hash grid "
+                               "L=16 F=2 T=2^19 + SDF MLP 48-64-16 + colour MLP 48-64-64-16, first and second order backward, "
+                               "compositing, Adam",
+                   "target_batch": TARGET, "rays_per_step": n_rays, "marched_samples_per_step": counters["samples"],
+                   "inference_batch": n_inf, "compacted_before_rollover": counters["compacted"], "loss": counters["loss"]},
+        "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_sample": ALGO_BYTES[dom], "samples_per_launch": per_launch,
+                     "avg_launch_us": kernels[dom]["avg_us"]},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cams, rgba, bits, sdf_w)
+    return result
+
+
+def run_grid_workload(args):
+    """BASELINE configs[1]: hash-grid encoding only, forward + backward on 2^18 uniform points."""
+    import torch
+    from neus2_amd import capi
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding
+    lib = capi.lib()
+    g = GridEncoding()
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    params = ((torch.rand(g.n_params(), device="cuda", generator=gen) * 2 - 1) * 1e-4).half()
+    grads = torch.zeros_like(params)
+    g.set_params(params, grads)
+    x = torch.rand((3, TARGET), device="cuda", generator=gen)
+    dy = torch.randn((32, TARGET), device="cuda", generator=gen).half()
+
+    def step():
+        _, ctx = g.forward(x, prepare_input_gradients=True)
+        g.backward(ctx, x, dy, want_input_grad=True, mode=GRAD_OVERWRITE)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.n2_profile_reset()
+    lib.n2_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.n2_profile_enable(0)
+    kernels = {}
+    for name in ("grid_forward", "grid_backward_params"):
+        ms, n = profile_read(lib, name)
+        kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
+    dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    achieved = ALGO_BYTES[dom] * TARGET / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    return {"metric": "hash-grid fwd+bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "hash-grid encoding only, forward + backward (BASELINE configs[1])", "batch": TARGET},
+            "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+            "kernels": kernels}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=["step", "grid"], default="step")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs the hot path on ONE GPU (the reference has no multi-GPU path and the "
+                         "benchmark metric is quoted on 1 GPU); run with --gpus 1")
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (there is no CPU fallback of the product path)")
+    result = run_step_workload(args) if args.workload == "step" else run_grid_workload(args)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
