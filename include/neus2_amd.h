@@ -113,6 +113,18 @@ int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const f
                                     const float* d_dL_ddLdx, const n2_half* d_dL_dy, n2_half* d_dL_ddLdy,
                                     float* d_dL_dx, n2_grad_mode mode);
 
+/* First- and second-order parameter gradients in ONE scatter pass: the fusion of the two calls above as
+ * NerfNetwork::backward_impl issues them back to back (nerf_network.h:419-429 then :534-544).  Each table
+ * entry receives dL_dy*weight + dL_dy_second*(second-order coefficient) as a single packed fp16 atomic,
+ * which halves the atomic traffic of the backward pass.  No dL_dx outputs.
+ *  d_dL_dy          fp16 SoA output_width x N: first-order output gradient
+ *  d_dL_ddLdx       fp32 SoA 3 x N;  d_dL_dy_second fp16 SoA output_width x N (see backward_backward_input)
+ *  d_dL_ddLdy       NULL or fp16 SoA output_width x N
+ *  mode             OVERWRITE or ACCUMULATE */
+int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                           uint32_t dim_stride, uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx,
+                           const n2_half* d_dL_dy_second, n2_half* d_dL_ddLdy, n2_grad_mode mode);
+
 /* Test hook for the bit-exact contract: entry index (without the level offset)
  * of the 8 trilinear corners, uint32 [n_levels][8][N], corner c uses +1 on
  * dimension d iff bit d of c is set (takikawa_encoding.cuh:82-92). */

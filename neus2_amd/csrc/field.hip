@@ -134,24 +134,33 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 	o[10] = (hf)c[6];
 }
 
-// dL_drgb = rows 0..2 of dL_doutput (rest zero); variance gradient = sum of row 7.
-__global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ dL_drgb,
-                                                                 float* __restrict__ var_acc) {
-	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+// dL_drgb = rows 0..2 of dL_doutput (rest zero); variance gradient = sum of row 7
+// (workgroup reduction, then one atomic per 1024 samples: same-address atomics serialise).
+constexpr uint32_t PREP_BLOCK = 1024;
+__global__ void __launch_bounds__(PREP_BLOCK) field_backward_prep_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ dL_drgb,
+                                                                         float* __restrict__ var_acc) {
+	__shared__ float part[PREP_BLOCK / 64];
+	const uint32_t i = blockIdx.x * PREP_BLOCK + threadIdx.x;
 	float s = 0.f;
 	if (i < N) {
 		const hf* src = dL_dout + (size_t)i * 16;
 		typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-		half8 lo = {src[0], src[1], src[2], (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
+		const half8 in = *reinterpret_cast<const half8*>(src);
+		half8 lo = {in[0], in[1], in[2], (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
 		half8 hi = {(hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
 		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16) = lo;
 		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16 + 8) = hi;
-		s = (float)src[7];
+		s = (float)in[7];
 	}
-	// wave reduction, then one atomic per wave
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-	if ((threadIdx.x & 63) == 0 && s != 0.f) atomicAdd(var_acc, s);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		float t = 0.f;
+		for (uint32_t w = 0; w < PREP_BLOCK / 64; ++w) t += part[w];
+		if (t != 0.f) atomicAdd(var_acc, t);
+	}
 }
 
 __global__ void __launch_bounds__(FB) field_add_density_gradient_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ d_sdf_out_row0) {
@@ -365,7 +374,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	hipStream_t s = n2_stream(stream);
 	const hf* dL = reinterpret_cast<const hf*>(d_dL_doutput);
 	if (int rc = n2_fill_zero_u32(s, f->var_acc, 16)) return rc;
-	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, dL, f->dL_drgb, f->var_acc);
+	field_backward_prep_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->dL_drgb, f->var_acc);
 	N2_LAUNCH_CHECK();
 	// colour net
 	if (int rc = n2_mlp_backward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, reinterpret_cast<const n2_half*>(f->dL_drgb),
@@ -375,18 +384,18 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient
 	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
 	                             N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), mode)) return rc;
-	// grid, first order
-	if (int rc = n2_grid_backward(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), nullptr,
-	                              nullptr, mode)) return rc;
 	// dL/dnormal and the variance gradient
 	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->v,
 	                                                             f->d_density_in, f->var_acc, f->grads + f->off_var,
 	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();
-	// second order: grid (its dL_ddLdy lands in rows 3.. of the MLP's second-order input), then the SDF net
-	if (int rc = n2_grid_backward_backward_input(f->grid, stream, d_coords, 7, 1, n, f->v,
-	                                             reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n),
-	                                             reinterpret_cast<n2_half*>(f->d_density_in + (size_t)3 * n), nullptr, N2_GRAD_ACCUMULATE)) return rc;
+	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
+	// Overwrite followed by backward_backward_input with Accumulate); the second-order dL_ddLdy lands in
+	// rows 3.. of the MLP's second-order input
+	if (int rc = n2_grid_backward_fused(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
+	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n),
+	                                    reinterpret_cast<n2_half*>(f->d_density_in + (size_t)3 * n), mode)) return rc;
+	// second order through the SDF net
 	return n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
 	                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE);
 }

@@ -176,35 +176,94 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_indices_kernel(N2LevelTable t
 }
 
 // ----------------------------------------------------------------------------
-// backward: parameter scatter (packed fp16 atomics) ...
+// backward: parameter scatter (packed fp16 atomics), first and second order in
+// one pass.
+//
+// Atomics retire at a fixed rate per REQUEST, and lanes of one instruction that
+// hit the same 8 bytes travel as one request.  Corners that differ only in x
+// are neighbours in the table (dense levels: index + 1; hashed levels: the x
+// term enters the hash with prime 1, so even x and x+1 differ in bit 0 only).
+// A point is therefore handled by a PAIR of adjacent lanes: lane bit 0 selects
+// the x corner, each lane issues the four (y, z) corners.  That halves the
+// number of atomic requests against one lane per point.
+//
+// Per corner c of level l the two contributions are
+//   first order   dL_dy[l,f] * weight_c
+//   second order  g[l,f] * scale_l * sum_d v_d * s_{c,d} * prod_{d' != d} w_{c,d'}
+// and they leave as ONE packed fp16 atomic (one rounding instead of two).
 // ----------------------------------------------------------------------------
-template <uint32_t MODE>
-__device__ __forceinline__ void grid_scatter_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
-                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
-                                                   const __half* __restrict__ dL_dy, __half2* __restrict__ grads) {
-	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, tab.scale[level]);
-	uint32_t e[8];
-	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
+constexpr uint32_t PAIR_POINTS = GRID_BLOCK / 2;  // points per workgroup and level
+
+template <uint32_t MODE, bool FIRST, bool SECOND, bool WANT_OUT>
+__device__ __forceinline__ void grid_scatter_pair(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t b, uint32_t N,
+                                                  const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                  const __half* __restrict__ dL_dy, const float* __restrict__ v,
+                                                  const __half* __restrict__ g2, const __half2* __restrict__ params,
+                                                  __half2* __restrict__ grads, __half* __restrict__ dL_ddLdy) {
+	const float scale = tab.scale[level];
+	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
 	const size_t row = (size_t)level * 2;
-	const float g0 = __half2float(dL_dy[row * N + i]);
-	const float g1 = __half2float(dL_dy[(row + 1) * N + i]);
-	if (g0 == 0.f && g1 == 0.f) return;
-	__half2* G = grads + tab.offset[level];
+	float a0 = 0.f, a1 = 0.f, c0 = 0.f, c1 = 0.f, v0 = 0.f, v1 = 0.f, v2 = 0.f;
+	if (FIRST) {
+		a0 = __half2float(dL_dy[row * N + i]);
+		a1 = __half2float(dL_dy[(row + 1) * N + i]);
+	}
+	if (SECOND) {
+		c0 = __half2float(g2[row * N + i]);
+		c1 = __half2float(g2[(row + 1) * N + i]);
+		v0 = v[i] * scale; v1 = v[(size_t)N + i] * scale; v2 = v[(size_t)2 * N + i] * scale;
+	}
+	const bool skip = !SECOND && a0 == 0.f && a1 == 0.f;  // nothing to add (both lanes of a pair agree)
+	const float wx = b ? p.w[0] : 1.f - p.w[0];
+	const float sx = b ? 1.f : -1.f;
+	const uint32_t gx = p.c[0] + b;
+	const __half2* P = params + tab.offset[level];
+	__half2* G = grads ? grads + tab.offset[level] : nullptr;
+	float o0 = 0.f, o1 = 0.f;
 #pragma unroll
-	for (uint32_t k = 0; k < 8; ++k) {
-		const float wt = n2_corner_weight(p, k);
-		unsafeAtomicAdd(&G[e[k]], __floats2half2_rn(g0 * wt, g1 * wt));
+	for (uint32_t k = 0; k < 4; ++k) {
+		const uint32_t y = k & 1u, z = k >> 1;
+		const uint32_t e = n2_entry<MODE>(entries, res, gx, p.c[1] + y, p.c[2] + z);
+		const float wy = y ? p.w[1] : 1.f - p.w[1], wz = z ? p.w[2] : 1.f - p.w[2];
+		float r0 = 0.f, r1 = 0.f;
+		if (FIRST) {
+			const float wt = wx * wy * wz;
+			r0 = a0 * wt;
+			r1 = a1 * wt;
+		}
+		if (SECOND) {
+			const float sy = y ? 1.f : -1.f, sz = z ? 1.f : -1.f;
+			const float coef = v0 * sx * wy * wz + v1 * sy * wx * wz + v2 * sz * wx * wy;
+			r0 = fmaf(c0, coef, r0);
+			r1 = fmaf(c1, coef, r1);
+			if (WANT_OUT) {
+				const float2 val = __half22float2(P[e]);
+				o0 = fmaf(coef, val.x, o0);
+				o1 = fmaf(coef, val.y, o1);
+			}
+		}
+		if (G && !skip) unsafeAtomicAdd(&G[e], __floats2half2_rn(r0, r1));
+	}
+	if (SECOND && WANT_OUT) {
+		// lane b finishes feature b: it needs the partner's partial sum of that feature
+		const float mine = b ? o1 : o0, theirs = __shfl_xor(b ? o0 : o1, 1);
+		dL_ddLdy[(row + b) * N + i] = __float2half_rn(mine + theirs);
 	}
 }
 
-__global__ void __launch_bounds__(GRID_BLOCK) grid_backward_params_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
-                                                                          const float* __restrict__ xyz, uint32_t point_stride,
-                                                                          uint32_t dim_stride, const __half* __restrict__ dL_dy,
-                                                                          __half2* __restrict__ grads) {
+template <bool FIRST, bool SECOND, bool WANT_OUT>
+__global__ void __launch_bounds__(GRID_BLOCK) grid_scatter_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                                  const float* __restrict__ xyz, uint32_t point_stride,
+                                                                  uint32_t dim_stride, const __half* __restrict__ dL_dy,
+                                                                  const float* __restrict__ v, const __half* __restrict__ g2,
+                                                                  const __half2* __restrict__ params, __half2* __restrict__ grads,
+                                                                  __half* __restrict__ dL_ddLdy) {
 	const uint32_t level = blockIdx.x / tiles;
-	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
-	if (i >= N) return;
-#define CALL(M) grid_scatter_point<M>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, grads)
+	const uint32_t i = (blockIdx.x - level * tiles) * PAIR_POINTS + (threadIdx.x >> 1);
+	const uint32_t b = threadIdx.x & 1u;
+	if (i >= N) return;  // both lanes of a pair share i, so pairs leave together
+#define CALL(M) grid_scatter_pair<M, FIRST, SECOND, WANT_OUT>(tab, level, i, b, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, grads, dL_ddLdy)
 	N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
 }
@@ -439,6 +498,26 @@ static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2
 	return N2_OK;
 }
 
+static inline uint32_t n_pair_tiles(uint32_t n_points) { return (n_points + PAIR_POINTS - 1) / PAIR_POINTS; }
+
+// One scatter pass with any combination of first-order (dL_dy) and second-order (v, g2) terms.
+static int launch_scatter(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
+                          const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy) {
+	const uint32_t tiles = n_pair_tiles(n_points);
+	const dim3 gd(tiles * grid->tab.n_levels), bd(GRID_BLOCK);
+	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
+#define LAUNCH(F, S, O) grid_scatter_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
+                                                                       grid->params, grads, dL_ddLdy)
+	if (first && second && out) LAUNCH(true, true, true);
+	else if (first && second) LAUNCH(true, true, false);
+	else if (second && out) LAUNCH(false, true, true);
+	else if (second) LAUNCH(false, true, false);
+	else LAUNCH(true, false, false);
+#undef LAUNCH
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
 N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
                             uint32_t dim_stride, uint32_t n_points, const n2_half* d_dL_dy, const float* d_dy_dx,
                             float* d_dL_dx, n2_grad_mode mode) {
@@ -448,19 +527,32 @@ N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_
 	hipStream_t s = n2_stream(stream);
 	if (int rc = prepare_grads(grid, "n2_grid_backward", s, mode)) return rc;
 	if (n_points == 0) return N2_OK;
-	const uint32_t tiles = n_tiles(n_points);
 	if (mode != N2_GRAD_IGNORE) {
 		N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
-		grid_backward_params_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
-			grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, reinterpret_cast<const __half*>(d_dL_dy), grid->grads);
-		N2_LAUNCH_CHECK();
+		if (int rc = launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), nullptr,
+		                            nullptr, grid->grads, nullptr)) return rc;
 	}
 	if (d_dL_dx) {
-		grid_backward_input_kernel<<<dim3(tiles), dim3(GRID_BLOCK), 0, s>>>(
+		grid_backward_input_kernel<<<dim3(n_tiles(n_points)), dim3(GRID_BLOCK), 0, s>>>(
 			n_points, grid->tab.n_levels * grid->n_features, reinterpret_cast<const __half*>(d_dL_dy), d_dy_dx, d_dL_dx);
 		N2_LAUNCH_CHECK();
 	}
 	return N2_OK;
+}
+
+N2_API int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
+                                  uint32_t dim_stride, uint32_t n_points, const n2_half* d_dL_dy,
+                                  const float* d_dL_ddLdx, const n2_half* d_dL_dy_second, n2_half* d_dL_ddLdy,
+                                  n2_grad_mode mode) {
+	if (int rc = check_batch(grid, "n2_grid_backward_fused", d_xyz, point_stride, dim_stride, n_points)) return rc;
+	N2_REQUIRE((d_dL_dy && d_dL_ddLdx && d_dL_dy_second) || n_points == 0, "n2_grid_backward_fused: d_dL_dy, d_dL_ddLdx and d_dL_dy_second are required");
+	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_grid_backward_fused: mode must be OVERWRITE or ACCUMULATE");
+	hipStream_t s = n2_stream(stream);
+	if (int rc = prepare_grads(grid, "n2_grid_backward_fused", s, mode)) return rc;
+	if (n_points == 0) return N2_OK;
+	N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
+	return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), d_dL_ddLdx,
+	                      reinterpret_cast<const __half*>(d_dL_dy_second), grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy));
 }
 
 N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz,
@@ -476,8 +568,12 @@ N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, 
 	if (d_dL_dx) {
 		if (int rc = n2_fill_zero_u32(s, d_dL_dx, sizeof(float) * 3 * (size_t)n_points)) return rc;
 	}
-	const uint32_t tiles = n_tiles(n_points);
 	N2ProfScope prof(N2_PROF_GRID_SECOND_ORDER, s);
+	if (!d_dL_dx) {
+		return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, nullptr, d_dL_ddLdx, reinterpret_cast<const __half*>(d_dL_dy),
+		                      mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy));
+	}
+	const uint32_t tiles = n_tiles(n_points);
 	grid_bbi_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(
 		grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, d_dL_ddLdx, reinterpret_cast<const __half*>(d_dL_dy),
 		grid->params, mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy), d_dL_dx);

@@ -619,15 +619,25 @@ __global__ void __launch_bounds__(MLP_BLOCK) mlp_bbi_kernel(const hf* __restrict
 	}
 }
 
-// grads (fp16) = [grads +] sum over slabs
+// grads (fp16) = [grads +] sum over slabs.  16 parameters x 16 slab groups per workgroup: every
+// lane adds up n_slabs/16 partial sums (coalesced across the 16 parameters), LDS folds the groups.
 __global__ void __launch_bounds__(256) mlp_reduce_partials_kernel(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params,
                                                                   hf* __restrict__ grads, int accumulate) {
-	const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-	if (i >= n_params) return;
+	__shared__ float fold[16][17];
+	const uint32_t pl = threadIdx.x & 15, grp = threadIdx.x >> 4;
+	const uint32_t i = blockIdx.x * 16 + pl;
 	float s = 0.f;
-	for (uint32_t k = 0; k < n_slabs; ++k) s += partials[(size_t)k * n_params + i];
-	if (accumulate) s += (float)grads[i];
-	grads[i] = (hf)s;
+	if (i < n_params)
+		for (uint32_t k = grp; k < n_slabs; k += 16) s += partials[(size_t)k * n_params + i];
+	fold[grp][pl] = s;
+	__syncthreads();
+	if (grp == 0 && i < n_params) {
+		float t = 0.f;
+#pragma unroll
+		for (int k = 0; k < 16; ++k) t += fold[k][pl];
+		if (accumulate) t += (float)grads[i];
+		grads[i] = (hf)t;
+	}
 }
 
 // ----------------------------------------------------------------------------
@@ -734,7 +744,7 @@ N2_API int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_in
 }
 
 static int reduce_partials(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
-	mlp_reduce_partials_kernel<<<dim3((mlp->n_params + 255) / 256), dim3(256), 0, s>>>(mlp->workspace, n_slabs, mlp->n_params,
+	mlp_reduce_partials_kernel<<<dim3((mlp->n_params + 15) / 16), dim3(256), 0, s>>>(mlp->workspace, n_slabs, mlp->n_params,
 		mlp->grads, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();
 	return N2_OK;

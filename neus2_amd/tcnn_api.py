@@ -27,7 +27,7 @@ def _positions(xyz):
     if not xyz.is_contiguous():
         raise N2Error("positions must be contiguous")
     if xyz.dim() == 2 and xyz.shape[0] == 3:
-        return xyz, 1, xyz.shape[1], xyz.shape[1]
+        return xyz, 1, max(xyz.shape[1], 1), xyz.shape[1]
     if xyz.dim() == 2 and xyz.shape[1] >= 3:
         return xyz, xyz.shape[1], 1, xyz.shape[0]
     raise N2Error(f"positions must be 3 x N or N x C, got {tuple(xyz.shape)}")
@@ -112,6 +112,21 @@ class GridEncoding:
                                                          C.c_uint32(n), ptr(dL_ddLdx), ptr(dL_dy), ptr(o), ptr(dx),
                                                          C.c_int(mode)), "n2_grid_backward_backward_input")
         return o, dx
+
+    def backward_fused(self, xyz, dL_dy, dL_ddLdx, dL_dy_second, want_dL_ddLdy=True, mode=GRAD_OVERWRITE):
+        """backward (parameter gradients only) + backward_backward_input in one scatter pass."""
+        x, ps, ds, n = _positions(xyz)
+        w = self.output_width()
+        for t, what in ((dL_dy, "dL_dy"), (dL_dy_second, "dL_dy_second")):
+            if t.dtype != torch.float16 or tuple(t.shape) != (w, n) or not t.is_contiguous():
+                raise N2Error(f"{what} must be a contiguous fp16 [output_width, N] tensor")
+        if dL_ddLdx.dtype != torch.float32 or tuple(dL_ddLdx.shape) != (3, n) or not dL_ddLdx.is_contiguous():
+            raise N2Error("dL_ddLdx must be a contiguous fp32 [3, N] tensor")
+        o = torch.empty((w, n), dtype=torch.float16, device=x.device) if want_dL_ddLdy else None
+        check(capi.lib().n2_grid_backward_fused(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds), C.c_uint32(n),
+                                                ptr(dL_dy), ptr(dL_ddLdx), ptr(dL_dy_second), ptr(o), C.c_int(mode)),
+              "n2_grid_backward_fused")
+        return o
 
     def corner_indices(self, xyz):
         x, ps, ds, n = _positions(xyz)
