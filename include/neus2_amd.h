@@ -80,6 +80,14 @@ int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolutio
  * gradient buffer (n_params, may be NULL until a backward needs it). */
 int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients);
 
+/* Optional scratch for the parameter-gradient scatter (the reference takes temporaries from tcnn's arena).
+ * With it, batches of >= 4096 points scatter through an LDS counting sort (no global atomics, fp32
+ * accumulation); without it, or for tables with more than 2^19 entries per level, packed fp16 global
+ * atomics are used.  Results agree within the stated tolerance either way.
+ * n2_grid_workspace_bytes returns 0 when the table shape does not support the sorted path. */
+uint64_t n2_grid_workspace_bytes(const n2_grid_t* grid, uint32_t max_points);
+int n2_grid_set_workspace(n2_grid_t* grid, void* d_workspace, uint64_t n_bytes, uint32_t max_points);
+
 /* Encoding::forward(stream, input, &output, use_inference_params, prepare_input_gradients),
  * nerf_network.h:184-190 and inference at :671-676.
  *  d_xyz      positions in [0,1]^3; coordinate d of point i at d_xyz[i*point_stride + d*dim_stride]

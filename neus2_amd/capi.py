@@ -64,6 +64,8 @@ def lib():
         for name in ("n2_grid_n_params", "n2_grid_output_width", "n2_grid_n_levels"):
             getattr(_lib, name).restype = C.c_uint32
             getattr(_lib, name).argtypes = [C.c_void_p]
+        _lib.n2_grid_workspace_bytes.restype = C.c_uint64
+        _lib.n2_grid_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
         _lib.n2_grid_destroy.restype = None
         _lib.n2_grid_destroy.argtypes = [C.c_void_p]
         for name in ("n2_mlp_n_params", "n2_mlp_input_width", "n2_mlp_output_width"):

@@ -40,6 +40,7 @@ struct n2_field {
 	float* var_acc;    // [4]
 	void* ws_sdf;
 	void* ws_rgb;
+	void* ws_grid;
 };
 
 constexpr uint32_t FB = 256;
@@ -269,7 +270,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, total;
+	uint64_t sdf_in, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -292,6 +293,7 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.var_acc = take(16);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
+	c.ws_grid = take(n2_grid_workspace_bytes(f->grid, (uint32_t)nbw));
 	c.total = o;
 	return c;
 }
@@ -324,8 +326,11 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->var_acc = reinterpret_cast<float*>(b + c.var_acc);
 	f->ws_sdf = b + c.ws_sdf;
 	f->ws_rgb = b + c.ws_rgb;
+	f->ws_grid = b + c.ws_grid;
 	if (int rc = n2_mlp_set_workspace(f->sdf, f->ws_sdf, n2_mlp_workspace_bytes(f->sdf))) return rc;
-	return n2_mlp_set_workspace(f->rgb, f->ws_rgb, n2_mlp_workspace_bytes(f->rgb));
+	if (int rc = n2_mlp_set_workspace(f->rgb, f->ws_rgb, n2_mlp_workspace_bytes(f->rgb))) return rc;
+	const uint64_t gb = n2_grid_workspace_bytes(f->grid, max_batch_backward);
+	return n2_grid_set_workspace(f->grid, gb ? f->ws_grid : nullptr, gb, max_batch_backward);
 }
 
 static int check_field(const n2_field_t* f, const char* fn, uint32_t n) {

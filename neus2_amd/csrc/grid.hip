@@ -19,6 +19,10 @@ struct n2_grid {
 	uint32_t n_params;
 	const __half2* params;
 	__half2* grads;
+	// optional scratch of the bucketed scatter
+	unsigned char* ws;
+	uint64_t ws_bytes;
+	uint32_t ws_max_points;
 };
 
 // ----------------------------------------------------------------------------
@@ -357,6 +361,201 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bbi_kernel(N2LevelTable tab, 
 }
 
 // ----------------------------------------------------------------------------
+// bucketed scatter: parameter gradients WITHOUT global atomics
+//
+// Global atomics retire at ~2e10 requests/s on this part however they are
+// issued, which caps the scatter above at ~55 us per level.  Loads, stores and
+// LDS atomics are two orders of magnitude faster, so the scatter is turned
+// into a two-kernel counting sort on entry ranges:
+//
+//  bin     one workgroup per (level, tile of 1024 points): computes the 8192
+//          (entry, value) records of the tile, sorts them in LDS by bucket
+//          (bucket = entry / 8192, at most 64 per level) and writes the sorted
+//          tile (64 KiB, fully coalesced) plus its 65 bucket offsets.
+//  reduce  one workgroup per (level, bucket[, tile group]): walks the bucket's
+//          run in every tile (contiguous, ~1 KiB each), accumulates in an LDS
+//          table of 8192 fp32 pairs with LDS atomics, and writes the bucket's
+//          entries with plain stores.  Coarse levels have few buckets, so their
+//          work is split over tile groups and folded with (few, contention-free)
+//          global atomics.
+// Accumulation is fp32 until the single rounding to fp16 at the store, which
+// also removes the rounding drift of chained fp16 atomics.
+// ----------------------------------------------------------------------------
+constexpr uint32_t BKT_ENTRIES = 8192;   // entries per bucket: 64 KiB of fp32 pairs in LDS
+constexpr uint32_t BKT_SHIFT = 13;
+constexpr uint32_t BKT_MAX = 64;         // buckets per level (entries <= 2^19)
+constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
+constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
+constexpr uint32_t BIN_PER_THREAD = BIN_POINTS / GRID_BLOCK;  // 4
+
+struct N2BucketPlan {
+	uint32_t wg_begin[N2_MAX_LEVELS + 1];  // first reduce workgroup of each level
+	uint32_t n_buckets[N2_MAX_LEVELS];
+	uint32_t groups[N2_MAX_LEVELS];        // tile groups per bucket
+};
+
+template <uint32_t MODE, bool FIRST, bool SECOND, bool WANT_OUT>
+__device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
+                                               const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                               const __half* __restrict__ dL_dy, const float* __restrict__ v,
+                                               const __half* __restrict__ g2, const __half2* __restrict__ params,
+                                               __half* __restrict__ dL_ddLdy, uint32_t* e_out, uint32_t* val_out) {
+	const float scale = tab.scale[level];
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	uint32_t e[8];
+	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
+	const size_t row = (size_t)level * 2;
+	float a0 = 0.f, a1 = 0.f, c0 = 0.f, c1 = 0.f, v0 = 0.f, v1 = 0.f, v2 = 0.f;
+	if (FIRST) {
+		a0 = __half2float(dL_dy[row * N + i]);
+		a1 = __half2float(dL_dy[(row + 1) * N + i]);
+	}
+	if (SECOND) {
+		c0 = __half2float(g2[row * N + i]);
+		c1 = __half2float(g2[(row + 1) * N + i]);
+		v0 = v[i] * scale; v1 = v[(size_t)N + i] * scale; v2 = v[(size_t)2 * N + i] * scale;
+	}
+	const __half2* P = params + tab.offset[level];
+	float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		const float w0 = (k & 1u) ? p.w[0] : 1.f - p.w[0];
+		const float w1 = (k & 2u) ? p.w[1] : 1.f - p.w[1];
+		const float w2 = (k & 4u) ? p.w[2] : 1.f - p.w[2];
+		float r0 = 0.f, r1 = 0.f;
+		if (FIRST) {
+			const float wt = w0 * w1 * w2;
+			r0 = a0 * wt;
+			r1 = a1 * wt;
+		}
+		if (SECOND) {
+			const float s0 = (k & 1u) ? 1.f : -1.f, s1 = (k & 2u) ? 1.f : -1.f, s2 = (k & 4u) ? 1.f : -1.f;
+			const float coef = v0 * s0 * w1 * w2 + v1 * s1 * w0 * w2 + v2 * s2 * w0 * w1;
+			r0 = fmaf(c0, coef, r0);
+			r1 = fmaf(c1, coef, r1);
+			if (WANT_OUT) {
+				const float2 val = __half22float2(P[e[k]]);
+				o0 = fmaf(coef, val.x, o0);
+				o1 = fmaf(coef, val.y, o1);
+			}
+		}
+		e_out[k] = e[k];
+		const __half2 h = __floats2half2_rn(r0, r1);
+		val_out[k] = *reinterpret_cast<const uint32_t*>(&h);
+	}
+	if (SECOND && WANT_OUT) {
+		dL_ddLdy[row * N + i] = __float2half_rn(o0);
+		dL_ddLdy[(row + 1) * N + i] = __float2half_rn(o1);
+	}
+}
+
+template <bool FIRST, bool SECOND, bool WANT_OUT>
+__global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                              const float* __restrict__ xyz, uint32_t point_stride,
+                                                              uint32_t dim_stride, const __half* __restrict__ dL_dy,
+                                                              const float* __restrict__ v, const __half* __restrict__ g2,
+                                                              const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
+                                                              uint2* __restrict__ records, uint16_t* __restrict__ offsets) {
+	__shared__ uint32_t hist[BKT_MAX];
+	__shared__ uint32_t prefix[BKT_MAX + 1];
+	__shared__ uint2 staging[BIN_RECORDS];
+	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
+	if (threadIdx.x < BKT_MAX) hist[threadIdx.x] = 0;
+	__syncthreads();
+	// records of this thread: entry | rank << 19 after the counting step
+	uint32_t re[BIN_PER_THREAD * 8], rv[BIN_PER_THREAD * 8];
+	uint32_t live = 0;
+#pragma unroll
+	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
+		const uint32_t i = tile * BIN_POINTS + j * GRID_BLOCK + threadIdx.x;
+		if (i < N) {
+			live |= 1u << j;
+#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, re + 8 * j, rv + 8 * j)
+			N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+#pragma unroll
+			for (uint32_t k = 0; k < 8; ++k) {
+				const uint32_t rank = atomicAdd(&hist[re[8 * j + k] >> BKT_SHIFT], 1u);
+				re[8 * j + k] |= rank << 19;
+			}
+		}
+	}
+	__syncthreads();
+	if (threadIdx.x < 64) {  // one wave scans the 64 counters
+		const uint32_t c = hist[threadIdx.x];
+		uint32_t s = c;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) {
+			const uint32_t u = __shfl_up(s, o);
+			if ((int)threadIdx.x >= o) s += u;
+		}
+		prefix[threadIdx.x] = s - c;
+		if (threadIdx.x == 63) prefix[64] = s;
+	}
+	__syncthreads();
+#pragma unroll
+	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
+		if (live & (1u << j)) {
+#pragma unroll
+			for (uint32_t k = 0; k < 8; ++k) {
+				const uint32_t e = re[8 * j + k] & 0x7FFFFu, rank = re[8 * j + k] >> 19;
+				staging[prefix[e >> BKT_SHIFT] + rank] = make_uint2(e & (BKT_ENTRIES - 1u), rv[8 * j + k]);
+			}
+		}
+	}
+	__syncthreads();
+	const uint32_t total = prefix[64];
+	uint2* out = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
+	for (uint32_t t = threadIdx.x; t < total; t += GRID_BLOCK) out[t] = staging[t];
+	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
+}
+
+__global__ void __launch_bounds__(GRID_BLOCK) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
+                                                                 const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
+                                                                 __half2* __restrict__ grads, int accumulate) {
+	__shared__ float2 acc[BKT_ENTRIES];
+	// which (level, bucket, group) is this workgroup?
+	uint32_t level = 0;
+	while (blockIdx.x >= plan.wg_begin[level + 1]) ++level;
+	const uint32_t local = blockIdx.x - plan.wg_begin[level];
+	const uint32_t G = plan.groups[level];
+	const uint32_t bucket = local / G, group = local - bucket * G;
+	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += GRID_BLOCK) acc[e] = make_float2(0.f, 0.f);
+	__syncthreads();
+	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+	float* accf = reinterpret_cast<float*>(acc);
+	for (uint32_t tile = group + G * wave; tile < tiles; tile += G * (GRID_BLOCK / 64)) {
+		const uint16_t* off = offsets + ((size_t)level * tiles + tile) * (BKT_MAX + 1) + bucket;
+		const uint32_t begin = off[0], end = off[1];
+		const uint2* run = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
+		for (uint32_t t = begin + lane; t < end; t += 64) {
+			const uint2 r = run[t];
+			const __half2 h = *reinterpret_cast<const __half2*>(&r.y);
+			const float2 f = __half22float2(h);
+			atomicAdd(&accf[2 * r.x], f.x);      // LDS atomics
+			atomicAdd(&accf[2 * r.x + 1], f.y);
+		}
+	}
+	__syncthreads();
+	const uint32_t entries = tab.entries[level];
+	__half2* Gd = grads + tab.offset[level];
+	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += GRID_BLOCK) {
+		const uint32_t idx = bucket * BKT_ENTRIES + e;
+		if (idx >= entries) break;
+		const float2 a = acc[e];
+		if (G > 1) {
+			// several tile groups fold into the same entries (coarse levels only)
+			if (a.x != 0.f || a.y != 0.f) unsafeAtomicAdd(&Gd[idx], __floats2half2_rn(a.x, a.y));
+		} else if (accumulate) {
+			const float2 old = __half22float2(Gd[idx]);
+			Gd[idx] = __floats2half2_rn(old.x + a.x, old.y + a.y);
+		} else {
+			Gd[idx] = __floats2half2_rn(a.x, a.y);
+		}
+	}
+}
+
+// ----------------------------------------------------------------------------
 // host side
 // ----------------------------------------------------------------------------
 static uint32_t level_mode(uint32_t res, uint32_t entries) {
@@ -414,6 +613,9 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->n_params = (uint32_t)off * n_features_per_level;
 	g->params = nullptr;
 	g->grads = nullptr;
+	g->ws = nullptr;
+	g->ws_bytes = 0;
+	g->ws_max_points = 0;
 	*out = g;
 	return N2_OK;
 }
@@ -499,10 +701,83 @@ static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2
 }
 
 static inline uint32_t n_pair_tiles(uint32_t n_points) { return (n_points + PAIR_POINTS - 1) / PAIR_POINTS; }
+static inline uint32_t n_bin_tiles(uint32_t n_points) { return (n_points + BIN_POINTS - 1) / BIN_POINTS; }
+
+static bool bucket_supported(const n2_grid_t* grid) {
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l)
+		if (grid->tab.entries[l] > BKT_ENTRIES * BKT_MAX) return false;
+	return true;
+}
+static uint64_t bucket_ws_bytes(const n2_grid_t* grid, uint32_t max_points) {
+	const uint64_t tiles = n_bin_tiles(max_points), L = grid->tab.n_levels;
+	const uint64_t rec = L * tiles * BIN_RECORDS * sizeof(uint2);
+	const uint64_t off = (L * tiles * (BKT_MAX + 1) * sizeof(uint16_t) + 255) / 256 * 256;
+	return rec + off;
+}
+
+N2_API uint64_t n2_grid_workspace_bytes(const n2_grid_t* grid, uint32_t max_points) {
+	if (!grid || !bucket_supported(grid)) return 0;
+	return bucket_ws_bytes(grid, max_points);
+}
+
+N2_API int n2_grid_set_workspace(n2_grid_t* grid, void* d_workspace, uint64_t n_bytes, uint32_t max_points) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_workspace: grid is null");
+	if (d_workspace == nullptr) {
+		grid->ws = nullptr; grid->ws_bytes = 0; grid->ws_max_points = 0;
+		return N2_OK;
+	}
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256 == 0, "n2_grid_set_workspace: workspace must be 256-byte aligned");
+	N2_REQUIRE(n_bytes >= n2_grid_workspace_bytes(grid, max_points), "n2_grid_set_workspace: %llu bytes given, %llu needed for %u points",
+	           (unsigned long long)n_bytes, (unsigned long long)n2_grid_workspace_bytes(grid, max_points), max_points);
+	grid->ws = reinterpret_cast<unsigned char*>(d_workspace);
+	grid->ws_bytes = n_bytes;
+	grid->ws_max_points = bucket_supported(grid) ? max_points : 0;
+	return N2_OK;
+}
+
+// Parameter gradients through the bin + reduce kernels.  The gradient buffer has been zeroed for OVERWRITE.
+static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
+                           const __half* dL_dy, const float* v, const __half* g2, __half* dL_ddLdy, bool accumulate) {
+	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
+	uint2* records = reinterpret_cast<uint2*>(grid->ws);
+	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + (uint64_t)L * tiles * BIN_RECORDS * sizeof(uint2));
+	const dim3 gd(tiles * L), bd(GRID_BLOCK);
+	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
+#define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
+                                                                   grid->params, dL_ddLdy, records, offsets)
+	if (first && second && out) LAUNCH(true, true, true);
+	else if (first && second) LAUNCH(true, true, false);
+	else if (second && out) LAUNCH(false, true, true);
+	else if (second) LAUNCH(false, true, false);
+	else LAUNCH(true, false, false);
+#undef LAUNCH
+	N2_LAUNCH_CHECK();
+	N2BucketPlan plan;
+	uint32_t wg = 0;
+	for (uint32_t l = 0; l < L; ++l) {
+		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES;
+		// aim at <= ~64k records per reduce workgroup: a level holds 8 records per point
+		const uint64_t per_bucket = (uint64_t)n_points * 8 / nb;
+		uint32_t groups = (uint32_t)((per_bucket + 65535) / 65536);
+		if (groups > tiles) groups = tiles;
+		if (groups < 1) groups = 1;
+		plan.wg_begin[l] = wg;
+		plan.n_buckets[l] = nb;
+		plan.groups[l] = groups;
+		wg += nb * groups;
+	}
+	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
+	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; }
+	grid_reduce_kernel<<<dim3(wg), bd, 0, s>>>(grid->tab, plan, tiles, records, offsets, grid->grads, accumulate ? 1 : 0);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
 
 // One scatter pass with any combination of first-order (dL_dy) and second-order (v, g2) terms.
 static int launch_scatter(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
-                          const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy) {
+                          const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy, bool accumulate) {
+	if (grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 4 * BIN_POINTS)
+		return launch_bucketed(grid, s, d_xyz, point_stride, dim_stride, n_points, dL_dy, v, g2, dL_ddLdy, accumulate);
 	const uint32_t tiles = n_pair_tiles(n_points);
 	const dim3 gd(tiles * grid->tab.n_levels), bd(GRID_BLOCK);
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
@@ -530,7 +805,7 @@ N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_
 	if (mode != N2_GRAD_IGNORE) {
 		N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
 		if (int rc = launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), nullptr,
-		                            nullptr, grid->grads, nullptr)) return rc;
+		                            nullptr, grid->grads, nullptr, mode == N2_GRAD_ACCUMULATE)) return rc;
 	}
 	if (d_dL_dx) {
 		grid_backward_input_kernel<<<dim3(n_tiles(n_points)), dim3(GRID_BLOCK), 0, s>>>(
@@ -552,7 +827,8 @@ N2_API int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const flo
 	if (n_points == 0) return N2_OK;
 	N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
 	return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), d_dL_ddLdx,
-	                      reinterpret_cast<const __half*>(d_dL_dy_second), grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy));
+	                      reinterpret_cast<const __half*>(d_dL_dy_second), grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy),
+	                      mode == N2_GRAD_ACCUMULATE);
 }
 
 N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz,
@@ -571,7 +847,7 @@ N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, 
 	N2ProfScope prof(N2_PROF_GRID_SECOND_ORDER, s);
 	if (!d_dL_dx) {
 		return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, nullptr, d_dL_ddLdx, reinterpret_cast<const __half*>(d_dL_dy),
-		                      mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy));
+		                      mode == N2_GRAD_IGNORE ? nullptr : grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy), mode == N2_GRAD_ACCUMULATE);
 	}
 	const uint32_t tiles = n_tiles(n_points);
 	grid_bbi_kernel<<<dim3(tiles * grid->tab.n_levels), dim3(GRID_BLOCK), 0, s>>>(

@@ -80,6 +80,17 @@ class GridEncoding:
         check(capi.lib().n2_grid_set_params(self._h, ptr(params), ptr(gradients)), "n2_grid_set_params")
         self._params, self._grads = params, gradients
 
+    def reserve_scatter_workspace(self, max_points):
+        """Scratch that lets backward passes of >= 4096 points sort their updates in LDS instead of issuing
+        global atomics.  Returns False when the table shape does not support it."""
+        nbytes = int(capi.lib().n2_grid_workspace_bytes(self._h, C.c_uint32(max_points)))
+        if nbytes == 0:
+            return False
+        self._scatter_ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        check(capi.lib().n2_grid_set_workspace(self._h, ptr(self._scatter_ws), C.c_uint64(nbytes), C.c_uint32(max_points)),
+              "n2_grid_set_workspace")
+        return True
+
     def forward(self, xyz, prepare_input_gradients=False):
         """Returns (out fp16 [width, N], ctx) where ctx holds dy_dx when requested."""
         x, ps, ds, n = _positions(xyz)
