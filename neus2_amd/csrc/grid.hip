@@ -510,47 +510,139 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
 }
 
-__global__ void __launch_bounds__(GRID_BLOCK) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
-                                                                 const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
-                                                                 __half2* __restrict__ grads, int accumulate) {
-	__shared__ float2 acc[BKT_ENTRIES];
+// LDS float atomics retire about one lane every three clocks on this part, integer ones at ~9 (32-bit) and
+// ~5.5 (64-bit) lanes per clock.  The reduce therefore accumulates in 64-bit fixed point: a record holds
+// fp16 values, i.e. multiples of 2^-24 below 2^16, so value * 2^32 is an exact integer below 2^48 and the
+// sum of a whole bucket stays far inside 64 bits.  The accumulation is exact and independent of order.
+constexpr uint32_t RED_BLOCK = 1024;              // 16 waves; the 128 KiB table allows one workgroup per CU
+constexpr uint32_t RED_CHUNK = 2048;              // tiles whose runs are gathered per pass
+constexpr uint32_t RED_PER_THREAD = RED_CHUNK / RED_BLOCK;
+constexpr float FIX_SCALE = 4294967296.0f;        // 2^32
+
+__device__ __forceinline__ unsigned long long to_fixed(float x) { return (unsigned long long)(long long)(x * FIX_SCALE); }
+__device__ __forceinline__ float from_fixed(unsigned long long q) { return (float)((double)(long long)q * (1.0 / 4294967296.0)); }
+
+__global__ void __launch_bounds__(RED_BLOCK) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
+                                                                const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
+                                                                __half2* __restrict__ grads, int accumulate) {
+	__shared__ unsigned long long acc[2 * BKT_ENTRIES];  // 128 KiB
+	__shared__ uint32_t run_src[RED_CHUNK];               // index of the run's first record in `records`
+	__shared__ uint16_t run_len[RED_CHUNK];
+	__shared__ uint32_t item_pos[RED_CHUNK + 1];          // exclusive prefix of the runs' item counts
+	__shared__ uint32_t wave_tot[RED_BLOCK / 64];
 	// which (level, bucket, group) is this workgroup?
 	uint32_t level = 0;
 	while (blockIdx.x >= plan.wg_begin[level + 1]) ++level;
 	const uint32_t local = blockIdx.x - plan.wg_begin[level];
 	const uint32_t G = plan.groups[level];
 	const uint32_t bucket = local / G, group = local - bucket * G;
-	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += GRID_BLOCK) acc[e] = make_float2(0.f, 0.f);
-	__syncthreads();
+	for (uint32_t e = threadIdx.x; e < 2 * BKT_ENTRIES; e += RED_BLOCK) acc[e] = 0ull;
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-	float* accf = reinterpret_cast<float*>(acc);
-	for (uint32_t tile = group + G * wave; tile < tiles; tile += G * (GRID_BLOCK / 64)) {
-		const uint16_t* off = offsets + ((size_t)level * tiles + tile) * (BKT_MAX + 1) + bucket;
-		const uint32_t begin = off[0], end = off[1];
-		const uint2* run = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
-		for (uint32_t t = begin + lane; t < end; t += 64) {
-			const uint2 r = run[t];
-			const __half2 h = *reinterpret_cast<const __half2*>(&r.y);
-			const float2 f = __half22float2(h);
-			atomicAdd(&accf[2 * r.x], f.x);      // LDS atomics
-			atomicAdd(&accf[2 * r.x + 1], f.y);
+	const uint32_t my_tiles = (tiles > group) ? (tiles - group + G - 1) / G : 0;  // tiles group, group + G, ...
+	const size_t level_tile0 = (size_t)level * tiles;
+	const uint2* base = records + level_tile0 * BIN_RECORDS;
+	for (uint32_t c0 = 0; c0 < my_tiles; c0 += RED_CHUNK) {
+		__syncthreads();
+		// every thread fetches the bucket's run bounds of 4 tiles (independent loads); a run is cut into items
+		// of 128 records and the items of all runs are numbered consecutively (block scan of the item counts)
+		uint32_t cnt[RED_PER_THREAD], sum = 0;
+#pragma unroll
+		for (uint32_t j = 0; j < RED_PER_THREAD; ++j) {
+			const uint32_t k = threadIdx.x * RED_PER_THREAD + j, t = c0 + k;
+			cnt[j] = 0;
+			if (t < my_tiles) {
+				const size_t tile = level_tile0 + group + (size_t)t * G;
+				const uint16_t* off = offsets + tile * (BKT_MAX + 1) + bucket;
+				const uint32_t begin = off[0], end = off[1];
+				run_src[k] = (uint32_t)((tile - level_tile0) * BIN_RECORDS) + begin;
+				run_len[k] = (uint16_t)(end - begin);
+				cnt[j] = (end - begin + 127u) >> 7;
+			}
+			sum += cnt[j];
+		}
+		uint32_t incl = sum;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) {
+			const uint32_t u = __shfl_up(incl, o);
+			if ((int)lane >= o) incl += u;
+		}
+		if (lane == 63) wave_tot[wave] = incl;
+		__syncthreads();
+		uint32_t run = incl - sum;
+		for (uint32_t w = 0; w < wave; ++w) run += wave_tot[w];
+#pragma unroll
+		for (uint32_t j = 0; j < RED_PER_THREAD; ++j) {
+			item_pos[threadIdx.x * RED_PER_THREAD + j] = run;
+			run += cnt[j];
+		}
+		if (threadIdx.x == RED_BLOCK - 1) item_pos[RED_CHUNK] = run;
+		__syncthreads();
+		const uint32_t n_items = item_pos[RED_CHUNK];
+		// a wave takes 4 items at a time (8 independent 8-byte loads per lane); the loads of the next 4 items are
+		// issued before the current ones are accumulated
+		auto fetch = [&](uint32_t i0, uint2 (&rec)[8], uint32_t& okmask) {
+			okmask = 0;
+#pragma unroll
+			for (uint32_t j = 0; j < 4; ++j) {
+				const uint32_t it = i0 + j;
+				uint32_t src = 0, n = 0, t0 = 0;
+				if (it < n_items) {
+					uint32_t lo = 0, hi = RED_CHUNK;  // last run k with item_pos[k] <= it
+#pragma unroll
+					for (int step = 0; step < 11; ++step) {
+						const uint32_t mid = (lo + hi) >> 1;
+						if (item_pos[mid] <= it) lo = mid; else hi = mid;
+					}
+					src = run_src[lo]; n = run_len[lo]; t0 = (it - item_pos[lo]) << 7;
+				}
+#pragma unroll
+				for (uint32_t h = 0; h < 2; ++h) {
+					const uint32_t t = t0 + h * 64 + lane;
+					const bool ok = t < n;
+					okmask |= (ok ? 1u : 0u) << (2 * j + h);
+					rec[2 * j + h] = ok ? base[(size_t)src + t] : make_uint2(0u, 0u);
+				}
+			}
+		};
+		constexpr uint32_t STRIDE = (RED_BLOCK / 64) * 4;
+		uint2 cur[8], nxt[8];
+		uint32_t cur_ok = 0, nxt_ok = 0;
+		uint32_t i0 = wave * 4;
+		if (i0 < n_items) fetch(i0, cur, cur_ok);
+		for (; i0 < n_items; i0 += STRIDE) {
+			const bool more = i0 + STRIDE < n_items;
+			if (more) fetch(i0 + STRIDE, nxt, nxt_ok);
+#pragma unroll
+			for (uint32_t q = 0; q < 8; ++q) {
+				if (cur_ok & (1u << q)) {
+					const __half2 hh = *reinterpret_cast<const __half2*>(&cur[q].y);
+					const float2 f = __half22float2(hh);
+					atomicAdd(&acc[2 * cur[q].x], to_fixed(f.x));  // LDS integer atomics
+					atomicAdd(&acc[2 * cur[q].x + 1], to_fixed(f.y));
+				}
+			}
+			if (more) {
+#pragma unroll
+				for (uint32_t q = 0; q < 8; ++q) cur[q] = nxt[q];
+				cur_ok = nxt_ok;
+			}
 		}
 	}
 	__syncthreads();
 	const uint32_t entries = tab.entries[level];
 	__half2* Gd = grads + tab.offset[level];
-	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += GRID_BLOCK) {
+	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) {
 		const uint32_t idx = bucket * BKT_ENTRIES + e;
 		if (idx >= entries) break;
-		const float2 a = acc[e];
+		const float ax = from_fixed(acc[2 * e]), ay = from_fixed(acc[2 * e + 1]);
 		if (G > 1) {
 			// several tile groups fold into the same entries (coarse levels only)
-			if (a.x != 0.f || a.y != 0.f) unsafeAtomicAdd(&Gd[idx], __floats2half2_rn(a.x, a.y));
+			if (ax != 0.f || ay != 0.f) unsafeAtomicAdd(&Gd[idx], __floats2half2_rn(ax, ay));
 		} else if (accumulate) {
 			const float2 old = __half22float2(Gd[idx]);
-			Gd[idx] = __floats2half2_rn(old.x + a.x, old.y + a.y);
+			Gd[idx] = __floats2half2_rn(old.x + ax, old.y + ay);
 		} else {
-			Gd[idx] = __floats2half2_rn(a.x, a.y);
+			Gd[idx] = __floats2half2_rn(ax, ay);
 		}
 	}
 }
@@ -768,7 +860,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	}
 	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
 	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; }
-	grid_reduce_kernel<<<dim3(wg), bd, 0, s>>>(grid->tab, plan, tiles, records, offsets, grid->grads, accumulate ? 1 : 0);
+	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, records, offsets, grid->grads, accumulate ? 1 : 0);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
