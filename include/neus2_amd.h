@@ -414,6 +414,11 @@ typedef struct n2_trainer_config {
 	uint32_t max_rays_per_batch;    /* upper bound of n_rays in a step */
 	uint32_t max_samples;           /* capacity for marched samples; the reference uses 16 x target (src/testbed_nerf.cu:3719) */
 	float loss_scale;               /* 128, testbed.h:237 */
+	uint32_t prefetch_samples;      /* non-zero: each step also starts the NEXT step's sample generation (same n_rays and
+	                                   n_inference, seed + 1) on a stream the trainer owns, so that it overlaps this step's
+	                                   field kernels; a following step called with other arguments regenerates in line.
+	                                   Results are identical either way.  The trainer must then be driven from one stream
+	                                   (or from streams the caller orders against each other). */
 } n2_trainer_config;
 
 /* All device memory a trainer uses (parameters, optimiser state, every temporary) lives in one

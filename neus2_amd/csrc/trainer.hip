@@ -1,7 +1,10 @@
 // One training step on one GPU: sample generation, field forward over all
 // marched samples, compositing / loss / compaction, roll-over to the target
 // batch size, field forward + backward (first and second order), Adam.
-// Everything is enqueued on the caller's stream; no host synchronisation.
+// Everything is enqueued on the caller's stream, without host synchronisation,
+// except that the sample generator of the FOLLOWING step (which depends only on
+// the scene and the seed) may run ahead on a stream the trainer owns, into the
+// other of two sample sets, while this step's field kernels occupy the GPU.
 #include "n2_common.h"
 
 #include <cstring>
@@ -21,17 +24,20 @@ struct n2_trainer {
 	float* m1;
 	float* m2;
 	uint32_t* steps;
-	// per-step buffers
-	float* coords;            // [max_samples][7]
+	// per-step buffers; everything the sample generator writes exists twice
+	struct SampleSet {
+		float* coords;            // [max_samples][7]
+		uint32_t* numsteps;       // [max_rays][2]
+		uint32_t* ray_indices;    // [max_rays]
+		float* rgb_target;        // [max_rays][3]
+		uint32_t* counters;       // [0] live rays, [1] marched samples
+		void* ws_sampler;
+	} sets[2];
 	hf* mlp_out;              // [max(max_samples, target)][16]
 	hf* dloss;                // [target][16]
 	float* coords_compacted;  // [target][7]
-	uint32_t* numsteps;       // [max_rays][2]
-	uint32_t* ray_indices;    // [max_rays]
-	float* rgb_target;        // [max_rays][3]
 	float* ray_loss;          // [max_rays]
 	uint32_t* counters;       // [0] live rays, [1] marched samples, [2] compacted samples (+ [4] as float: loss)
-	void* ws_sampler;
 	void* ws_composite;
 	uint64_t ws_sampler_bytes, ws_composite_bytes;
 	void* ws_field;
@@ -41,11 +47,17 @@ struct n2_trainer {
 	const float* rgba;
 	const uint8_t* bitfield;
 	uint32_t n_rays_total;
+	// sample generation running ahead of the step that uses it
+	hipStream_t side;
+	hipEvent_t ev_main, ev_ready;
+	bool pf_valid;
+	uint32_t pf_set, pf_n_rays, pf_n_inference, pf_seed, pf_ray_base;
+	uint32_t last_set;
 };
 
 struct TrainerCarve {
-	uint64_t master, params, grads, m1, m2, steps, coords, mlp_out, dloss, coords_compacted, numsteps, ray_indices, rgb_target, ray_loss,
-		counters, ws_sampler, ws_composite, ws_field, total;
+	uint64_t master, params, grads, m1, m2, steps, coords[2], mlp_out, dloss, coords_compacted, numsteps[2], ray_indices[2], rgb_target[2],
+		set_counters[2], ray_loss, counters, ws_sampler[2], ws_composite, ws_field, total;
 };
 
 static inline uint64_t a256(uint64_t x) { return (x + 255) / 256 * 256; }
@@ -63,16 +75,19 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	c.m1 = take(4 * np);
 	c.m2 = take(4 * np);
 	c.steps = take(4 * np);
-	c.coords = take(28 * S);
+	for (int i = 0; i < 2; ++i) c.coords[i] = take(28 * S);
 	c.mlp_out = take(32 * (S > T ? S : T));
 	c.dloss = take(32 * T);
 	c.coords_compacted = take(28 * T);
-	c.numsteps = take(8 * R);
-	c.ray_indices = take(4 * R);
-	c.rgb_target = take(12 * R);
+	for (int i = 0; i < 2; ++i) {
+		c.numsteps[i] = take(8 * R);
+		c.ray_indices[i] = take(4 * R);
+		c.rgb_target[i] = take(12 * R);
+		c.set_counters[i] = take(64);
+	}
 	c.ray_loss = take(4 * R);
 	c.counters = take(64);
-	c.ws_sampler = take(n2_sampler_workspace_bytes((uint32_t)R));
+	for (int i = 0; i < 2; ++i) c.ws_sampler[i] = take(n2_sampler_workspace_bytes((uint32_t)R));
 	c.ws_composite = take(n2_composite_workspace_bytes((uint32_t)R));
 	c.ws_field = take(n2_field_workspace_bytes(f, (uint32_t)(S > T ? S : T), (uint32_t)T));
 	c.total = o;
@@ -104,11 +119,11 @@ __global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, co
 	if (i < n) params[i] = (hf)master[i];
 }
 
-// sum of the per-ray losses of the live rays (one workgroup)
-__global__ void __launch_bounds__(1024) trainer_loss_sum_kernel(const uint32_t* __restrict__ ray_counter, uint32_t max_rays,
-                                                                const float* __restrict__ ray_loss, float* __restrict__ out) {
+// sum of the per-ray losses of the live rays (one workgroup); also publishes the sample set's counters
+__global__ void __launch_bounds__(1024) trainer_loss_sum_kernel(const uint32_t* __restrict__ set_counters, uint32_t max_rays,
+                                                                const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
 	__shared__ float part[16];
-	const uint32_t n = min(*ray_counter, max_rays);
+	const uint32_t n = min(set_counters[0], max_rays);
 	float s = 0.f;
 	for (uint32_t i = threadIdx.x; i < n; i += 1024) s += ray_loss[i];
 #pragma unroll
@@ -118,7 +133,9 @@ __global__ void __launch_bounds__(1024) trainer_loss_sum_kernel(const uint32_t* 
 	if (threadIdx.x == 0) {
 		float t = 0.f;
 		for (int w = 0; w < 16; ++w) t += part[w];
-		*out = t;
+		counters[0] = set_counters[0];
+		counters[1] = set_counters[1];
+		reinterpret_cast<float*>(counters)[4] = t;
 	}
 }
 
@@ -152,17 +169,20 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->m1 = reinterpret_cast<float*>(b + c.m1);
 	t->m2 = reinterpret_cast<float*>(b + c.m2);
 	t->steps = reinterpret_cast<uint32_t*>(b + c.steps);
-	t->coords = reinterpret_cast<float*>(b + c.coords);
+	for (int i = 0; i < 2; ++i) {
+		t->sets[i].coords = reinterpret_cast<float*>(b + c.coords[i]);
+		t->sets[i].numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps[i]);
+		t->sets[i].ray_indices = reinterpret_cast<uint32_t*>(b + c.ray_indices[i]);
+		t->sets[i].rgb_target = reinterpret_cast<float*>(b + c.rgb_target[i]);
+		t->sets[i].counters = reinterpret_cast<uint32_t*>(b + c.set_counters[i]);
+		t->sets[i].ws_sampler = b + c.ws_sampler[i];
+	}
 	t->mlp_out = reinterpret_cast<hf*>(b + c.mlp_out);
 	t->dloss = reinterpret_cast<hf*>(b + c.dloss);
 	t->coords_compacted = reinterpret_cast<float*>(b + c.coords_compacted);
-	t->numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps);
-	t->ray_indices = reinterpret_cast<uint32_t*>(b + c.ray_indices);
-	t->rgb_target = reinterpret_cast<float*>(b + c.rgb_target);
 	t->ray_loss = reinterpret_cast<float*>(b + c.ray_loss);
 	t->counters = reinterpret_cast<uint32_t*>(b + c.counters);
-	t->ws_sampler = b + c.ws_sampler;
-	t->ws_sampler_bytes = c.ws_composite - c.ws_sampler;
+	t->ws_sampler_bytes = c.ws_sampler[1] - c.ws_sampler[0];
 	t->ws_composite = b + c.ws_composite;
 	t->ws_composite_bytes = c.ws_field - c.ws_composite;
 	t->ws_field = b + c.ws_field;
@@ -171,12 +191,20 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	if (rc == N2_OK) rc = n2_field_set_workspace(t->field, t->ws_field, c.total - c.ws_field, S, cfg->target_batch_size);
 	// optimiser state, gradients, counters and every per-step buffer start at zero (padding rows of a
 	// batch are then valid positions with zero gradient)
-	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.grads, c.coords - c.grads);
-	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.coords, c.ws_sampler - c.coords);
+	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.grads, c.coords[0] - c.grads);
+	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.coords[0], c.ws_sampler[0] - c.coords[0]);
 	if (rc == N2_OK && hipStreamSynchronize(nullptr) != hipSuccess) { n2_set_error("n2_trainer_create: workspace initialisation failed"); rc = N2_ERR_HIP; }
+	if (rc == N2_OK && cfg->prefetch_samples) {
+		// default priority on purpose: the stream only has to run beside the caller's, not ahead of it
+		if (hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking) != hipSuccess ||
+		    hipEventCreateWithFlags(&t->ev_main, hipEventDisableTiming) != hipSuccess ||
+		    hipEventCreateWithFlags(&t->ev_ready, hipEventDisableTiming) != hipSuccess) {
+			n2_set_error("n2_trainer_create: cannot create the sample-generation stream");
+			rc = N2_ERR_HIP;
+		}
+	}
 	if (rc != N2_OK) {
-		n2_field_destroy(t->field);
-		delete t;
+		n2_trainer_destroy(t);
 		return rc;
 	}
 	*out = t;
@@ -185,6 +213,9 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 
 N2_API void n2_trainer_destroy(n2_trainer_t* t) {
 	if (!t) return;
+	if (t->side) { (void)hipStreamSynchronize(t->side); (void)hipStreamDestroy(t->side); }
+	if (t->ev_main) (void)hipEventDestroy(t->ev_main);
+	if (t->ev_ready) (void)hipEventDestroy(t->ev_ready);
 	n2_field_destroy(t->field);
 	delete t;
 }
@@ -210,6 +241,9 @@ N2_API n2_field_t* n2_trainer_field(n2_trainer_t* t) { return t ? t->field : nul
 N2_API int n2_trainer_set_scene(n2_trainer_t* t, const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba, const uint8_t* d_bitfield) {
 	N2_REQUIRE(t != nullptr, "n2_trainer_set_scene: trainer is null");
 	N2_REQUIRE(d_cameras && d_rgba && d_bitfield && n_images > 0, "n2_trainer_set_scene: null scene buffer or no images");
+	// a sample generation that is still running ahead reads the previous scene
+	if (t->side) N2_HIP(hipStreamSynchronize(t->side));
+	t->pf_valid = false;
 	t->cameras = d_cameras; t->n_images = n_images; t->rgba = d_rgba; t->bitfield = d_bitfield;
 	return N2_OK;
 }
@@ -222,24 +256,51 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	           n_inference, t->cfg.max_samples);
 	hipStream_t s = n2_stream(stream);
 	const uint32_t T = t->cfg.target_batch_size;
-	uint32_t* ray_counter = t->counters;
-	uint32_t* sample_counter = t->counters + 1;
 	uint32_t* compacted_counter = t->counters + 2;
-	// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
-	if (int rc = n2_generate_training_samples(stream, n_rays, t->n_rays_total, seed, t->cameras, t->n_images, t->rgba, t->cfg.composite.background,
-	                                          t->bitfield, n_inference, ray_counter, sample_counter, t->ray_indices, t->numsteps, t->rgb_target,
-	                                          t->coords, t->ws_sampler, t->ws_sampler_bytes)) return rc;
-	t->n_rays_total += n_rays;
+	auto sample = [&](n2_trainer::SampleSet& set, hipStream_t on, uint32_t ray_base, uint32_t sd) {
+		// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
+		return n2_generate_training_samples(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,
+		                                    t->cfg.composite.background, t->bitfield, n_inference, set.counters, set.counters + 1, set.ray_indices,
+		                                    set.numsteps, set.rgb_target, set.coords, set.ws_sampler, t->ws_sampler_bytes);
+	};
+	uint32_t cur;
+	if (t->side) {
+		// everything enqueued by earlier steps precedes this marker: the set the generator overwrites next is free after it
+		N2_HIP(hipEventRecord(t->ev_main, s));
+		const bool hit = t->pf_valid && t->pf_n_rays == n_rays && t->pf_n_inference == n_inference && t->pf_seed == seed && t->pf_ray_base == t->n_rays_total;
+		if (hit) {
+			cur = t->pf_set;
+			N2_HIP(hipStreamWaitEvent(s, t->ev_ready, 0));
+		} else {
+			// a generation that ran ahead with other arguments is abandoned (it stays ordered on the side stream)
+			cur = t->pf_valid ? 1u - t->pf_set : 1u - t->last_set;
+			if (int rc = sample(t->sets[cur], s, t->n_rays_total, seed)) return rc;
+		}
+		t->n_rays_total += n_rays;
+		// the following step's samples, assuming the same ray count and the next seed
+		t->pf_valid = false;
+		N2_HIP(hipStreamWaitEvent(t->side, t->ev_main, 0));
+		if (int rc = sample(t->sets[1u - cur], t->side, t->n_rays_total, seed + 1)) return rc;
+		N2_HIP(hipEventRecord(t->ev_ready, t->side));
+		t->pf_valid = true; t->pf_set = 1u - cur; t->pf_n_rays = n_rays; t->pf_n_inference = n_inference; t->pf_seed = seed + 1; t->pf_ray_base = t->n_rays_total;
+	} else {
+		cur = 0;
+		if (int rc = sample(t->sets[0], s, t->n_rays_total, seed)) return rc;
+		t->n_rays_total += n_rays;
+	}
+	t->last_set = cur;
+	const n2_trainer::SampleSet& set = t->sets[cur];
+	const uint32_t* ray_counter = set.counters;
 	// field over every marched sample
-	if (int rc = n2_field_forward(t->field, stream, t->coords, n_inference, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	if (int rc = n2_field_forward(t->field, stream, set.coords, n_inference, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
 	// compositing, loss, gradients w.r.t. the outputs, compaction
 	n2_composite_config cc = t->cfg.composite;
 	cc.n_rays_norm = n_rays;
 	cc.loss_scale = t->cfg.loss_scale;
-	if (int rc = n2_composite_loss(stream, &cc, n_rays, ray_counter, t->numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), t->coords,
-	                               t->rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
+	if (int rc = n2_composite_loss(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
+	                               set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
 	                               t->ws_composite, t->ws_composite_bytes)) return rc;
-	trainer_loss_sum_kernel<<<dim3(1), dim3(1024), 0, s>>>(ray_counter, n_rays, t->ray_loss, reinterpret_cast<float*>(t->counters + 4));
+	trainer_loss_sum_kernel<<<dim3(1), dim3(1024), 0, s>>>(ray_counter, n_rays, t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
 	// pad the compacted batch to exactly T samples
 	if (int rc = n2_fill_rollover_and_rescale_f16(stream, T, 16, compacted_counter, reinterpret_cast<n2_half*>(t->dloss))) return rc;

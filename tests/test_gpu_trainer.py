@@ -114,3 +114,35 @@ def test_trainer_errors(setup):
     t2 = Trainer(default_config(target_batch_size=256, max_rays_per_batch=64, max_samples=1024))
     with pytest.raises(N2Error, match="set_scene"):
         t2.step(n_rays=8, n_inference=1024)
+
+
+def test_samples_generated_ahead_give_the_same_steps():
+    """Generating the next step's samples on the trainer's own stream changes nothing but timing, also when a
+    step is called with other arguments than the ones the generation ran ahead with."""
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    cams = scene.cameras_on_sphere(6, 64)
+    rgba = scene.render_sphere_images(cams)
+    bits = scene.sphere_bitfield()
+    T = 2048
+    d_cams, d_rgba, d_bits = pack_cameras(cams), dev(rgba), dev(bits)
+    # (n_rays, seed): consecutive seeds hit the generation that ran ahead, the others miss it
+    plan = [(200, 0), (200, 1), (200, 2), (260, 3), (260, 4), (260, 9), (260, 10), (120, 11)]
+    runs = []
+    for ahead in (False, True):
+        tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=512, max_samples=16 * T, prefetch_samples=ahead))
+        tr.set_scene(d_cams, len(cams), d_rgba, d_bits)
+        tr.initialize_params(seed=5, sdf_mlp_weights=None)
+        log = []
+        for n_rays, seed in plan:
+            tr.step(n_rays=n_rays, n_inference=16 * T, seed=seed)
+            log.append(tr.read_counters())
+        runs.append((log, host(tr.master).copy()))
+        del tr
+    (log_a, m_a), (log_b, m_b) = runs
+    for a, b in zip(log_a, log_b):
+        assert (a["rays"], a["samples"]) == (b["rays"], b["samples"]) and a["rays"] > 0
+        assert abs(a["compacted"] - b["compacted"]) <= max(2, 0.005 * a["compacted"])
+        assert abs(a["loss"] - b["loss"]) <= 0.01 * abs(a["loss"]) + 1e-6
+    assert cos_sim(m_a - m_a.mean(), m_b - m_b.mean()) > 0.999
+    assert np.abs(m_a - m_b).max() < 2e-2
