@@ -56,7 +56,7 @@ def test_trainer_config_struct_matches_header():
     from neus2_amd import capi
     assert ctypes.sizeof(capi.FieldConfig) == 32 and ctypes.sizeof(capi.AdamConfig) == 20
     assert ctypes.sizeof(capi.CompositeConfig) == 28 and ctypes.sizeof(capi.Camera) == 80
-    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 16
+    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 20
     L = capi.lib()
     cfg = capi.TrainerConfig()
     assert L.n2_trainer_workspace_bytes(ctypes.byref(cfg)) == 0  # all-zero config is rejected on the host
