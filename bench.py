@@ -23,7 +23,15 @@ HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 #   grid backward (parameter scatter): 12 (xyz) + 64 (dL_dy, 32 fp16) + 128 x 4 (packed fp16 atomics) = 588
 #   grid forward:                      12 (xyz) + 128 x 4 (gathers) + 64 (32 fp16 out)             = 588
 #   grid second order:                 12 + 12 (v) + 64 (dL_dy) + 64 (dL_ddLdy) + 128 x 4           = 664
+# In a training step the first- and second-order parameter scatters run as ONE merged pass (one write per corner),
+# timed under "grid_backward_params": its algorithmic bytes are those of the second-order pass alone, 664 (the
+# two passes the reference launches would be 588 + 664).
 ALGO_BYTES = {"grid_backward_params": 588, "grid_forward": 588, "grid_second_order": 664}
+STEP_ALGO_BYTES = {"grid_backward_params": 664, "grid_forward": 588}
+# MFMA work of one launch of the colour-network backward (the largest matrix kernel of a step), per sample:
+# recomputed forward 2 x (48x64 + 64x64) + data backward 2 x (16x64 + 64x64 + 64x48) + weight gradients 2 x (48x64 + 64x64 + 64x16)
+COLOUR_BACKWARD_FLOPS = 14336 + 16384 + 16384
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8}
 
@@ -112,11 +120,18 @@ def run_step_workload(args):
         ms, n = profile_read(lib, name)
         if n:
             kernels[name] = {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_us": ms / n * 1e3}
-    dom = max((k for k in ALGO_BYTES if k in kernels), key=lambda k: kernels[k]["ms_per_step"])
+    dom = max((k for k in STEP_ALGO_BYTES if k in kernels), key=lambda k: kernels[k]["ms_per_step"])
     # per-launch batch of the dominant kernel: the backward kernels always see the 2^18 compacted batch; the forward
     # also runs over the marched samples, so use the average batch per launch
     per_launch = TARGET if dom != "grid_forward" else (TARGET + n_inf) / 2
-    achieved = ALGO_BYTES[dom] * per_launch / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    achieved = STEP_ALGO_BYTES[dom] * per_launch / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    if args.calibrate_copy:
+        # a plain copy of known size in the same process: the scale of the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.empty(args.calibrate_copy << 20, dtype=torch.uint8, device="cuda").zero_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
     result = {
         "metric": "SDF train samples/sec @2^18 batch (1 GPU)",
         "value": args.steps * TARGET / elapsed,
@@ -133,7 +148,7 @@ def run_step_workload(args):
                    "inference_batch": n_inf, "compacted_before_rollover": counters["compacted"], "loss": counters["loss"]},
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_sample": ALGO_BYTES[dom], "samples_per_launch": per_launch,
+                     "algorithmic_bytes_per_sample": STEP_ALGO_BYTES[dom], "samples_per_launch": per_launch,
                      "avg_launch_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
     }
@@ -193,6 +208,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=["step", "grid"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs the hot path on ONE GPU (the reference has no multi-GPU path and the "
