@@ -34,7 +34,7 @@ constexpr int MLP_WIDTH = 64;
 constexpr int MLP_OUT = 16;
 constexpr int MLP_BLOCK = 256;      // 4 waves
 constexpr int MLP_TILE = 64;        // samples per wave iteration
-constexpr int MLP_MAX_SLABS = 256;  // workgroups of the weight-gradient kernels
+constexpr int MLP_MAX_SLABS = 512;  // workgroups of the weight-gradient kernels (two per CU)
 constexpr int STAGE_LD = 72;        // halves per staged row: 64 samples + 8 pad (keeps 16-byte alignment)
 
 struct n2_mlp {
@@ -79,15 +79,14 @@ __device__ __forceinline__ half8 wTfrag_chained(const hf* W, int ld, int m, int 
 	return f;
 }
 
-// B operands of both sample tiles for K-chunk c from an SoA matrix (rows x N):
-// rows 16c + 8g + e, sample pair at column `col` (even, already clamped).
-__device__ __forceinline__ void bfrag_soa(const hf* __restrict__ M, size_t N, uint32_t col, int c, int g, int n_rows,
-                                          half8& t0, half8& t1) {
+// B operands of both sample tiles for K-chunk c from an SoA matrix (rows x N): rows 16c + 8g + e,
+// sample pair at column `col`.  off8 = 8*g*N + col is the only per-lane part of the address; the
+// row part is uniform, so every load is "scalar base + one shared 32-bit lane offset".
+__device__ __forceinline__ void bfrag_soa(const hf* __restrict__ M, uint32_t N, uint32_t off8, int c, int n_rows, half8& t0, half8& t1) {
 #pragma unroll
 	for (int e = 0; e < 8; ++e) {
-		const int k = 16 * c + 8 * g + e;
 		half2v v = {(hf)0, (hf)0};
-		if (k < n_rows) v = *reinterpret_cast<const half2v*>(M + (size_t)k * N + col);
+		if (16 * c + e < n_rows) v = *reinterpret_cast<const half2v*>(M + (size_t)(16 * c + e) * N + off8);
 		t0[e] = v[0];
 		t1[e] = v[1];
 	}
@@ -180,7 +179,7 @@ __device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N
 		t0 = *reinterpret_cast<const half8*>(dY + (size_t)col * MLP_OUT + 8 * g);
 		t1 = *reinterpret_cast<const half8*>(dY + (size_t)(col + 1) * MLP_OUT + 8 * g);
 	} else {
-		bfrag_soa(dY, N, col, 0, g, MLP_OUT, t0, t1);
+		bfrag_soa(dY, (uint32_t)N, 8u * g * (uint32_t)N + col, 0, MLP_OUT, t0, t1);
 	}
 }
 
@@ -199,424 +198,479 @@ __device__ __forceinline__ void store_soa(hf* __restrict__ M, size_t N, uint32_t
 	}
 }
 
+// natural-K input operands of both sample tiles of a wave's 64 samples
+template <int IC>
+__device__ __forceinline__ void load_input(const hf* __restrict__ X, size_t N, uint32_t col, int g, half8 (&x)[2][IC]) {
+#pragma unroll
+	for (int c = 0; c < IC; ++c) bfrag_soa(X, (uint32_t)N, 8u * g * (uint32_t)N + col, c, 16 * IC, x[0][c], x[1][c]);
+}
+
 // ----------------------------------------------------------------------------
-// weights of one network in registers
+// Weight fragments in LDS.
+// A workgroup builds every MFMA operand the kernels need once, in "fragment
+// form": fragment f is 64 lanes x 16 bytes at F + f*512 halves, so a wave reads
+// an operand with one conflict-free 16-byte LDS load per lane.  Keeping the
+// weights out of the register file is what lets two workgroups share a CU.
 // ----------------------------------------------------------------------------
-template <int IN_CHUNKS, int N_HIDDEN>
-struct FwdWeights {
-	half8 w0[2][IN_CHUNKS];
-	half8 wh[N_HIDDEN > 1 ? N_HIDDEN - 1 : 1][2][4];
-	half8 wo[4];
-	__device__ __forceinline__ void load(const hf* W, int n, int g) {
-		constexpr int IN_W = 16 * IN_CHUNKS;
-#pragma unroll
-		for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-			for (int c = 0; c < IN_CHUNKS; ++c) w0[mt][c] = wfrag_natural(W, IN_W, 32 * mt + n, c, g);
-		const hf* Wk = W + MLP_WIDTH * IN_W;
-#pragma unroll
-		for (int k = 0; k < N_HIDDEN - 1; ++k) {
-#pragma unroll
-			for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-				for (int c = 0; c < 4; ++c) wh[k][mt][c] = wfrag_chained(Wk, MLP_WIDTH, 32 * mt + n, c, g);
-			Wk += MLP_WIDTH * MLP_WIDTH;
-		}
-#pragma unroll
-		for (int c = 0; c < 4; ++c) {
-			half8 z;
-#pragma unroll
-			for (int e = 0; e < 8; ++e) z[e] = (hf)0;
-			wo[c] = (n < MLP_OUT) ? wfrag_chained(Wk, MLP_WIDTH, n, c, g) : z;
-		}
-	}
+template <int IC, int NH>
+struct FragMap {
+	static constexpr int IN_W = 16 * IC, IN_MT = (IN_W + 31) / 32;
+	static constexpr int W0 = 0;                      // [mt][c]    W_0 rows 32mt+n, natural K            (A of the sample-lane chain)
+	static constexpr int WH = W0 + 2 * IC;            // [k][mt][c] hidden weights, chained K
+	static constexpr int WO = WH + (NH - 1) * 8;      // [c]        W_out rows n < 16, chained K
+	static constexpr int FWD_COUNT = WO + 4;
+	static constexpr int WOT = FWD_COUNT;             // [mt]       W_out^T rows 32mt+n, K = 16 outputs
+	static constexpr int WHT = WOT + 2;               // [k][mt][c] hidden weights transposed, chained K
+	static constexpr int W0T = WHT + (NH - 1) * 8;    // [mt][c]    W_0^T rows 32mt+n (< IN_W), chained K
+	static constexpr int SEL = W0T + IN_MT * 4;       // [c]        selects input rows 16c.. into feature tile c/2
+	static constexpr int ID = SEL + IC;               //            16 x 32 identity
+	static constexpr int COUNT = ID + 1;
 };
 
-// Forward through the hidden layers for one 64-sample tile: fills h[k][t][c]
-// (post-activation, fp16, chained operand form) for every hidden layer k.
-template <int IN_CHUNKS, int N_HIDDEN>
-__device__ __forceinline__ void forward_hidden(const FwdWeights<IN_CHUNKS, N_HIDDEN>& w, const half8 (&x)[2][IN_CHUNKS],
-                                               half8 (&h)[N_HIDDEN][2][4]) {
+__device__ __forceinline__ half8 zero8() {
+	half8 z;
 #pragma unroll
-	for (int t = 0; t < 2; ++t) {
+	for (int e = 0; e < 8; ++e) z[e] = (hf)0;
+	return z;
+}
+
+template <int IC, int NH>
+__device__ __forceinline__ void build_frags(hf* F, const hf* __restrict__ W, int count) {
+	using M = FragMap<IC, NH>;
+	const hf* W_hid = W + MLP_WIDTH * M::IN_W;
+	const hf* W_out = W_hid + (NH - 1) * MLP_WIDTH * MLP_WIDTH;
+	for (int idx = threadIdx.x; idx < count * 64; idx += MLP_BLOCK) {
+		const int f = idx >> 6, l = idx & 63, n = l & 31, g = l >> 5;
+		half8 v = zero8();
+		if (f < M::WH) {
+			v = wfrag_natural(W, M::IN_W, 32 * (f / IC) + n, f % IC, g);
+		} else if (f < M::WO) {
+			const int q = f - M::WH;
+			v = wfrag_chained(W_hid + (q >> 3) * MLP_WIDTH * MLP_WIDTH, MLP_WIDTH, 32 * ((q >> 2) & 1) + n, q & 3, g);
+		} else if (f < M::WOT) {
+			if (n < MLP_OUT) v = wfrag_chained(W_out, MLP_WIDTH, n, f - M::WO, g);
+		} else if (f < M::WHT) {
+			v = wTfrag_natural(W_out, MLP_WIDTH, 32 * (f - M::WOT) + n, 0, g, MLP_OUT);
+		} else if (f < M::W0T) {
+			const int q = f - M::WHT;
+			v = wTfrag_chained(W_hid + (q >> 3) * MLP_WIDTH * MLP_WIDTH, MLP_WIDTH, 32 * ((q >> 2) & 1) + n, q & 3, g);
+		} else if (f < M::SEL) {
+			const int q = f - M::W0T, m = 32 * (q >> 2) + n;
+			if (m < M::IN_W) v = wTfrag_chained(W, M::IN_W, m, q & 3, g);
+		} else if (f < M::ID) {
+			const int c = f - M::SEL;
+#pragma unroll
+			for (int e = 0; e < 8; ++e) v[e] = (16 * c + 8 * g + e == 32 * (c >> 1) + n) ? (hf)1 : (hf)0;
+		} else {
+#pragma unroll
+			for (int e = 0; e < 8; ++e) v[e] = (8 * g + e == n) ? (hf)1 : (hf)0;
+		}
+		*reinterpret_cast<half8*>(F + (size_t)idx * 8) = v;
+	}
+	__syncthreads();
+}
+
+// Ends one 32-sample tile: keeps the compiler from interleaving two tiles and from hoisting the
+// (loop-invariant) fragment loads into registers, which is exactly the register pressure to avoid.
+__device__ __forceinline__ void tile_fence() {
+	__builtin_amdgcn_sched_barrier(0);
+	asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ half8 frag(const hf* F, int f, int lane) { return *reinterpret_cast<const half8*>(F + f * 512 + lane * 8); }
+
+// fp16 rounding of a D tile into its two chained operands (no activation)
+__device__ __forceinline__ void plain_pack(const float16v& d, half8& lo, half8& hi) {
+#pragma unroll
+	for (int e = 0; e < 8; ++e) {
+		lo[e] = (hf)d[e];
+		hi[e] = (hf)d[8 + e];
+	}
+}
+
+// A register set that is the B operand of a matrix X (K x 32 samples, lane = sample) is at the same
+// time the A operand of X^T.  Swapping the two MFMA arguments of D = W X therefore yields
+// D^T = X^T W^T: the same activations with lane = neuron and the 32 samples along the registers.
+// Packed, a D^T tile is directly an operand of the batch-reduction products dW = dh h^T
+// (K = samples), so the weight gradients need no transposition through memory.
+
+// hidden layers, sample-lane form, for one 32-sample tile
+template <int IC, int NH>
+__device__ __forceinline__ void hidden_S(const hf* F, int lane, const half8 (&x)[IC], half8 (&h)[NH][4]) {
+	using M = FragMap<IC, NH>;
+#pragma unroll
+	for (int mt = 0; mt < 2; ++mt) {
+		float16v acc = zero16();
+#pragma unroll
+		for (int c = 0; c < IC; ++c) acc = N2_MFMA(frag(F, M::W0 + mt * IC + c, lane), x[c], acc);
+		relu_pack(acc, h[0][2 * mt], h[0][2 * mt + 1]);
+	}
+#pragma unroll
+	for (int k = 1; k < NH; ++k)
 #pragma unroll
 		for (int mt = 0; mt < 2; ++mt) {
 			float16v acc = zero16();
 #pragma unroll
-			for (int c = 0; c < IN_CHUNKS; ++c) acc = N2_MFMA(w.w0[mt][c], x[t][c], acc);
-			relu_pack(acc, h[0][t][2 * mt], h[0][t][2 * mt + 1]);
+			for (int c = 0; c < 4; ++c) acc = N2_MFMA(frag(F, M::WH + (k - 1) * 8 + mt * 4 + c, lane), h[k - 1][c], acc);
+			relu_pack(acc, h[k][2 * mt], h[k][2 * mt + 1]);
 		}
+}
+// neuron-lane form of neuron tile nt of hidden layer k (k = 0: from the input, else from layer k-1 in sample-lane form)
+template <int IC, int NH>
+__device__ __forceinline__ void hidden_N(const hf* F, int lane, int k, int nt, const half8 (&x)[IC], const half8 (&h)[NH][4], half8 (&out)[2]) {
+	using M = FragMap<IC, NH>;
+	float16v acc = zero16();
+	if (k == 0) {
+#pragma unroll
+		for (int c = 0; c < IC; ++c) acc = N2_MFMA(x[c], frag(F, M::W0 + nt * IC + c, lane), acc);
+	} else {
+#pragma unroll
+		for (int c = 0; c < 4; ++c) acc = N2_MFMA(h[k - 1][c], frag(F, M::WH + (k - 1) * 8 + nt * 4 + c, lane), acc);
 	}
+	relu_pack(acc, out[0], out[1]);
+}
+// input rows of feature tile nt in feature-lane form (exact: products with 0 and 1)
+template <int IC, int NH>
+__device__ __forceinline__ void input_N(const hf* F, int lane, int nt, const half8 (&x)[IC], half8 (&out)[2]) {
+	using M = FragMap<IC, NH>;
+	float16v acc = zero16();
 #pragma unroll
-	for (int k = 1; k < N_HIDDEN; ++k) {
-#pragma unroll
-		for (int t = 0; t < 2; ++t) {
-#pragma unroll
-			for (int mt = 0; mt < 2; ++mt) {
-				float16v acc = zero16();
-#pragma unroll
-				for (int c = 0; c < 4; ++c) acc = N2_MFMA(w.wh[k - 1][mt][c], h[k - 1][t][c], acc);
-				relu_pack(acc, h[k][t][2 * mt], h[k][t][2 * mt + 1]);
-			}
-		}
-	}
+	for (int c = 0; c < IC; ++c)
+		if ((c >> 1) == nt) acc = N2_MFMA(x[c], frag(F, M::SEL + c, lane), acc);
+	plain_pack(acc, out[0], out[1]);
 }
 
-template <int IN_CHUNKS>
-__device__ __forceinline__ void load_input(const hf* __restrict__ X, size_t N, uint32_t col, int g, half8 (&x)[2][IN_CHUNKS]) {
+template <int IC>
+__device__ __forceinline__ void split_pairs(const half8 (&p)[2][IC], int t, half8 (&x)[IC]) {
 #pragma unroll
-	for (int c = 0; c < IN_CHUNKS; ++c) bfrag_soa(X, N, col, c, g, 16 * IN_CHUNKS, x[0][c], x[1][c]);
+	for (int c = 0; c < IC; ++c) x[c] = p[t][c];
 }
 
 // ----------------------------------------------------------------------------
 // forward kernel
 // ----------------------------------------------------------------------------
-template <int IN_CHUNKS, int N_HIDDEN>
-__global__ void __launch_bounds__(MLP_BLOCK) mlp_forward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
-                                                                hf* __restrict__ Y, int out_aos, hf* __restrict__ hidden) {
+template <int IC, int NH, bool WANT_HIDDEN>
+__global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_forward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
+                                                                   hf* __restrict__ Y, int out_aos, hf* __restrict__ hidden) {
+	using M = FragMap<IC, NH>;
+	extern __shared__ __align__(16) unsigned char smem[];
+	hf* F = reinterpret_cast<hf*>(smem);
+	build_frags<IC, NH>(F, W, M::FWD_COUNT);
 	const int lane = threadIdx.x & 63, n = lane & 31, g = lane >> 5;
 	const uint32_t n_tiles = (N + MLP_TILE - 1) / MLP_TILE;
 	const uint32_t wave_gid = blockIdx.x * (MLP_BLOCK / 64) + (threadIdx.x >> 6), n_waves = gridDim.x * (MLP_BLOCK / 64);
-	FwdWeights<IN_CHUNKS, N_HIDDEN> w;
-	w.load(W, n, g);
 	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
-		const uint32_t b0 = tile * MLP_TILE, col_raw = b0 + 2 * n;
+		const uint32_t col_raw = tile * MLP_TILE + 2 * n;
 		const bool valid = col_raw < N;
 		const uint32_t col = valid ? col_raw : N - 2;
-		half8 x[2][IN_CHUNKS];
-		load_input<IN_CHUNKS>(X, N, col, g, x);
-		half8 h[N_HIDDEN][2][4];
-		forward_hidden<IN_CHUNKS, N_HIDDEN>(w, x, h);
-		float16v out[2][1];
+		const uint32_t off4 = 4u * g * N + col;
+		half8 xp[2][IC];
+		load_input<IC>(X, N, col, g, xp);
+		half4 keep[2];  // tile 0's output rows, held until tile 1's are known (SoA stores move sample pairs)
 #pragma unroll
 		for (int t = 0; t < 2; ++t) {
-			out[t][0] = zero16();
+			half8 x[IC], h[NH][4];
+			split_pairs<IC>(xp, t, x);
+			hidden_S<IC, NH>(F, lane, x, h);
+			float16v out = zero16();
 #pragma unroll
-			for (int c = 0; c < 4; ++c) out[t][0] = N2_MFMA(w.wo[c], h[N_HIDDEN - 1][t][c], out[t][0]);
-		}
-		if (out_aos) {
+			for (int c = 0; c < 4; ++c) out = N2_MFMA(frag(F, M::WO + c, lane), h[NH - 1][c], out);
+			// registers 0..3 hold rows 4g..4g+3, registers 4..7 rows 8+4g..8+4g+3
+			const half4 lo = half4{(hf)out[0], (hf)out[1], (hf)out[2], (hf)out[3]}, hi = half4{(hf)out[4], (hf)out[5], (hf)out[6], (hf)out[7]};
 			if (valid) {
-				// rows 4g..4g+3 (r = 0..3) and 8+4g..8+4g+3 (r = 4..7) of each sample
-#pragma unroll
-				for (int t = 0; t < 2; ++t) {
+				if (out_aos) {
 					hf* y = Y + (size_t)(col + t) * MLP_OUT;
-					*reinterpret_cast<half4*>(y + 4 * g) = half4{(hf)out[t][0][0], (hf)out[t][0][1], (hf)out[t][0][2], (hf)out[t][0][3]};
-					*reinterpret_cast<half4*>(y + 8 + 4 * g) = half4{(hf)out[t][0][4], (hf)out[t][0][5], (hf)out[t][0][6], (hf)out[t][0][7]};
+					*reinterpret_cast<half4*>(y + 4 * g) = lo;
+					*reinterpret_cast<half4*>(y + 8 + 4 * g) = hi;
+				} else if (t == 0) {
+					keep[0] = lo; keep[1] = hi;
+				} else {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						*reinterpret_cast<half2v*>(Y + (size_t)e * N + off4) = half2v{keep[0][e], lo[e]};
+						*reinterpret_cast<half2v*>(Y + (size_t)(8 + e) * N + off4) = half2v{keep[1][e], hi[e]};
+					}
+				}
+				if (WANT_HIDDEN) {
+#pragma unroll
+					for (int k = 0; k < NH; ++k)
+#pragma unroll
+						for (int c = 0; c < 4; ++c)
+#pragma unroll
+							for (int e = 0; e < 8; ++e) {
+								const int neuron = 16 * c + 4 * g + (e & 3) + ((e >> 2) << 3);
+								hidden[((size_t)k * MLP_WIDTH + neuron) * N + col + t] = h[k][c][e];
+							}
 				}
 			}
-		} else {
-			store_soa<1>(Y, N, col, valid, out, g, MLP_OUT);
-		}
-		if (hidden && valid) {
-#pragma unroll
-			for (int k = 0; k < N_HIDDEN; ++k)
-#pragma unroll
-				for (int c = 0; c < 4; ++c)
-#pragma unroll
-					for (int e = 0; e < 8; ++e) {
-						const int neuron = 16 * c + 4 * g + (e & 3) + ((e >> 2) << 3);
-						*reinterpret_cast<half2v*>(hidden + ((size_t)k * MLP_WIDTH + neuron) * N + col) = half2v{h[k][0][c][e], h[k][1][c][e]};
-					}
+			tile_fence();
 		}
 	}
 }
 
 // ----------------------------------------------------------------------------
-// weight-gradient accumulation helpers
+// weight-gradient accumulators of one wave
 // ----------------------------------------------------------------------------
-// acc[mt][nt] += A_staged(64 rows) x B^T over the 64 samples of the tile.
-// B comes from a second staged matrix.
-template <int NT>
-__device__ __forceinline__ void outer_staged(float16v (&acc)[2][NT], const hf* SA, const hf* SB, int n, int g) {
-	stage_sync();
+// A wave with role r owns the gradient rows of neuron tile r (neurons 32r .. 32r+31):
+//   gW0[nt]    : dW_0  rows 32r + drow, columns 32nt + n
+//   gWh[k][nt] : dW_k+1 rows 32r + drow, columns 32nt + n
+//   gWo        : dW_out rows drow (< 16), columns 32r + n
+template <int IC, int NH>
+struct GradAcc {
+	static constexpr int IN_MT = (16 * IC + 31) / 32;
+	float16v gW0[IN_MT], gWh[NH > 1 ? NH - 1 : 1][2], gWo;
+	__device__ __forceinline__ void clear() {
 #pragma unroll
-	for (int c = 0; c < 4; ++c) {
-		half8 a[2], b[NT];
+		for (int nt = 0; nt < IN_MT; ++nt) gW0[nt] = zero16();
 #pragma unroll
-		for (int mt = 0; mt < 2; ++mt) a[mt] = stage_frag(SA, 32 * mt + n, c, g);
-#pragma unroll
-		for (int nt = 0; nt < NT; ++nt) b[nt] = stage_frag(SB, 32 * nt + n, c, g);
-#pragma unroll
-		for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-			for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = N2_MFMA(a[mt], b[nt], acc[mt][nt]);
+		for (int k = 0; k < NH - 1; ++k) { gWh[k][0] = zero16(); gWh[k][1] = zero16(); }
+		gWo = zero16();
 	}
-}
-// B comes straight from an SoA global matrix with n_rows valid rows.
-template <int NT>
-__device__ __forceinline__ void outer_global(float16v (&acc)[2][NT], const hf* SA, const hf* __restrict__ M, size_t N, uint32_t b0,
-                                             int n_rows, bool aos16, int unit_row, int n, int g) {
-	stage_sync();
+	// visit every accumulator element this lane holds: fn(parameter index, value)
+	template <typename Fn>
+	__device__ __forceinline__ void for_each(int role, int n, int g, Fn fn) {
+		constexpr int IN_W = 16 * IC;
 #pragma unroll
-	for (int c = 0; c < 4; ++c) {
-		half8 a[2], b[NT];
+		for (int nt = 0; nt < IN_MT; ++nt)
 #pragma unroll
-		for (int mt = 0; mt < 2; ++mt) a[mt] = stage_frag(SA, 32 * mt + n, c, g);
+			for (int r = 0; r < 16; ++r)
+				if (32 * nt + n < IN_W) fn((32 * role + drow(r, g)) * IN_W + 32 * nt + n, gW0[nt][r]);
 #pragma unroll
-		for (int nt = 0; nt < NT; ++nt)
-			b[nt] = unit_row >= 0 ? batch_frag_unit(N, b0, 32 * nt + n, unit_row, c, g)
-			      : aos16 ? batch_frag_aos16(M, N, b0, 32 * nt + n, c, g) : batch_frag_soa(M, N, b0, 32 * nt + n, n_rows, c, g);
+		for (int k = 0; k < NH - 1; ++k)
 #pragma unroll
-		for (int mt = 0; mt < 2; ++mt)
+			for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-			for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = N2_MFMA(a[mt], b[nt], acc[mt][nt]);
+				for (int r = 0; r < 16; ++r) fn(MLP_WIDTH * IN_W + k * MLP_WIDTH * MLP_WIDTH + (32 * role + drow(r, g)) * MLP_WIDTH + 32 * nt + n, gWh[k][nt][r]);
+#pragma unroll
+		for (int r = 0; r < 16; ++r)
+			if (drow(r, g) < MLP_OUT) fn(MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + drow(r, g) * MLP_WIDTH + 32 * role + n, gWo[r]);
 	}
-}
-
-// Add a wave's D tiles (rows = 64 "left" indices, cols = 32*NT "right" indices)
-// into the workgroup's fp32 LDS image of a weight matrix.
-// transposed = false: left is the weight's row (out), right its column (in): W[left*ld + right]
-// transposed = true : left is the column, right the row:                   W[right*ld + left]
-template <int NT>
-__device__ __forceinline__ void flush_acc(float* Wl, int ld, bool transposed, int n_right, const float16v (&acc)[2][NT], int n, int g) {
-#pragma unroll
-	for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-		for (int nt = 0; nt < NT; ++nt) {
-			const int right = 32 * nt + n;
-			if (right >= n_right) continue;
-#pragma unroll
-			for (int r = 0; r < 16; ++r) {
-				const int left = 32 * mt + drow(r, g);
-				atomicAdd(&Wl[transposed ? right * ld + left : left * ld + right], acc[mt][nt][r]);
-			}
-		}
-}
+	// Sum the four waves of a workgroup (waves 0,1 and 2,3 hold the same roles) in an fp32 LDS image
+	// of the parameters and write it as this workgroup's slab.  Plain LDS stores only.
+	__device__ __forceinline__ void write_slab(float* Wl, float* __restrict__ slab, int n_params, int wave, int role, int n, int g) {
+		__syncthreads();  // every wave is done with the fragments the image overlays
+		if (wave < 2) for_each(role, n, g, [&](int i, float v) { Wl[i] = v; });
+		__syncthreads();
+		if (wave >= 2) for_each(role, n, g, [&](int i, float v) { Wl[i] += v; });
+		__syncthreads();
+		for (int i = threadIdx.x; i < n_params; i += MLP_BLOCK) slab[i] = Wl[i];
+	}
+};
 
 // ----------------------------------------------------------------------------
 // backward kernel: recomputes the hidden activations, then
 //   dL_dh_last = mask * W_out^T dL_dy ; ... ; dL_dx = W_0^T dL_dh_0
 //   dW_out = dL_dy h_last^T ; dW_k = dL_dh_k h_{k-1}^T ; dW_0 = dL_dh_0 x^T
-// Weight gradients are summed per workgroup in fp32 and written to one slab of
-// `partials` per workgroup; a second tiny kernel reduces the slabs.
+// With WANT_DW two waves (roles 0 and 1) work on the same 64 samples; each accumulates the gradient
+// rows of one neuron tile (and computes one row tile of dL_dx), both run the cheap data chain.
+// Weight gradients are summed per workgroup in fp32 and written to one slab of `partials` per
+// workgroup; a second tiny kernel reduces the slabs.
 // ----------------------------------------------------------------------------
-template <int IN_CHUNKS, int N_HIDDEN, bool WANT_DX, bool WANT_DW>
-__global__ void __launch_bounds__(MLP_BLOCK) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
-                                                                 const hf* __restrict__ dY, int dy_aos, int unit_row,
-                                                                 hf* __restrict__ dX, float* __restrict__ partials) {
-	constexpr int IN_W = 16 * IN_CHUNKS;
-	constexpr int IN_MT = (IN_W + 31) / 32;
-	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (N_HIDDEN - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
+template <int IC, int NH, bool WANT_DX, bool WANT_DW>
+__global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
+                                                                    const hf* __restrict__ dY, int dy_aos, int unit_row,
+                                                                    hf* __restrict__ dX, float* __restrict__ partials) {
+	using M = FragMap<IC, NH>;
+	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT, ROLES = WANT_DW ? 2 : 1;
+	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
 	extern __shared__ __align__(16) unsigned char smem[];
+	hf* F = reinterpret_cast<hf*>(smem);
+	build_frags<IC, NH>(F, W, M::COUNT);
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, g = lane >> 5;
+	const int role = WANT_DW ? __builtin_amdgcn_readfirstlane(wave & 1) : 0;
 	const uint32_t n_tiles = (N + MLP_TILE - 1) / MLP_TILE;
-	const uint32_t wave_gid = blockIdx.x * (MLP_BLOCK / 64) + wave, n_waves = gridDim.x * (MLP_BLOCK / 64);
-	hf* SA = reinterpret_cast<hf*>(smem) + (size_t)wave * 2 * MLP_WIDTH * STAGE_LD;
-	hf* SB = SA + MLP_WIDTH * STAGE_LD;
+	const uint32_t slot = (blockIdx.x * (MLP_BLOCK / 64) + wave) / ROLES, n_slots = gridDim.x * (MLP_BLOCK / 64) / ROLES;
+	GradAcc<IC, NH> acc;
+	if (WANT_DW) acc.clear();
 
-	FwdWeights<IN_CHUNKS, N_HIDDEN> w;
-	w.load(W, n, g);
-	// transposed weights for the data path
-	const hf* W_out = W + MLP_WIDTH * IN_W + (N_HIDDEN - 1) * MLP_WIDTH * MLP_WIDTH;
-	half8 woT[2];
-#pragma unroll
-	for (int mt = 0; mt < 2; ++mt) woT[mt] = wTfrag_natural(W_out, MLP_WIDTH, 32 * mt + n, 0, g, MLP_OUT);
-	half8 whT[N_HIDDEN > 1 ? N_HIDDEN - 1 : 1][2][4];
-#pragma unroll
-	for (int k = 0; k < N_HIDDEN - 1; ++k)
-#pragma unroll
-		for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-			for (int c = 0; c < 4; ++c) whT[k][mt][c] = wTfrag_chained(W + MLP_WIDTH * IN_W + k * MLP_WIDTH * MLP_WIDTH, MLP_WIDTH, 32 * mt + n, c, g);
-	half8 w0T[IN_MT][4];
-	if (WANT_DX) {
-#pragma unroll
-		for (int mt = 0; mt < IN_MT; ++mt)
-#pragma unroll
-			for (int c = 0; c < 4; ++c) {
-				half8 z;
-#pragma unroll
-				for (int e = 0; e < 8; ++e) z[e] = (hf)0;
-				w0T[mt][c] = (32 * mt + n < IN_W) ? wTfrag_chained(W, IN_W, 32 * mt + n, c, g) : z;
-			}
-	}
-
-	float16v gW0[2][IN_MT], gWh[N_HIDDEN > 1 ? N_HIDDEN - 1 : 1][2][2], gWo[2][1];
-	if (WANT_DW) {
-#pragma unroll
-		for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-			for (int nt = 0; nt < IN_MT; ++nt) gW0[mt][nt] = zero16();
-#pragma unroll
-			for (int k = 0; k < N_HIDDEN - 1; ++k) { gWh[k][mt][0] = zero16(); gWh[k][mt][1] = zero16(); }
-			gWo[mt][0] = zero16();
-		}
-	}
-
-	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
-		const uint32_t b0 = tile * MLP_TILE, col_raw = b0 + 2 * n;
+	for (uint32_t tile = slot; tile < n_tiles; tile += n_slots) {
+		const uint32_t col_raw = tile * MLP_TILE + 2 * n;
 		const bool valid = col_raw < N;
 		const uint32_t col = valid ? col_raw : N - 2;
-		half8 x[2][IN_CHUNKS];
-		load_input<IN_CHUNKS>(X, N, col, g, x);
-		half8 h[N_HIDDEN][2][4];
-		forward_hidden<IN_CHUNKS, N_HIDDEN>(w, x, h);
-		half8 dy[2];
-		outgrad_frag(dY, N, col, g, dy_aos != 0, unit_row, dy[0], dy[1]);
-		if (!valid) {
+		const uint32_t off4 = 4u * g * N + col;
+		half8 xp[2][IC], dyp[2];
+		load_input<IC>(X, N, col, g, xp);
+		outgrad_frag(dY, N, col, g, dy_aos != 0, unit_row, dyp[0], dyp[1]);
+		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
+		constexpr int DX_TILES = WANT_DW ? 1 : IN_MT;  // with two roles each computes one row tile of dL_dx
+		half8 dx_keep[DX_TILES][2];                    // tile 0's rows until tile 1's are known (sample-pair stores)
 #pragma unroll
-			for (int e = 0; e < 8; ++e) { dy[0][e] = (hf)0; dy[1][e] = (hf)0; }
-		}
-		// dL_dh of the last hidden layer
-		half8 dh[2][4];
-#pragma unroll
-		for (int t = 0; t < 2; ++t)
-#pragma unroll
-			for (int mt = 0; mt < 2; ++mt) {
-				float16v acc = N2_MFMA(woT[mt], dy[t], zero16());
-				mask_pack(acc, h[N_HIDDEN - 1][t][2 * mt], h[N_HIDDEN - 1][t][2 * mt + 1], dh[t][2 * mt], dh[t][2 * mt + 1]);
-			}
-		if (WANT_DW) {
-			// dW_out^T [neuron][o] += h_last dY^T
-			stage_store(SA, h[N_HIDDEN - 1], n, g);
-			outer_global<1>(gWo, SA, dY, N, b0, MLP_OUT, dy_aos != 0, unit_row, n, g);
-		}
-#pragma unroll
-		for (int k = N_HIDDEN - 1; k >= 1; --k) {
+		for (int t = 0; t < 2; ++t) {
+			half8 x[IC], h[NH][4], dh[4];
+			split_pairs<IC>(xp, t, x);
+			const half8 dy = dyp[t];
+			hidden_S<IC, NH>(F, lane, x, h);
+			// ---- output layer ----
+			// dhN: gradient of the pre-activations of the current layer, neuron tile `role`, neuron-lane form
+			half8 dhN[2];
 			if (WANT_DW) {
-				// dW_k [out][in] += dh_k h_{k-1}^T
-				stage_store(SA, dh, n, g);
-				stage_store(SB, h[k - 1], n, g);
-				outer_staged<2>(gWh[k - 1], SA, SB, n, g);
+				half8 hN[2], dyN[2];
+				hidden_N<IC, NH>(F, lane, NH - 1, role, x, h, hN);
+				plain_pack(N2_MFMA(dy, frag(F, M::ID, lane), zero16()), dyN[0], dyN[1]);
+				acc.gWo = N2_MFMA(dyN[0], hN[0], acc.gWo);
+				acc.gWo = N2_MFMA(dyN[1], hN[1], acc.gWo);
+				mask_pack(N2_MFMA(dy, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], dhN[0], dhN[1]);
 			}
-			half8 dprev[2][4];
 #pragma unroll
-			for (int t = 0; t < 2; ++t)
+			for (int mt = 0; mt < 2; ++mt)
+				mask_pack(N2_MFMA(frag(F, M::WOT + mt, lane), dy, zero16()), h[NH - 1][2 * mt], h[NH - 1][2 * mt + 1], dh[2 * mt], dh[2 * mt + 1]);
+			// ---- hidden layers, last to first ----
+#pragma unroll
+			for (int k = NH - 1; k >= 1; --k) {
+				if (WANT_DW) {
+#pragma unroll
+					for (int nt = 0; nt < 2; ++nt) {
+						half8 hN[2];
+						hidden_N<IC, NH>(F, lane, k - 1, nt, x, h, hN);
+						acc.gWh[k - 1][nt] = N2_MFMA(dhN[0], hN[0], acc.gWh[k - 1][nt]);
+						acc.gWh[k - 1][nt] = N2_MFMA(dhN[1], hN[1], acc.gWh[k - 1][nt]);
+					}
+					half8 hN[2];
+					hidden_N<IC, NH>(F, lane, k - 1, role, x, h, hN);
+					float16v a = zero16();
+#pragma unroll
+					for (int c = 0; c < 4; ++c) a = N2_MFMA(dh[c], frag(F, M::WHT + (k - 1) * 8 + role * 4 + c, lane), a);
+					mask_pack(a, hN[0], hN[1], dhN[0], dhN[1]);
+				}
+				half8 dprev[4];
 #pragma unroll
 				for (int mt = 0; mt < 2; ++mt) {
-					float16v acc = zero16();
+					float16v a = zero16();
 #pragma unroll
-					for (int c = 0; c < 4; ++c) acc = N2_MFMA(whT[k - 1][mt][c], dh[t][c], acc);
-					mask_pack(acc, h[k - 1][t][2 * mt], h[k - 1][t][2 * mt + 1], dprev[t][2 * mt], dprev[t][2 * mt + 1]);
+					for (int c = 0; c < 4; ++c) a = N2_MFMA(frag(F, M::WHT + (k - 1) * 8 + mt * 4 + c, lane), dh[c], a);
+					mask_pack(a, h[k - 1][2 * mt], h[k - 1][2 * mt + 1], dprev[2 * mt], dprev[2 * mt + 1]);
 				}
 #pragma unroll
-			for (int t = 0; t < 2; ++t)
+				for (int c = 0; c < 4; ++c) dh[c] = dprev[c];
+			}
+			// ---- first layer ----
+			if (WANT_DW) {
 #pragma unroll
-				for (int c = 0; c < 4; ++c) dh[t][c] = dprev[t][c];
-		}
-		if (WANT_DW) {
-			// dW_0 [neuron][input] += dh_0 x^T
-			stage_store(SA, dh, n, g);
-			outer_global<IN_MT>(gW0, SA, X, N, b0, IN_W, false, -1, n, g);
-		}
-		if (WANT_DX) {
-			float16v dx[2][IN_MT];
-#pragma unroll
-			for (int t = 0; t < 2; ++t)
-#pragma unroll
-				for (int mt = 0; mt < IN_MT; ++mt) {
-					dx[t][mt] = zero16();
-#pragma unroll
-					for (int c = 0; c < 4; ++c) dx[t][mt] = N2_MFMA(w0T[mt][c], dh[t][c], dx[t][mt]);
+				for (int nt = 0; nt < IN_MT; ++nt) {
+					half8 xN[2];
+					input_N<IC, NH>(F, lane, nt, x, xN);
+					acc.gW0[nt] = N2_MFMA(dhN[0], xN[0], acc.gW0[nt]);
+					acc.gW0[nt] = N2_MFMA(dhN[1], xN[1], acc.gW0[nt]);
 				}
-			store_soa<IN_MT>(dX, N, col, valid, dx, g, IN_W);
+			}
+			if (WANT_DX) {
+#pragma unroll
+				for (int j = 0; j < DX_TILES; ++j) {
+					const int mt = WANT_DW ? role : j;
+					if (mt >= IN_MT) continue;
+					float16v d = zero16();
+#pragma unroll
+					for (int c = 0; c < 4; ++c) d = N2_MFMA(frag(F, M::W0T + mt * 4 + c, lane), dh[c], d);
+					half8 lo, hi;
+					plain_pack(d, lo, hi);
+					if (t == 0) {
+						dx_keep[j][0] = lo; dx_keep[j][1] = hi;
+					} else if (valid) {
+#pragma unroll
+						for (int e = 0; e < 8; ++e) {
+							// rows 32mt + drow(e, g) and 32mt + drow(8 + e, g); the 4g part is in off4
+							const int r0 = 32 * mt + 8 * (e >> 2) + (e & 3), r1 = r0 + 16;
+							if (r0 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r0 * N + off4) = half2v{dx_keep[j][0][e], lo[e]};
+							if (r1 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r1 * N + off4) = half2v{dx_keep[j][1][e], hi[e]};
+						}
+					}
+				}
+			}
+			tile_fence();
 		}
 	}
-
-	if (WANT_DW) {
-		__syncthreads();
-		float* Wl = reinterpret_cast<float*>(smem);
-		for (int i = threadIdx.x; i < N_PARAMS; i += MLP_BLOCK) Wl[i] = 0.f;
-		__syncthreads();
-		flush_acc<IN_MT>(Wl, IN_W, false, IN_W, gW0, n, g);
-#pragma unroll
-		for (int k = 0; k < N_HIDDEN - 1; ++k) flush_acc<2>(Wl + MLP_WIDTH * IN_W + k * MLP_WIDTH * MLP_WIDTH, MLP_WIDTH, false, MLP_WIDTH, gWh[k], n, g);
-		flush_acc<1>(Wl + MLP_WIDTH * IN_W + (N_HIDDEN - 1) * MLP_WIDTH * MLP_WIDTH, MLP_WIDTH, true, MLP_OUT, gWo, n, g);
-		__syncthreads();
-		float* slab = partials + (size_t)blockIdx.x * N_PARAMS;
-		for (int i = threadIdx.x; i < N_PARAMS; i += MLP_BLOCK) slab[i] = Wl[i];
-	}
+	if (WANT_DW) acc.write_slab(reinterpret_cast<float*>(smem), partials + (size_t)blockIdx.x * N_PARAMS, N_PARAMS, wave, role, n, g);
 }
 
 // ----------------------------------------------------------------------------
 // second-order kernel (one hidden layer):
 //   m = 1[W_0 x > 0];  a = m * (W_0 v);  b = m * (W_out^T g)
 //   dW_0 += b v^T;  dW_out += g a^T;  dL_ddLdy = W_out a
+// Same two-role scheme as the backward kernel.
 // ----------------------------------------------------------------------------
-template <int IN_CHUNKS>
-__global__ void __launch_bounds__(MLP_BLOCK) mlp_bbi_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
-                                                            const hf* __restrict__ V, const hf* __restrict__ G, int unit_row,
-                                                            hf* __restrict__ dLddY, float* __restrict__ partials) {
-	constexpr int IN_W = 16 * IN_CHUNKS;
-	constexpr int IN_MT = (IN_W + 31) / 32;
+template <int IC>
+__global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_bbi_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
+                                                               const hf* __restrict__ V, const hf* __restrict__ G, int unit_row,
+                                                               hf* __restrict__ dLddY, float* __restrict__ partials) {
+	using M = FragMap<IC, 1>;
+	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + MLP_OUT * MLP_WIDTH;
 	extern __shared__ __align__(16) unsigned char smem[];
+	hf* F = reinterpret_cast<hf*>(smem);
+	build_frags<IC, 1>(F, W, M::COUNT);
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, g = lane >> 5;
+	const int role = __builtin_amdgcn_readfirstlane(wave & 1);
 	const uint32_t n_tiles = (N + MLP_TILE - 1) / MLP_TILE;
-	const uint32_t wave_gid = blockIdx.x * (MLP_BLOCK / 64) + wave, n_waves = gridDim.x * (MLP_BLOCK / 64);
-	hf* SA = reinterpret_cast<hf*>(smem) + (size_t)wave * 2 * MLP_WIDTH * STAGE_LD;
-
-	FwdWeights<IN_CHUNKS, 1> w;
-	w.load(W, n, g);
-	const hf* W_out = W + MLP_WIDTH * IN_W;
-	half8 woT[2];
-#pragma unroll
-	for (int mt = 0; mt < 2; ++mt) woT[mt] = wTfrag_natural(W_out, MLP_WIDTH, 32 * mt + n, 0, g, MLP_OUT);
-	float16v gW0[2][IN_MT], gWo[2][1];
-#pragma unroll
-	for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-		for (int nt = 0; nt < IN_MT; ++nt) gW0[mt][nt] = zero16();
-		gWo[mt][0] = zero16();
-	}
-	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
-		const uint32_t b0 = tile * MLP_TILE, col_raw = b0 + 2 * n;
+	const uint32_t slot = (blockIdx.x * (MLP_BLOCK / 64) + wave) / 2, n_slots = gridDim.x * (MLP_BLOCK / 64) / 2;
+	GradAcc<IC, 1> acc;
+	acc.clear();
+	for (uint32_t tile = slot; tile < n_tiles; tile += n_slots) {
+		const uint32_t col_raw = tile * MLP_TILE + 2 * n;
 		const bool valid = col_raw < N;
 		const uint32_t col = valid ? col_raw : N - 2;
-		half8 x[2][IN_CHUNKS], v[2][IN_CHUNKS], gg[2];
-		load_input<IN_CHUNKS>(X, N, col, g, x);
-		load_input<IN_CHUNKS>(V, N, col, g, v);
-		outgrad_frag(G, N, col, g, false, unit_row, gg[0], gg[1]);
+		const uint32_t off4 = 4u * g * N + col;
+		half8 xp[2][IC], vp[2][IC], gp[2];
+		load_input<IC>(X, N, col, g, xp);
+		load_input<IC>(V, N, col, g, vp);
+		outgrad_frag(G, N, col, g, false, unit_row, gp[0], gp[1]);
 		if (!valid) {
+			gp[0] = zero8(); gp[1] = zero8();
 #pragma unroll
-			for (int e = 0; e < 8; ++e) {
-				gg[0][e] = (hf)0; gg[1][e] = (hf)0;
-#pragma unroll
-				for (int c = 0; c < IN_CHUNKS; ++c) { v[0][c][e] = (hf)0; v[1][c][e] = (hf)0; }
-			}
+			for (int c = 0; c < IC; ++c) { vp[0][c] = zero8(); vp[1][c] = zero8(); }
 		}
-		half8 h[1][2][4];
-		forward_hidden<IN_CHUNKS, 1>(w, x, h);
-		half8 a[2][4], b[2][4];
+		half4 keep[2];
 #pragma unroll
-		for (int t = 0; t < 2; ++t)
+		for (int t = 0; t < 2; ++t) {
+			half8 x[IC], v[IC], h[1][4];
+			split_pairs<IC>(xp, t, x);
+			split_pairs<IC>(vp, t, v);
+			const half8 gg = gp[t];
+			if (partials) {
+				half8 hN[2], aN[2], bN[2], gN[2];
+				hidden_N<IC, 1>(F, lane, 0, role, x, h, hN);  // the mask of neuron tile `role`, neuron-lane form
+				float16v a = zero16();
 #pragma unroll
-			for (int mt = 0; mt < 2; ++mt) {
-				float16v acc = zero16();
+				for (int c = 0; c < IC; ++c) a = N2_MFMA(v[c], frag(F, M::W0 + role * IC + c, lane), a);
+				mask_pack(a, hN[0], hN[1], aN[0], aN[1]);
+				mask_pack(N2_MFMA(gg, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], bN[0], bN[1]);
+				plain_pack(N2_MFMA(gg, frag(F, M::ID, lane), zero16()), gN[0], gN[1]);
+				acc.gWo = N2_MFMA(gN[0], aN[0], acc.gWo);
+				acc.gWo = N2_MFMA(gN[1], aN[1], acc.gWo);
 #pragma unroll
-				for (int c = 0; c < IN_CHUNKS; ++c) acc = N2_MFMA(w.w0[mt][c], v[t][c], acc);
-				mask_pack(acc, h[0][t][2 * mt], h[0][t][2 * mt + 1], a[t][2 * mt], a[t][2 * mt + 1]);
-				float16v accb = N2_MFMA(woT[mt], gg[t], zero16());
-				mask_pack(accb, h[0][t][2 * mt], h[0][t][2 * mt + 1], b[t][2 * mt], b[t][2 * mt + 1]);
+				for (int nt = 0; nt < IN_MT; ++nt) {
+					half8 vN[2];
+					input_N<IC, 1>(F, lane, nt, v, vN);
+					acc.gW0[nt] = N2_MFMA(bN[0], vN[0], acc.gW0[nt]);
+					acc.gW0[nt] = N2_MFMA(bN[1], vN[1], acc.gW0[nt]);
+				}
 			}
-		if (partials) {
-			stage_store(SA, b, n, g);
-			outer_global<IN_MT>(gW0, SA, V, N, b0, IN_W, false, -1, n, g);
-			stage_store(SA, a, n, g);
-			outer_global<1>(gWo, SA, G, N, b0, MLP_OUT, false, unit_row, n, g);
-		}
-		if (dLddY) {
-			float16v out[2][1];
+			if (dLddY && role == 0) {
+				hidden_S<IC, 1>(F, lane, x, h);
+				half8 a[4];
 #pragma unroll
-			for (int t = 0; t < 2; ++t) {
-				out[t][0] = zero16();
+				for (int mt = 0; mt < 2; ++mt) {
+					float16v d = zero16();
 #pragma unroll
-				for (int c = 0; c < 4; ++c) out[t][0] = N2_MFMA(w.wo[c], a[t][c], out[t][0]);
+					for (int c = 0; c < IC; ++c) d = N2_MFMA(frag(F, M::W0 + mt * IC + c, lane), v[c], d);
+					mask_pack(d, h[0][2 * mt], h[0][2 * mt + 1], a[2 * mt], a[2 * mt + 1]);
+				}
+				float16v out = zero16();
+#pragma unroll
+				for (int c = 0; c < 4; ++c) out = N2_MFMA(frag(F, M::WO + c, lane), a[c], out);
+				const half4 lo = half4{(hf)out[0], (hf)out[1], (hf)out[2], (hf)out[3]}, hi = half4{(hf)out[4], (hf)out[5], (hf)out[6], (hf)out[7]};
+				if (t == 0) {
+					keep[0] = lo; keep[1] = hi;
+				} else if (valid) {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						*reinterpret_cast<half2v*>(dLddY + (size_t)e * N + off4) = half2v{keep[0][e], lo[e]};
+						*reinterpret_cast<half2v*>(dLddY + (size_t)(8 + e) * N + off4) = half2v{keep[1][e], hi[e]};
+					}
+				}
 			}
-			store_soa<1>(dLddY, N, col, valid, out, g, MLP_OUT);
+			tile_fence();
 		}
 	}
-	if (partials) {
-		__syncthreads();
-		float* Wl = reinterpret_cast<float*>(smem);
-		for (int i = threadIdx.x; i < N_PARAMS; i += MLP_BLOCK) Wl[i] = 0.f;
-		__syncthreads();
-		flush_acc<IN_MT>(Wl, IN_W, false, IN_W, gW0, n, g);
-		flush_acc<1>(Wl + MLP_WIDTH * IN_W, MLP_WIDTH, true, MLP_OUT, gWo, n, g);
-		__syncthreads();
-		float* slab = partials + (size_t)blockIdx.x * N_PARAMS;
-		for (int i = threadIdx.x; i < N_PARAMS; i += MLP_BLOCK) slab[i] = Wl[i];
-	}
+	if (partials) acc.write_slab(reinterpret_cast<float*>(smem), partials + (size_t)blockIdx.x * N_PARAMS, N_PARAMS, wave, role, n, g);
 }
 
 // grads (fp16) = [grads +] sum over slabs.  16 parameters x 16 slab groups per workgroup: every
@@ -696,17 +750,21 @@ static int check_mlp_batch(const n2_mlp_t* mlp, const char* fn, const void* d_in
 	N2_REQUIRE(mlp != nullptr, "%s: mlp is null", fn);
 	N2_REQUIRE(mlp->params != nullptr, "%s: n2_mlp_set_params has not been called", fn);
 	N2_REQUIRE(n % 8 == 0, "%s: batch size %u is not a multiple of 8", fn, n);
-	N2_REQUIRE(n <= (1u << 30), "%s: batch size %u exceeds 2^30", fn, n);
+	N2_REQUIRE(n <= (1u << 28), "%s: batch size %u exceeds 2^28 (per-lane offsets are 32-bit)", fn, n);
 	N2_REQUIRE(d_input != nullptr || n == 0, "%s: d_input is null", fn);
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_input) % 16 == 0, "%s: d_input must be 16-byte aligned", fn);
 	return N2_OK;
 }
 
-static inline uint32_t stream_grid(uint32_t n, uint32_t max_blocks) {
+// workgroups of a launch: every wave (or pair of waves when two roles share a tile) takes 64-sample
+// tiles in a grid-stride loop; never more than two workgroups per CU, which build the weight fragments once
+static inline uint32_t stream_grid(uint32_t n, uint32_t waves_per_tile) {
 	const uint32_t tiles = (n + MLP_TILE - 1) / MLP_TILE;
-	const uint32_t blocks = (tiles + (MLP_BLOCK / 64) - 1) / (MLP_BLOCK / 64);
-	return blocks < max_blocks ? blocks : max_blocks;
+	const uint32_t tiles_per_block = (MLP_BLOCK / 64) / waves_per_tile;
+	const uint32_t blocks = (tiles + tiles_per_block - 1) / tiles_per_block;
+	return blocks < (uint32_t)MLP_MAX_SLABS ? blocks : (uint32_t)MLP_MAX_SLABS;
 }
+static inline size_t frag_bytes(int n_frags) { return (size_t)n_frags * 64 * 16; }
 
 #define MLP_DISPATCH(in_w, n_hidden, CALL)                                            \
 	do {                                                                              \
@@ -732,11 +790,17 @@ N2_API int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_in
 	N2_REQUIRE(out_layout == N2_LAYOUT_SOA || out_layout == N2_LAYOUT_AOS, "n2_mlp_forward: bad layout %d", (int)out_layout);
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0 && reinterpret_cast<uintptr_t>(d_hidden) % 16 == 0,
 	           "n2_mlp_forward: outputs must be 16-byte aligned");
-	const dim3 grid(stream_grid(n, 2048)), block(MLP_BLOCK);
+	const dim3 grid(stream_grid(n, 1)), block(MLP_BLOCK);
 	N2ProfScope prof(N2_PROF_MLP_FORWARD, n2_stream(stream));
 #define CALL(IC, NH)                                                                                                     \
-	mlp_forward_kernel<IC, NH><<<grid, block, 0, n2_stream(stream)>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
-		reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0, reinterpret_cast<hf*>(d_hidden))
+	do {                                                                                                                 \
+		if (d_hidden)                                                                                                    \
+			mlp_forward_kernel<IC, NH, true><<<grid, block, frag_bytes(FragMap<IC, NH>::FWD_COUNT), n2_stream(stream)>>>(mlp->params, \
+				reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0, reinterpret_cast<hf*>(d_hidden)); \
+		else                                                                                                             \
+			mlp_forward_kernel<IC, NH, false><<<grid, block, frag_bytes(FragMap<IC, NH>::FWD_COUNT), n2_stream(stream)>>>(mlp->params, \
+				reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0, nullptr); \
+	} while (0)
 	MLP_DISPATCH(mlp->in_w, mlp->n_hidden, CALL);
 #undef CALL
 	N2_LAUNCH_CHECK();
@@ -758,8 +822,6 @@ static int check_grad_mode(const n2_mlp_t* mlp, const char* fn, n2_grad_mode mod
 	}
 	return N2_OK;
 }
-
-static constexpr size_t STAGE_BYTES = (size_t)(MLP_BLOCK / 64) * 2 * MLP_WIDTH * STAGE_LD * sizeof(hf);
 
 template <typename K>
 static int allow_lds(K kernel, size_t bytes) {
@@ -783,9 +845,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 		return N2_OK;
 	}
 	if (!want_dw && !want_dx) return N2_OK;
-	const uint32_t blocks = stream_grid(n, want_dw ? MLP_MAX_SLABS : 2048);
-	const size_t lds_stage = want_dw ? STAGE_BYTES : 0;
-	const size_t lds = want_dw ? (lds_stage > mlp->n_params * sizeof(float) ? lds_stage : mlp->n_params * sizeof(float)) : 0;
+	const uint32_t blocks = stream_grid(n, want_dw ? 2 : 1);
 	const hf* X = reinterpret_cast<const hf*>(d_input);
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
@@ -793,6 +853,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 #define LAUNCH(IC, NH, DX, DW)                                                                                      \
 	do {                                                                                                            \
+		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT); /* >= the fp32 parameter image laid over it */      \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
 		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, mlp->workspace); \
 	} while (0)
@@ -842,14 +903,13 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 		return N2_OK;
 	}
 	if (!want_dw && !d_dL_ddLdoutput) return N2_OK;
-	const uint32_t blocks = stream_grid(n, MLP_MAX_SLABS);
-	const size_t lds = STAGE_BYTES > mlp->n_params * sizeof(float) ? STAGE_BYTES : mlp->n_params * sizeof(float);
+	const uint32_t blocks = stream_grid(n, 2);
 	N2ProfScope prof(N2_PROF_MLP_SECOND_ORDER, s);
 	switch (mlp->in_w / 16) {
 #define CASE(IC)                                                                                                           \
 	case IC:                                                                                                               \
-		if (int rc = allow_lds(mlp_bbi_kernel<IC>, lds)) return rc;                                                        \
-		mlp_bbi_kernel<IC><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
+		if (int rc = allow_lds(mlp_bbi_kernel<IC>, frag_bytes(FragMap<IC, 1>::COUNT))) return rc;                          \
+		mlp_bbi_kernel<IC><<<dim3(blocks), dim3(MLP_BLOCK), frag_bytes(FragMap<IC, 1>::COUNT), s>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
 			reinterpret_cast<const hf*>(d_dL_ddLdinput), reinterpret_cast<const hf*>(d_dL_doutput), unit_row,              \
 			reinterpret_cast<hf*>(d_dL_ddLdoutput), want_dw ? mlp->workspace : nullptr);                                   \
 		break;
