@@ -171,22 +171,30 @@ __global__ void __launch_bounds__(FB) field_add_density_gradient_kernel(uint32_t
 }
 
 // v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
-// second-order MLP input rows 0..2 = half(v), rows [3 + enc_w, sdf_in_w) = 0; variance gradient written.
+// second-order MLP input rows 0..2 = half(v), rows 3 .. 3+enc_w = dy_dx v (the encoding's
+// backward_backward_input output dL_ddLdoutput, taken from the Jacobian the forward stored instead of
+// gathering the table again), rows [3 + enc_w, sdf_in_w) = 0; variance gradient written.
 __global__ void __launch_bounds__(FB) field_second_order_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, const hf* __restrict__ d_rgb_in,
-                                                                     const hf* __restrict__ dL_dout, float ek_batch, float* __restrict__ v,
-                                                                     hf* __restrict__ d_density_in, const float* __restrict__ var_acc,
-                                                                     hf* __restrict__ var_grad, int accumulate) {
+                                                                     const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
+                                                                     float* __restrict__ v, hf* __restrict__ d_density_in,
+                                                                     const float* __restrict__ var_acc, hf* __restrict__ var_grad, int accumulate) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + var_acc[0]) : (hf)var_acc[0];
 	if (i >= N) return;
 	const hf* g = dL_dout + (size_t)i * 16;
+	float vv[3];
 #pragma unroll
 	for (int d = 0; d < 3; ++d) {
 		float x = (float)d_rgb_in[(size_t)(35 + d) * N + i];
 		x += (float)g[4 + d] / ek_batch;
 		x += (float)g[8 + d];
+		vv[d] = x;
 		v[(size_t)d * N + i] = x;
 		d_density_in[(size_t)d * N + i] = (hf)x;
+	}
+	for (uint32_t r = 0; r < enc_w; ++r) {
+		const float* j = dy_dx + ((size_t)r * N + i) * 3;
+		d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
 	}
 	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
 }
@@ -390,16 +398,14 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
 	                             N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), mode)) return rc;
 	// dL/dnormal and the variance gradient
-	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->v,
+	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
 	                                                             f->d_density_in, f->var_acc, f->grads + f->off_var,
 	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
-	// Overwrite followed by backward_backward_input with Accumulate); the second-order dL_ddLdy lands in
-	// rows 3.. of the MLP's second-order input
+	// Overwrite followed by backward_backward_input with Accumulate)
 	if (int rc = n2_grid_backward_fused(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
-	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n),
-	                                    reinterpret_cast<n2_half*>(f->d_density_in + (size_t)3 * n), mode)) return rc;
+	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n), nullptr, mode)) return rc;
 	// second order through the SDF net
 	return n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
 	                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE);

@@ -399,9 +399,11 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
                                                const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
                                                const __half* __restrict__ dL_dy, const float* __restrict__ v,
                                                const __half* __restrict__ g2, const __half2* __restrict__ params,
-                                               __half* __restrict__ dL_ddLdy, uint32_t* e_out, uint32_t* val_out) {
+                                               __half* __restrict__ dL_ddLdy, uint32_t* e_out, float* r0_out, float* r1_out,
+                                               uint32_t* cell) {
 	const float scale = tab.scale[level];
 	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	cell[0] = p.c[0]; cell[1] = p.c[1]; cell[2] = p.c[2];
 	uint32_t e[8];
 	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
 	const size_t row = (size_t)level * 2;
@@ -440,8 +442,8 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
 			}
 		}
 		e_out[k] = e[k];
-		const __half2 h = __floats2half2_rn(r0, r1);
-		val_out[k] = *reinterpret_cast<const uint32_t*>(&h);
+		r0_out[k] = r0;
+		r1_out[k] = r1;
 	}
 	if (SECOND && WANT_OUT) {
 		dL_ddLdy[row * N + i] = __float2half_rn(o0);
@@ -449,8 +451,16 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
 	}
 }
 
+// Samples arrive in ray order, so on the coarser levels consecutive samples (= consecutive lanes)
+// fall into the same cell and would hit the same eight entries.  When fewer than MERGE_MAX_HEADS
+// runs of equal cells make up a wave, the runs are summed across lanes in fp32 (segmented scan) and
+// only the last lane of a run emits records: fewer records, and no pile-up on a few hot entries in
+// the sort's counters or the reduce's accumulators.
+constexpr uint32_t MERGE_MAX_HEADS = 40;
+constexpr uint32_t REC_SKIP = 0xFFFFFFFFu;
+
 template <bool FIRST, bool SECOND, bool WANT_OUT>
-__global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+__global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
                                                               const float* __restrict__ xyz, uint32_t point_stride,
                                                               uint32_t dim_stride, const __half* __restrict__ dL_dy,
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
@@ -459,25 +469,55 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 	__shared__ uint32_t hist[BKT_MAX];
 	__shared__ uint32_t prefix[BKT_MAX + 1];
 	__shared__ uint2 staging[BIN_RECORDS];
-	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
+	const uint32_t level = first_level + blockIdx.x / tiles, tile = blockIdx.x % tiles;
+	const uint32_t lane = threadIdx.x & 63u;
 	if (threadIdx.x < BKT_MAX) hist[threadIdx.x] = 0;
 	__syncthreads();
-	// records of this thread: entry | rank << 19 after the counting step
+	// records of this thread: entry | rank << 19 after the counting step (REC_SKIP: merged into a later lane)
 	uint32_t re[BIN_PER_THREAD * 8], rv[BIN_PER_THREAD * 8];
-	uint32_t live = 0;
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
 		const uint32_t i = tile * BIN_POINTS + j * GRID_BLOCK + threadIdx.x;
-		if (i < N) {
-			live |= 1u << j;
-#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, re + 8 * j, rv + 8 * j)
+		const bool valid = i < N;
+		uint32_t e[8], cell[3] = {0, 0, 0};
+		float r0[8], r1[8];
+#pragma unroll
+		for (uint32_t k = 0; k < 8; ++k) { e[k] = 0; r0[k] = 0.f; r1[k] = 0.f; }
+		if (valid) {
+#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell)
 			N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
+		}
+		// runs of equal cells among the wave's 64 consecutive points
+		const uint32_t up_x = __shfl_up(cell[0], 1), up_y = __shfl_up(cell[1], 1), up_z = __shfl_up(cell[2], 1);
+		const int up_valid = __shfl_up((int)valid, 1);
+		const bool head = lane == 0 || !valid || !up_valid || cell[0] != up_x || cell[1] != up_y || cell[2] != up_z;
+		const unsigned long long heads = __ballot(head);
+		bool emit = valid;
+		if (__popcll(heads) <= MERGE_MAX_HEADS) {
+			// first lane of this lane's run, and whether the next lane starts a new one
+			const uint32_t start = 63u - (uint32_t)__clzll(heads & (~0ull >> (63u - lane)));
+			emit = valid && (lane == 63u || ((heads >> (lane + 1u)) & 1ull));
 #pragma unroll
-			for (uint32_t k = 0; k < 8; ++k) {
-				const uint32_t rank = atomicAdd(&hist[re[8 * j + k] >> BKT_SHIFT], 1u);
-				re[8 * j + k] |= rank << 19;
+			for (uint32_t d = 1; d < 64; d <<= 1) {
+				const bool take = lane >= start + d;
+#pragma unroll
+				for (uint32_t k = 0; k < 8; ++k) {
+					const float t0 = __shfl_up(r0[k], d), t1 = __shfl_up(r1[k], d);
+					if (take) { r0[k] += t0; r1[k] += t1; }
+				}
 			}
+		}
+#pragma unroll
+		for (uint32_t k = 0; k < 8; ++k) {
+			uint32_t rec = REC_SKIP;
+			if (emit) {
+				const uint32_t rank = atomicAdd(&hist[e[k] >> BKT_SHIFT], 1u);
+				rec = e[k] | (rank << 19);
+			}
+			re[8 * j + k] = rec;
+			const __half2 h = __floats2half2_rn(r0[k], r1[k]);
+			rv[8 * j + k] = *reinterpret_cast<const uint32_t*>(&h);
 		}
 	}
 	__syncthreads();
@@ -495,9 +535,9 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 	__syncthreads();
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
-		if (live & (1u << j)) {
 #pragma unroll
-			for (uint32_t k = 0; k < 8; ++k) {
+		for (uint32_t k = 0; k < 8; ++k) {
+			if (re[8 * j + k] != REC_SKIP) {
 				const uint32_t e = re[8 * j + k] & 0x7FFFFu, rank = re[8 * j + k] >> 19;
 				staging[prefix[e >> BKT_SHIFT] + rank] = make_uint2(e & (BKT_ENTRIES - 1u), rv[8 * j + k]);
 			}
@@ -831,11 +871,12 @@ N2_API int n2_grid_set_workspace(n2_grid_t* grid, void* d_workspace, uint64_t n_
 static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
                            const __half* dL_dy, const float* v, const __half* g2, __half* dL_ddLdy, bool accumulate) {
 	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
+	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
+	const dim3 bd(GRID_BLOCK);
 	uint2* records = reinterpret_cast<uint2*>(grid->ws);
 	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + (uint64_t)L * tiles * BIN_RECORDS * sizeof(uint2));
-	const dim3 gd(tiles * L), bd(GRID_BLOCK);
-	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
-#define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
+	const dim3 gd(tiles * L);
+#define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
                                                                    grid->params, dL_ddLdy, records, offsets)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);

@@ -2,12 +2,16 @@
 // backward_backward_input) behind the n2_mlp_* C ABI.
 //
 // Shape of the problem: 48->64->16 (SDF net) and 48->64->64->16 (colour net) at
-// 2^18 samples are ~8-16 kflop per sample against 128+ bytes per sample of
-// activations, so every kernel here is bound by HBM, not by MFMA.  The design
-// therefore minimises bytes: a wave keeps a 64-sample tile entirely in
-// registers from the first layer to the last (MFMA accumulators are re-packed
-// in place into the next layer's B operand), hidden activations are never
-// written to memory, and the backward passes recompute them from the input.
+// 2^18 samples are ~8-47 kflop per sample against 128+ bytes per sample of
+// activations: far from the MFMA peak, so what matters is bytes, instruction
+// count and occupancy.  A wave keeps a sample tile entirely in registers from
+// the first layer to the last (MFMA accumulators are re-packed in place into
+// the next layer's B operand), hidden activations are never written to memory
+// and the backward passes recompute them from the input.  Weights live in LDS
+// as ready-made MFMA operands (not in registers), and the batch-reduction
+// products of the weight gradients take their operands from a second set of
+// MFMAs with swapped arguments (see hidden_N) instead of a transposition
+// through memory.
 //
 // MFMA tiling (v_mfma_f32_32x32x16_f16, wave64):
 //   A (32 x 16, weights)      lane l holds A[l%32][8*(l/32) + 0..7]
@@ -35,7 +39,6 @@ constexpr int MLP_OUT = 16;
 constexpr int MLP_BLOCK = 256;      // 4 waves
 constexpr int MLP_TILE = 64;        // samples per wave iteration
 constexpr int MLP_MAX_SLABS = 512;  // workgroups of the weight-gradient kernels (two per CU)
-constexpr int STAGE_LD = 72;        // halves per staged row: 64 samples + 8 pad (keeps 16-byte alignment)
 
 struct n2_mlp {
 	uint32_t in_w, n_hidden, n_params;
@@ -119,56 +122,6 @@ __device__ __forceinline__ float16v zero16() {
 // row index inside a 32-row D tile held in register r by lane group g
 __device__ __forceinline__ int drow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 
-// Write both sample tiles of a chained operand set (4 chunks = 64 neurons) to a
-// staging matrix [64][STAGE_LD] so that rows can be re-read along the batch.
-__device__ __forceinline__ void stage_sync() {
-	// staging buffers are private to a wave: order its LDS writes and reads
-	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-	__builtin_amdgcn_wave_barrier();
-	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-__device__ __forceinline__ void stage_store(hf* S, const half8 (&f)[2][4], int n, int g) {
-	stage_sync();
-#pragma unroll
-	for (int c = 0; c < 4; ++c) {
-#pragma unroll
-		for (int e = 0; e < 8; ++e) {
-			const int neuron = 16 * c + 4 * g + (e & 3) + ((e >> 2) << 3);
-			*reinterpret_cast<half2v*>(S + neuron * STAGE_LD + 2 * n) = half2v{f[0][c][e], f[1][c][e]};
-		}
-	}
-}
-// A operand along the batch: row `row` of a staged matrix, samples 16c + 8g + 0..7
-__device__ __forceinline__ half8 stage_frag(const hf* S, int row, int c, int g) {
-	return *reinterpret_cast<const half8*>(S + row * STAGE_LD + 16 * c + 8 * g);
-}
-// B operand along the batch from an SoA global matrix: row `row`, samples b0 + 16c + 8g + 0..7
-__device__ __forceinline__ half8 batch_frag_soa(const hf* __restrict__ M, size_t N, uint32_t b0, int row, int n_rows, int c, int g) {
-	const uint32_t col = b0 + 16 * c + 8 * g;
-	half8 z;
-#pragma unroll
-	for (int e = 0; e < 8; ++e) z[e] = (hf)0;
-	if (row < n_rows && col < N) z = *reinterpret_cast<const half8*>(M + (size_t)row * N + col);
-	return z;
-}
-// the constant matrix e_{unit_row} 1^T restricted to valid samples
-__device__ __forceinline__ half8 batch_frag_unit(size_t N, uint32_t b0, int row, int unit_row, int c, int g) {
-	const uint32_t col = b0 + 16 * c + 8 * g;
-	half8 z;
-#pragma unroll
-	for (int e = 0; e < 8; ++e) z[e] = (row == unit_row && col < N) ? (hf)1 : (hf)0;
-	return z;
-}
-__device__ __forceinline__ half8 batch_frag_aos16(const hf* __restrict__ M, size_t N, uint32_t b0, int row, int c, int g) {
-	half8 z;
-#pragma unroll
-	for (int e = 0; e < 8; ++e) {
-		const uint32_t col = b0 + 16 * c + 8 * g + e;
-		z[e] = (row < MLP_OUT && col < N) ? M[(size_t)col * MLP_OUT + row] : (hf)0;
-	}
-	return z;
-}
-
 // 16-row operand (network output gradient) as B operand of both tiles, K = 16
 __device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N, uint32_t col, int g, bool aos, int unit_row, half8& t0, half8& t1) {
 	if (unit_row >= 0) {
@@ -180,21 +133,6 @@ __device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N
 		t1 = *reinterpret_cast<const half8*>(dY + (size_t)(col + 1) * MLP_OUT + 8 * g);
 	} else {
 		bfrag_soa(dY, (uint32_t)N, 8u * g * (uint32_t)N + col, 0, MLP_OUT, t0, t1);
-	}
-}
-
-// Store rows [0, n_rows) of D tiles (both sample tiles) of a 32*MT-row result to an SoA matrix.
-template <int MT>
-__device__ __forceinline__ void store_soa(hf* __restrict__ M, size_t N, uint32_t col, bool valid, const float16v (&d)[2][MT],
-                                          int g, int n_rows) {
-	if (!valid) return;
-#pragma unroll
-	for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-		for (int r = 0; r < 16; ++r) {
-			const int row = 32 * mt + drow(r, g);
-			if (row < n_rows) *reinterpret_cast<half2v*>(M + (size_t)row * N + col) = half2v{(hf)d[0][mt][r], (hf)d[1][mt][r]};
-		}
 	}
 }
 

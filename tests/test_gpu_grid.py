@@ -221,11 +221,12 @@ def test_backward_fused_equals_first_plus_second_order(setup, n):
     assert none is None and rel_l2(host(d_grads), 2 * ref) < 2e-2
 
 
-@pytest.mark.parametrize("kind", ["uniform", "clustered"])
+@pytest.mark.parametrize("kind", ["uniform", "clustered", "rays"])
 def test_sorted_scatter_path(oracle, kind):
-    """With a scatter workspace, batches of >= 4096 points go through the LDS counting sort (no global atomics,
-    fp32 accumulation): tighter agreement with the fp32 oracle than the atomic path, on uniform points and on
-    points packed into a few cells (the contention case)."""
+    """With a scatter workspace, batches of >= 4096 points go through the run-length kernel (coarsest levels) and the
+    LDS counting sort (the others): fp32 / exact accumulation, tighter agreement with the fp32 oracle than the
+    atomic path, on uniform points, on points packed into a few cells (the contention case) and on points in ray
+    order (consecutive samples share cells on the coarse levels, so runs are merged before they are written)."""
     from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_OVERWRITE, GridEncoding
     og = oracle.Grid(CFG["n_levels"], CFG["log2_hashmap_size"], CFG["base_resolution"], CFG["per_level_scale"])
     gg = GridEncoding(**CFG)
@@ -238,8 +239,16 @@ def test_sorted_scatter_path(oracle, kind):
     assert gg.reserve_scatter_workspace(1 << 15)
     if kind == "uniform":
         xyz = rng.random((3, n), dtype=np.float32)
-    else:
+    elif kind == "clustered":
         xyz = (0.4 + 0.02 * rng.random((3, n))).astype(np.float32)
+    else:
+        per_ray = 97  # not a divisor of the 32-sample runs a lane walks
+        n_rays = (n + per_ray - 1) // per_ray
+        o = 0.3 + 0.4 * rng.random((n_rays, 1, 3))
+        d = rng.standard_normal((n_rays, 1, 3))
+        d /= np.linalg.norm(d, axis=-1, keepdims=True)
+        k = np.arange(per_ray).reshape(1, per_ray, 1) - per_ray // 2
+        xyz = np.clip(o + d * k * (np.sqrt(3.0) / 1024), 0, 1).reshape(-1, 3)[:n].T.astype(np.float32).copy()
     dy = q16(rng.standard_normal((32, n)))
     g2 = q16(rng.standard_normal((32, n)) * 0.1)
     v = (rng.standard_normal((3, n)) * 1e-3).astype(np.float32)
