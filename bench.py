@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the NeuS2 SDF-field hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice] [--no-cpu-baseline]
 
 A step is one full static NeuS2 training step (BASELINE config 4) on a synthetic scene: an analytic sphere of
 radius 0.3, Lambertian-textured, seen by 64 cameras at 512x512 on a sphere of radius 2; rays are marched through a
@@ -168,6 +168,7 @@ def run_grid_workload(args):
     params = ((torch.rand(g.n_params(), device="cuda", generator=gen) * 2 - 1) * 1e-4).half()
     grads = torch.zeros_like(params)
     g.set_params(params, grads)
+    g.reserve_scatter_workspace(TARGET)
     x = torch.rand((3, TARGET), device="cuda", generator=gen)
     dy = torch.randn((32, TARGET), device="cuda", generator=gen).half()
 
@@ -201,12 +202,126 @@ def run_grid_workload(args):
             "kernels": kernels}
 
 
+def run_sdf_workload(args):
+    """BASELINE configs[2]: grid + SDF MLP with the eikonal second-order path on 2^18 uniform points: forward,
+    normals, backward of mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 through the encoding and the MLP weights."""
+    import numpy as np
+    import torch
+    from neus2_amd import capi
+    from neus2_amd.sdf_net import SdfNet
+    lib = capi.lib()
+    net = SdfNet(max_batch=TARGET)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    P = ((torch.rand(net.grid.n_params(), device="cuda", generator=gen) * 2 - 1) * 1e-4).half()
+    W = torch.from_numpy(np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy"))).cuda().half()
+    gP, gW = torch.zeros_like(P), torch.zeros_like(W)
+    net.set_params(P, gP, W, gW)
+    x = torch.rand((3, TARGET), device="cuda", generator=gen)
+    loss = None
+
+    def step():
+        nonlocal loss
+        loss = net.loss_backward(net.forward(x))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.n2_profile_reset()
+    lib.n2_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.n2_profile_enable(0)
+    kernels, total = {}, 0.0
+    for name in PROF:
+        ms, n = profile_read(lib, name)
+        if n:
+            kernels[name] = {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_us": ms / n * 1e3}
+            total += ms / args.steps
+    sc = kernels["grid_backward_params"]["avg_us"] * 1e-6
+    achieved = ALGO_BYTES["grid_second_order"] * TARGET / sc / 1e9
+    return {"metric": "SDF net + eikonal fwd/bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "hash grid + SDF MLP 48-64-16, forward, normals, first and second order backward of "
+                                   "mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 (BASELINE configs[2]); 2^18 uniform points; element-wise "
+                                   "glue between the kernels runs in torch and is inside the wall clock",
+                       "batch": TARGET, "loss": float(loss), "kernel_ms_per_step": total},
+            "roofline": {"kernel": "grid_backward_params (merged first+second order scatter)", "bound": "hbm", "achieved": achieved,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                         "algorithmic_bytes_per_sample": ALGO_BYTES["grid_second_order"], "samples_per_launch": TARGET,
+                         "avg_launch_us": kernels["grid_backward_params"]["avg_us"]},
+            "kernels": kernels}
+
+
+def run_lattice_workload(args):
+    """BASELINE configs[4]: SDF inference for mesh extraction (hash grid + SDF MLP forward, fp16) over the 512^3
+    lattice p = (i, j, k) / 512, in chunks of 2^22 points; a step is one chunk, chunks are visited in order."""
+    import numpy as np
+    import torch
+    from neus2_amd import capi
+    from neus2_amd.tcnn_api import NerfNetwork
+    from neus2_amd.training import initial_parameters
+    lib = capi.lib()
+    CH, RES = 1 << 22, 512
+    net = NerfNetwork()
+    offs = net.param_offsets()
+    p = initial_parameters(offs, 48, seed=1, sdf_mlp_weights=np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy")))
+    params = torch.from_numpy(p).cuda().half()
+    net.set_params(params, None)
+    net.reserve(CH)
+    n_chunks = RES ** 3 // CH
+    use = min(n_chunks, max(args.steps, 1) + args.warmup)
+    # lattice coordinates of the chunks that will be visited, x fastest (generated once, resident in HBM)
+    idx = torch.arange(use * CH, device="cuda", dtype=torch.int64)
+    xyz = torch.stack(((idx % RES).float() / RES, ((idx // RES) % RES).float() / RES, (idx // (RES * RES)).float() / RES))
+    xyz = xyz.view(3, use, CH).permute(1, 0, 2).contiguous()  # [chunk][3][CH]
+    del idx
+
+    def chunk(k):
+        k %= use
+        return net.sdf(xyz[k])
+
+    for k in range(args.warmup):
+        out = chunk(k)
+    torch.cuda.synchronize()
+    lib.n2_profile_reset()
+    lib.n2_profile_enable(1)
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        out = chunk(args.warmup + k)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.n2_profile_enable(0)
+    kernels = {}
+    for name in ("grid_forward", "mlp_forward"):
+        ms, n = profile_read(lib, name)
+        kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
+    gf = kernels["grid_forward"]["avg_us"] * 1e-6
+    achieved = (12 + 128 * 4 + 64) * CH / gf / 1e9
+    mlp_tflops = 8192 * CH / (kernels["mlp_forward"]["avg_us"] * 1e-6) / 1e12
+    return {"metric": "SDF inference points/sec over a 512^3 lattice in 2^22-point chunks (1 GPU)", "value": args.steps * CH / elapsed,
+            "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "hash grid + SDF MLP forward over the 512^3 lattice (BASELINE configs[4]), geometric-init SDF MLP, "
+                                   "grid U(-1e-4, 1e-4) seed 1", "chunk": CH, "chunks_in_lattice": n_chunks,
+                       "sdf_mean_abs": float(out[0].float().abs().mean())},
+            "roofline": {"kernel": "grid_forward", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": 588,
+                         "samples_per_launch": CH, "avg_launch_us": kernels["grid_forward"]["avg_us"]},
+            "mfma": {"kernel": "mlp_forward (SDF net 48-64-16)", "flops_per_sample": 8192, "achieved_tflops": mlp_tflops,
+                     "peak_tflops": MFMA_PEAK_TFLOPS, "frac": mlp_tflops / MFMA_PEAK_TFLOPS},
+            "kernels": kernels}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=["step", "grid"], default="step")
+    ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
@@ -217,7 +332,7 @@ def main():
     import torch
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (there is no CPU fallback of the product path)")
-    result = run_step_workload(args) if args.workload == "step" else run_grid_workload(args)
+    result = {"step": run_step_workload, "grid": run_grid_workload, "sdf": run_sdf_workload, "lattice": run_lattice_workload}[args.workload](args)
     print(json.dumps(result))
 
 

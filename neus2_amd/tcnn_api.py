@@ -91,10 +91,14 @@ class GridEncoding:
               "n2_grid_set_workspace")
         return True
 
-    def forward(self, xyz, prepare_input_gradients=False):
-        """Returns (out fp16 [width, N], ctx) where ctx holds dy_dx when requested."""
+    def forward(self, xyz, prepare_input_gradients=False, out=None):
+        """Returns (out fp16 [width, N], ctx) where ctx holds dy_dx when requested; ``out`` may be a [width, N]
+        row block of a wider matrix (the encoding rows of the network input, nerf_network.h:184-190)."""
         x, ps, ds, n = _positions(xyz)
-        out = torch.empty((self.output_width(), n), dtype=torch.float16, device=x.device)
+        if out is None:
+            out = torch.empty((self.output_width(), n), dtype=torch.float16, device=x.device)
+        else:
+            _check_half(out, (self.output_width(), n), "grid output")
         dy_dx = torch.empty((self.output_width(), n, 3), dtype=torch.float32, device=x.device) \
             if prepare_input_gradients else None
         check(capi.lib().n2_grid_forward(self._h, _stream(), ptr(x), C.c_uint32(ps), C.c_uint32(ds), C.c_uint32(n),
@@ -220,11 +224,22 @@ class FullyFusedMLP:
                                          ptr(dx), C.c_int(mode)), "n2_mlp_backward")
         return dx
 
+    def input_gradient(self, x, dim=0):
+        """d output[dim] / d input for every sample (Network::input_gradient, nerf_network.h:229): fp16 [in_width, N]."""
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        d = torch.empty((self.input_width(), n), dtype=torch.float16, device=x.device)
+        check(capi.lib().n2_mlp_input_gradient(self._h, _stream(), C.c_uint32(dim), ptr(x), C.c_uint32(n), ptr(d)),
+              "n2_mlp_input_gradient")
+        return d
+
     def backward_backward_input(self, x, dL_ddLdinput, dL_doutput, want_dL_ddLdoutput=False, mode=GRAD_ACCUMULATE):
+        """dL_doutput None: the first-order output gradient was e_0 for every sample (the SDF's own gradient)."""
         n = x.shape[1]
         _check_half(x, (self.input_width(), n), "mlp input")
         _check_half(dL_ddLdinput, (self.input_width(), n), "dL_ddLdinput")
-        _check_half(dL_doutput, (16, n), "dL_doutput")
+        if dL_doutput is not None:
+            _check_half(dL_doutput, (16, n), "dL_doutput")
         o = torch.empty((16, n), dtype=torch.float16, device=x.device) if want_dL_ddLdoutput else None
         check(capi.lib().n2_mlp_backward_backward_input(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(dL_ddLdinput),
                                                         ptr(dL_doutput), ptr(o), C.c_int(mode)),
