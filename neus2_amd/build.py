@@ -63,5 +63,25 @@ def build_library(force=False, verbose=False):
     return LIB
 
 
+SHIM_SRC = os.path.join(ROOT, "tests", "cpp", "shim_check.cpp")
+SHIM_BIN = os.path.join(ROOT, "tests", "cpp", "shim_check")
+
+
+def build_shim_check(force=False):
+    """The C++ program that drives the library through include/neus2_amd.hpp (host compiler only: the shim and the
+    C ABI carry no device code)."""
+    deps = [SHIM_SRC, LIB] + glob.glob(os.path.join(ROOT, "include", "*.h*"))
+    if not force and not _newer(deps, SHIM_BIN):
+        return SHIM_BIN
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
+           "-I", "/opt/rocm/include", SHIM_SRC, "-o", SHIM_BIN, "-L", PKG, "-lneus2_amd", "-L", "/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../neus2_amd", "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("shim_check build failed:\n" + r.stderr)
+    return SHIM_BIN
+
+
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv, verbose=True))
+    print(build_shim_check(force="--force" in sys.argv))

@@ -63,3 +63,15 @@ def test_level_table_matches_oracle(oracle):
         assert np.array_equal(sc, g.scale) and np.array_equal(res, g.resolution)
         assert np.array_equal(ent, g.entries) and np.array_equal(off, g.offset)
         L.n2_grid_destroy(h)
+
+
+def test_cpp_shim_host_checks():
+    """The header-only C++ shim (tcnn method names over the C ABI) compiles with the host compiler and its
+    host-only behaviour holds: shapes, parameter counts, matrix views, errors as std::runtime_error."""
+    import subprocess
+    from neus2_amd.build import build_library, build_shim_check
+    build_library()
+    exe = build_shim_check()
+    r = subprocess.run([exe, "host"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    assert "shim host checks ok" in r.stdout
