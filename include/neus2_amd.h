@@ -75,6 +75,12 @@ uint32_t n2_grid_n_levels(const n2_grid_t* grid);
 int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolution, uint32_t* entries,
                         uint32_t* offset);
 
+/* Tuning knob without a counterpart in the reference: the relative cost of one tile of points on each level
+ * (n_levels values > 0).  The gather kernels split the levels over the GPU's 8 XCDs in proportion to it so
+ * that each XCD's L2 holds only the tables of its own levels.  Defaults: 1 for hashed levels, 0.6 for dense ones.
+ * Results do not depend on it. */
+int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs);
+
 /* Encoding::set_params(params, inference_params, backward_params, gradients),
  * nerf_network.h:746-753.  One fp16 parameter buffer (n_params) and one fp16
  * gradient buffer (n_params, may be NULL until a backward needs it). */

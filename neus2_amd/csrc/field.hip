@@ -28,6 +28,7 @@ struct n2_field {
 	uint32_t max_batch, max_batch_bwd;
 	// carved from the workspace
 	hf* sdf_in;        // [sdf_in_w][N]
+	float* xyz;        // [3][N]  positions of the last forward, row per coordinate (the grid kernels read each row 16 times)
 	hf* rgb_in;        // [48][N]
 	float* dy_dx;      // [enc_w][N][3]
 	hf* dsdf_din;      // [sdf_in_w][N]  d sdf / d (SDF net input)
@@ -51,12 +52,17 @@ constexpr uint32_t FB = 256;
 // rows 0..2 = half(x) - half(0.5) (computed in half precision like the reference's
 // (T)pos - (T)0.5f), rows [3 + enc_w, sdf_in_w) = 0.
 __global__ void __launch_bounds__(FB) field_pack_sdf_input_kernel(const float* __restrict__ xyz, uint32_t ps, uint32_t ds, uint32_t N,
-                                                                  hf* __restrict__ sdf_in, uint32_t enc_w, uint32_t sdf_in_w) {
+                                                                  hf* __restrict__ sdf_in, uint32_t enc_w, uint32_t sdf_in_w,
+                                                                  float* __restrict__ xyz_rows) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
 	const float* q = xyz + (size_t)i * ps;
 #pragma unroll
-	for (int d = 0; d < 3; ++d) sdf_in[(size_t)d * N + i] = (hf)q[(size_t)d * ds] - (hf)0.5f;
+	for (int d = 0; d < 3; ++d) {
+		const float x = q[(size_t)d * ds];
+		sdf_in[(size_t)d * N + i] = (hf)x - (hf)0.5f;
+		xyz_rows[(size_t)d * N + i] = x;
+	}
 	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) sdf_in[(size_t)r * N + i] = (hf)0;
 }
 
@@ -278,7 +284,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -288,6 +294,7 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	uint64_t n = nf;
 	auto take = [&](uint64_t bytes) { const uint64_t at = o; o = align256(o + bytes); return at; };
 	c.sdf_in = take(2ull * f->sdf_in_w * n);
+	c.xyz = take(12ull * n);
 	c.rgb_in = take(2ull * f->rgb_in_w * n);
 	c.dy_dx = take(12ull * f->enc_w * n);
 	c.dsdf_din = take(2ull * f->sdf_in_w * n);
@@ -322,6 +329,7 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	unsigned char* b = reinterpret_cast<unsigned char*>(d_workspace);
 	f->ws = b; f->ws_bytes = n_bytes; f->max_batch = max_batch; f->max_batch_bwd = max_batch_backward;
 	f->sdf_in = reinterpret_cast<hf*>(b + c.sdf_in);
+	f->xyz = reinterpret_cast<float*>(b + c.xyz);
 	f->rgb_in = reinterpret_cast<hf*>(b + c.rgb_in);
 	f->dy_dx = reinterpret_cast<float*>(b + c.dy_dx);
 	f->dsdf_din = reinterpret_cast<hf*>(b + c.dsdf_din);
@@ -358,9 +366,9 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	N2_REQUIRE(d_coords != nullptr && d_output != nullptr, "n2_field_forward: null buffer");
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "n2_field_forward: d_output must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
-	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w);
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
 	N2_LAUNCH_CHECK();
-	if (int rc = n2_grid_forward(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
+	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
 	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<n2_half*>(f->rgb_in),
 	                            N2_LAYOUT_SOA, nullptr)) return rc;
 	if (int rc = n2_mlp_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
@@ -404,7 +412,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_LAUNCH_CHECK();
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)
-	if (int rc = n2_grid_backward_fused(f->grid, stream, d_coords, 7, 1, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
+	if (int rc = n2_grid_backward_fused(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
 	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n), nullptr, mode)) return rc;
 	// second order through the SDF net
 	return n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
@@ -419,9 +427,9 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	N2_REQUIRE(ps >= 1 && ds >= 1, "%s: strides must be >= 1", fn);
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "%s: d_output must be 16-byte aligned", fn);
 	hipStream_t s = n2_stream(stream);
-	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->enc_w, f->sdf_in_w);
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
 	N2_LAUNCH_CHECK();
-	if (int rc = n2_grid_forward(f->grid, stream, d_xyz, ps, ds, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), nullptr)) return rc;
+	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), nullptr)) return rc;
 	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, d_output, N2_LAYOUT_SOA, nullptr)) return rc;
 	field_add_bias_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, (hf)f->sdf_bias, reinterpret_cast<hf*>(d_output));
 	N2_LAUNCH_CHECK();

@@ -3,11 +3,14 @@
 // backward_backward_input, behind the n2_grid_* C ABI.
 //
 // Work decomposition: one workgroup handles a tile of points for ONE level.
-// Workgroup ids are level-major (all tiles of level 0, then level 1, ...).
-// The hardware deals consecutive workgroup ids round-robin over the 8 XCDs,
-// so at any moment every XCD works on the same level and its private 4 MiB
-// L2 only has to hold that level's table (<= 2 MiB at T = 2^19) while the
-// points stream through.
+// The gather kernels number their (level, tile) work items level-major and cut
+// that list into 8 contiguous pieces of equal estimated cost, one per XCD: the
+// hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so
+// workgroup id b runs on XCD b % 8 and takes item number b / 8 of that XCD's
+// piece.  Each XCD then streams all points through about two levels, and its
+// private 4 MiB L2 fetches only those levels' tables (<= 2 MiB each at
+// T = 2^19) instead of all 24 MiB.  (With plain level-major ids every XCD
+// walks every level and the table crosses the fabric 8 times per launch.)
 #include "n2_common.h"
 
 #include <cmath>
@@ -19,6 +22,8 @@ struct n2_grid {
 	uint32_t n_params;
 	const __half2* params;
 	__half2* grads;
+	// relative cost of one tile of each level (balances the levels over the XCDs)
+	float level_cost[N2_MAX_LEVELS];
 	// optional scratch of the bucketed scatter
 	unsigned char* ws;
 	uint64_t ws_bytes;
@@ -95,68 +100,83 @@ __device__ __forceinline__ float n2_corner_weight(const N2Point& p, uint32_t k) 
 	}
 
 constexpr uint32_t GRID_BLOCK = 256;
+constexpr uint32_t N_XCD = 8;  // gfx950: 8 XCDs, workgroup ids are dealt round-robin
+
+// Piece x of the level-major item list [begin[x], begin[x + 1]) belongs to XCD x.
+struct N2XcdPlan {
+	uint32_t begin[N_XCD + 1];
+};
+
+// The (level, tile) item of this workgroup, or false if its XCD's piece is shorter than the longest one.
+__device__ __forceinline__ bool n2_xcd_item(const N2XcdPlan& plan, uint32_t tiles, uint32_t& level, uint32_t& tile) {
+	const uint32_t xcd = blockIdx.x % N_XCD, item = plan.begin[xcd] + blockIdx.x / N_XCD;
+	if (item >= plan.begin[xcd + 1]) return false;
+	level = item / tiles;
+	tile = item - level * tiles;
+	return true;
+}
 
 // ----------------------------------------------------------------------------
 // forward
 // ----------------------------------------------------------------------------
+// A point is handled by a PAIR of adjacent lanes: lane bit 0 selects the x corner, each lane gathers the four
+// (y, z) corners of its x.  The two x corners are neighbours in the table (dense levels: index + 1; hashed
+// levels: x enters the hash with prime 1), so the two lanes of a pair read the same cache line almost always and
+// the memory pipeline, which looks up one line per clock, sees half as many lines per point.  The pair then
+// exchanges its partial sums and lane b finishes feature b.
+constexpr uint32_t FWD_POINTS = GRID_BLOCK / 2;  // points per workgroup and level
+
 template <uint32_t MODE, bool WANT_DYDX>
-__device__ __forceinline__ void grid_forward_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
-                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
-                                                   const __half2* __restrict__ params, __half* __restrict__ out,
-                                                   float* __restrict__ dy_dx) {
+__device__ __forceinline__ void grid_forward_pair(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t b, uint32_t N,
+                                                  const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                  const __half2* __restrict__ params, __half* __restrict__ out,
+                                                  float* __restrict__ dy_dx) {
 	const float scale = tab.scale[level];
 	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
 	const __half2* P = params + tab.offset[level];
 	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
-	uint32_t e[8];
-	n2_corner_entries<MODE>(p, entries, res, e);
-	float2 v[8];
+	const uint32_t gx = p.c[0] + b;
+	float2 v[4];
 #pragma unroll
-	for (uint32_t k = 0; k < 8; ++k) v[k] = __half22float2(P[e[k]]);
-	float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-	for (uint32_t k = 0; k < 8; ++k) {
-		const float wt = n2_corner_weight(p, k);
-		a0 = fmaf(wt, v[k].x, a0);
-		a1 = fmaf(wt, v[k].y, a1);
-	}
-	const size_t row = (size_t)level * 2;
-	out[row * N + i] = __float2half_rn(a0);
-	out[(row + 1) * N + i] = __float2half_rn(a1);
+	for (uint32_t k = 0; k < 4; ++k) v[k] = __half22float2(P[n2_entry<MODE>(entries, res, gx, p.c[1] + (k & 1u), p.c[2] + (k >> 1))]);
+	const float wy = p.w[1], wz = p.w[2], uy = 1.f - wy, uz = 1.f - wz;
+	// this lane's x plane: bilinear value s, and its y and z differences ty, tz (k = y + 2 z)
+	float2 s, ty, tz;
+	s.x = fmaf(uy * uz, v[0].x, fmaf(wy * uz, v[1].x, fmaf(uy * wz, v[2].x, wy * wz * v[3].x)));
+	s.y = fmaf(uy * uz, v[0].y, fmaf(wy * uz, v[1].y, fmaf(uy * wz, v[2].y, wy * wz * v[3].y)));
 	if (WANT_DYDX) {
-		float g0[3], g1[3];
-#pragma unroll
-		for (int gd = 0; gd < 3; ++gd) {
-			const int d1 = (gd + 1) % 3, d2 = (gd + 2) % 3;
-			float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-			for (uint32_t k = 0; k < 8; ++k) {
-				if ((k >> gd) & 1u) continue;
-				float wt = ((k >> d1) & 1u) ? p.w[d1] : 1.f - p.w[d1];
-				wt *= ((k >> d2) & 1u) ? p.w[d2] : 1.f - p.w[d2];
-				const uint32_t kr = k | (1u << gd);
-				s0 = fmaf(wt, v[kr].x - v[k].x, s0);
-				s1 = fmaf(wt, v[kr].y - v[k].y, s1);
-			}
-			g0[gd] = s0 * scale;
-			g1[gd] = s1 * scale;
-		}
-		float* j0 = dy_dx + (row * N + i) * 3;
-		float* j1 = dy_dx + ((row + 1) * N + i) * 3;
-		j0[0] = g0[0]; j0[1] = g0[1]; j0[2] = g0[2];
-		j1[0] = g1[0]; j1[1] = g1[1]; j1[2] = g1[2];
+		ty.x = fmaf(uz, v[1].x - v[0].x, wz * (v[3].x - v[2].x));
+		ty.y = fmaf(uz, v[1].y - v[0].y, wz * (v[3].y - v[2].y));
+		tz.x = fmaf(uy, v[2].x - v[0].x, wy * (v[3].x - v[1].x));
+		tz.y = fmaf(uy, v[2].y - v[0].y, wy * (v[3].y - v[1].y));
+	}
+	// lane b keeps feature b of its own plane and receives feature b of the partner's plane
+	const float s_mine = b ? s.y : s.x, s_other = __shfl_xor(b ? s.x : s.y, 1);
+	const float s_lo = b ? s_other : s_mine, s_hi = b ? s_mine : s_other;  // x corner 0 / 1
+	const float wx = p.w[0], ux = 1.f - wx;
+	const size_t row = (size_t)level * 2 + b;
+	out[row * N + i] = __float2half_rn(fmaf(ux, s_lo, wx * s_hi));
+	if (WANT_DYDX) {
+		const float ty_mine = b ? ty.y : ty.x, ty_other = __shfl_xor(b ? ty.x : ty.y, 1);
+		const float tz_mine = b ? tz.y : tz.x, tz_other = __shfl_xor(b ? tz.x : tz.y, 1);
+		const float w_mine = b ? wx : ux, w_other = b ? ux : wx;
+		float* j = dy_dx + (row * N + i) * 3;
+		j[0] = (s_hi - s_lo) * scale;
+		j[1] = fmaf(w_mine, ty_mine, w_other * ty_other) * scale;
+		j[2] = fmaf(w_mine, tz_mine, w_other * tz_other) * scale;
 	}
 }
 
 template <bool WANT_DYDX>
-__global__ void __launch_bounds__(GRID_BLOCK) grid_forward_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+__global__ void __launch_bounds__(GRID_BLOCK) grid_forward_kernel(N2LevelTable tab, N2XcdPlan plan, uint32_t N, uint32_t tiles,
                                                                   const float* __restrict__ xyz, uint32_t point_stride,
                                                                   uint32_t dim_stride, const __half2* __restrict__ params,
                                                                   __half* __restrict__ out, float* __restrict__ dy_dx) {
-	const uint32_t level = blockIdx.x / tiles;
-	const uint32_t i = (blockIdx.x - level * tiles) * GRID_BLOCK + threadIdx.x;
-	if (i >= N) return;
-#define CALL(M) grid_forward_point<M, WANT_DYDX>(tab, level, i, N, xyz, point_stride, dim_stride, params, out, dy_dx)
+	uint32_t level, tile;
+	if (!n2_xcd_item(plan, tiles, level, tile)) return;
+	const uint32_t i = tile * FWD_POINTS + (threadIdx.x >> 1), b = threadIdx.x & 1u;
+	if (i >= N) return;  // both lanes of a pair share i, so pairs leave together
+#define CALL(M) grid_forward_pair<M, WANT_DYDX>(tab, level, i, b, N, xyz, point_stride, dim_stride, params, out, dy_dx)
 	N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
 }
@@ -452,11 +472,20 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
 }
 
 // Samples arrive in ray order, so on the coarser levels consecutive samples (= consecutive lanes)
-// fall into the same cell and would hit the same eight entries.  When fewer than MERGE_MAX_HEADS
-// runs of equal cells make up a wave, the runs are summed across lanes in fp32 (segmented scan) and
-// only the last lane of a run emits records: fewer records, and no pile-up on a few hot entries in
-// the sort's counters or the reduce's accumulators.
+// fall into the same cell and would hit the same eight entries.  When runs of equal cells are long
+// enough (at most MERGE_MAX_HEADS runs in a wave), they are summed across lanes in fp32 and only the
+// last lane of a run emits records: fewer records, and no pile-up on a few hot entries in the sort's
+// counters or the reduce's accumulators.  The sums are segmented scans inside rows of 16 lanes, which
+// the data-parallel-primitive lane shifts do at full ALU rate without touching LDS; a run that
+// crosses a row boundary simply emits one record per row.
 constexpr uint32_t MERGE_MAX_HEADS = 40;
+constexpr unsigned long long ROW_HEADS = 0x0001000100010001ull;  // first lane of each 16-lane row
+
+// value of the lane D places below in the same 16-lane row (0 if that leaves the row)
+template <int D>
+__device__ __forceinline__ float n2_row_shr(float x) {
+	return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x110 + D, 0xf, 0xf, false));
+}
 constexpr uint32_t REC_SKIP = 0xFFFFFFFFu;
 
 template <bool FIRST, bool SECOND, bool WANT_OUT>
@@ -492,21 +521,24 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 		const uint32_t up_x = __shfl_up(cell[0], 1), up_y = __shfl_up(cell[1], 1), up_z = __shfl_up(cell[2], 1);
 		const int up_valid = __shfl_up((int)valid, 1);
 		const bool head = lane == 0 || !valid || !up_valid || cell[0] != up_x || cell[1] != up_y || cell[2] != up_z;
-		const unsigned long long heads = __ballot(head);
+		const unsigned long long heads = __ballot(head) | ROW_HEADS;
 		bool emit = valid;
 		if (__popcll(heads) <= MERGE_MAX_HEADS) {
-			// first lane of this lane's run, and whether the next lane starts a new one
+			// first lane of this lane's run (same row), and whether the next lane starts a new one
 			const uint32_t start = 63u - (uint32_t)__clzll(heads & (~0ull >> (63u - lane)));
 			emit = valid && (lane == 63u || ((heads >> (lane + 1u)) & 1ull));
-#pragma unroll
-			for (uint32_t d = 1; d < 64; d <<= 1) {
-				const bool take = lane >= start + d;
-#pragma unroll
-				for (uint32_t k = 0; k < 8; ++k) {
-					const float t0 = __shfl_up(r0[k], d), t1 = __shfl_up(r1[k], d);
-					if (take) { r0[k] += t0; r1[k] += t1; }
-				}
+			const uint32_t depth = lane - start;  // lanes of the run below this one
+#define N2_SCAN_STEP(D)                                               \
+			{                                                         \
+				const bool take = depth >= D;                         \
+				_Pragma("unroll") for (uint32_t k = 0; k < 8; ++k) {  \
+					const float t0 = n2_row_shr<D>(r0[k]), t1 = n2_row_shr<D>(r1[k]); \
+					r0[k] += take ? t0 : 0.f;                         \
+					r1[k] += take ? t1 : 0.f;                         \
+				}                                                     \
 			}
+			N2_SCAN_STEP(1) N2_SCAN_STEP(2) N2_SCAN_STEP(4) N2_SCAN_STEP(8)
+#undef N2_SCAN_STEP
 		}
 #pragma unroll
 		for (uint32_t k = 0; k < 8; ++k) {
@@ -734,6 +766,8 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 		g->tab.entries[l] = n;
 		g->tab.offset[l] = (uint32_t)off;
 		g->tab.mode[l] = level_mode(res, n);
+		// hashed levels gather from all over their table; the dense ones mostly hit lines their neighbours fetched
+		g->level_cost[l] = (g->tab.mode[l] == N2_LEVEL_HASH || g->tab.mode[l] == N2_LEVEL_HASH_MOD) ? 1.0f : 0.6f;
 		off += n;
 	}
 	if (off * n_features_per_level > 0x7FFFFFFFull) {
@@ -769,6 +803,15 @@ N2_API int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* re
 	return N2_OK;
 }
 
+N2_API int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs) {
+	N2_REQUIRE(grid != nullptr && costs != nullptr, "n2_grid_set_level_costs: null argument");
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
+		N2_REQUIRE(costs[l] > 0.f && costs[l] <= 1e6f, "n2_grid_set_level_costs: cost of level %u must be in (0, 1e6]", l);
+	}
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) grid->level_cost[l] = costs[l];
+	return N2_OK;
+}
+
 N2_API int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients) {
 	N2_REQUIRE(grid != nullptr, "n2_grid_set_params: grid is null");
 	N2_REQUIRE(d_params != nullptr, "n2_grid_set_params: d_params is null");
@@ -793,19 +836,50 @@ static int check_batch(const n2_grid_t* grid, const char* fn, const float* d_xyz
 
 static inline uint32_t n_tiles(uint32_t n_points) { return (n_points + GRID_BLOCK - 1) / GRID_BLOCK; }
 
+// Cuts the level-major list of n_levels x tiles items into N_XCD contiguous pieces of equal estimated cost.
+// Returns the length of the longest piece (the launch needs N_XCD times that many workgroups).
+static uint32_t make_xcd_plan(const n2_grid_t* grid, uint32_t tiles, N2XcdPlan& plan) {
+	const uint32_t L = grid->tab.n_levels;
+	double total = 0.0;
+	for (uint32_t l = 0; l < L; ++l) total += (double)grid->level_cost[l] * tiles;
+	plan.begin[0] = 0;
+	uint32_t level = 0, longest = 0;
+	double before = 0.0;  // cost of the levels below `level`
+	for (uint32_t x = 1; x < N_XCD; ++x) {
+		const double target = total * x / N_XCD;
+		while (level + 1 < L && before + (double)grid->level_cost[level] * tiles <= target) {
+			before += (double)grid->level_cost[level] * tiles;
+			++level;
+		}
+		double in_level = (target - before) / grid->level_cost[level];
+		if (in_level < 0.0) in_level = 0.0;
+		if (in_level > tiles) in_level = tiles;
+		uint32_t b = level * tiles + (uint32_t)(in_level + 0.5);
+		if (b < plan.begin[x - 1]) b = plan.begin[x - 1];
+		plan.begin[x] = b;
+	}
+	plan.begin[N_XCD] = L * tiles;
+	for (uint32_t x = 0; x < N_XCD; ++x) {
+		const uint32_t len = plan.begin[x + 1] - plan.begin[x];
+		if (len > longest) longest = len;
+	}
+	return longest;
+}
+
 N2_API int n2_grid_forward(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz, uint32_t point_stride,
                            uint32_t dim_stride, uint32_t n_points, n2_half* d_out, float* d_dy_dx) {
 	if (int rc = check_batch(grid, "n2_grid_forward", d_xyz, point_stride, dim_stride, n_points)) return rc;
 	if (n_points == 0) return N2_OK;
 	N2_REQUIRE(d_out != nullptr, "n2_grid_forward: d_out is null");
-	const uint32_t tiles = n_tiles(n_points);
-	const dim3 grid_dim(tiles * grid->tab.n_levels), block(GRID_BLOCK);
+	const uint32_t tiles = (n_points + FWD_POINTS - 1) / FWD_POINTS;
+	N2XcdPlan plan;
+	const dim3 grid_dim(make_xcd_plan(grid, tiles, plan) * N_XCD), block(GRID_BLOCK);
 	N2ProfScope prof(N2_PROF_GRID_FORWARD, n2_stream(stream));
 	if (d_dy_dx) {
-		grid_forward_kernel<true><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride,
+		grid_forward_kernel<true><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, plan, n_points, tiles, d_xyz, point_stride,
 			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), d_dy_dx);
 	} else {
-		grid_forward_kernel<false><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride,
+		grid_forward_kernel<false><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, plan, n_points, tiles, d_xyz, point_stride,
 			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), nullptr);
 	}
 	N2_LAUNCH_CHECK();
