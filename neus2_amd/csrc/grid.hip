@@ -406,7 +406,8 @@ constexpr uint32_t BKT_SHIFT = 13;
 constexpr uint32_t BKT_MAX = 64;         // buckets per level (entries <= 2^19)
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
 constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
-constexpr uint32_t BIN_PER_THREAD = BIN_POINTS / GRID_BLOCK;  // 4
+constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: two workgroups (2 x 64 KiB staging) keep 4 waves on every SIMD
+constexpr uint32_t BIN_PER_THREAD = BIN_POINTS / BIN_BLOCK;  // 2
 
 struct N2BucketPlan {
 	uint32_t wg_begin[N2_MAX_LEVELS + 1];  // first reduce workgroup of each level
@@ -489,7 +490,7 @@ __device__ __forceinline__ float n2_row_shr(float x) {
 constexpr uint32_t REC_SKIP = 0xFFFFFFFFu;
 
 template <bool FIRST, bool SECOND, bool WANT_OUT>
-__global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
+__global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
                                                               const float* __restrict__ xyz, uint32_t point_stride,
                                                               uint32_t dim_stride, const __half* __restrict__ dL_dy,
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
@@ -506,7 +507,7 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 	uint32_t re[BIN_PER_THREAD * 8], rv[BIN_PER_THREAD * 8];
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
-		const uint32_t i = tile * BIN_POINTS + j * GRID_BLOCK + threadIdx.x;
+		const uint32_t i = tile * BIN_POINTS + j * BIN_BLOCK + threadIdx.x;
 		const bool valid = i < N;
 		uint32_t e[8], cell[3] = {0, 0, 0};
 		float r0[8], r1[8];
@@ -578,7 +579,7 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bin_kernel(N2LevelTable tab, 
 	__syncthreads();
 	const uint32_t total = prefix[64];
 	uint2* out = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
-	for (uint32_t t = threadIdx.x; t < total; t += GRID_BLOCK) out[t] = staging[t];
+	for (uint32_t t = threadIdx.x; t < total; t += BIN_BLOCK) out[t] = staging[t];
 	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
 }
 
@@ -946,7 +947,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
                            const __half* dL_dy, const float* v, const __half* g2, __half* dL_ddLdy, bool accumulate) {
 	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
-	const dim3 bd(GRID_BLOCK);
+	const dim3 bd(BIN_BLOCK);
 	uint2* records = reinterpret_cast<uint2*>(grid->ws);
 	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + (uint64_t)L * tiles * BIN_RECORDS * sizeof(uint2));
 	const dim3 gd(tiles * L);
