@@ -32,6 +32,10 @@ STEP_ALGO_BYTES = {"grid_backward_params": 664, "grid_forward": 588}
 # recomputed forward 2 x (48x64 + 64x64) + data backward 2 x (16x64 + 64x64 + 64x48) + weight gradients 2 x (48x64 + 64x64 + 64x16)
 COLOUR_BACKWARD_FLOPS = 14336 + 16384 + 16384
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
+# HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
+# (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
+# scatter pair = bin (49.9 + 158.2 MiB) + reduce (181.0 + 24.3 MiB); forward = 80.7 + 112.1 MiB
+STEP_TRAFFIC_BYTES = {"grid_backward_params": int(413.4 * 2**20), "grid_forward": int(192.8 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8}
 
@@ -147,7 +151,8 @@ def run_step_workload(args):
                    "target_batch": TARGET, "rays_per_step": n_rays, "marched_samples_per_step": counters["samples"],
                    "inference_batch": n_inf, "compacted_before_rollover": counters["compacted"], "loss": counters["loss"]},
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": STEP_TRAFFIC_BYTES.get(dom),
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated; recorded from profiles/)",
                      "algorithmic_bytes_per_sample": STEP_ALGO_BYTES[dom], "samples_per_launch": per_launch,
                      "avg_launch_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
