@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the NeuS2 SDF-field hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice|occupancy] [--no-cpu-baseline]
 
 A step is one full static NeuS2 training step (BASELINE config 4) on a synthetic scene: an analytic sphere of
 radius 0.3, Lambertian-textured, seen by 64 cameras at 512x512 on a sphere of radius 2; rays are marched through a
@@ -321,12 +321,71 @@ def run_lattice_workload(args):
             "kernels": kernels}
 
 
+def run_occupancy_workload(args):
+    """The occupancy-grid update that precedes training steps (the reference runs it every step for the first 32 steps,
+    then every 2nd ... 16th): a step is one update_density_grid_nerf over all 128^3 cells (uniform samples), i.e. sample
+    generation, NerfNetwork::density on 2^21 points, max-splat, decayed maximum, mean, bitfield and its mip levels."""
+    import numpy as np
+    import torch
+    from neus2_amd import capi
+    from neus2_amd.training import GRID_CELLS, OccupancyGrid, Trainer, default_config
+    lib = capi.lib()
+    tr = Trainer(default_config(target_batch_size=TARGET, max_rays_per_batch=1 << 16, max_samples=1 << 21))
+    sdf_w = np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy"))
+    tr.initialize_params(seed=1337, sdf_mlp_weights=sdf_w)
+    occ = OccupancyGrid(1, seed=1337, max_chunk=1 << 21)
+    for _ in range(args.warmup):
+        occ.update(tr._field, GRID_CELLS, 0)
+    torch.cuda.synchronize()
+    lib.n2_profile_reset()
+    lib.n2_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        occ.update(tr._field, GRID_CELLS, 0)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.n2_profile_enable(0)
+    kernels = {}
+    for name in ("grid_forward", "mlp_forward"):
+        ms, n = profile_read(lib, name)
+        kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
+    gf = kernels["grid_forward"]["avg_us"] * 1e-6
+    achieved = 588 * GRID_CELLS / gf / 1e9
+    result = {"metric": "occupancy-grid cells updated per second (128^3 cells per update, 1 GPU)", "value": args.steps * GRID_CELLS / elapsed,
+              "unit": "cells/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+              "config": {"workload": "update_density_grid_nerf over all 128^3 cells of one cascade: PCG32 sample generation, field density "
+                                     "(hash grid + SDF MLP forward) on 2^21 points, max-splat, decayed maximum, mean, bitfield + 7 mips",
+                         "cells": GRID_CELLS, "occupied_fraction": float(np.unpackbits(occ.bitfield[:GRID_CELLS // 8].cpu().numpy()).mean())},
+              "roofline": {"kernel": "grid_forward", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": 588,
+                           "samples_per_launch": GRID_CELLS, "avg_launch_us": kernels["grid_forward"]["avg_us"]},
+              "kernels": kernels}
+    if not args.no_cpu_baseline:
+        from oracle import oracle as orc
+        from oracle.field import Field
+        f = Field(fp16=True)
+        p16 = tr.params.float().cpu().numpy()
+        ref = orc.OccupancyGrid(1, seed=1337)
+        n = 1 << 17
+        best = None
+        for _ in range(3):
+            t0 = time.time()
+            ref.update(lambda xyz: f.density(p16, xyz)[0], 0.95, n, 0)
+            dt = time.time() - t0
+            best = dt if best is None else min(best, dt)
+        result["cpu_baseline"] = {"value": n / best, "unit": "cells/s", "cores": orc.num_threads(), "kind": "port",
+                                  "sample": f"one update with 2^17 uniform samples (1/16 of the cells; the mean/bitfield part still covers all "
+                                            f"128^3 cells), best of 3, {best * 1e3:.0f} ms"}
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice"], default="step")
+    ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice", "occupancy"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
@@ -337,7 +396,8 @@ def main():
     import torch
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (there is no CPU fallback of the product path)")
-    result = {"step": run_step_workload, "grid": run_grid_workload, "sdf": run_sdf_workload, "lattice": run_lattice_workload}[args.workload](args)
+    result = {"step": run_step_workload, "grid": run_grid_workload, "sdf": run_sdf_workload, "lattice": run_lattice_workload,
+              "occupancy": run_occupancy_workload}[args.workload](args)
     print(json.dumps(result))
 
 

@@ -445,6 +445,12 @@ n2_field_t* n2_trainer_field(n2_trainer_t* trainer);
 int n2_trainer_set_scene(n2_trainer_t* trainer, const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
                          const uint8_t* d_bitfield);
 
+/* Call before the bitfield passed to n2_trainer_set_scene is rewritten in place (an occupancy-grid update): waits for a
+ * sample generation that is running ahead on the trainer's own stream and discards it, so that the next step marches
+ * through the new bitfield like the reference does (training_prep_nerf runs before train_nerf_step,
+ * src/testbed.cu:2658-2674).  No counterpart in the reference, which generates its samples inside the step. */
+int n2_trainer_invalidate_prefetch(n2_trainer_t* trainer);
+
 /*  n_rays       rays to draw this step (<= max_rays_per_batch)
  *  n_inference  how many marched samples the first forward covers (a multiple of 8, <= max_samples); the
  *               reference uses the sample count measured in earlier steps, rounded up to 128
@@ -457,6 +463,52 @@ int n2_trainer_step(n2_trainer_t* trainer, n2_stream_t stream, uint32_t n_rays, 
  * (counters.update_after_training, src/testbed_nerf.cu:3406-3429). */
 int n2_trainer_read_counters(n2_trainer_t* trainer, n2_stream_t stream, uint32_t* rays, uint32_t* samples,
                              uint32_t* compacted, float* loss);
+
+/* ------------------------------------------------------------------------
+ * Occupancy grid: the running density estimate on 128^3 cells per cascade, and the morton-ordered
+ * 1-bit-per-cell bitfield with 8 mip levels (level m at byte m * 128^3 / 8) that the sample generator
+ * marches through.  Testbed::update_density_grid_nerf and update_density_grid_mean_and_bitfield,
+ * src/testbed_nerf.cu:3286-3391; kernels generate_grid_samples_nerf_nonuniform (:630-660),
+ * splat_grid_samples_nerf_max_nearest_neighbor (:662-680), ema_grid_samples_nerf (:698-727),
+ * grid_to_bitfield (:738-764), bitfield_max_pool (:766-786).  Unit aabb; threshold
+ * min(NERF_MIN_OPTICAL_THICKNESS = 0.1, mean density of the first cascade).
+ * Random numbers: PCG32 seeded as pcg32(seed) (the reference's density_grid_rng, src/testbed.cu:2090),
+ * passed to each sample launch by value and advanced by 2^32 afterwards.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_occupancy n2_occupancy_t;
+
+typedef struct n2_occupancy_buffers {
+	float* density_grid;      /* [n_cascades][128^3] running estimate */
+	float* density_grid_tmp;  /* [n_cascades][128^3] maxima splatted by the last update */
+	uint8_t* bitfield;        /* [8][128^3 / 8] */
+	float* mean;              /* [1] mean of max(density, 0) over the first cascade */
+	float* positions;         /* [n_samples][3] sample positions of the last update */
+	uint32_t* indices;        /* [n_samples] their cells */
+	uint32_t n_samples, n_cascades, ema_step;
+	uint64_t rng_state, rng_inc;
+} n2_occupancy_buffers;
+
+/*  n_cascades  max_cascade + 1 (1 for aabb_scale 1, src/testbed_nerf.cu:3077-3080) */
+int n2_occupancy_create(uint32_t n_cascades, uint64_t seed, n2_occupancy_t** out);
+void n2_occupancy_destroy(n2_occupancy_t* occupancy);
+/*  max_samples  largest n_uniform + n_nonuniform of an update
+ *  max_chunk    largest batch the field accepts (its workspace's max_batch); densities are evaluated in chunks */
+uint64_t n2_occupancy_workspace_bytes(const n2_occupancy_t* occupancy, uint32_t max_samples, uint32_t max_chunk);
+int n2_occupancy_set_workspace(n2_occupancy_t* occupancy, void* d_workspace, uint64_t n_bytes, uint32_t max_samples,
+                               uint32_t max_chunk);
+/* The training_step == 0 branch of update_density_grid_nerf (:3310-3329): zero grid, ema step 0. */
+int n2_occupancy_reset(n2_occupancy_t* occupancy, n2_stream_t stream);
+/* update_density_grid_nerf(decay, n_uniform, n_nonuniform, stream): sample cells, evaluate NerfNetwork::density,
+ * max-splat, decayed maximum, mean, bitfield and mips.  training_prep_nerf (:3989-4002) calls it with
+ * (128^3 * n_cascades, 0) for the first 256 steps and a quarter of that for each kind afterwards, decay 0.95. */
+int n2_occupancy_update(n2_occupancy_t* occupancy, n2_field_t* field, n2_stream_t stream, float decay, uint32_t n_uniform,
+                        uint32_t n_nonuniform);
+/* update_density_grid_mean_and_bitfield alone (after the density grid was written from outside, e.g. a snapshot);
+ * uses the partial sums of the last n2_occupancy_update. */
+int n2_occupancy_update_bitfield(n2_occupancy_t* occupancy, n2_stream_t stream);
+int n2_occupancy_view(n2_occupancy_t* occupancy, n2_occupancy_buffers* out);
+/* Restores the host-side state that n2_occupancy_view reports (resuming from a saved state). */
+int n2_occupancy_set_state(n2_occupancy_t* occupancy, uint32_t ema_step, uint64_t rng_state, uint64_t rng_inc);
 
 /* ------------------------------------------------------------------------
  * Optional event timing of the dominant kernels (off by default; the reference has only

@@ -48,6 +48,13 @@ class TrainerConfig(C.Structure):
                 ("loss_scale", C.c_float), ("prefetch_samples", C.c_uint32)]
 
 
+class OccupancyBuffers(C.Structure):
+    """struct n2_occupancy_buffers"""
+    _fields_ = [("density_grid", C.c_void_p), ("density_grid_tmp", C.c_void_p), ("bitfield", C.c_void_p), ("mean", C.c_void_p),
+                ("positions", C.c_void_p), ("indices", C.c_void_p), ("n_samples", C.c_uint32), ("n_cascades", C.c_uint32),
+                ("ema_step", C.c_uint32), ("rng_state", C.c_uint64), ("rng_inc", C.c_uint64)]
+
+
 class N2Error(RuntimeError):
     """A C-ABI call returned a non-zero status (mirrors the reference's std::runtime_error)."""
 
@@ -91,6 +98,10 @@ def lib():
         _lib.n2_trainer_field.argtypes = [C.c_void_p]
         _lib.n2_field_destroy.restype = None
         _lib.n2_field_destroy.argtypes = [C.c_void_p]
+        _lib.n2_occupancy_workspace_bytes.restype = C.c_uint64
+        _lib.n2_occupancy_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32]
+        _lib.n2_occupancy_destroy.restype = None
+        _lib.n2_occupancy_destroy.argtypes = [C.c_void_p]
     return _lib
 
 

@@ -248,6 +248,13 @@ N2_API int n2_trainer_set_scene(n2_trainer_t* t, const n2_camera* d_cameras, uin
 	return N2_OK;
 }
 
+N2_API int n2_trainer_invalidate_prefetch(n2_trainer_t* t) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_invalidate_prefetch: trainer is null");
+	if (t->side) N2_HIP(hipStreamSynchronize(t->side));
+	t->pf_valid = false;
+	return N2_OK;
+}
+
 N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays, uint32_t n_inference, uint32_t seed) {
 	N2_REQUIRE(t != nullptr, "n2_trainer_step: trainer is null");
 	N2_REQUIRE(t->cameras != nullptr, "n2_trainer_step: n2_trainer_set_scene has not been called");

@@ -83,6 +83,94 @@ class RayBudget:
         return True
 
 
+GRID_CELLS = 128 ** 3  # NERF_GRIDSIZE()^3, nerf.h:24-26
+
+
+def density_grid_update_plan(training_step, n_cascades=1):
+    """Which occupancy update Testbed::train runs before step ``training_step`` (src/testbed.cu:2658-2674 and
+    training_prep_nerf, src/testbed_nerf.cu:3989-4002): None when the step is skipped, else
+    (n_uniform, n_nonuniform).  The update runs every clamp(step / 16, 1, 16) steps; the first 256 steps
+    sample every cell once, later ones a quarter of the cells uniformly and a quarter among occupied cells."""
+    skip = min(max(training_step // 16, 1), 16)
+    if training_step % skip != 0:
+        return None
+    n = GRID_CELLS * n_cascades
+    return (n, 0) if training_step < 256 else (n // 4, n // 4)
+
+
+class OccupancyGrid:
+    """The density grid and its bitfield (Testbed::Nerf::density_grid / density_grid_bitfield), updated through
+    the C ABI from a field's density."""
+
+    def __init__(self, n_cascades=1, seed=1337, max_chunk=1 << 21, device="cuda"):
+        L = capi.lib()
+        self._h = C.c_void_p()
+        check(L.n2_occupancy_create(C.c_uint32(n_cascades), C.c_uint64(seed), C.byref(self._h)), "n2_occupancy_create")
+        self.n_cascades = n_cascades
+        self.max_samples = GRID_CELLS * n_cascades
+        nbytes = int(L.n2_occupancy_workspace_bytes(self._h, C.c_uint32(self.max_samples), C.c_uint32(max_chunk)))
+        if nbytes == 0:
+            raise N2Error("n2_occupancy_workspace_bytes: " + L.n2_last_error().decode())
+        self._ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        check(L.n2_occupancy_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes), C.c_uint32(self.max_samples),
+                                           C.c_uint32(max_chunk)), "n2_occupancy_set_workspace")
+        self.reset()
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) is not None and self._h.value:
+                capi.lib().n2_occupancy_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+    @staticmethod
+    def _stream():
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def reset(self):
+        check(capi.lib().n2_occupancy_reset(self._h, self._stream()), "n2_occupancy_reset")
+
+    def update(self, field_handle, n_uniform, n_nonuniform, decay=0.95):
+        """decay: Testbed::Nerf::Training::density_grid_decay (testbed.h:635)."""
+        check(capi.lib().n2_occupancy_update(self._h, field_handle, self._stream(), C.c_float(decay), C.c_uint32(n_uniform),
+                                             C.c_uint32(n_nonuniform)), "n2_occupancy_update")
+
+    def update_bitfield(self):
+        check(capi.lib().n2_occupancy_update_bitfield(self._h, self._stream()), "n2_occupancy_update_bitfield")
+
+    def view(self):
+        v = capi.OccupancyBuffers()
+        check(capi.lib().n2_occupancy_view(self._h, C.byref(v)), "n2_occupancy_view")
+        return v
+
+    def _tensor(self, address, nbytes, dtype):
+        off = address - self._ws.data_ptr()
+        return self._ws[off:off + nbytes].view(dtype)
+
+    @property
+    def density_grid(self):
+        return self._tensor(self.view().density_grid, 4 * GRID_CELLS * self.n_cascades, torch.float32)
+
+    @property
+    def density_grid_tmp(self):
+        return self._tensor(self.view().density_grid_tmp, 4 * GRID_CELLS * self.n_cascades, torch.float32)
+
+    @property
+    def bitfield(self):
+        """uint8 [8 * 128^3 / 8]; the first 128^3 / 8 bytes are what the sample generator reads."""
+        return self._tensor(self.view().bitfield, GRID_CELLS, torch.uint8)
+
+    @property
+    def mean(self):
+        return self._tensor(self.view().mean, 4, torch.float32)
+
+    def last_samples(self):
+        v = self.view()
+        return (self._tensor(v.positions, 12 * v.n_samples, torch.float32).view(-1, 3),
+                self._tensor(v.indices, 4 * v.n_samples, torch.int32))
+
+
 class Trainer:
     def __init__(self, cfg=None, device="cuda"):
         self.cfg = cfg if cfg is not None else default_config()
@@ -131,8 +219,35 @@ class Trainer:
     def set_scene(self, cameras, n_images, rgba, bitfield):
         """cameras: device byte tensor (tcnn_api.pack_cameras); rgba fp32 [pixels, 4]; bitfield uint8."""
         self._scene = (cameras, rgba, bitfield)  # keep alive
+        self._n_images = n_images
         check(capi.lib().n2_trainer_set_scene(self._h, ptr(cameras), C.c_uint32(n_images), ptr(rgba), ptr(bitfield)),
               "n2_trainer_set_scene")
+
+    def attach_occupancy(self, occupancy):
+        """From now on the rays march through ``occupancy``'s bitfield, which training_prep keeps up to date
+        (the reference's own density grid instead of a bitfield supplied with the scene)."""
+        if self._scene is None:
+            raise N2Error("attach_occupancy: call set_scene first")
+        self.occupancy = occupancy
+        cameras, rgba, _ = self._scene
+        n_images = self._n_images
+        self.set_scene(cameras, n_images, rgba, occupancy.bitfield)
+
+    def training_prep(self):
+        """Testbed::train's occupancy-grid cadence for the step about to run (src/testbed.cu:2658-2674).
+        Returns the (n_uniform, n_nonuniform) update that ran, or None."""
+        occ = getattr(self, "occupancy", None)
+        if occ is None:
+            return None
+        plan = density_grid_update_plan(self.step_index, occ.n_cascades)
+        if plan is None:
+            return None
+        # a sample generation running ahead reads the bitfield that is about to change
+        check(capi.lib().n2_trainer_invalidate_prefetch(self._h), "n2_trainer_invalidate_prefetch")
+        if self.step_index == 0:
+            occ.reset()
+        occ.update(self._field, plan[0], plan[1])
+        return plan
 
     def step(self, n_rays=None, n_inference=None, seed=None):
         n_rays = self.budget.rays_per_batch if n_rays is None else n_rays

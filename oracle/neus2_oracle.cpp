@@ -28,6 +28,13 @@
 //   orc_field_*               autograd of a torch restatement of
 //                             nerf_network.h's composition               pinned
 //   orc_composite_*           closed-form cases + finite differences     pinned
+//   orc_pcg32_*               published PCG32 outputs for seed (42, 54),
+//                             advance(n) == n draws                      pinned
+//     (agreement with the pcg32 class of the absent fork: parity unpinned)
+//   orc_generate_grid_samples integer index closed form (bijection at full
+//                             coverage), positions inside their cell     pinned
+//   orc_splat_grid_max / orc_ema_grid / orc_grid_mean / orc_grid_to_bitfield
+//                             numpy restatements, brute-force pooling    pinned
 //   fp16 rounding order inside the reference MLP (fp16 accumulate):
 //                             parity unpinned (source absent)
 //
@@ -926,5 +933,160 @@ ORC_API void orc_generate_training_samples(uint32_t n_rays, uint32_t n_rays_tota
 		numsteps[2 * s + 1] = base[i];
 		for (int k = 0; k < 3; ++k) rgb_target[(size_t)s * 3 + k] = r.target[k];
 		march(r, bitfield, coords + (size_t)base[i] * 7, cnt[i]);
+	}
+}
+
+// ---------------------------------------------------------------------------
+// Occupancy-grid update: update_density_grid_nerf and
+// update_density_grid_mean_and_bitfield, src/testbed_nerf.cu:3286-3391, with
+// their kernels (:630-660 sample generation, :662-680 max splat, :698-727 decay
+// + max, :738-764 threshold to bits, :766-786 mip pooling).  The density itself
+// comes from the field (NerfNetwork::density), evaluated by the caller.
+//
+// Random numbers: the reference passes a tcnn::pcg32 by value, skips it ahead
+// by 4*i and draws four floats.  The class lives in the absent submodule; what
+// is restated here is the published PCG32 (XSH-RR 64/32, M. O'Neill) in the
+// form of W. Jakob's pcg32.h that tiny-cuda-nn ships: seeding, next_uint,
+// next_float = bits((u >> 9) | 0x3f800000) - 1, and the O(log n) skip-ahead.
+// Pinned by the generator's published first outputs for seed (42, 54) and by
+// advance(n) == n draws; agreement with the fork itself is unpinned.
+// ---------------------------------------------------------------------------
+struct Pcg32 {
+	uint64_t state, inc;
+};
+static const uint64_t PCG32_MULT = 0x5851f42d4c957f2dULL;
+
+static inline uint32_t pcg32_next_uint(Pcg32& r) {
+	const uint64_t old = r.state;
+	r.state = old * PCG32_MULT + r.inc;
+	const uint32_t xorshifted = (uint32_t)(((old >> 18u) ^ old) >> 27u);
+	const uint32_t rot = (uint32_t)(old >> 59u);
+	return (xorshifted >> rot) | (xorshifted << ((~rot + 1u) & 31));
+}
+static inline Pcg32 pcg32_seed(uint64_t initstate, uint64_t initseq) {
+	Pcg32 r;
+	r.state = 0u;
+	r.inc = (initseq << 1u) | 1u;
+	pcg32_next_uint(r);
+	r.state += initstate;
+	pcg32_next_uint(r);
+	return r;
+}
+static inline float pcg32_next_float(Pcg32& r) {
+	const uint32_t u = (pcg32_next_uint(r) >> 9) | 0x3f800000u;
+	float f;
+	memcpy(&f, &u, 4);
+	return f - 1.0f;
+}
+static inline void pcg32_advance(Pcg32& r, uint64_t delta) {
+	uint64_t cur_mult = PCG32_MULT, cur_plus = r.inc, acc_mult = 1u, acc_plus = 0u;
+	while (delta > 0) {
+		if (delta & 1) {
+			acc_mult *= cur_mult;
+			acc_plus = acc_plus * cur_mult + cur_plus;
+		}
+		cur_plus = (cur_mult + 1) * cur_plus;
+		cur_mult *= cur_mult;
+		delta /= 2;
+	}
+	r.state = acc_mult * r.state + acc_plus;
+}
+
+ORC_API void orc_pcg32_seed(uint64_t initstate, uint64_t initseq, uint64_t* state_inc) {
+	const Pcg32 r = pcg32_seed(initstate, initseq);
+	state_inc[0] = r.state; state_inc[1] = r.inc;
+}
+// draws n values after skipping `skip` draws; updates state_inc to the generator's state afterwards
+ORC_API void orc_pcg32_draw(uint64_t* state_inc, uint64_t skip, uint32_t n, uint32_t* out_uint, float* out_float) {
+	Pcg32 r{state_inc[0], state_inc[1]};
+	pcg32_advance(r, skip);
+	for (uint32_t i = 0; i < n; ++i) {
+		if (out_float) out_float[i] = pcg32_next_float(r);
+		else out_uint[i] = pcg32_next_uint(r);
+	}
+	state_inc[0] = r.state;
+}
+ORC_API void orc_pcg32_advance(uint64_t* state_inc, uint64_t delta) {
+	Pcg32 r{state_inc[0], state_inc[1]};
+	pcg32_advance(r, delta);
+	state_inc[0] = r.state;
+}
+
+static const uint32_t GRID_CELLS = GRIDSIZE * GRIDSIZE * GRIDSIZE;
+
+// generate_grid_samples_nerf_nonuniform (:630-660) for the unit aabb (warp_position is the identity).
+//  rng      generator state {state, inc}, taken by value as in the reference
+//  grid_in  n_cascades * 128^3 running densities; out: positions [n][3], indices [n]
+ORC_API void orc_generate_grid_samples(uint32_t n_elements, const uint64_t* rng, uint32_t step, const float* grid_in, uint32_t n_cascades,
+                                       float thresh, float* positions, uint32_t* indices) {
+	#pragma omp parallel for schedule(static)
+	for (uint32_t i = 0; i < n_elements; ++i) {
+		Pcg32 r{rng[0], rng[1]};
+		pcg32_advance(r, (uint64_t)i * 4);
+		const uint32_t level = (uint32_t)(pcg32_next_float(r) * n_cascades) % n_cascades;
+		uint32_t idx = 0;
+		for (uint32_t j = 0; j < 10; ++j) {
+			idx = ((i + step * n_elements) * 56924617u + j * 19349663u + 96925573u) % GRID_CELLS;
+			idx += level * GRID_CELLS;
+			if (grid_in[idx] > thresh) break;
+		}
+		const uint32_t pos_idx = idx % GRID_CELLS;
+		uint32_t c[3];
+		orc_morton3d_invert(pos_idx, c);
+		const float scale = scalbnf(1.0f, (int)level);
+		for (int d = 0; d < 3; ++d) {
+			const float u = pcg32_next_float(r);
+			positions[(size_t)i * 3 + d] = (((float)c[d] + u) / (float)GRIDSIZE - 0.5f) * scale + 0.5f;
+		}
+		indices[i] = idx;
+	}
+}
+
+// splat_grid_samples_nerf_max_nearest_neighbor (:662-680): maximum through the unsigned bit pattern
+ORC_API void orc_splat_grid_max(uint32_t n_elements, const uint32_t* indices, const float* density, float* grid_tmp) {
+	for (uint32_t i = 0; i < n_elements; ++i) {
+		uint32_t a, b;
+		memcpy(&a, &grid_tmp[indices[i]], 4);
+		memcpy(&b, &density[i], 4);
+		if (b > a) memcpy(&grid_tmp[indices[i]], &b, 4);
+	}
+}
+
+// ema_grid_samples_nerf (:698-727): decayed maximum; negative cells stay untouched
+ORC_API void orc_ema_grid(uint32_t n_elements, float decay, float* grid, const float* grid_tmp) {
+	for (uint32_t i = 0; i < n_elements; ++i) {
+		const float prev = grid[i];
+		grid[i] = (prev < 0.f) ? prev : fmaxf(prev * decay, grid_tmp[i]);
+	}
+}
+
+// mean of max(v, 0) over the first cascade (:3383), accumulated in double
+ORC_API float orc_grid_mean(const float* grid) {
+	double s = 0.0;
+	for (uint32_t i = 0; i < GRID_CELLS; ++i) s += (double)fmaxf(grid[i], 0.f);
+	return (float)(s / GRID_CELLS);
+}
+
+// grid_to_bitfield (:738-764) over all 8 cascades and bitfield_max_pool (:766-786) for levels 1..7.
+//  bitfield  8 * 128^3 / 8 bytes, level m at byte m * 128^3 / 8
+ORC_API void orc_grid_to_bitfield(const float* grid, uint32_t n_cascades, float mean, float min_optical_thickness, uint8_t* bitfield) {
+	const uint32_t level_bytes = GRID_CELLS / 8, n_levels = 8;
+	const float thresh = std::min(min_optical_thickness, mean);
+	for (uint32_t i = 0; i < level_bytes * n_levels; ++i) {
+		uint8_t bits = 0;
+		if (i < level_bytes * n_cascades)
+			for (uint32_t j = 0; j < 8; ++j) bits |= grid[(size_t)i * 8 + j] > thresh ? (uint8_t)(1u << j) : 0;
+		bitfield[i] = bits;
+	}
+	for (uint32_t level = 1; level < n_levels; ++level) {
+		const uint8_t* prev = bitfield + (size_t)(level - 1) * level_bytes;
+		uint8_t* next = bitfield + (size_t)level * level_bytes;
+		for (uint32_t i = 0; i < GRID_CELLS / 64; ++i) {
+			uint8_t bits = 0;
+			for (uint32_t j = 0; j < 8; ++j) bits |= prev[i * 8 + j] > 0 ? (uint8_t)(1u << j) : 0;
+			uint32_t c[3];
+			orc_morton3d_invert(i, c);
+			next[orc_morton3d(c[0] + GRIDSIZE / 8, c[1] + GRIDSIZE / 8, c[2] + GRIDSIZE / 8)] |= bits;
+		}
 	}
 }

@@ -263,3 +263,100 @@ def generate_training_samples(n_rays, n_rays_total, seed, cameras, rgba, backgro
                                         _fp(target), _fp(coords))
     return dict(ray_counter=int(ray_counter.value), sample_counter=int(sample_counter.value), ray_indices=ray_indices,
                 numsteps=numsteps, rgb_target=target, coords=coords)
+
+
+# ---------------------------------------------------------------------------
+# occupancy-grid update (src/testbed_nerf.cu:3286-3391)
+# ---------------------------------------------------------------------------
+_u64 = C.POINTER(C.c_uint64)
+GRID_CELLS = 128 ** 3
+MIN_OPTICAL_THICKNESS = 0.1  # NERF_MIN_OPTICAL_THICKNESS() with SDF_GRID 0, src/testbed_nerf.cu:39, 65
+
+
+class Pcg32:
+    """Published PCG32 in the form tiny-cuda-nn ships (pcg32(initstate, initseq = 1))."""
+
+    def __init__(self, initstate=None, initseq=1):
+        self.s = np.zeros(2, np.uint64)
+        if initstate is None:  # default-constructed generator
+            self.s[0], self.s[1] = 0x853c49e6748fea9b, 0xda3e39cb94b95bdb
+        else:
+            lib().orc_pcg32_seed(C.c_uint64(initstate), C.c_uint64(initseq), self.s.ctypes.data_as(_u64))
+
+    def copy(self):
+        r = Pcg32()
+        r.s[:] = self.s
+        return r
+
+    def next_uints(self, n, skip=0):
+        out = np.zeros(n, np.uint32)
+        lib().orc_pcg32_draw(self.s.ctypes.data_as(_u64), C.c_uint64(skip), C.c_uint32(n), _up(out), None)
+        return out
+
+    def next_floats(self, n, skip=0):
+        out = np.zeros(n, np.float32)
+        lib().orc_pcg32_draw(self.s.ctypes.data_as(_u64), C.c_uint64(skip), C.c_uint32(n), None, _fp(out))
+        return out
+
+    def advance(self, delta=1 << 32):
+        lib().orc_pcg32_advance(self.s.ctypes.data_as(_u64), C.c_uint64(delta))
+
+
+def generate_grid_samples(n, rng, step, grid, n_cascades, thresh):
+    """generate_grid_samples_nerf_nonuniform: positions [n, 3] and cell indices [n] (rng is taken by value)."""
+    grid = _f32(grid)
+    pos, idx = np.zeros((n, 3), np.float32), np.zeros(n, np.uint32)
+    if n:
+        lib().orc_generate_grid_samples(C.c_uint32(n), rng.s.ctypes.data_as(_u64), C.c_uint32(step), _fp(grid), C.c_uint32(n_cascades),
+                                        C.c_float(thresh), _fp(pos), _up(idx))
+    return pos, idx
+
+
+def splat_grid_max(indices, density, grid_tmp):
+    density = _f32(density)
+    lib().orc_splat_grid_max(C.c_uint32(len(indices)), _up(indices), _fp(density), _fp(grid_tmp))
+
+
+def ema_grid(grid, grid_tmp, decay):
+    lib().orc_ema_grid(C.c_uint32(grid.size), C.c_float(decay), _fp(grid), _fp(grid_tmp))
+
+
+def grid_mean(grid):
+    lib().orc_grid_mean.restype = C.c_float
+    return float(lib().orc_grid_mean(_fp(grid)))
+
+
+def grid_to_bitfield(grid, n_cascades, mean):
+    bits = np.zeros(8 * GRID_CELLS // 8, np.uint8)
+    lib().orc_grid_to_bitfield(_fp(grid), C.c_uint32(n_cascades), C.c_float(mean), C.c_float(MIN_OPTICAL_THICKNESS),
+                               bits.ctypes.data_as(C.POINTER(C.c_uint8)))
+    return bits
+
+
+class OccupancyGrid:
+    """State and update of the density grid: Testbed::update_density_grid_nerf + update_density_grid_mean_and_bitfield.
+    ``density_fn(xyz [3, n]) -> [n]`` stands for NerfNetwork::density."""
+
+    def __init__(self, n_cascades=1, seed=1337):
+        self.n_cascades = n_cascades
+        self.grid = np.zeros(n_cascades * GRID_CELLS, np.float32)
+        self.rng = Pcg32(seed)
+        self.ema_step = 0
+        self.mean = 0.0
+        self.bitfield = np.zeros(GRID_CELLS, np.uint8)
+
+    def update(self, density_fn, decay, n_uniform, n_nonuniform, chunk=1 << 18):
+        tmp = np.zeros_like(self.grid)
+        p0, i0 = generate_grid_samples(n_uniform, self.rng, self.ema_step, self.grid, self.n_cascades, -0.01)
+        self.rng.advance()
+        p1, i1 = generate_grid_samples(n_nonuniform, self.rng, self.ema_step, self.grid, self.n_cascades, MIN_OPTICAL_THICKNESS)
+        self.rng.advance()
+        pos, idx = np.concatenate([p0, p1]), np.concatenate([i0, i1])
+        dens = np.concatenate([density_fn(np.ascontiguousarray(pos[a:a + chunk].T)) for a in range(0, len(pos), chunk)]) \
+            if len(pos) else np.zeros(0, np.float32)
+        splat_grid_max(idx, dens, tmp)
+        ema_grid(self.grid, tmp, decay)
+        self.ema_step += 1
+        self.mean = grid_mean(self.grid)
+        self.bitfield = grid_to_bitfield(self.grid, self.n_cascades, self.mean)
+        return dict(positions=pos, indices=idx, density=dens, tmp=tmp)
