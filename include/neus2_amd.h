@@ -300,7 +300,7 @@ int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, 
  * Adam on fp32 master weights with an fp16 working copy: tcnn's Adam as the
  * trainer runs it, Trainer::optimizer_step(stream, LOSS_SCALE) at
  * src/testbed_nerf.cu:3498, hyper-parameters from configs/nerf/base.json:13-26
- * (the Ema and ExponentialDecay wrappers around it are not part of this path).
+ * (the Ema wrapper is n2_ema_step, the ExponentialDecay wrapper is host logic over n2_trainer_set_learning_rate).
  * Per parameter i:  g = grad/loss_scale;  i >= n_matrix_params and g == 0: skipped entirely;
  * i < n_matrix_params: g += l2_reg*w;  moments with beta1/beta2;  per-parameter step counter t;
  * w -= lr*sqrt(1-beta2^t)/(1-beta1^t) * m/(sqrt(v)+epsilon);  fp16 copy refreshed.
@@ -312,6 +312,12 @@ typedef struct n2_adam_config {
 	float epsilon;       /* 1e-15 */
 	float l2_reg;        /* 1e-6 */
 } n2_adam_config;
+
+/* tcnn's EmaOptimizer step after nested step `step` (1-based), over all parameters:
+ *   tmp = (tmp*decay*(1 - decay^(step-1)) + w*(1 - decay)) / (1 - decay^step);  ema = half(tmp)
+ *  d_weights fp16 working weights (read), d_tmp fp32 moving average (read/written), d_ema fp16 copy (written). */
+int n2_ema_step(n2_stream_t stream, uint32_t n_params, float decay, uint32_t step, const n2_half* d_weights, float* d_tmp,
+                n2_half* d_ema);
 
 /* All buffers hold n_params elements and are caller-owned device memory:
  *  d_master fp32 weights, d_params fp16 copy (written), d_gradients fp16 (read),
@@ -425,6 +431,8 @@ typedef struct n2_trainer_config {
 	                                   field kernels; a following step called with other arguments regenerates in line.
 	                                   Results are identical either way.  The trainer must then be driven from one stream
 	                                   (or from streams the caller orders against each other). */
+	float ema_decay;                /* 0: plain Adam.  In (0, 1): the Ema wrapper of configs/nerf/base.json:5-7 (0.95) keeps a
+	                                   bias-corrected moving average of the fp16 weights as the inference parameters */
 } n2_trainer_config;
 
 /* All device memory a trainer uses (parameters, optimiser state, every temporary) lives in one
@@ -444,6 +452,25 @@ n2_field_t* n2_trainer_field(n2_trainer_t* trainer);
 /* Training images, cameras and the occupancy bitfield (see n2_generate_training_samples). */
 int n2_trainer_set_scene(n2_trainer_t* trainer, const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
                          const uint8_t* d_bitfield);
+
+/* The ExponentialDecay wrapper (configs/nerf/base.json:8-12) is host logic: after nested step t, if t >= decay_start and
+ * (t - decay_start) % decay_interval == 0, the learning rate is multiplied by decay_base.  The caller applies it here. */
+int n2_trainer_set_learning_rate(n2_trainer_t* trainer, float learning_rate);
+
+/* Optimizer state inside the workspace (what Trainer::serialize(include_optimizer_state) stores, src/testbed.cu:3134-3137):
+ * Adam moments and per-parameter step counters, the fp32 moving average of the Ema wrapper (NULL without it) and the
+ * parameters to use for inference (the Ema copy when it exists, else the working copy). */
+typedef struct n2_trainer_optimizer_buffers {
+	float* first_moments;
+	float* second_moments;
+	uint32_t* param_steps;
+	float* ema_weights;
+	n2_half* inference_params;
+	uint32_t optimizer_steps;
+	float learning_rate;
+} n2_trainer_optimizer_buffers;
+int n2_trainer_optimizer_state(n2_trainer_t* trainer, n2_trainer_optimizer_buffers* out);
+int n2_trainer_set_optimizer_steps(n2_trainer_t* trainer, uint32_t steps);
 
 /* Call before the bitfield passed to n2_trainer_set_scene is rewritten in place (an occupancy-grid update): waits for a
  * sample generation that is running ahead on the trainer's own stream and discards it, so that the next step marches

@@ -45,7 +45,14 @@ class TrainerConfig(C.Structure):
     """struct n2_trainer_config"""
     _fields_ = [("field", FieldConfig), ("adam", AdamConfig), ("composite", CompositeConfig),
                 ("target_batch_size", C.c_uint32), ("max_rays_per_batch", C.c_uint32), ("max_samples", C.c_uint32),
-                ("loss_scale", C.c_float), ("prefetch_samples", C.c_uint32)]
+                ("loss_scale", C.c_float), ("prefetch_samples", C.c_uint32), ("ema_decay", C.c_float)]
+
+
+class TrainerOptimizerBuffers(C.Structure):
+    """struct n2_trainer_optimizer_buffers"""
+    _fields_ = [("first_moments", C.c_void_p), ("second_moments", C.c_void_p), ("param_steps", C.c_void_p),
+                ("ema_weights", C.c_void_p), ("inference_params", C.c_void_p), ("optimizer_steps", C.c_uint32),
+                ("learning_rate", C.c_float)]
 
 
 class OccupancyBuffers(C.Structure):

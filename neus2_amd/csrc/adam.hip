@@ -4,6 +4,8 @@
 // one step) cost only the 2-byte gradient read.
 #include "n2_common.h"
 
+#include <cmath>
+
 typedef _Float16 hf;
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 
@@ -77,6 +79,48 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 	N2ProfScope prof(N2_PROF_ADAM, n2_stream(stream));
 	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(*config, n_params, n_matrix_params, loss_scale,
 		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+// Ema wrapper around the nested optimizer (configs/nerf/base.json:5-7, tcnn's EmaOptimizer): the bias-corrected
+// exponential moving average of the fp16 working weights, kept in fp32 with an fp16 copy for inference.  Unlike Adam
+// it touches every parameter in every step.
+__global__ void __launch_bounds__(256) ema_step_kernel(uint32_t n, float decay, float debias_old, float debias_new, const hf* __restrict__ weights,
+                                                       float* __restrict__ tmp, hf* __restrict__ ema) {
+	const uint32_t i0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+	if (i0 >= n) return;
+	if (i0 + 4 <= n) {
+		const half4 w = *reinterpret_cast<const half4*>(weights + i0);
+		float4 t = *reinterpret_cast<float4*>(tmp + i0);
+		t.x = (t.x * decay * debias_old + (float)w[0] * (1.f - decay)) / debias_new;
+		t.y = (t.y * decay * debias_old + (float)w[1] * (1.f - decay)) / debias_new;
+		t.z = (t.z * decay * debias_old + (float)w[2] * (1.f - decay)) / debias_new;
+		t.w = (t.w * decay * debias_old + (float)w[3] * (1.f - decay)) / debias_new;
+		*reinterpret_cast<float4*>(tmp + i0) = t;
+		*reinterpret_cast<half4*>(ema + i0) = half4{(hf)t.x, (hf)t.y, (hf)t.z, (hf)t.w};
+	} else {
+		for (uint32_t i = i0; i < n; ++i) {
+			const float v = (tmp[i] * decay * debias_old + (float)weights[i] * (1.f - decay)) / debias_new;
+			tmp[i] = v;
+			ema[i] = (hf)v;
+		}
+	}
+}
+
+N2_API int n2_ema_step(n2_stream_t stream, uint32_t n_params, float decay, uint32_t step, const n2_half* d_weights, float* d_tmp,
+                       n2_half* d_ema) {
+	if (n_params == 0) return N2_OK;
+	N2_REQUIRE(d_weights && d_tmp && d_ema, "n2_ema_step: null buffer");
+	N2_REQUIRE(decay > 0.f && decay < 1.f, "n2_ema_step: decay %g outside (0, 1)", (double)decay);
+	N2_REQUIRE(step >= 1, "n2_ema_step: step counts from 1 (the nested optimizer's step that just ran)");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_tmp) % 16 == 0 && reinterpret_cast<uintptr_t>(d_weights) % 8 == 0 && reinterpret_cast<uintptr_t>(d_ema) % 8 == 0,
+	           "n2_ema_step: buffers must be 16-byte (fp32) / 8-byte (fp16) aligned");
+	const float debias_old = 1.f - (float)pow((double)decay, (double)(step - 1));
+	const float debias_new = 1.f - (float)pow((double)decay, (double)step);
+	const uint32_t quads = (n_params + 3) / 4;
+	ema_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(n_params, decay, debias_old, debias_new,
+		reinterpret_cast<const hf*>(d_weights), d_tmp, reinterpret_cast<hf*>(d_ema));
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -24,6 +24,9 @@ struct n2_trainer {
 	float* m1;
 	float* m2;
 	uint32_t* steps;
+	float* ema_tmp;   // fp32 moving average of the fp16 weights (null without the Ema wrapper)
+	hf* ema;          // its fp16 copy: the inference parameters
+	uint32_t optimizer_steps;  // nested optimizer steps taken so far
 	// per-step buffers; everything the sample generator writes exists twice
 	struct SampleSet {
 		float* coords;            // [max_samples][7]
@@ -56,7 +59,7 @@ struct n2_trainer {
 };
 
 struct TrainerCarve {
-	uint64_t master, params, grads, m1, m2, steps, coords[2], mlp_out, dloss, coords_compacted, numsteps[2], ray_indices[2], rgb_target[2],
+	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], mlp_out, dloss, coords_compacted, numsteps[2], ray_indices[2], rgb_target[2],
 		set_counters[2], ray_loss, counters, ws_sampler[2], ws_composite, ws_field, total;
 };
 
@@ -75,6 +78,9 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	c.m1 = take(4 * np);
 	c.m2 = take(4 * np);
 	c.steps = take(4 * np);
+	const bool ema = cfg->ema_decay > 0.f;
+	c.ema_tmp = take(ema ? 4 * np : 0);
+	c.ema = take(ema ? 2 * np : 0);
 	for (int i = 0; i < 2; ++i) c.coords[i] = take(28 * S);
 	c.mlp_out = take(32 * (S > T ? S : T));
 	c.dloss = take(32 * T);
@@ -102,6 +108,7 @@ static int check_cfg(const n2_trainer_config* cfg, const char* fn) {
 	           cfg->max_samples);
 	N2_REQUIRE(cfg->max_rays_per_batch >= 1, "%s: max_rays_per_batch must be positive", fn);
 	N2_REQUIRE(cfg->loss_scale > 0.f, "%s: loss_scale must be positive", fn);
+	N2_REQUIRE(cfg->ema_decay >= 0.f && cfg->ema_decay < 1.f, "%s: ema_decay %g outside [0, 1)", fn, (double)cfg->ema_decay);
 	return N2_OK;
 }
 
@@ -169,6 +176,9 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->m1 = reinterpret_cast<float*>(b + c.m1);
 	t->m2 = reinterpret_cast<float*>(b + c.m2);
 	t->steps = reinterpret_cast<uint32_t*>(b + c.steps);
+	t->ema_tmp = cfg->ema_decay > 0.f ? reinterpret_cast<float*>(b + c.ema_tmp) : nullptr;
+	t->ema = cfg->ema_decay > 0.f ? reinterpret_cast<hf*>(b + c.ema) : nullptr;
+	t->optimizer_steps = 0;
 	for (int i = 0; i < 2; ++i) {
 		t->sets[i].coords = reinterpret_cast<float*>(b + c.coords[i]);
 		t->sets[i].numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps[i]);
@@ -315,8 +325,39 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	// forward + backward on the compacted batch, then the optimiser
 	if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
 	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
-	return n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                    reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps);
+	if (int rc = n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
+	                          reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps)) return rc;
+	t->optimizer_steps += 1;
+	if (t->ema) {
+		return n2_ema_step(stream, t->n_params, t->cfg.ema_decay, t->optimizer_steps, reinterpret_cast<const n2_half*>(t->params), t->ema_tmp,
+		                   reinterpret_cast<n2_half*>(t->ema));
+	}
+	return N2_OK;
+}
+
+N2_API int n2_trainer_set_learning_rate(n2_trainer_t* t, float learning_rate) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_set_learning_rate: trainer is null");
+	N2_REQUIRE(learning_rate >= 0.f, "n2_trainer_set_learning_rate: negative learning rate");
+	t->cfg.adam.learning_rate = learning_rate;
+	return N2_OK;
+}
+
+N2_API int n2_trainer_optimizer_state(n2_trainer_t* t, n2_trainer_optimizer_buffers* out) {
+	N2_REQUIRE(t != nullptr && out != nullptr, "n2_trainer_optimizer_state: null argument");
+	out->first_moments = t->m1;
+	out->second_moments = t->m2;
+	out->param_steps = t->steps;
+	out->ema_weights = t->ema_tmp;
+	out->inference_params = reinterpret_cast<n2_half*>(t->ema ? t->ema : t->params);
+	out->optimizer_steps = t->optimizer_steps;
+	out->learning_rate = t->cfg.adam.learning_rate;
+	return N2_OK;
+}
+
+N2_API int n2_trainer_set_optimizer_steps(n2_trainer_t* t, uint32_t steps) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_set_optimizer_steps: trainer is null");
+	t->optimizer_steps = steps;
+	return N2_OK;
 }
 
 N2_API int n2_trainer_read_counters(n2_trainer_t* t, n2_stream_t stream, uint32_t* rays, uint32_t* samples, uint32_t* compacted, float* loss) {

@@ -19,7 +19,7 @@ def next_multiple(x, m):
 
 def default_config(target_batch_size=1 << 18, max_rays_per_batch=1 << 16, max_samples=None, n_levels=16,
                    log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447, ek_loss_weight=0.01,
-                   background=(1.0, 1.0, 1.0), learning_rate=1e-3, prefetch_samples=True):
+                   background=(1.0, 1.0, 1.0), learning_rate=1e-3, prefetch_samples=True, ema_decay=0.0):
     """configs/nerf/base.json, with the level count / growth factor BASELINE's configs fix."""
     if max_samples is None:
         max_samples = 16 * target_batch_size  # src/testbed_nerf.cu:3719
@@ -32,7 +32,23 @@ def default_config(target_batch_size=1 << 18, max_rays_per_batch=1 << 16, max_sa
     cfg.max_samples = max_samples
     cfg.loss_scale = 128.0
     cfg.prefetch_samples = 1 if prefetch_samples else 0
+    cfg.ema_decay = ema_decay  # configs/nerf/base.json:5-7 wraps Adam in Ema(0.95); 0 leaves plain Adam
     return cfg
+
+
+class ExponentialDecay:
+    """tcnn's ExponentialDecay wrapper with the settings of configs/nerf/base.json:8-12: after nested step t, the
+    learning rate is multiplied by decay_base whenever t >= decay_start and (t - decay_start) % decay_interval == 0."""
+
+    def __init__(self, base_learning_rate=1e-3, decay_start=20000, decay_interval=10000, decay_base=0.33):
+        self.learning_rate = float(np.float32(base_learning_rate))
+        self.decay_start, self.decay_interval, self.decay_base = decay_start, decay_interval, decay_base
+
+    def after_step(self, steps_done):
+        """Returns the learning rate of the next step; ``steps_done`` counts the nested steps including the last one."""
+        if steps_done >= self.decay_start and (steps_done - self.decay_start) % self.decay_interval == 0:
+            self.learning_rate = float(np.float32(self.learning_rate) * np.float32(self.decay_base))
+        return self.learning_rate
 
 
 def initial_parameters(offsets, sdf_in_width, seed=1337, sdf_mlp_weights=None):
@@ -197,6 +213,7 @@ class Trainer:
         self._scene = None
         self.budget = RayBudget(self.cfg.target_batch_size, self.cfg.max_rays_per_batch, self.cfg.max_samples)
         self.step_index = 0
+        self.lr_schedule = None  # an ExponentialDecay, when the optimizer configuration nests one
 
     def __del__(self):
         try:
@@ -256,6 +273,30 @@ class Trainer:
         check(capi.lib().n2_trainer_step(self._h, self._stream(), C.c_uint32(n_rays), C.c_uint32(n_inference),
                                          C.c_uint32(seed)), "n2_trainer_step")
         self.step_index += 1
+        if self.lr_schedule is not None:
+            before = self.lr_schedule.learning_rate
+            lr = self.lr_schedule.after_step(self.optimizer_state().optimizer_steps)
+            if lr != before:
+                check(capi.lib().n2_trainer_set_learning_rate(self._h, C.c_float(lr)), "n2_trainer_set_learning_rate")
+
+    def optimizer_state(self):
+        s = capi.TrainerOptimizerBuffers()
+        check(capi.lib().n2_trainer_optimizer_state(self._h, C.byref(s)), "n2_trainer_optimizer_state")
+        return s
+
+    def _view(self, address, count, dtype):
+        off = address - self._ws.data_ptr()
+        return self._ws[off:off + count * torch.empty(0, dtype=dtype).element_size()].view(dtype)
+
+    @property
+    def inference_params(self):
+        """fp16 parameters to render / extract with: the Ema copy when the wrapper is on, else the working copy."""
+        return self._view(self.optimizer_state().inference_params, self.n_params, torch.float16)
+
+    @property
+    def ema_weights(self):
+        s = self.optimizer_state()
+        return None if not s.ema_weights else self._view(s.ema_weights, self.n_params, torch.float32)
 
     def read_counters(self):
         r, s, c, l = C.c_uint32(), C.c_uint32(), C.c_uint32(), C.c_float()

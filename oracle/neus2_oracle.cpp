@@ -1090,3 +1090,28 @@ ORC_API void orc_grid_to_bitfield(const float* grid, uint32_t n_cascades, float 
 		}
 	}
 }
+
+// ---------------------------------------------------------------------------
+// Optimizer wrappers of configs/nerf/base.json:5-13 around Adam, as tiny-cuda-nn publishes them (the fork's
+// copies are absent: parity with it unpinned).
+//  Ema: after the nested step number t (1-based), per weight
+//     tmp = (tmp * decay * (1 - decay^(t-1)) + w16 * (1 - decay)) / (1 - decay^t),  ema16 = half(tmp)
+//  i.e. the bias-corrected exponential moving average of the fp16 working weights; it becomes the inference copy.
+//  ExponentialDecay: after nested step t, if t >= decay_start and (t - decay_start) % decay_interval == 0 the
+//  nested learning rate is multiplied by decay_base.
+// ---------------------------------------------------------------------------
+ORC_API void orc_ema_step(uint32_t n, float decay, uint32_t step, const float* weights16, float* tmp, float* ema16) {
+	const float debias_old = 1.f - (float)std::pow((double)decay, (double)(step - 1));
+	const float debias_new = 1.f - (float)std::pow((double)decay, (double)step);
+	for (uint32_t i = 0; i < n; ++i) {
+		const float v = (tmp[i] * decay * debias_old + weights16[i] * (1.f - decay)) / debias_new;
+		tmp[i] = v;
+		ema16[i] = round_fp16(v);
+	}
+}
+ORC_API float orc_exponential_decay_lr(float base_lr, uint32_t decay_start, uint32_t decay_interval, float decay_base, uint32_t steps_done) {
+	float lr = base_lr;
+	for (uint32_t t = 1; t <= steps_done; ++t)
+		if (t >= decay_start && (t - decay_start) % decay_interval == 0) lr *= decay_base;
+	return lr;
+}

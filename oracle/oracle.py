@@ -360,3 +360,20 @@ class OccupancyGrid:
         self.mean = grid_mean(self.grid)
         self.bitfield = grid_to_bitfield(self.grid, self.n_cascades, self.mean)
         return dict(positions=pos, indices=idx, density=dens, tmp=tmp)
+
+
+# ---------------------------------------------------------------------------
+# optimizer wrappers (configs/nerf/base.json:5-13)
+# ---------------------------------------------------------------------------
+def ema_step(weights16, tmp, step, decay=0.95):
+    """One Ema step after nested step ``step`` (1-based); tmp (float32) is updated in place, returns the fp16-rounded EMA."""
+    weights16 = _f32(weights16)
+    out = np.zeros_like(weights16)
+    lib().orc_ema_step(C.c_uint32(weights16.size), C.c_float(decay), C.c_uint32(step), _fp(weights16), _fp(tmp), _fp(out))
+    return out
+
+
+def exponential_decay_lr(base_lr, steps_done, decay_start=20000, decay_interval=10000, decay_base=0.33):
+    lib().orc_exponential_decay_lr.restype = C.c_float
+    return float(lib().orc_exponential_decay_lr(C.c_float(base_lr), C.c_uint32(decay_start), C.c_uint32(decay_interval),
+                                                C.c_float(decay_base), C.c_uint32(steps_done)))

@@ -56,10 +56,46 @@ def test_trainer_config_struct_matches_header():
     from neus2_amd import capi
     assert ctypes.sizeof(capi.FieldConfig) == 32 and ctypes.sizeof(capi.AdamConfig) == 20
     assert ctypes.sizeof(capi.CompositeConfig) == 28 and ctypes.sizeof(capi.Camera) == 80
-    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 20
+    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 24
+    assert ctypes.sizeof(capi.OccupancyBuffers) == 6 * 8 + 3 * 4 + 4 + 2 * 8 and ctypes.sizeof(capi.TrainerOptimizerBuffers) == 5 * 8 + 8
     L = capi.lib()
     cfg = capi.TrainerConfig()
     assert L.n2_trainer_workspace_bytes(ctypes.byref(cfg)) == 0  # all-zero config is rejected on the host
     from neus2_amd.training import default_config
     n = L.n2_trainer_workspace_bytes(ctypes.byref(default_config()))
     assert 3 * 2 ** 30 < n < 6 * 2 ** 30
+
+
+def test_exponential_decay_schedule(oracle):
+    """Host mirror of tcnn's ExponentialDecay (configs/nerf/base.json:8-12) against the oracle's step-by-step loop."""
+    from neus2_amd.training import ExponentialDecay
+    sched = ExponentialDecay(1e-3, decay_start=20, decay_interval=10, decay_base=0.33)
+    for t in range(1, 75):
+        lr = sched.after_step(t)
+        want = oracle.exponential_decay_lr(1e-3, t, 20, 10, 0.33)
+        assert abs(lr - want) <= 1e-7 * want, (t, lr, want)
+    # closed form: the rate has been multiplied once at each of the steps 20, 30, ..., 70
+    assert abs(sched.learning_rate - 1e-3 * 0.33 ** 6) < 1e-9
+    # the published defaults leave the first 19999 steps alone
+    d = ExponentialDecay()
+    assert all(d.after_step(t) == d.learning_rate for t in (1, 100, 19999)) and abs(d.after_step(20000) - 3.3e-4) < 1e-9
+
+
+def test_ema_oracle_closed_forms(oracle):
+    rng = np.random.default_rng(0)
+    decay = 0.95
+    # constant weights: the bias-corrected average equals them at every step
+    w = rng.standard_normal(1000).astype(np.float16).astype(np.float32)
+    tmp = np.zeros_like(w)
+    for t in range(1, 30):
+        ema = oracle.ema_step(w, tmp, t, decay)
+        np.testing.assert_allclose(tmp, w, rtol=2e-6, atol=1e-9)
+        np.testing.assert_array_equal(ema, tmp.astype(np.float16).astype(np.float32))
+    # changing weights: sum of (1 - d) d^(t-k) w_k over the steps, divided by 1 - d^t
+    ws = rng.standard_normal((12, 64)).astype(np.float16).astype(np.float32)
+    tmp = np.zeros(64, np.float32)
+    for t in range(1, 13):
+        oracle.ema_step(ws[t - 1], tmp, t, decay)
+        k = np.arange(1, t + 1)
+        want = ((1 - decay) * decay ** (t - k)[:, None] * ws[:t].astype(np.float64)).sum(0) / (1 - decay ** t)
+        np.testing.assert_allclose(tmp, want, rtol=1e-5, atol=1e-6)
