@@ -530,12 +530,80 @@ int n2_occupancy_reset(n2_occupancy_t* occupancy, n2_stream_t stream);
  * (128^3 * n_cascades, 0) for the first 256 steps and a quarter of that for each kind afterwards, decay 0.95. */
 int n2_occupancy_update(n2_occupancy_t* occupancy, n2_field_t* field, n2_stream_t stream, float decay, uint32_t n_uniform,
                         uint32_t n_nonuniform);
-/* update_density_grid_mean_and_bitfield alone (after the density grid was written from outside, e.g. a snapshot);
- * uses the partial sums of the last n2_occupancy_update. */
+/* update_density_grid_mean_and_bitfield alone (after the density grid was written from outside, e.g. a snapshot). */
 int n2_occupancy_update_bitfield(n2_occupancy_t* occupancy, n2_stream_t stream);
 int n2_occupancy_view(n2_occupancy_t* occupancy, n2_occupancy_buffers* out);
 /* Restores the host-side state that n2_occupancy_view reports (resuming from a saved state). */
 int n2_occupancy_set_state(n2_occupancy_t* occupancy, uint32_t ema_step, uint64_t rng_state, uint64_t rng_inc);
+
+/* ------------------------------------------------------------------------
+ * Snapshot files: MessagePack of the network configuration plus a "snapshot" object, the format of
+ * Testbed::save_snapshot / load_snapshot (src/testbed.cu:3134-3244): n_params, params_type, params_binary,
+ * [optimizer], density_grid_size, density_grid_binary (fp16), nerf { aabb_scale, rgb { rays_per_batch,
+ * measured_batch_size, measured_batch_size_before_compaction } }, training_step, loss.
+ * Device pointers in, device pointers out; the file image lives in host memory in between.
+ * ---------------------------------------------------------------------- */
+typedef struct n2_snapshot n2_snapshot_t;
+
+typedef struct n2_snapshot_desc {
+	const uint8_t* config_msgpack;   /* host: an encoded MessagePack map (the network configuration, m_network_config); its entries
+	                                    become the file's top-level entries.  May be NULL */
+	uint64_t config_bytes;
+	uint32_t n_params;
+	const n2_half* d_params;         /* fp16 working parameters (written as params_type "__half") */
+	uint32_t include_optimizer_state;
+	const float* d_first_moments;    /* Adam state, n_params each (only with include_optimizer_state) */
+	const float* d_second_moments;
+	const uint32_t* d_param_steps;
+	const float* d_ema_weights;      /* fp32 moving average of the Ema wrapper, or NULL */
+	uint32_t optimizer_steps;
+	float learning_rate;
+	const float* d_density_grid;     /* fp32, density_grid_cells = n_cascades * 128^3 (0: never populated) */
+	uint64_t density_grid_cells;
+	void* d_scratch;                 /* device scratch for the fp16 copy of the density grid: 2 bytes per cell */
+	uint64_t scratch_bytes;
+	uint32_t aabb_scale;
+	uint32_t rays_per_batch, measured_batch_size, measured_batch_size_before_compaction;
+	uint32_t training_step;
+	float loss;
+} n2_snapshot_desc;
+
+/* Testbed::save_snapshot(path, include_optimizer_state).  Synchronises with the stream. */
+int n2_snapshot_save(const char* path, const n2_snapshot_desc* desc, n2_stream_t stream);
+
+typedef struct n2_snapshot_info {
+	uint32_t n_params;
+	uint32_t params_are_fp32;        /* params_type "float" (newer tiny-cuda-nn) instead of "__half" */
+	uint32_t density_grid_size;
+	uint64_t density_grid_cells;
+	uint32_t aabb_scale;
+	uint32_t rays_per_batch, measured_batch_size, measured_batch_size_before_compaction;
+	uint32_t training_step;
+	float loss;
+	uint32_t has_optimizer_state, has_ema_weights;
+	uint32_t optimizer_steps;
+	float learning_rate;
+} n2_snapshot_info;
+
+typedef struct n2_snapshot_targets {
+	uint32_t n_params;               /* of the model that receives the parameters: must match the file */
+	float* d_master;                 /* fp32 master weights (any of the pointers may be NULL: that part is not loaded) */
+	n2_half* d_params;               /* fp16 working copy */
+	float* d_density_grid;           /* fp32, density_grid_cells cells; follow with n2_occupancy_update_bitfield */
+	uint64_t density_grid_cells;
+	float* d_first_moments;
+	float* d_second_moments;
+	uint32_t* d_param_steps;
+	float* d_ema_weights;
+	void* d_scratch;                 /* device staging: max(params_binary bytes, 2 bytes per density cell) */
+	uint64_t scratch_bytes;
+} n2_snapshot_targets;
+
+/* Testbed::load_snapshot: reads and checks the file ("does not contain a snapshot", parameter count, grid size). */
+int n2_snapshot_open(const char* path, n2_snapshot_t** out, n2_snapshot_info* info);
+/* Copies the requested parts to the device, converting fp16 <-> fp32 as needed.  Synchronises with the stream. */
+int n2_snapshot_read(n2_snapshot_t* snapshot, n2_stream_t stream, const n2_snapshot_targets* targets);
+void n2_snapshot_close(n2_snapshot_t* snapshot);
 
 /* ------------------------------------------------------------------------
  * Optional event timing of the dominant kernels (off by default; the reference has only

@@ -107,6 +107,8 @@ def lib():
         _lib.n2_field_destroy.argtypes = [C.c_void_p]
         _lib.n2_occupancy_workspace_bytes.restype = C.c_uint64
         _lib.n2_occupancy_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32]
+        _lib.n2_snapshot_close.restype = None
+        _lib.n2_snapshot_close.argtypes = [C.c_void_p]
         _lib.n2_occupancy_destroy.restype = None
         _lib.n2_occupancy_destroy.argtypes = [C.c_void_p]
     return _lib

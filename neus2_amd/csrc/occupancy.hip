@@ -129,6 +129,8 @@ __global__ void __launch_bounds__(OCC_BLOCK) occ_splat_kernel(uint32_t n, const 
 
 // ema_grid_samples_nerf (:698-727), fused with the partial sums of max(v, 0) over the first cascade (:3383).
 // A block covers 8192 consecutive cells; its partial sum is built in a fixed order, so the mean is reproducible.
+// MERGE false: only the partial sums (the grid was written from outside).
+template <bool MERGE>
 __global__ void __launch_bounds__(OCC_BLOCK) occ_ema_kernel(uint32_t n_elements, float decay, float* __restrict__ grid, const float* __restrict__ tmp,
                                                             float* __restrict__ partial) {
 	__shared__ float red[OCC_BLOCK / 64];
@@ -137,9 +139,11 @@ __global__ void __launch_bounds__(OCC_BLOCK) occ_ema_kernel(uint32_t n_elements,
 	for (uint32_t k = 0; k < 32; ++k) {
 		const uint32_t i = base + k * OCC_BLOCK + threadIdx.x;
 		if (i < n_elements) {
-			const float prev = grid[i];
-			const float val = (prev < 0.f) ? prev : fmaxf(prev * decay, tmp[i]);
-			grid[i] = val;
+			float val = grid[i];
+			if (MERGE) {
+				val = (val < 0.f) ? val : fmaxf(val * decay, tmp[i]);
+				grid[i] = val;
+			}
 			sum += fmaxf(val, 0.f);
 		}
 	}
@@ -282,9 +286,19 @@ N2_API int n2_occupancy_reset(n2_occupancy_t* occ, n2_stream_t stream) {
 
 static inline dim3 ogrid(uint64_t n) { return dim3((uint32_t)((n + OCC_BLOCK - 1) / OCC_BLOCK)); }
 
+static int occ_bitfield_from_partials(n2_occupancy_t* occ, hipStream_t s);
+
 N2_API int n2_occupancy_update_bitfield(n2_occupancy_t* occ, n2_stream_t stream) {
 	N2_REQUIRE(occ != nullptr && occ->ws != nullptr, "n2_occupancy_update_bitfield: no workspace");
 	hipStream_t s = n2_stream(stream);
+	const uint32_t n_elements = occ->n_cascades * OCC_CELLS;
+	occ_ema_kernel<false><<<dim3((n_elements + OCC_BLOCK * 32 - 1) / (OCC_BLOCK * 32)), dim3(OCC_BLOCK), 0, s>>>(n_elements, 1.f, occ->grid, occ->tmp,
+	                                                                                                             occ->partial);
+	N2_LAUNCH_CHECK();
+	return occ_bitfield_from_partials(occ, s);
+}
+
+static int occ_bitfield_from_partials(n2_occupancy_t* occ, hipStream_t s) {
 	const uint32_t n_bytes = OCC_LEVELS * OCC_LEVEL_BYTES;
 	occ_mean_kernel<<<dim3(1), dim3(OCC_MEAN_BLOCKS), 0, s>>>(occ->partial, occ->mean);
 	N2_LAUNCH_CHECK();
@@ -332,12 +346,12 @@ N2_API int n2_occupancy_update(n2_occupancy_t* occ, n2_field_t* field, n2_stream
 		occ_splat_kernel<<<ogrid(m), dim3(OCC_BLOCK), 0, s>>>(m, occ->indices + a, occ->mlp_out, occ->tmp);
 		N2_LAUNCH_CHECK();
 	}
-	occ_ema_kernel<<<dim3((n_elements + OCC_BLOCK * 32 - 1) / (OCC_BLOCK * 32)), dim3(OCC_BLOCK), 0, s>>>(n_elements, decay, occ->grid, occ->tmp,
-	                                                                                                      occ->partial);
+	occ_ema_kernel<true><<<dim3((n_elements + OCC_BLOCK * 32 - 1) / (OCC_BLOCK * 32)), dim3(OCC_BLOCK), 0, s>>>(n_elements, decay, occ->grid, occ->tmp,
+	                                                                                                            occ->partial);
 	N2_LAUNCH_CHECK();
 	occ->ema_step += 1;
 	occ->last_n = n;
-	return n2_occupancy_update_bitfield(occ, stream);
+	return occ_bitfield_from_partials(occ, s);
 }
 
 N2_API int n2_occupancy_view(n2_occupancy_t* occ, n2_occupancy_buffers* out) {

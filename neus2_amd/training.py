@@ -84,6 +84,7 @@ class RayBudget:
         self.target, self.max_rays, self.max_samples = target_batch_size, max_rays, max_samples
         self.rays_per_batch = min(rays_per_batch, max_rays)
         self.measured_before_compaction = 0
+        self.measured = 0  # counters_rgb.measured_batch_size: samples the rays kept after compaction
 
     def n_inference(self):
         if self.measured_before_compaction == 0:
@@ -94,6 +95,7 @@ class RayBudget:
         if compacted == 0 or samples == 0:
             return False  # the reference warns and stops training (src/testbed_nerf.cu:3536-3542)
         self.measured_before_compaction = min(int(samples), self.max_samples)
+        self.measured = int(compacted)
         r = next_multiple(self.rays_per_batch * self.target / compacted, BATCH_SIZE_GRANULARITY)
         self.rays_per_batch = int(min(max(r, BATCH_SIZE_GRANULARITY), self.max_rays))
         return True

@@ -1,0 +1,119 @@
+"""Snapshot save / load through the C ABI: the file decodes with an independent MessagePack implementation to the
+device contents, and a trainer restored from it continues exactly like the one that wrote it."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, host
+from neus2_amd import scene
+from test_snapshot_format import CONFIG, reference_style_file
+
+msgpack = pytest.importorskip("msgpack")
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+CELLS = 128 ** 3
+
+
+def make_trainer(ema=0.95):
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import OccupancyGrid, Trainer, default_config
+    cams = scene.cameras_on_sphere(8, 96)
+    rgba = scene.render_sphere_images(cams)
+    tr = Trainer(default_config(target_batch_size=4096, max_rays_per_batch=2048, max_samples=1 << 17, ema_decay=ema))
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), dev(scene.sphere_bitfield()))
+    tr.initialize_params(seed=5, sdf_mlp_weights=np.load(os.path.join(GOLD, "sdf_mlp_weights_48.npy")))
+    tr.attach_occupancy(OccupancyGrid(1, seed=11, max_chunk=1 << 17))
+    return tr
+
+
+def run_steps(tr, n):
+    log = []
+    for _ in range(n):
+        tr.training_prep()
+        tr.step(n_rays=256, n_inference=1 << 17)
+        c, _ = tr.update_budget()
+        log.append((c["rays"], c["samples"], c["compacted"], c["loss"]))
+    return log
+
+
+def test_file_contents_and_exact_resume(tmp_path):
+    from neus2_amd.snapshot import load_snapshot, save_snapshot, snapshot_info
+    tr = make_trainer()
+    run_steps(tr, 3)
+    path = tmp_path / "step3.msgpack"
+    save_snapshot(path, tr, tr.occupancy, config=CONFIG, include_optimizer_state=True, loss=0.25)
+    # ---- the file, read by another implementation ----
+    doc = msgpack.unpackb(path.read_bytes(), raw=False, strict_map_key=False)
+    assert {k: doc[k] for k in CONFIG} == CONFIG
+    snap = doc["snapshot"]
+    assert snap["n_params"] == tr.n_params and snap["params_type"] == "__half" and snap["density_grid_size"] == 128
+    np.testing.assert_array_equal(np.frombuffer(snap["params_binary"], np.float16), tr.params.cpu().numpy())
+    np.testing.assert_array_equal(np.frombuffer(snap["density_grid_binary"], np.float16), tr.occupancy.density_grid.cpu().numpy().astype(np.float16))
+    assert snap["training_step"] == 3 and snap["loss"] == 0.25 and snap["nerf"]["aabb_scale"] == 1
+    assert snap["nerf"]["rgb"]["rays_per_batch"] == tr.budget.rays_per_batch
+    assert snap["nerf"]["rgb"]["measured_batch_size_before_compaction"] == tr.budget.measured_before_compaction
+    adam = snap["optimizer"]["nested"]["nested"]
+    st = tr.optimizer_state()
+    assert adam["current_step"] == 3 and abs(adam["base_learning_rate"] - 1e-3) < 1e-9
+    np.testing.assert_array_equal(np.frombuffer(adam["first_moments_binary"], np.float32), tr._view(st.first_moments, tr.n_params, torch.float32).cpu().numpy())
+    np.testing.assert_array_equal(np.frombuffer(adam["param_steps_binary"], np.uint32),
+                                  tr._view(st.param_steps, tr.n_params, torch.int32).cpu().numpy().view(np.uint32))
+    np.testing.assert_array_equal(np.frombuffer(snap["optimizer"]["ema_weights_binary"], np.float32), tr.ema_weights.cpu().numpy())
+    info = snapshot_info(path)
+    assert info.n_params == tr.n_params and info.training_step == 3 and info.has_optimizer_state and info.has_ema_weights
+    assert info.density_grid_cells == CELLS and info.optimizer_steps == 3
+    # ---- resume: a fresh trainer restored from the file continues bit for bit like the original ----
+    tr2 = make_trainer()
+    load_snapshot(path, tr2, tr2.occupancy)
+    np.testing.assert_array_equal(host(tr2.params), host(tr.params))
+    np.testing.assert_array_equal(host(tr2.master), host(tr.params))  # fp16 file: the master restarts from the rounded weights
+    np.testing.assert_array_equal(host(tr2.occupancy.density_grid), tr.occupancy.density_grid.cpu().numpy().astype(np.float16).astype(np.float32))
+    np.testing.assert_array_equal(host(tr2.inference_params), host(tr.inference_params))
+    assert tr2.step_index == 3 and tr2.optimizer_state().optimizer_steps == 3
+    # the original continues from the same rounded state so that both see identical inputs
+    load_snapshot(path, tr, tr.occupancy)
+    v, v2 = tr.occupancy.view(), tr2.occupancy.view()
+    from neus2_amd import capi
+    import ctypes as C
+    capi.check(capi.lib().n2_occupancy_set_state(tr2.occupancy._h, C.c_uint32(v.ema_step), C.c_uint64(v.rng_state), C.c_uint64(v.rng_inc)))
+    np.testing.assert_array_equal(host(tr2.occupancy.bitfield), host(tr.occupancy.bitfield))
+    assert run_steps(tr, 2) == run_steps(tr2, 2)
+    np.testing.assert_array_equal(host(tr2.master), host(tr.master))
+    np.testing.assert_array_equal(host(tr2.ema_weights), host(tr.ema_weights))
+
+
+def test_loads_files_of_another_writer_and_checks_shapes(tmp_path):
+    """A file in the reference's layout written by the msgpack package (fp32 parameters, as newer tiny-cuda-nn stores them)."""
+    from neus2_amd import capi
+    from neus2_amd.snapshot import load_snapshot
+    tr = make_trainer(ema=0.0)
+    n = tr.n_params
+    rng = np.random.default_rng(1)
+    w = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    grid = rng.random(CELLS).astype(np.float16)
+    doc = reference_style_file()
+    doc["snapshot"].update(n_params=n, params_type="float", params_binary=w.tobytes(), density_grid_binary=grid.tobytes())
+    p = tmp_path / "other.msgpack"
+    p.write_bytes(msgpack.packb(doc, use_bin_type=True))
+    info = load_snapshot(p, tr, tr.occupancy)
+    assert info.params_are_fp32 == 1 and not info.has_optimizer_state
+    np.testing.assert_array_equal(host(tr.master), w)
+    np.testing.assert_array_equal(host(tr.params), w.astype(np.float16).astype(np.float32))
+    np.testing.assert_array_equal(host(tr.occupancy.density_grid), grid.astype(np.float32))
+    # mean and bitfield were rebuilt from the loaded grid (update_density_grid_mean_and_bitfield)
+    mean = float(host(tr.occupancy.mean)[0])
+    assert abs(mean - grid.astype(np.float64).mean()) < 1e-4
+    bits = np.unpackbits(host(tr.occupancy.bitfield)[:CELLS // 8], bitorder="little").astype(bool)
+    np.testing.assert_array_equal(bits, grid.astype(np.float32) > np.float32(min(0.1, mean)))
+    assert tr.step_index == 1234 and tr.budget.rays_per_batch == 4096
+    # wrong parameter count / cascade count: the reference's errors, not a fault
+    doc["snapshot"].update(n_params=24, params_binary=w[:24].tobytes())
+    p.write_bytes(msgpack.packb(doc, use_bin_type=True))
+    with pytest.raises(capi.N2Error, match="parameters"):
+        load_snapshot(p, tr, tr.occupancy)
+    doc["snapshot"].update(n_params=n, params_binary=w.tobytes(), density_grid_binary=grid[:CELLS // 2].tobytes())
+    p.write_bytes(msgpack.packb(doc, use_bin_type=True))
+    with pytest.raises(capi.N2Error, match="cascades"):
+        load_snapshot(p, tr, tr.occupancy)
