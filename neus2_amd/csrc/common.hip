@@ -52,6 +52,7 @@ int n2_set_u32(hipStream_t stream, uint32_t* d_ptr, uint32_t value) {
 namespace {
 struct ProfState {
 	bool enabled = false;
+	uint32_t mask = 0xFFFFFFFFu;                  // ids that are timed while enabled
 	std::vector<hipEvent_t> pool;                 // recycled events
 	std::vector<hipEvent_t> pending[N2_PROF_COUNT];  // begin/end pairs, not yet read
 	float total_ms[N2_PROF_COUNT] = {};
@@ -87,7 +88,7 @@ void prof_collect(int id) {
 }  // namespace
 
 void n2_prof_begin(int id, hipStream_t stream) {
-	if (!g_prof.enabled) return;
+	if (!g_prof.enabled || !((g_prof.mask >> id) & 1u)) return;
 	hipEvent_t e = prof_take();
 	if (!e) return;
 	(void)hipEventRecord(e, stream);
@@ -107,6 +108,11 @@ void n2_prof_end(int id, hipStream_t stream) {
 
 N2_API int n2_profile_enable(int enable) {
 	g_prof.enabled = enable != 0;
+	return N2_OK;
+}
+
+N2_API int n2_profile_select(uint32_t id_mask) {
+	g_prof.mask = id_mask;
 	return N2_OK;
 }
 
