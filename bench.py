@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the NeuS2 SDF-field hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice|occupancy] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice|occupancy|mesh] [--no-cpu-baseline]
 
 A step is one full static NeuS2 training step (BASELINE config 4) on a synthetic scene: an analytic sphere of
 radius 0.3, Lambertian-textured, seen by 64 cameras at 512x512 on a sphere of radius 2; rays are marched through a
@@ -395,12 +395,48 @@ def run_occupancy_workload(args):
     return result
 
 
+def run_mesh_workload(args):
+    """The consumer of BASELINE configs[4]: marching cubes over the 512^3 SDF lattice (count, prefix sums, vertices, faces,
+    normals).  The lattice is evaluated once, untimed (that part is `--workload lattice`); a step is one full extraction."""
+    import numpy as np
+    import torch
+    from neus2_amd.mesh import density_on_grid, marching_cubes
+    from neus2_amd.training import Trainer, default_config
+    RES = 512
+    tr = Trainer(default_config(target_batch_size=TARGET, max_rays_per_batch=1 << 12, max_samples=1 << 22))
+    tr.initialize_params(seed=1, sdf_mlp_weights=np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy")))
+    d = density_on_grid(tr._field, (RES, RES, RES), chunk=1 << 22)
+    for _ in range(args.warmup):
+        v, t, n = marching_cubes(d, 0.0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        v, t, n = marching_cubes(d, 0.0)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    n_pts = RES ** 3
+    # algorithmic bytes per lattice point: density read once by each of count, vertices, faces (12) + two counters written,
+    # scanned (read + write, twice) and read back (8 + 16 + 16 + 8 = 48); output vertices / indices / normals are small
+    algo = 60
+    achieved = algo * n_pts / (elapsed / args.steps) / 1e9
+    return {"metric": "marching-cubes lattice points/sec over a 512^3 SDF lattice (1 GPU)", "value": args.steps * n_pts / elapsed, "unit": "points/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "marching cubes (shared vertices, deterministic numbering, vertex normals) over the 512^3 lattice of the "
+                                   "geometric-init SDF network, threshold 0; wall clock of the whole extraction including its one host "
+                                   "synchronisation and output allocation", "lattice": [RES, RES, RES], "vertices": int(v.shape[0]),
+                       "triangles": int(t.shape[0])},
+            "roofline": {"kernel": "marching cubes, all kernels of one extraction", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": algo,
+                         "samples_per_launch": n_pts, "avg_launch_us": elapsed / args.steps * 1e6}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice", "occupancy"], default="step")
+    ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice", "occupancy", "mesh"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
@@ -412,7 +448,7 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (there is no CPU fallback of the product path)")
     result = {"step": run_step_workload, "grid": run_grid_workload, "sdf": run_sdf_workload, "lattice": run_lattice_workload,
-              "occupancy": run_occupancy_workload}[args.workload](args)
+              "occupancy": run_occupancy_workload, "mesh": run_mesh_workload}[args.workload](args)
     print(json.dumps(result))
 
 

@@ -537,6 +537,37 @@ int n2_occupancy_view(n2_occupancy_t* occupancy, n2_occupancy_buffers* out);
 int n2_occupancy_set_state(n2_occupancy_t* occupancy, uint32_t ema_step, uint64_t rng_state, uint64_t rng_inc);
 
 /* ------------------------------------------------------------------------
+ * Mesh extraction: marching cubes with shared vertices over a density lattice, marching_cubes_gpu
+ * (src/marching_cubes.cu:794-822; gen_vertices :276-329, gen_faces :377-718), the lattice itself
+ * (Testbed::get_density_on_grid, src/testbed_nerf.cu:4082-4133) and the area-weighted vertex normals of
+ * accumulate_1ring (src/marching_cubes.cu:331-366).
+ * density[x + y*rx + z*rx*ry]; inside = density > thresh; vertex at dt = (thresh - f0)/(f1 - f0) along a cut edge,
+ * times (aabb_max - aabb_min)/res plus aabb_min.  Vertices are numbered by lattice point (x fastest) and edge
+ * direction, triangles by cube (the reference's order is an atomicAdd race).  The case table is derived on the host;
+ * it has the contour of the reference's table on every cube face in all 256 cases (same surface and orientation),
+ * with the polygons of some cases cut into triangles along other diagonals.
+ * ---------------------------------------------------------------------- */
+/* The derived case table: 256 rows of up to 5 edge triples, -1 terminated (the layout of the reference's
+ * triangle_table, src/marching_cubes.cu:400-657). */
+int n2_marching_cubes_table(int8_t* out_256x16);
+uint64_t n2_marching_cubes_workspace_bytes(const uint32_t res[3]);
+/* First pass: counts (the reference's "count only" launches, :807-811).  Synchronises with the stream. */
+int n2_marching_cubes_count(n2_stream_t stream, const uint32_t res[3], const float aabb_min[3], const float aabb_max[3],
+                            float thresh, const float* d_density, void* d_workspace, uint64_t workspace_bytes,
+                            uint32_t* n_vertices, uint32_t* n_triangles);
+/* Second pass with the workspace of the first: d_vertices fp32 [n_vertices][3], d_indices uint32 [n_triangles][3],
+ * d_normals fp32 [n_vertices][3] or NULL (not normalised, like the reference's). */
+int n2_marching_cubes_emit(n2_stream_t stream, const uint32_t res[3], const float aabb_min[3], const float aabb_max[3],
+                           float thresh, const float* d_density, const void* d_workspace, float* d_vertices,
+                           uint32_t* d_indices, float* d_normals, uint32_t n_vertices, uint32_t n_triangles);
+/* get_density_on_grid: the field's SDF (row 0 of NerfNetwork::sdf, fp16 widened to fp32) at the lattice points
+ * (x, y, z)/res * (aabb_max - aabb_min) + aabb_min, evaluated `chunk` points at a time (a multiple of 8, at most the
+ * field's max_batch; the reference uses 2^20).  d_density fp32 [rx*ry*rz]. */
+uint64_t n2_density_on_grid_scratch_bytes(uint32_t chunk);
+int n2_density_on_grid(n2_field_t* field, n2_stream_t stream, const uint32_t res[3], const float aabb_min[3],
+                       const float aabb_max[3], float* d_density, void* d_scratch, uint64_t scratch_bytes, uint32_t chunk);
+
+/* ------------------------------------------------------------------------
  * Snapshot files: MessagePack of the network configuration plus a "snapshot" object, the format of
  * Testbed::save_snapshot / load_snapshot (src/testbed.cu:3134-3244): n_params, params_type, params_binary,
  * [optimizer], density_grid_size, density_grid_binary (fp16), nerf { aabb_scale, rgb { rays_per_batch,
