@@ -408,6 +408,13 @@ int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n
                                  uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
                                  uint64_t workspace_bytes);
 
+/* Training images as the loader decodes them (8-bit sRGB RGBA, stb_image order) -> what the ray generator reads (fp32
+ * RGBA, linear, premultiplied by alpha): convert_rgba32 (src/nerf_loader.cu:59-81) with its white/black-is-transparent
+ * and mask-colour rules, then the Byte branch of read_rgba (common_device.cuh:635-655): srgb_to_linear(c/255)*alpha,
+ * alpha = a/255; a pixel equal to 0x00FF00FF afterwards (the mask marker) becomes (-1, -1, -1, -1). */
+int n2_convert_rgba8(n2_stream_t stream, uint64_t n_pixels, const uint8_t* d_rgba8, float* d_rgba, int white_transparent,
+                     int black_transparent, uint32_t mask_color);
+
 /* ------------------------------------------------------------------------
  * One training step: counterpart of Testbed::train_nerf_step followed by
  * Trainer::optimizer_step (src/testbed_nerf.cu:3717-3987, 3498):

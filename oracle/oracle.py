@@ -377,3 +377,32 @@ def exponential_decay_lr(base_lr, steps_done, decay_start=20000, decay_interval=
     lib().orc_exponential_decay_lr.restype = C.c_float
     return float(lib().orc_exponential_decay_lr(C.c_float(base_lr), C.c_uint32(decay_start), C.c_uint32(decay_interval),
                                                 C.c_float(decay_base), C.c_uint32(steps_done)))
+
+
+# ---------------------------------------------------------------------------
+# training images (src/nerf_loader.cu:59-81, common_device.cuh:31-37, 635-655)
+# ---------------------------------------------------------------------------
+def srgb_to_linear(c):
+    c = np.asarray(c, np.float32)
+    with np.errstate(invalid="ignore"):
+        return np.where(c <= np.float32(0.04045), c / np.float32(12.92),
+                        np.power((c + np.float32(0.055)) / np.float32(1.055), np.float32(2.4))).astype(np.float32)
+
+
+def convert_rgba8(rgba8, white_transparent=False, black_transparent=False, mask_color=0):
+    """uint8 [n, 4] -> float32 [n, 4]: convert_rgba32's transparency rules, then read_rgba's Byte branch."""
+    px = np.ascontiguousarray(rgba8, np.uint8).reshape(-1, 4).copy()
+    rgb = px[:, :3]
+    if white_transparent:
+        px[(rgb == 255).all(1), 3] = 0
+    if black_transparent:
+        px[(rgb == 0).all(1), 3] = 0
+    word = px.view(np.uint32).ravel()
+    masked = word == np.uint32(0x00FF00FF)
+    if mask_color:
+        masked |= word == np.uint32(mask_color)
+    a = px[:, 3].astype(np.float32) * np.float32(1.0 / 255.0)
+    lin = srgb_to_linear(px[:, :3].astype(np.float32) * np.float32(1.0 / 255.0))
+    out = np.concatenate([lin * a[:, None], a[:, None]], 1).astype(np.float32)
+    out[masked] = -1.0
+    return out
