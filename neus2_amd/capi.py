@@ -72,6 +72,14 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise N2Error(f"{LIB_PATH} is missing: build it with `python -m neus2_amd.build` "
                           "(there is no CPU or eager fallback)")
+        # torch owns the device memory and streams this library is handed, so both must share ONE HIP runtime: torch
+        # ships its own copy, and whichever copy is loaded first serves every later request for that library name.
+        # Loading torch first makes its copy the shared one (the other order leaves two runtimes that do not see each
+        # other's allocations).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = C.CDLL(LIB_PATH)
         _lib.n2_last_error.restype = C.c_char_p
         _lib.n2_version.restype = C.c_char_p
