@@ -592,7 +592,14 @@ constexpr uint32_t RED_CHUNK = 2048;              // tiles whose runs are gather
 constexpr uint32_t RED_PER_THREAD = RED_CHUNK / RED_BLOCK;
 constexpr float FIX_SCALE = 4294967296.0f;        // 2^32
 
-__device__ __forceinline__ unsigned long long to_fixed(float x) { return (unsigned long long)(long long)(x * FIX_SCALE); }
+// x * 2^32 as a two's complement 64-bit integer, for |x| < 2^31 with at most 24 significant bits (any fp16 value):
+// the high word is floor(x), the low word fract(x) * 2^32, both exact.  Five ALU operations instead of the generic
+// float -> int64 sequence.
+__device__ __forceinline__ unsigned long long to_fixed(float x) {
+	const float fl = floorf(x);
+	const uint32_t hi = (uint32_t)(int32_t)fl, lo = (uint32_t)((x - fl) * FIX_SCALE);
+	return ((unsigned long long)hi << 32) | lo;
+}
 __device__ __forceinline__ float from_fixed(unsigned long long q) { return (float)((double)(long long)q * (1.0 / 4294967296.0)); }
 
 __global__ void __launch_bounds__(RED_BLOCK) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
