@@ -209,6 +209,11 @@ int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, u
 int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
                           n2_half* d_dinput);
 
+/* forward and input_gradient(dim) of the same batch in one pass over the input (the reference calls them back to back
+ * on the SDF net, nerf_network.h:212 and :229); results equal those of the two separate calls. */
+int n2_mlp_forward_and_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
+                                      n2_half* d_output, n2_layout out_layout, n2_half* d_dinput);
+
 /* Network::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
  * dL_ddLdoutput, dL_dinput, use_inference_params, mode): the second-order pass the
  * reference fork adds for the eikonal loss, nerf_network.h:560-571.  One hidden

@@ -369,10 +369,9 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
-	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<n2_half*>(f->rgb_in),
-	                            N2_LAYOUT_SOA, nullptr)) return rc;
-	if (int rc = n2_mlp_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
-	                                   reinterpret_cast<n2_half*>(f->dsdf_din))) return rc;
+	// SDF net forward (into rows 0..15 of the colour net's input) and d sdf / d input in one pass over the input
+	if (int rc = n2_mlp_forward_and_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
+	                                               reinterpret_cast<n2_half*>(f->rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->dsdf_din))) return rc;
 	field_normals_rgb_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->enc_w, f->dsdf_din, f->dy_dx, f->normal, f->rgb_in);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_mlp_forward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_output, N2_LAYOUT_AOS, nullptr)) return rc;

@@ -403,10 +403,13 @@ struct GradAcc {
 // Weight gradients are summed per workgroup in fp32 and written to one slab of `partials` per
 // workgroup; a second tiny kernel reduces the slabs.
 // ----------------------------------------------------------------------------
-template <int IC, int NH, bool WANT_DX, bool WANT_DW>
+// WANT_Y: the forward output is written as well (the recomputed hidden activations are at hand): forward and input
+// gradient of the SDF net in one pass over its input.
+template <int IC, int NH, bool WANT_DX, bool WANT_DW, bool WANT_Y = false>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
                                                                     const hf* __restrict__ dY, int dy_aos, int unit_row,
-                                                                    hf* __restrict__ dX, float* __restrict__ partials) {
+                                                                    hf* __restrict__ dX, float* __restrict__ partials,
+                                                                    hf* __restrict__ Y = nullptr, int y_aos = 0) {
 	using M = FragMap<IC, NH>;
 	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT, ROLES = WANT_DW ? 2 : 1;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
@@ -431,12 +434,34 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_backward_kernel(const hf* __
 		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
 		constexpr int DX_TILES = WANT_DW ? 1 : IN_MT;  // with two roles each computes one row tile of dL_dx
 		half8 dx_keep[DX_TILES][2];                    // tile 0's rows until tile 1's are known (sample-pair stores)
+		half4 y_keep[2];
 #pragma unroll
 		for (int t = 0; t < 2; ++t) {
 			half8 x[IC], h[NH][4], dh[4];
 			split_pairs<IC>(xp, t, x);
 			const half8 dy = dyp[t];
 			hidden_S<IC, NH>(F, lane, x, h);
+			if (WANT_Y) {
+				float16v out = zero16();
+#pragma unroll
+				for (int c = 0; c < 4; ++c) out = N2_MFMA(frag(F, M::WO + c, lane), h[NH - 1][c], out);
+				const half4 lo = half4{(hf)out[0], (hf)out[1], (hf)out[2], (hf)out[3]}, hi = half4{(hf)out[4], (hf)out[5], (hf)out[6], (hf)out[7]};
+				if (valid) {
+					if (y_aos) {
+						hf* y = Y + (size_t)(col + t) * MLP_OUT;
+						*reinterpret_cast<half4*>(y + 4 * g) = lo;
+						*reinterpret_cast<half4*>(y + 8 + 4 * g) = hi;
+					} else if (t == 0) {
+						y_keep[0] = lo; y_keep[1] = hi;
+					} else {
+#pragma unroll
+						for (int e = 0; e < 4; ++e) {
+							*reinterpret_cast<half2v*>(Y + (size_t)e * N + off4) = half2v{y_keep[0][e], lo[e]};
+							*reinterpret_cast<half2v*>(Y + (size_t)(8 + e) * N + off4) = half2v{y_keep[1][e], hi[e]};
+						}
+					}
+				}
+			}
 			// ---- output layer ----
 			// dhN: gradient of the pre-activations of the current layer, neuron tile `role`, neuron-lane form
 			half8 dhN[2];
@@ -769,7 +794,8 @@ static int allow_lds(K kernel, size_t bytes) {
 
 // unit_row >= 0: dL_doutput is the constant e_{unit_row} and d_dL_doutput is not read
 static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
-                             const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode) {
+                             const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode,
+                             n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
@@ -795,18 +821,36 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
 		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, mlp->workspace); \
 	} while (0)
+#define LAUNCH_Y(IC, NH)                                                                                            \
+	do {                                                                                                            \
+		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT);                                                      \
+		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, true, false, true>, lds)) return rc;                     \
+		mlp_backward_kernel<IC, NH, true, false, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, \
+			mlp->workspace, reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0);                  \
+	} while (0)
 #define CALL(IC, NH)                                   \
 	do {                                               \
-		if (want_dx && want_dw) LAUNCH(IC, NH, true, true);    \
+		if (d_output) LAUNCH_Y(IC, NH);                        \
+		else if (want_dx && want_dw) LAUNCH(IC, NH, true, true);    \
 		else if (want_dx) LAUNCH(IC, NH, true, false);         \
 		else LAUNCH(IC, NH, false, true);                      \
 	} while (0)
 	MLP_DISPATCH(mlp->in_w, mlp->n_hidden, CALL);
 #undef CALL
 #undef LAUNCH
+#undef LAUNCH_Y
 	N2_LAUNCH_CHECK();
 	if (want_dw) return reduce_partials(mlp, s, blocks, mode);
 	return N2_OK;
+}
+
+N2_API int n2_mlp_forward_and_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
+                                             n2_half* d_output, n2_layout out_layout, n2_half* d_dinput) {
+	N2_REQUIRE(dim < (uint32_t)MLP_OUT, "n2_mlp_forward_and_input_gradient: output dimension %u out of range", dim);
+	N2_REQUIRE((d_output != nullptr && d_dinput != nullptr) || n == 0, "n2_mlp_forward_and_input_gradient: null output");
+	N2_REQUIRE(out_layout == N2_LAYOUT_SOA || out_layout == N2_LAYOUT_AOS, "n2_mlp_forward_and_input_gradient: bad layout %d", (int)out_layout);
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "n2_mlp_forward_and_input_gradient: d_output must be 16-byte aligned");
+	return mlp_backward_impl(mlp, stream, d_input, n, nullptr, N2_LAYOUT_SOA, (int)dim, d_dinput, N2_GRAD_IGNORE, d_output, out_layout);
 }
 
 N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,

@@ -233,6 +233,16 @@ class FullyFusedMLP:
               "n2_mlp_input_gradient")
         return d
 
+    def forward_and_input_gradient(self, x, dim=0, out_layout=LAYOUT_SOA, out=None):
+        """forward and input_gradient(dim) in one pass over the input: (y, d output[dim] / d input)."""
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        y = self._out(n, out_layout, x.device) if out is None else out
+        d = torch.empty((self.input_width(), n), dtype=torch.float16, device=x.device)
+        check(capi.lib().n2_mlp_forward_and_input_gradient(self._h, _stream(), C.c_uint32(dim), ptr(x), C.c_uint32(n), ptr(y),
+                                                           C.c_int(out_layout), ptr(d)), "n2_mlp_forward_and_input_gradient")
+        return y, d
+
     def backward_backward_input(self, x, dL_ddLdinput, dL_doutput, want_dL_ddLdoutput=False, mode=GRAD_ACCUMULATE):
         """dL_doutput None: the first-order output gradient was e_0 for every sample (the SDF's own gradient)."""
         n = x.shape[1]

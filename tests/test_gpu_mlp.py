@@ -145,3 +145,19 @@ def test_mlp_errors(oracle):
         m.backward_backward_input(x, x, torch.zeros((16, 64), dtype=torch.float16, device="cuda"))
     y, _ = m.forward(torch.zeros((48, 0), dtype=torch.float16, device="cuda"))
     assert y.shape == (16, 0)
+
+
+@pytest.mark.parametrize("in_w,n_hidden", [(48, 1), (48, 2), (32, 1), (64, 2)])
+@pytest.mark.parametrize("n", [8, 200, 4096 + 72])
+def test_forward_and_input_gradient_equals_the_two_calls(oracle, in_w, n_hidden, n):
+    """The fused pass writes exactly what forward and input_gradient write separately (same arithmetic, one read of x)."""
+    from neus2_amd.tcnn_api import LAYOUT_AOS, LAYOUT_SOA
+    om, gm, W, *_, rng = make(oracle, in_w, n_hidden, 7)
+    x = dev(q16(rng.standard_normal((in_w, n))), torch.float16)
+    for dim in (0, 5):
+        y_ref, _ = gm.forward(x, LAYOUT_SOA)
+        d_ref = gm.input_gradient(x, dim)
+        y, d = gm.forward_and_input_gradient(x, dim, LAYOUT_SOA)
+        assert torch.equal(y, y_ref) and torch.equal(d, d_ref)
+        y2, d2 = gm.forward_and_input_gradient(x, dim, LAYOUT_AOS)
+        assert torch.equal(y2.t().contiguous(), y_ref) and torch.equal(d2, d_ref)
