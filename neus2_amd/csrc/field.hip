@@ -126,9 +126,10 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 // 11..15 keep what the colour net wrote.
 __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __restrict__ coords, uint32_t N, const hf* __restrict__ sdf_out,
                                                                  hf bias, const float* __restrict__ normal, const hf* __restrict__ variance,
-                                                                 hf* __restrict__ output) {
+                                                                 hf* __restrict__ output, float* __restrict__ var_acc) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
+	if (i == 0) var_acc[0] = 0.f;  // the backward of this batch accumulates the variance gradient here
 	hf* o = output + (size_t)i * 16;
 	const float* c = coords + (size_t)i * 7;
 	o[3] = sdf_out[i] + bias;
@@ -376,7 +377,7 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_mlp_forward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_output, N2_LAYOUT_AOS, nullptr)) return rc;
 	field_finish_output_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->rgb_in, (hf)f->sdf_bias, f->normal, f->params + f->off_var,
-	                                                         reinterpret_cast<hf*>(d_output));
+	                                                         reinterpret_cast<hf*>(d_output), f->var_acc);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
@@ -393,7 +394,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0, "n2_field_backward: d_dL_doutput must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
 	const hf* dL = reinterpret_cast<const hf*>(d_dL_doutput);
-	if (int rc = n2_fill_zero_u32(s, f->var_acc, 16)) return rc;
+	// (the variance accumulator was cleared by the forward of this batch)
 	field_backward_prep_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->dL_drgb, f->var_acc);
 	N2_LAUNCH_CHECK();
 	// colour net

@@ -906,12 +906,30 @@ N2_API int n2_grid_corner_indices(n2_grid_t* grid, n2_stream_t stream, const flo
 	return N2_OK;
 }
 
-static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2_grad_mode mode) {
+static bool uses_bucketed(const n2_grid_t* grid, uint32_t n_points);
+static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_points, uint32_t tiles);
+
+// OVERWRITE: the gradient buffer starts from zero.  The bucketed scatter writes every entry of a level whose buckets
+// have one workgroup each, so only levels whose buckets are split over several workgroups (they add with atomics) need
+// clearing beforehand.
+static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2_grad_mode mode, uint32_t n_points) {
 	N2_REQUIRE(mode == N2_GRAD_IGNORE || mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "%s: bad gradient mode %d", fn, (int)mode);
 	if (mode == N2_GRAD_IGNORE) return N2_OK;
 	N2_REQUIRE(grid->grads != nullptr, "%s: gradient mode %d needs a gradient buffer (n2_grid_set_params)", fn, (int)mode);
-	if (mode == N2_GRAD_OVERWRITE) return n2_fill_zero_u32(stream, grid->grads, (size_t)grid->n_params * sizeof(__half));
-	return N2_OK;
+	if (mode != N2_GRAD_OVERWRITE) return N2_OK;
+	if (!uses_bucketed(grid, n_points)) return n2_fill_zero_u32(stream, grid->grads, (size_t)grid->n_params * sizeof(__half));
+	const uint32_t tiles = (n_points + 1023u) / 1024u;
+	uint32_t first = 0xFFFFFFFFu, last = 0;
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
+		if (bucket_groups(grid, l, n_points, tiles) > 1) {
+			if (first == 0xFFFFFFFFu) first = l;
+			last = l;
+		}
+	}
+	if (first == 0xFFFFFFFFu) return N2_OK;
+	// one fill over the span of those levels (they are the coarse, small ones): 16-byte aligned because every level holds a multiple of 8 entries
+	const size_t begin = (size_t)grid->tab.offset[first] * sizeof(__half2), end = (size_t)grid->tab.offset[last + 1] * sizeof(__half2);
+	return n2_fill_zero_u32(stream, reinterpret_cast<unsigned char*>(grid->grads) + begin, end - begin);
 }
 
 static inline uint32_t n_pair_tiles(uint32_t n_points) { return (n_points + PAIR_POINTS - 1) / PAIR_POINTS; }
@@ -927,6 +945,19 @@ static uint64_t bucket_ws_bytes(const n2_grid_t* grid, uint32_t max_points) {
 	const uint64_t rec = L * tiles * BIN_RECORDS * sizeof(uint2);
 	const uint64_t off = (L * tiles * (BKT_MAX + 1) * sizeof(uint16_t) + 255) / 256 * 256;
 	return rec + off;
+}
+
+static bool uses_bucketed(const n2_grid_t* grid, uint32_t n_points) {
+	return grid->grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 4 * BIN_POINTS;
+}
+// workgroups per bucket of a level: aim at <= ~64k records per reduce workgroup (a level holds 8 records per point)
+static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_points, uint32_t tiles) {
+	const uint32_t nb = (grid->tab.entries[level] + BKT_ENTRIES - 1) / BKT_ENTRIES;
+	const uint64_t per_bucket = (uint64_t)n_points * 8 / nb;
+	uint32_t groups = (uint32_t)((per_bucket + 65535) / 65536);
+	if (groups > tiles) groups = tiles;
+	if (groups < 1) groups = 1;
+	return groups;
 }
 
 N2_API uint64_t n2_grid_workspace_bytes(const n2_grid_t* grid, uint32_t max_points) {
@@ -971,11 +1002,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	uint32_t wg = 0;
 	for (uint32_t l = 0; l < L; ++l) {
 		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES;
-		// aim at <= ~64k records per reduce workgroup: a level holds 8 records per point
-		const uint64_t per_bucket = (uint64_t)n_points * 8 / nb;
-		uint32_t groups = (uint32_t)((per_bucket + 65535) / 65536);
-		if (groups > tiles) groups = tiles;
-		if (groups < 1) groups = 1;
+		const uint32_t groups = bucket_groups(grid, l, n_points, tiles);
 		plan.wg_begin[l] = wg;
 		plan.n_buckets[l] = nb;
 		plan.groups[l] = groups;
@@ -991,7 +1018,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 // One scatter pass with any combination of first-order (dL_dy) and second-order (v, g2) terms.
 static int launch_scatter(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
                           const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy, bool accumulate) {
-	if (grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 4 * BIN_POINTS)
+	if (grads != nullptr && uses_bucketed(grid, n_points))
 		return launch_bucketed(grid, s, d_xyz, point_stride, dim_stride, n_points, dL_dy, v, g2, dL_ddLdy, accumulate);
 	const uint32_t tiles = n_pair_tiles(n_points);
 	const dim3 gd(tiles * grid->tab.n_levels), bd(GRID_BLOCK);
@@ -1015,7 +1042,7 @@ N2_API int n2_grid_backward(n2_grid_t* grid, n2_stream_t stream, const float* d_
 	N2_REQUIRE(d_dL_dy != nullptr || n_points == 0, "n2_grid_backward: d_dL_dy is null");
 	N2_REQUIRE(d_dL_dx == nullptr || d_dy_dx != nullptr, "n2_grid_backward: d_dL_dx needs the d_dy_dx context of the forward");
 	hipStream_t s = n2_stream(stream);
-	if (int rc = prepare_grads(grid, "n2_grid_backward", s, mode)) return rc;
+	if (int rc = prepare_grads(grid, "n2_grid_backward", s, mode, n_points)) return rc;
 	if (n_points == 0) return N2_OK;
 	if (mode != N2_GRAD_IGNORE) {
 		N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
@@ -1038,7 +1065,7 @@ N2_API int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const flo
 	N2_REQUIRE((d_dL_dy && d_dL_ddLdx && d_dL_dy_second) || n_points == 0, "n2_grid_backward_fused: d_dL_dy, d_dL_ddLdx and d_dL_dy_second are required");
 	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_grid_backward_fused: mode must be OVERWRITE or ACCUMULATE");
 	hipStream_t s = n2_stream(stream);
-	if (int rc = prepare_grads(grid, "n2_grid_backward_fused", s, mode)) return rc;
+	if (int rc = prepare_grads(grid, "n2_grid_backward_fused", s, mode, n_points)) return rc;
 	if (n_points == 0) return N2_OK;
 	N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
 	return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), d_dL_ddLdx,
@@ -1053,7 +1080,7 @@ N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, 
 	if (int rc = check_batch(grid, "n2_grid_backward_backward_input", d_xyz, point_stride, dim_stride, n_points)) return rc;
 	N2_REQUIRE((d_dL_ddLdx != nullptr && d_dL_dy != nullptr) || n_points == 0, "n2_grid_backward_backward_input: d_dL_ddLdx and d_dL_dy are required");
 	hipStream_t s = n2_stream(stream);
-	if (int rc = prepare_grads(grid, "n2_grid_backward_backward_input", s, mode)) return rc;
+	if (int rc = prepare_grads(grid, "n2_grid_backward_backward_input", s, mode, d_dL_dx ? 0u : n_points)) return rc;
 	if (n_points == 0) return N2_OK;
 	if (mode == N2_GRAD_IGNORE && !d_dL_ddLdy && !d_dL_dx) return N2_OK;
 	if (d_dL_dx) {

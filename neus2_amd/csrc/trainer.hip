@@ -126,23 +126,36 @@ __global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, co
 	if (i < n) params[i] = (hf)master[i];
 }
 
-// sum of the per-ray losses of the live rays (one workgroup); also publishes the sample set's counters
-__global__ void __launch_bounds__(1024) trainer_loss_sum_kernel(const uint32_t* __restrict__ set_counters, uint32_t max_rays,
-                                                                const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
-	__shared__ float part[16];
-	const uint32_t n = min(set_counters[0], max_rays);
-	float s = 0.f;
-	for (uint32_t i = threadIdx.x; i < n; i += 1024) s += ray_loss[i];
+// After compositing, in one launch: pad the compacted batch to exactly T samples (fill_rollover_and_rescale on the fp16
+// output gradients, fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916) and, in the last workgroup, sum the
+// per-ray losses of the live rays and publish the sample set's counters.
+__global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, const uint32_t* __restrict__ n_in_ptr, hf* __restrict__ dloss,
+                                                                   float* __restrict__ coords, uint32_t blocks_f16, uint32_t blocks_f32,
+                                                                   const uint32_t* __restrict__ set_counters, uint32_t max_rays,
+                                                                   const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
+	const uint32_t n_in = *n_in_ptr;
+	if (blockIdx.x < blocks_f16) {
+		const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, lim = (size_t)n_in * 16;
+		if (n_in == 0 || i < lim || i >= (size_t)T * 16) return;
+		dloss[i] = (hf)((float)dloss[i % lim] * (float)n_in / (float)T);
+	} else if (blockIdx.x < blocks_f16 + blocks_f32) {
+		const size_t i = (size_t)(blockIdx.x - blocks_f16) * 256 + threadIdx.x, lim = (size_t)n_in * 7;
+		if (n_in == 0 || i < lim || i >= (size_t)T * 7) return;
+		coords[i] = coords[i % lim];
+	} else {
+		__shared__ float part[4];
+		const uint32_t n = min(set_counters[0], max_rays);
+		float s = 0.f;
+		for (uint32_t i = threadIdx.x; i < n; i += 256) s += ray_loss[i];
 #pragma unroll
-	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
-	__syncthreads();
-	if (threadIdx.x == 0) {
-		float t = 0.f;
-		for (int w = 0; w < 16; ++w) t += part[w];
-		counters[0] = set_counters[0];
-		counters[1] = set_counters[1];
-		reinterpret_cast<float*>(counters)[4] = t;
+		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+		if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+		__syncthreads();
+		if (threadIdx.x == 0) {
+			counters[0] = set_counters[0];
+			counters[1] = set_counters[1];
+			reinterpret_cast<float*>(counters)[4] = (part[0] + part[1]) + (part[2] + part[3]);
+		}
 	}
 }
 
@@ -317,11 +330,11 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	if (int rc = n2_composite_loss(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
 	                               set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
 	                               t->ws_composite, t->ws_composite_bytes)) return rc;
-	trainer_loss_sum_kernel<<<dim3(1), dim3(1024), 0, s>>>(ray_counter, n_rays, t->ray_loss, t->counters);
+	// pad the compacted batch to exactly T samples; loss sum and counters
+	const uint32_t blocks_f16 = (uint32_t)(((size_t)T * 16 + 255) / 256), blocks_f32 = (uint32_t)(((size_t)T * 7 + 255) / 256);
+	trainer_finish_batch_kernel<<<dim3(blocks_f16 + blocks_f32 + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, blocks_f16,
+	                                                                                  blocks_f32, ray_counter, n_rays, t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
-	// pad the compacted batch to exactly T samples
-	if (int rc = n2_fill_rollover_and_rescale_f16(stream, T, 16, compacted_counter, reinterpret_cast<n2_half*>(t->dloss))) return rc;
-	if (int rc = n2_fill_rollover_f32(stream, T, 7, compacted_counter, t->coords_compacted)) return rc;
 	// forward + backward on the compacted batch, then the optimiser
 	if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
 	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
