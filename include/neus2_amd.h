@@ -214,6 +214,14 @@ int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const
 int n2_mlp_forward_and_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
                                       n2_half* d_output, n2_layout out_layout, n2_half* d_dinput);
 
+/* Weight gradients are summed per workgroup and a small second launch folds those partial sums into the gradient buffer.
+ * With deferred reduction switched on, n2_mlp_backward / n2_mlp_backward_backward_input leave their partial sums pending
+ * (the gradient buffer is NOT up to date until n2_mlp_reduce_deferred has run; after a pending pass only ACCUMULATE may
+ * follow) and n2_mlp_reduce_deferred folds everything pending for up to two networks in one launch.  Off by default;
+ * no counterpart in the reference, which uses GEMMs for the weight gradients. */
+int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable);
+int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b /* may be NULL */, n2_stream_t stream);
+
 /* Network::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
  * dL_ddLdoutput, dL_dinput, use_inference_params, mode): the second-order pass the
  * reference fork adds for the eikonal loss, nerf_network.h:560-571.  One hidden

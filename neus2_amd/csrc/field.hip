@@ -242,6 +242,8 @@ N2_API int n2_field_create(const n2_field_config* cfg, n2_field_t** out) {
 		rc = n2_mlp_create(f->sdf_in_w, cfg->sdf_hidden_layers, &f->sdf);
 	}
 	if (rc == N2_OK) rc = n2_mlp_create(f->rgb_in_w, cfg->rgb_hidden_layers, &f->rgb);
+	if (rc == N2_OK) rc = n2_mlp_set_deferred_reduction(f->sdf, 1);
+	if (rc == N2_OK) rc = n2_mlp_set_deferred_reduction(f->rgb, 1);
 	if (rc != N2_OK) {
 		n2_field_destroy(f);
 		return rc;
@@ -415,8 +417,11 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	if (int rc = n2_grid_backward_fused(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
 	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n), nullptr, mode)) return rc;
 	// second order through the SDF net
-	return n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
-	                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE);
+	if (int rc = n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
+	                                            reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE)) return rc;
+	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
+	// pending: one launch sums them
+	return n2_mlp_reduce_deferred(f->rgb, f->sdf, stream);
 }
 
 static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n,

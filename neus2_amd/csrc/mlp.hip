@@ -46,6 +46,10 @@ struct n2_mlp {
 	hf* grads;
 	float* workspace;
 	uint64_t workspace_bytes;
+	// deferred reduction: gradient-producing calls append their slabs and one later launch sums them all
+	bool deferred;
+	uint32_t pending_slabs;       // slabs written since the last reduction
+	n2_grad_mode pending_mode;    // mode of the first of the pending calls (later ones must accumulate)
 };
 
 // ----------------------------------------------------------------------------
@@ -640,18 +644,25 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_bbi_kernel(const hf* __restr
 // lane adds up n_slabs/16 partial sums (coalesced across the 16 parameters), LDS folds the groups.
 __global__ void __launch_bounds__(256) mlp_reduce_partials_kernel(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params,
                                                                   hf* __restrict__ grads, int accumulate) {
-	__shared__ float fold[16][17];
-	const uint32_t pl = threadIdx.x & 15, grp = threadIdx.x >> 4;
-	const uint32_t i = blockIdx.x * 16 + pl;
-	float s = 0.f;
-	if (i < n_params)
-		for (uint32_t k = grp; k < n_slabs; k += 16) s += partials[(size_t)k * n_params + i];
-	fold[grp][pl] = s;
+	// 32 consecutive parameters per workgroup (one 128-byte line of every slab), 8 groups of lanes share the slabs
+	__shared__ float fold[8][33];
+	const uint32_t pl = threadIdx.x & 31, grp = threadIdx.x >> 5;
+	const uint32_t i = blockIdx.x * 32 + pl;
+	float s0 = 0.f, s1 = 0.f;
+	if (i < n_params) {
+		uint32_t k = grp;
+		for (; k + 8 < n_slabs; k += 16) {  // two independent chains of loads
+			s0 += partials[(size_t)k * n_params + i];
+			s1 += partials[(size_t)(k + 8) * n_params + i];
+		}
+		if (k < n_slabs) s0 += partials[(size_t)k * n_params + i];
+	}
+	fold[grp][pl] = s0 + s1;
 	__syncthreads();
 	if (grp == 0 && i < n_params) {
 		float t = 0.f;
 #pragma unroll
-		for (int k = 0; k < 16; ++k) t += fold[k][pl];
+		for (int k = 0; k < 8; ++k) t += fold[k][pl];
 		if (accumulate) t += (float)grads[i];
 		grads[i] = (hf)t;
 	}
@@ -680,6 +691,9 @@ N2_API int n2_mlp_create(uint32_t in_width, uint32_t n_hidden_layers, n2_mlp_t**
 	m->grads = nullptr;
 	m->workspace = nullptr;
 	m->workspace_bytes = 0;
+	m->deferred = false;
+	m->pending_slabs = 0;
+	m->pending_mode = N2_GRAD_IGNORE;
 	*out = m;
 	return N2_OK;
 }
@@ -687,7 +701,10 @@ N2_API void n2_mlp_destroy(n2_mlp_t* mlp) { delete mlp; }
 N2_API uint32_t n2_mlp_n_params(const n2_mlp_t* mlp) { return mlp ? mlp->n_params : 0; }
 N2_API uint32_t n2_mlp_input_width(const n2_mlp_t* mlp) { return mlp ? mlp->in_w : 0; }
 N2_API uint32_t n2_mlp_output_width(const n2_mlp_t* mlp) { return mlp ? MLP_OUT : 0; }
-N2_API uint64_t n2_mlp_workspace_bytes(const n2_mlp_t* mlp) { return mlp ? (uint64_t)MLP_MAX_SLABS * mlp->n_params * sizeof(float) : 0; }
+constexpr uint32_t MLP_SLAB_SETS = 2;  // a backward and a second-order pass may be pending at the same time
+N2_API uint64_t n2_mlp_workspace_bytes(const n2_mlp_t* mlp) {
+	return mlp ? (uint64_t)MLP_SLAB_SETS * MLP_MAX_SLABS * mlp->n_params * sizeof(float) : 0;
+}
 
 N2_API int n2_mlp_set_params(n2_mlp_t* mlp, const n2_half* d_params, n2_half* d_gradients) {
 	N2_REQUIRE(mlp != nullptr, "n2_mlp_set_params: mlp is null");
@@ -770,10 +787,89 @@ N2_API int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_in
 	return N2_OK;
 }
 
-static int reduce_partials(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
-	mlp_reduce_partials_kernel<<<dim3((mlp->n_params + 15) / 16), dim3(256), 0, s>>>(mlp->workspace, n_slabs, mlp->n_params,
+// where the next gradient-producing kernel writes its slabs
+static float* next_slabs(n2_mlp_t* mlp) { return mlp->workspace + (size_t)mlp->pending_slabs * mlp->n_params; }
+
+static int reduce_now(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
+	mlp_reduce_partials_kernel<<<dim3((mlp->n_params + 31) / 32), dim3(256), 0, s>>>(mlp->workspace, n_slabs, mlp->n_params,
 		mlp->grads, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+// a kernel has just written n_slabs slabs at next_slabs(mlp)
+static int reduce_partials(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
+	if (!mlp->deferred) return reduce_now(mlp, s, n_slabs, mode);
+	if (mlp->pending_slabs == 0) mlp->pending_mode = mode;
+	mlp->pending_slabs += n_slabs;
+	return N2_OK;
+}
+
+// a gradient-producing call may run: room for its slabs, and a mode that can be folded into what is pending
+static int check_pending(n2_mlp_t* mlp, const char* fn, uint32_t n_slabs, n2_grad_mode mode) {
+	if (!mlp->deferred || mode == N2_GRAD_IGNORE) return N2_OK;
+	N2_REQUIRE(mlp->pending_slabs == 0 || mode == N2_GRAD_ACCUMULATE, "%s: with deferred reduction only ACCUMULATE can follow a pending gradient pass", fn);
+	N2_REQUIRE(mlp->pending_slabs + n_slabs <= MLP_SLAB_SETS * (uint32_t)MLP_MAX_SLABS, "%s: too many gradient passes pending (call n2_mlp_reduce_deferred)", fn);
+	return N2_OK;
+}
+
+N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
+	N2_REQUIRE(mlp != nullptr, "n2_mlp_set_deferred_reduction: mlp is null");
+	N2_REQUIRE(mlp->pending_slabs == 0, "n2_mlp_set_deferred_reduction: gradient passes are pending");
+	mlp->deferred = enable != 0;
+	return N2_OK;
+}
+
+// two parameter sets in one launch
+__global__ void __launch_bounds__(256) mlp_reduce_two_kernel(const float* __restrict__ pa, uint32_t slabs_a, uint32_t params_a, hf* __restrict__ ga, int acc_a,
+                                                             uint32_t blocks_a, const float* __restrict__ pb, uint32_t slabs_b, uint32_t params_b,
+                                                             hf* __restrict__ gb, int acc_b) {
+	__shared__ float fold[8][33];
+	const bool second = blockIdx.x >= blocks_a;
+	const float* partials = second ? pb : pa;
+	const uint32_t n_slabs = second ? slabs_b : slabs_a, n_params = second ? params_b : params_a;
+	hf* grads = second ? gb : ga;
+	const int accumulate = second ? acc_b : acc_a;
+	const uint32_t pl = threadIdx.x & 31, grp = threadIdx.x >> 5;
+	const uint32_t i = (second ? blockIdx.x - blocks_a : blockIdx.x) * 32 + pl;
+	float s0 = 0.f, s1 = 0.f;
+	if (i < n_params) {
+		uint32_t k = grp;
+		for (; k + 8 < n_slabs; k += 16) {
+			s0 += partials[(size_t)k * n_params + i];
+			s1 += partials[(size_t)(k + 8) * n_params + i];
+		}
+		if (k < n_slabs) s0 += partials[(size_t)k * n_params + i];
+	}
+	fold[grp][pl] = s0 + s1;
+	__syncthreads();
+	if (grp == 0 && i < n_params) {
+		float t = 0.f;
+#pragma unroll
+		for (int k = 0; k < 8; ++k) t += fold[k][pl];
+		if (accumulate) t += (float)grads[i];
+		grads[i] = (hf)t;
+	}
+}
+
+N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) {
+	N2_REQUIRE(a != nullptr, "n2_mlp_reduce_deferred: mlp is null");
+	hipStream_t s = n2_stream(stream);
+	if (b != nullptr && b->pending_slabs == 0) b = nullptr;
+	if (a->pending_slabs == 0) { a = b; b = nullptr; }
+	if (a == nullptr || a->pending_slabs == 0) return N2_OK;
+	if (b == nullptr) {
+		const int rc = reduce_now(a, s, a->pending_slabs, a->pending_mode);
+		a->pending_slabs = 0;
+		return rc;
+	}
+	const uint32_t blocks_a = (a->n_params + 31) / 32, blocks_b = (b->n_params + 31) / 32;
+	mlp_reduce_two_kernel<<<dim3(blocks_a + blocks_b), dim3(256), 0, s>>>(a->workspace, a->pending_slabs, a->n_params, a->grads,
+		a->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0, blocks_a, b->workspace, b->pending_slabs, b->n_params, b->grads,
+		b->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+	N2_LAUNCH_CHECK();
+	a->pending_slabs = 0;
+	b->pending_slabs = 0;
 	return N2_OK;
 }
 
@@ -810,6 +906,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	}
 	if (!want_dw && !want_dx) return N2_OK;
 	const uint32_t blocks = stream_grid(n, want_dw ? 2 : 1);
+	if (int rc = check_pending(mlp, "n2_mlp_backward", blocks, mode)) return rc;
 	const hf* X = reinterpret_cast<const hf*>(d_input);
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
@@ -819,7 +916,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	do {                                                                                                            \
 		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT); /* >= the fp32 parameter image laid over it */      \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
-		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, mlp->workspace); \
+		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, next_slabs(mlp)); \
 	} while (0)
 #define LAUNCH_Y(IC, NH)                                                                                            \
 	do {                                                                                                            \
@@ -886,6 +983,7 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 	}
 	if (!want_dw && !d_dL_ddLdoutput) return N2_OK;
 	const uint32_t blocks = stream_grid(n, 2);
+	if (int rc = check_pending(mlp, "n2_mlp_backward_backward_input", blocks, mode)) return rc;
 	N2ProfScope prof(N2_PROF_MLP_SECOND_ORDER, s);
 	switch (mlp->in_w / 16) {
 #define CASE(IC)                                                                                                           \
@@ -893,7 +991,7 @@ N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, con
 		if (int rc = allow_lds(mlp_bbi_kernel<IC>, frag_bytes(FragMap<IC, 1>::COUNT))) return rc;                          \
 		mlp_bbi_kernel<IC><<<dim3(blocks), dim3(MLP_BLOCK), frag_bytes(FragMap<IC, 1>::COUNT), s>>>(mlp->params, reinterpret_cast<const hf*>(d_input), n, \
 			reinterpret_cast<const hf*>(d_dL_ddLdinput), reinterpret_cast<const hf*>(d_dL_doutput), unit_row,              \
-			reinterpret_cast<hf*>(d_dL_ddLdoutput), want_dw ? mlp->workspace : nullptr);                                   \
+			reinterpret_cast<hf*>(d_dL_ddLdoutput), want_dw ? next_slabs(mlp) : nullptr);                                  \
 		break;
 		CASE(1) CASE(2) CASE(3) CASE(4)
 #undef CASE
