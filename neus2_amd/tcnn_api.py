@@ -243,6 +243,15 @@ class FullyFusedMLP:
                                                            C.c_int(out_layout), ptr(d)), "n2_mlp_forward_and_input_gradient")
         return y, d
 
+    def set_deferred_reduction(self, enable):
+        """Leave the per-workgroup weight-gradient sums of backward / backward_backward_input pending until
+        reduce_deferred (no tcnn counterpart: tcnn's weight gradients are GEMMs)."""
+        check(capi.lib().n2_mlp_set_deferred_reduction(self._h, C.c_int(1 if enable else 0)), "n2_mlp_set_deferred_reduction")
+
+    def reduce_deferred(self, other=None):
+        check(capi.lib().n2_mlp_reduce_deferred(self._h, other._h if other is not None else None, _stream()),
+              "n2_mlp_reduce_deferred")
+
     def backward_backward_input(self, x, dL_ddLdinput, dL_doutput, want_dL_ddLdoutput=False, mode=GRAD_ACCUMULATE):
         """dL_doutput None: the first-order output gradient was e_0 for every sample (the SDF's own gradient)."""
         n = x.shape[1]

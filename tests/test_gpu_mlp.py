@@ -161,3 +161,48 @@ def test_forward_and_input_gradient_equals_the_two_calls(oracle, in_w, n_hidden,
         assert torch.equal(y, y_ref) and torch.equal(d, d_ref)
         y2, d2 = gm.forward_and_input_gradient(x, dim, LAYOUT_AOS)
         assert torch.equal(y2.t().contiguous(), y_ref) and torch.equal(d2, d_ref)
+
+
+def test_deferred_reduction_sums_pending_passes_in_one_launch(oracle):
+    """backward(OVERWRITE) + second-order pass(ACCUMULATE) with the reduction deferred: the gradients appear only after
+    reduce_deferred, equal the oracle's sum, and two networks reduce in one call."""
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_OVERWRITE, LAYOUT_SOA, N2Error
+    om, gm, W, dW, dG, rng = make(oracle, 48, 1, 11)
+    om2, gm2, W2, dW2, dG2, _ = make(oracle, 32, 2, 12)
+    n = 8192 + 40
+    x = q16(rng.standard_normal((48, n)))
+    v = q16(rng.standard_normal((48, n)))
+    g = q16(rng.standard_normal((16, n)) * 0.1)
+    x2 = q16(rng.standard_normal((32, n)))
+    g2 = q16(rng.standard_normal((16, n)) * 0.1)
+    _, h = om.forward(W, x, round_hidden=True)
+    ref1 = om.backward(W, x, h, g)[1]
+    e0 = np.zeros((16, n), np.float32)
+    e0[0] = 1
+    ref2, _ = om.backward_backward_input(W, h, v, e0)
+    _, h2 = om2.forward(W2, x2, round_hidden=True)
+    ref3 = om2.backward(W2, x2, h2, g2)[1]
+    gm.set_deferred_reduction(True)
+    gm2.set_deferred_reduction(True)
+    dG.fill_(7.0)
+    dG2.fill_(7.0)
+    gm.backward(dev(x, torch.float16), dev(g, torch.float16), LAYOUT_SOA, want_input_grad=False, mode=GRAD_OVERWRITE)
+    gm.backward_backward_input(dev(x, torch.float16), dev(v, torch.float16), None, mode=GRAD_ACCUMULATE)
+    gm2.backward(dev(x2, torch.float16), dev(g2, torch.float16), LAYOUT_SOA, want_input_grad=False, mode=GRAD_OVERWRITE)
+    torch.cuda.synchronize()
+    assert (dG == 7.0).all() and (dG2 == 7.0).all()      # nothing folded yet
+    with pytest.raises(N2Error):                          # OVERWRITE cannot follow a pending pass
+        gm.backward(dev(x, torch.float16), dev(g, torch.float16), LAYOUT_SOA, want_input_grad=False, mode=GRAD_OVERWRITE)
+    with pytest.raises(N2Error):                          # nor can the switch be flipped with passes pending
+        gm.set_deferred_reduction(False)
+    gm.reduce_deferred(gm2)
+    assert_grad_close(host(dG), ref1 + ref2, what="deferred first + second order weight gradients")
+    assert_grad_close(host(dG2), ref3, what="deferred gradients of the second network")
+    # nothing pending: a second reduce is a no-op, and ACCUMULATE as first pending pass adds to the buffer
+    before = dG.clone()
+    gm.reduce_deferred()
+    assert torch.equal(before, dG)
+    gm.backward(dev(x, torch.float16), dev(g, torch.float16), LAYOUT_SOA, want_input_grad=False, mode=GRAD_ACCUMULATE)
+    gm.reduce_deferred()
+    assert_grad_close(host(dG), 2 * ref1 + ref2, what="accumulate through a deferred reduction")
+    gm.set_deferred_reduction(False)
