@@ -640,32 +640,60 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_bbi_kernel(const hf* __restr
 	if (partials) acc.write_slab(reinterpret_cast<float*>(smem), partials + (size_t)blockIdx.x * N_PARAMS, N_PARAMS, wave, role, n, g);
 }
 
-// grads (fp16) = [grads +] sum over slabs.  16 parameters x 16 slab groups per workgroup: every
-// lane adds up n_slabs/16 partial sums (coalesced across the 16 parameters), LDS folds the groups.
+// grads (fp16) = [grads +] sum over slabs.  A workgroup owns 32 consecutive parameters (one 128-byte line of every
+// slab): 8 lanes cover the line with 16-byte loads, 32 lane groups share the slabs, eight loads in flight per lane,
+// LDS folds the groups.  n_params is a multiple of 16, so lines are never ragged.
+__device__ __forceinline__ void mlp_reduce_line(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params, hf* __restrict__ grads,
+                                                int accumulate, uint32_t line, float (*fold)[33]) {
+	const uint32_t q = threadIdx.x & 7, grp = threadIdx.x >> 3;
+	const uint32_t i = line * 32 + q * 4;
+	float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+	if (i < n_params) {
+		const float* p = partials + i;
+		uint32_t k = grp;
+		for (; k + 7 * 32 < n_slabs; k += 8 * 32) {
+			float4 v[8];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(p + (size_t)(k + u * 32) * n_params);
+#pragma unroll
+			for (int u = 0; u < 8; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
+		}
+		for (; k < n_slabs; k += 32) {
+			const float4 v = *reinterpret_cast<const float4*>(p + (size_t)k * n_params);
+			acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+		}
+	}
+	fold[grp][q * 4 + 0] = acc.x;
+	fold[grp][q * 4 + 1] = acc.y;
+	fold[grp][q * 4 + 2] = acc.z;
+	fold[grp][q * 4 + 3] = acc.w;
+	__syncthreads();
+	// 8 lanes per parameter fold 4 groups each, then a shuffle tree
+	const uint32_t pl = threadIdx.x >> 3, part = threadIdx.x & 7;
+	float t = fold[part * 4][pl] + fold[part * 4 + 1][pl] + fold[part * 4 + 2][pl] + fold[part * 4 + 3][pl];
+	t += __shfl_xor(t, 1);
+	t += __shfl_xor(t, 2);
+	t += __shfl_xor(t, 4);
+	const uint32_t o = line * 32 + pl;
+	if (part == 0 && o < n_params) {
+		if (accumulate) t += (float)grads[o];
+		grads[o] = (hf)t;
+	}
+}
+
 __global__ void __launch_bounds__(256) mlp_reduce_partials_kernel(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params,
                                                                   hf* __restrict__ grads, int accumulate) {
-	// 32 consecutive parameters per workgroup (one 128-byte line of every slab), 8 groups of lanes share the slabs
-	__shared__ float fold[8][33];
-	const uint32_t pl = threadIdx.x & 31, grp = threadIdx.x >> 5;
-	const uint32_t i = blockIdx.x * 32 + pl;
-	float s0 = 0.f, s1 = 0.f;
-	if (i < n_params) {
-		uint32_t k = grp;
-		for (; k + 8 < n_slabs; k += 16) {  // two independent chains of loads
-			s0 += partials[(size_t)k * n_params + i];
-			s1 += partials[(size_t)(k + 8) * n_params + i];
-		}
-		if (k < n_slabs) s0 += partials[(size_t)k * n_params + i];
-	}
-	fold[grp][pl] = s0 + s1;
-	__syncthreads();
-	if (grp == 0 && i < n_params) {
-		float t = 0.f;
-#pragma unroll
-		for (int k = 0; k < 8; ++k) t += fold[k][pl];
-		if (accumulate) t += (float)grads[i];
-		grads[i] = (hf)t;
-	}
+	__shared__ float fold[32][33];
+	mlp_reduce_line(partials, n_slabs, n_params, grads, accumulate, blockIdx.x, fold);
+}
+
+// two parameter sets in one launch
+__global__ void __launch_bounds__(256) mlp_reduce_two_kernel(const float* __restrict__ pa, uint32_t slabs_a, uint32_t params_a, hf* __restrict__ ga, int acc_a,
+                                                             uint32_t blocks_a, const float* __restrict__ pb, uint32_t slabs_b, uint32_t params_b,
+                                                             hf* __restrict__ gb, int acc_b) {
+	__shared__ float fold[32][33];
+	if (blockIdx.x < blocks_a) mlp_reduce_line(pa, slabs_a, params_a, ga, acc_a, blockIdx.x, fold);
+	else mlp_reduce_line(pb, slabs_b, params_b, gb, acc_b, blockIdx.x - blocks_a, fold);
 }
 
 // ----------------------------------------------------------------------------
@@ -818,38 +846,6 @@ N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 	N2_REQUIRE(mlp->pending_slabs == 0, "n2_mlp_set_deferred_reduction: gradient passes are pending");
 	mlp->deferred = enable != 0;
 	return N2_OK;
-}
-
-// two parameter sets in one launch
-__global__ void __launch_bounds__(256) mlp_reduce_two_kernel(const float* __restrict__ pa, uint32_t slabs_a, uint32_t params_a, hf* __restrict__ ga, int acc_a,
-                                                             uint32_t blocks_a, const float* __restrict__ pb, uint32_t slabs_b, uint32_t params_b,
-                                                             hf* __restrict__ gb, int acc_b) {
-	__shared__ float fold[8][33];
-	const bool second = blockIdx.x >= blocks_a;
-	const float* partials = second ? pb : pa;
-	const uint32_t n_slabs = second ? slabs_b : slabs_a, n_params = second ? params_b : params_a;
-	hf* grads = second ? gb : ga;
-	const int accumulate = second ? acc_b : acc_a;
-	const uint32_t pl = threadIdx.x & 31, grp = threadIdx.x >> 5;
-	const uint32_t i = (second ? blockIdx.x - blocks_a : blockIdx.x) * 32 + pl;
-	float s0 = 0.f, s1 = 0.f;
-	if (i < n_params) {
-		uint32_t k = grp;
-		for (; k + 8 < n_slabs; k += 16) {
-			s0 += partials[(size_t)k * n_params + i];
-			s1 += partials[(size_t)(k + 8) * n_params + i];
-		}
-		if (k < n_slabs) s0 += partials[(size_t)k * n_params + i];
-	}
-	fold[grp][pl] = s0 + s1;
-	__syncthreads();
-	if (grp == 0 && i < n_params) {
-		float t = 0.f;
-#pragma unroll
-		for (int k = 0; k < 8; ++k) t += fold[k][pl];
-		if (accumulate) t += (float)grads[i];
-		grads[i] = (hf)t;
-	}
 }
 
 N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) {
