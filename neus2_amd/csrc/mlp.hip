@@ -99,21 +99,49 @@ __device__ __forceinline__ void bfrag_soa(const hf* __restrict__ M, uint32_t N, 
 	}
 }
 
+typedef short short8 __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+// fp16 rounding of eight D-tile registers starting at `base`, as four two-element conversions
+typedef float float2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ half8 round8(const float16v& d, int base) {
+	uint4v r;
+#pragma unroll
+	for (int w = 0; w < 4; ++w) {
+		const float2v p = {d[base + 2 * w], d[base + 2 * w + 1]};
+		r[w] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p, half2v));
+	}
+	return __builtin_bit_cast(half8, r);
+}
+// ReLU of rounded values as a packed 16-bit integer max with 0: every negative half (the sign bit makes it a negative
+// integer, -0 included) becomes +0, positive halves keep their bits.  relu(round(x)) == round(relu(x)).
+__device__ __forceinline__ half8 relu8(half8 v) {
+	const short8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+	return __builtin_bit_cast(half8, __builtin_elementwise_max(__builtin_bit_cast(short8, v), z));
+}
+// v where the saved activation is > 0, else 0.  Activations come out of relu8, so as 16-bit integers they are 0 or
+// positive and (0 - a) >> 15 (arithmetic) is all ones exactly for a > 0.  Written as the two packed 16-bit instructions
+// because the compiler otherwise turns the expression back into one compare and select per element.
+__device__ __forceinline__ uint32_t positive_mask2(uint32_t act_pair) {
+	uint32_t m;
+	asm("v_pk_sub_i16 %0, 0, %1\n\tv_pk_ashrrev_i16 %0, %2, %0" : "=v"(m) : "v"(act_pair), "s"(0x000F000Fu));
+	return m;
+}
+__device__ __forceinline__ half8 mask8(half8 v, half8 act) {
+	const uint4v a = __builtin_bit_cast(uint4v, act);
+	uint4v x = __builtin_bit_cast(uint4v, v);
+#pragma unroll
+	for (int w = 0; w < 4; ++w) x[w] &= positive_mask2(a[w]);
+	return __builtin_bit_cast(half8, x);
+}
 // ReLU + fp16 rounding of a D tile into the two chained B operands it holds
 __device__ __forceinline__ void relu_pack(const float16v& d, half8& lo, half8& hi) {
-#pragma unroll
-	for (int e = 0; e < 8; ++e) {
-		lo[e] = (hf)fmaxf(d[e], 0.f);
-		hi[e] = (hf)fmaxf(d[8 + e], 0.f);
-	}
+	lo = relu8(round8(d, 0));
+	hi = relu8(round8(d, 8));
 }
 // masked (by the sign of a saved activation) fp16 rounding of a D tile
 __device__ __forceinline__ void mask_pack(const float16v& d, const half8& act_lo, const half8& act_hi, half8& lo, half8& hi) {
-#pragma unroll
-	for (int e = 0; e < 8; ++e) {
-		lo[e] = (act_lo[e] > (hf)0) ? (hf)d[e] : (hf)0;
-		hi[e] = (act_hi[e] > (hf)0) ? (hf)d[8 + e] : (hf)0;
-	}
+	lo = mask8(round8(d, 0), act_lo);
+	hi = mask8(round8(d, 8), act_hi);
 }
 
 __device__ __forceinline__ float16v zero16() {
