@@ -126,6 +126,11 @@ __device__ __forceinline__ bool n2_xcd_item(const N2XcdPlan& plan, uint32_t tile
 // exchanges its partial sums and lane b finishes feature b.
 constexpr uint32_t FWD_POINTS = GRID_BLOCK / 2;  // points per workgroup and level
 
+// value held by the other lane of the pair (lane ^ 1): a quad permute [1, 0, 3, 2] inside the VALU, no LDS crossbar
+__device__ __forceinline__ float n2_pair_swap(float x) {
+	return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
+}
+
 template <uint32_t MODE, bool WANT_DYDX>
 __device__ __forceinline__ void grid_forward_pair(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t b, uint32_t N,
                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
@@ -151,14 +156,14 @@ __device__ __forceinline__ void grid_forward_pair(const N2LevelTable& tab, uint3
 		tz.y = fmaf(uy, v[2].y - v[0].y, wy * (v[3].y - v[1].y));
 	}
 	// lane b keeps feature b of its own plane and receives feature b of the partner's plane
-	const float s_mine = b ? s.y : s.x, s_other = __shfl_xor(b ? s.x : s.y, 1);
+	const float s_mine = b ? s.y : s.x, s_other = n2_pair_swap(b ? s.x : s.y);
 	const float s_lo = b ? s_other : s_mine, s_hi = b ? s_mine : s_other;  // x corner 0 / 1
 	const float wx = p.w[0], ux = 1.f - wx;
 	const size_t row = (size_t)level * 2 + b;
 	out[row * N + i] = __float2half_rn(fmaf(ux, s_lo, wx * s_hi));
 	if (WANT_DYDX) {
-		const float ty_mine = b ? ty.y : ty.x, ty_other = __shfl_xor(b ? ty.x : ty.y, 1);
-		const float tz_mine = b ? tz.y : tz.x, tz_other = __shfl_xor(b ? tz.x : tz.y, 1);
+		const float ty_mine = b ? ty.y : ty.x, ty_other = n2_pair_swap(b ? ty.x : ty.y);
+		const float tz_mine = b ? tz.y : tz.x, tz_other = n2_pair_swap(b ? tz.x : tz.y);
 		const float w_mine = b ? wx : ux, w_other = b ? ux : wx;
 		float* j = dy_dx + (row * N + i) * 3;
 		j[0] = (s_hi - s_lo) * scale;
@@ -271,7 +276,7 @@ __device__ __forceinline__ void grid_scatter_pair(const N2LevelTable& tab, uint3
 	}
 	if (SECOND && WANT_OUT) {
 		// lane b finishes feature b: it needs the partner's partial sum of that feature
-		const float mine = b ? o1 : o0, theirs = __shfl_xor(b ? o0 : o1, 1);
+		const float mine = b ? o1 : o0, theirs = n2_pair_swap(b ? o0 : o1);
 		dL_ddLdy[(row + b) * N + i] = __float2half_rn(mine + theirs);
 	}
 }
