@@ -81,6 +81,26 @@ int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolutio
  * Results do not depend on it. */
 int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs);
 
+/* Level mask of the grid encoding.
+ *  - n2_grid_set_max_level: GridEncoding::set_max_level as driven by Testbed::set_max_level (src/testbed.cu:1861-1866,
+ *    2618): max_level is the fraction of the levels in use, 1 = all.  Level l is switched off when
+ *    l >= (max_level * n_levels * n_features) / n_features + 1e-3 (fp32, tcnn's arithmetic): its output features and
+ *    dy_dx are zero, it receives no parameter gradient and its dL_ddLdy rows are zero.
+ *  - n2_grid_set_max_level_gpu: set_max_level_gpu (src/testbed_nerf.cu:3837, 3843, 3985): one fraction per point
+ *    (device pointer, n_points floats, read by every later call until reset with NULL) replaces the global one;
+ *    the reference fills it with random_val * 2 per ray when max_level_rand_training is on (:1305, 1440-1444).
+ *  - n2_grid_set_progressive + n2_grid_set_training_step: the encoding keys valid_level_scale, base_valid_level_scale,
+ *    base_training_step (configs/nerf/base.json:36-38) and Encoding::set_training_step (src/testbed.cu:2643-2646).
+ *    The arithmetic lives in the tcnn fork, which the reference tree does not hold: PARITY UNPINNED.  Implemented as
+ *    levels_in_use = clamp(floor(n_levels * (base_valid_level_scale + valid_level_scale * (step / base_training_step))
+ *    + 1e-3), 1, n_levels), with an integer division; base_training_step 0 (the default) switches the mask off.
+ *  - n2_grid_active_levels: levels in use under the global settings (per-point fractions not counted). */
+int n2_grid_set_max_level(n2_grid_t* grid, float max_level);
+int n2_grid_set_max_level_gpu(n2_grid_t* grid, const float* d_max_level);
+int n2_grid_set_progressive(n2_grid_t* grid, float base_valid_level_scale, float valid_level_scale, uint32_t base_training_step);
+int n2_grid_set_training_step(n2_grid_t* grid, uint32_t training_step);
+uint32_t n2_grid_active_levels(const n2_grid_t* grid);
+
 /* Encoding::set_params(params, inference_params, backward_params, gradients),
  * nerf_network.h:746-753.  One fp16 parameter buffer (n_params) and one fp16
  * gradient buffer (n_params, may be NULL until a backward needs it). */
@@ -261,6 +281,9 @@ typedef struct n2_field_config {
 int n2_field_create(const n2_field_config* config, n2_field_t** out);
 void n2_field_destroy(n2_field_t* field);
 
+/* The field's grid encoding (NerfNetwork::encoding(), used at src/testbed.cu:2643-2646 and src/testbed_nerf.cu:3837):
+ * owned by the field; for the level-mask setters above. */
+n2_grid_t* n2_field_encoding(n2_field_t* field);
 uint32_t n2_field_n_params(const n2_field_t* field);
 /* Offsets of the five segments [sdf mlp, colour mlp, grid, variance, end] in the parameter
  * vector; everything before offsets[2] is a matrix parameter for the optimiser

@@ -108,6 +108,15 @@ public:
 	void set_params(half_t* params, half_t* /*inference_params*/, half_t* /*backward_params*/, half_t* gradients) {
 		check(n2_grid_set_params(m_grid, params, gradients), "GridEncoding::set_params");
 	}
+	// level mask (GridEncoding::set_max_level / set_max_level_gpu, Encoding::set_training_step)
+	void set_max_level(float value) { check(n2_grid_set_max_level(m_grid, value), "GridEncoding::set_max_level"); }
+	void set_max_level_gpu(const float* d_value) { check(n2_grid_set_max_level_gpu(m_grid, d_value), "GridEncoding::set_max_level_gpu"); }
+	void set_progressive(float base_valid_level_scale, float valid_level_scale, uint32_t base_training_step) {
+		check(n2_grid_set_progressive(m_grid, base_valid_level_scale, valid_level_scale, base_training_step), "GridEncoding::set_progressive");
+	}
+	void set_training_step(int training_step) {
+		check(n2_grid_set_training_step(m_grid, training_step < 0 ? 0u : (uint32_t)training_step), "GridEncoding::set_training_step");
+	}
 	// scratch of the parameter-gradient scatter (tcnn: arena temporaries)
 	size_t workspace_bytes(uint32_t max_points) const { return n2_grid_workspace_bytes(m_grid, max_points); }
 	void set_workspace(void* d_workspace, size_t n_bytes, uint32_t max_points) {

@@ -83,7 +83,9 @@ def lib():
         _lib = C.CDLL(LIB_PATH)
         _lib.n2_last_error.restype = C.c_char_p
         _lib.n2_version.restype = C.c_char_p
-        for name in ("n2_grid_n_params", "n2_grid_output_width", "n2_grid_n_levels"):
+        _lib.n2_field_encoding.restype = C.c_void_p
+        _lib.n2_field_encoding.argtypes = [C.c_void_p]
+        for name in ("n2_grid_n_params", "n2_grid_output_width", "n2_grid_n_levels", "n2_grid_active_levels"):
             getattr(_lib, name).restype = C.c_uint32
             getattr(_lib, name).argtypes = [C.c_void_p]
         _lib.n2_grid_workspace_bytes.restype = C.c_uint64

@@ -266,6 +266,7 @@ N2_API void n2_field_destroy(n2_field_t* f) {
 	delete f;
 }
 
+N2_API n2_grid_t* n2_field_encoding(n2_field_t* field) { return field ? field->grid : nullptr; }
 N2_API uint32_t n2_field_n_params(const n2_field_t* f) { return f ? f->n_params : 0; }
 
 N2_API int n2_field_param_offsets(const n2_field_t* f, uint32_t offsets[5]) {

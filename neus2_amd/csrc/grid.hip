@@ -24,6 +24,9 @@ struct n2_grid {
 	__half2* grads;
 	// relative cost of one tile of each level (balances the levels over the XCDs)
 	float level_cost[N2_MAX_LEVELS];
+	// progressive training (base_training_step 0: off)
+	float base_valid_level_scale, valid_level_scale;
+	uint32_t base_training_step;
 	// optional scratch of the bucketed scatter
 	unsigned char* ws;
 	uint64_t ws_bytes;
@@ -42,6 +45,14 @@ __device__ __forceinline__ void n2_locate(float x, float scale, float& w, uint32
 	const float f = floorf(p);
 	cell = (uint32_t)(int32_t)f;
 	w = p - f;
+}
+
+// Level mask of tcnn's grid encoding: the limit is (max_level * n_output_features) / n_features_per_level in fp32
+// and a level is off when level >= limit + 1e-3; the progressive mask adds level >= valid_levels.
+__device__ __forceinline__ bool n2_level_masked(const N2LevelTable& tab, uint32_t level, uint32_t i) {
+	const float fraction = tab.max_level_gpu ? tab.max_level_gpu[i] : tab.max_level;
+	const float limit = (fraction * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
+	return (float)level >= limit + 1e-3f || level >= tab.valid_levels;
 }
 
 template <uint32_t MODE>
@@ -139,6 +150,15 @@ __device__ __forceinline__ void grid_forward_pair(const N2LevelTable& tab, uint3
 	const float scale = tab.scale[level];
 	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
 	const __half2* P = params + tab.offset[level];
+	const size_t row = (size_t)level * 2 + b;
+	if (n2_level_masked(tab, level, i)) {  // both lanes of a pair share i
+		out[row * N + i] = __float2half_rn(0.f);
+		if (WANT_DYDX) {
+			float* j = dy_dx + (row * N + i) * 3;
+			j[0] = 0.f; j[1] = 0.f; j[2] = 0.f;
+		}
+		return;
+	}
 	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
 	const uint32_t gx = p.c[0] + b;
 	float2 v[4];
@@ -159,7 +179,6 @@ __device__ __forceinline__ void grid_forward_pair(const N2LevelTable& tab, uint3
 	const float s_mine = b ? s.y : s.x, s_other = n2_pair_swap(b ? s.x : s.y);
 	const float s_lo = b ? s_other : s_mine, s_hi = b ? s_mine : s_other;  // x corner 0 / 1
 	const float wx = p.w[0], ux = 1.f - wx;
-	const size_t row = (size_t)level * 2 + b;
 	out[row * N + i] = __float2half_rn(fmaf(ux, s_lo, wx * s_hi));
 	if (WANT_DYDX) {
 		const float ty_mine = b ? ty.y : ty.x, ty_other = n2_pair_swap(b ? ty.x : ty.y);
@@ -231,8 +250,12 @@ __device__ __forceinline__ void grid_scatter_pair(const N2LevelTable& tab, uint3
                                                   __half2* __restrict__ grads, __half* __restrict__ dL_ddLdy) {
 	const float scale = tab.scale[level];
 	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
-	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
 	const size_t row = (size_t)level * 2;
+	if (n2_level_masked(tab, level, i)) {  // both lanes of a pair share i
+		if (SECOND && WANT_OUT) dL_ddLdy[(row + b) * N + i] = __float2half_rn(0.f);
+		return;
+	}
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
 	float a0 = 0.f, a1 = 0.f, c0 = 0.f, c1 = 0.f, v0 = 0.f, v1 = 0.f, v2 = 0.f;
 	if (FIRST) {
 		a0 = __half2float(dL_dy[row * N + i]);
@@ -327,10 +350,17 @@ __device__ __forceinline__ void grid_bbi_point(const N2LevelTable& tab, uint32_t
                                                const __half2* __restrict__ params, __half2* __restrict__ grads,
                                                __half* __restrict__ dL_ddLdy, float* __restrict__ dL_dx) {
 	const float scale = tab.scale[level];
+	const size_t row = (size_t)level * 2;
+	if (n2_level_masked(tab, level, i)) {
+		if (dL_ddLdy) {
+			dL_ddLdy[row * N + i] = __float2half_rn(0.f);
+			dL_ddLdy[(row + 1) * N + i] = __float2half_rn(0.f);
+		}
+		return;
+	}
 	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
 	uint32_t e[8];
 	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
-	const size_t row = (size_t)level * 2;
 	const float v0 = v[i] * scale, v1 = v[(size_t)N + i] * scale, v2 = v[(size_t)2 * N + i] * scale;
 	const float g0 = __half2float(dL_dy[row * N + i]);
 	const float g1 = __half2float(dL_dy[(row + 1) * N + i]);
@@ -513,7 +543,14 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
 		const uint32_t i = tile * BIN_POINTS + j * BIN_BLOCK + threadIdx.x;
-		const bool valid = i < N;
+		bool valid = i < N;
+		if (valid && n2_level_masked(tab, level, i)) {  // a switched-off level: no records, zero second-order output
+			valid = false;
+			if (SECOND && WANT_OUT) {
+				dL_ddLdy[(size_t)level * 2 * N + i] = __float2half_rn(0.f);
+				dL_ddLdy[((size_t)level * 2 + 1) * N + i] = __float2half_rn(0.f);
+			}
+		}
 		uint32_t e[8], cell[3] = {0, 0, 0};
 		float r0[8], r1[8];
 #pragma unroll
@@ -763,6 +800,13 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	N2_REQUIRE(g != nullptr, "n2_grid_create: out of host memory");
 	g->n_features = n_features_per_level;
 	g->tab.n_levels = n_levels;
+	g->tab.n_features = n_features_per_level;
+	g->tab.max_level = 1.0f;
+	g->tab.max_level_gpu = nullptr;
+	g->tab.valid_levels = n_levels;
+	g->base_valid_level_scale = 1.0f;
+	g->valid_level_scale = 0.0f;
+	g->base_training_step = 0;
 	uint64_t off = 0;
 	const float log2_b = std::log2(per_level_scale);
 	for (uint32_t l = 0; l < n_levels; ++l) {
@@ -823,6 +867,53 @@ N2_API int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs) {
 	}
 	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) grid->level_cost[l] = costs[l];
 	return N2_OK;
+}
+
+N2_API int n2_grid_set_max_level(n2_grid_t* grid, float max_level) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_max_level: grid is null");
+	N2_REQUIRE(max_level >= 0.f && max_level <= 1000.f, "n2_grid_set_max_level: max_level %g outside [0, 1000]", (double)max_level);
+	grid->tab.max_level = max_level;
+	return N2_OK;
+}
+
+N2_API int n2_grid_set_max_level_gpu(n2_grid_t* grid, const float* d_max_level) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_max_level_gpu: grid is null");
+	grid->tab.max_level_gpu = d_max_level;
+	return N2_OK;
+}
+
+N2_API int n2_grid_set_progressive(n2_grid_t* grid, float base_valid_level_scale, float valid_level_scale, uint32_t base_training_step) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_progressive: grid is null");
+	N2_REQUIRE(base_valid_level_scale >= 0.f && valid_level_scale >= 0.f, "n2_grid_set_progressive: scales must be >= 0");
+	grid->base_valid_level_scale = base_valid_level_scale;
+	grid->valid_level_scale = valid_level_scale;
+	grid->base_training_step = base_training_step;
+	if (base_training_step == 0) grid->tab.valid_levels = grid->tab.n_levels;
+	return N2_OK;
+}
+
+// levels in use at a training step: the fraction base + scale * (step / base_training_step), whole periods only,
+// of all levels, rounded down (after + 1e-3, so that a fraction that reaches 1 up to rounding gives every level),
+// at least one level and at most all of them
+N2_API int n2_grid_set_training_step(n2_grid_t* grid, uint32_t training_step) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_training_step: grid is null");
+	if (grid->base_training_step == 0) return N2_OK;
+	const float fraction = grid->base_valid_level_scale + grid->valid_level_scale * (float)(training_step / grid->base_training_step);
+	const float levels = fraction * (float)grid->tab.n_levels + 1e-3f;
+	uint32_t n = levels >= (float)grid->tab.n_levels ? grid->tab.n_levels : (uint32_t)levels;
+	if (n < 1) n = 1;
+	grid->tab.valid_levels = n;
+	return N2_OK;
+}
+
+N2_API uint32_t n2_grid_active_levels(const n2_grid_t* grid) {
+	if (!grid) return 0;
+	uint32_t n = 0;
+	const N2LevelTable& tab = grid->tab;
+	const float limit = (tab.max_level * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
+	for (uint32_t l = 0; l < tab.n_levels; ++l)
+		if (!((float)l >= limit + 1e-3f || l >= tab.valid_levels)) ++n;
+	return n;
 }
 
 N2_API int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients) {

@@ -51,6 +51,12 @@ struct N2LevelTable {
 	uint32_t offset[N2_MAX_LEVELS + 1];
 	uint32_t mode[N2_MAX_LEVELS];
 	uint32_t n_levels;
+	// level mask: level l is switched off (zero output, zero derivatives, no gradient) for point i when
+	//   l >= max_level * n_levels + 1e-3   (max_level = max_level_gpu[i] when that pointer is set)   or   l >= valid_levels
+	float max_level;               // fraction of the levels in use, 1 = all
+	const float* max_level_gpu;    // per point, or null
+	uint32_t valid_levels;         // progressive training: number of levels switched on so far
+	uint32_t n_features;
 };
 
 static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }

@@ -287,6 +287,8 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	hipStream_t s = n2_stream(stream);
 	const uint32_t T = t->cfg.target_batch_size;
 	uint32_t* compacted_counter = t->counters + 2;
+	// progressive level mask: the encoding is told the number of steps taken so far before every step
+	if (int rc = n2_grid_set_training_step(n2_field_encoding(t->field), t->optimizer_steps)) return rc;
 	auto sample = [&](n2_trainer::SampleSet& set, hipStream_t on, uint32_t ray_base, uint32_t sd) {
 		// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
 		return n2_generate_training_samples(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,

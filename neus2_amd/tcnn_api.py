@@ -44,10 +44,21 @@ class GridEncoding:
                                         C.c_float(per_level_scale), C.byref(self._h)), "n2_grid_create")
         self.n_levels = n_levels
         self._params = self._grads = None
+        self._owner = None
+
+    @classmethod
+    def _borrowed(cls, handle, owner):
+        """A view of a grid that another object owns (NerfNetwork.encoding()): never destroyed from here."""
+        g = cls.__new__(cls)
+        g._h = C.c_void_p(handle)
+        g._owner = owner
+        g._params = g._grads = None
+        g.n_levels = int(capi.lib().n2_grid_n_levels(g._h))
+        return g
 
     def __del__(self):
         try:
-            if getattr(self, "_h", None) is not None and self._h.value:
+            if getattr(self, "_owner", None) is None and getattr(self, "_h", None) is not None and self._h.value:
                 capi.lib().n2_grid_destroy(self._h)
                 self._h = C.c_void_p()
         except Exception:  # interpreter shutdown: the module globals may already be gone
@@ -79,6 +90,29 @@ class GridEncoding:
                 raise N2Error("grid params/gradients must be contiguous fp16 CUDA tensors of n_params elements")
         check(capi.lib().n2_grid_set_params(self._h, ptr(params), ptr(gradients)), "n2_grid_set_params")
         self._params, self._grads = params, gradients
+
+    def set_max_level(self, value):
+        """Fraction of the levels in use (GridEncoding::set_max_level, src/testbed.cu:1861-1866); 1 = all."""
+        check(capi.lib().n2_grid_set_max_level(self._h, C.c_float(value)), "n2_grid_set_max_level")
+
+    def set_max_level_gpu(self, per_point):
+        """One fraction per point (fp32 CUDA tensor, kept alive here) or None (src/testbed_nerf.cu:3837-3843, 3985)."""
+        if per_point is not None and (per_point.dtype != torch.float32 or not per_point.is_cuda or not per_point.is_contiguous()):
+            raise N2Error("max_level_gpu must be a contiguous fp32 CUDA tensor")
+        check(capi.lib().n2_grid_set_max_level_gpu(self._h, ptr(per_point)), "n2_grid_set_max_level_gpu")
+        self._max_level_gpu = per_point
+
+    def set_progressive(self, base_valid_level_scale, valid_level_scale, base_training_step):
+        """Encoding keys of configs/nerf/base.json:36-38; base_training_step 0 switches the progressive mask off."""
+        check(capi.lib().n2_grid_set_progressive(self._h, C.c_float(base_valid_level_scale), C.c_float(valid_level_scale),
+                                                 C.c_uint32(base_training_step)), "n2_grid_set_progressive")
+
+    def set_training_step(self, step):
+        """Encoding::set_training_step (src/testbed.cu:2643-2646)."""
+        check(capi.lib().n2_grid_set_training_step(self._h, C.c_uint32(max(0, int(step)))), "n2_grid_set_training_step")
+
+    def active_levels(self):
+        return int(capi.lib().n2_grid_active_levels(self._h))
 
     def reserve_scatter_workspace(self, max_points):
         """Scratch that lets backward passes of >= 4096 points sort their updates in LDS instead of issuing
@@ -290,6 +324,10 @@ class NerfNetwork:
 
     def n_params(self):
         return int(capi.lib().n2_field_n_params(self._h))
+
+    def encoding(self):
+        """The field's grid encoding (NerfNetwork::encoding(), src/testbed.cu:2643-2646), for the level-mask setters."""
+        return GridEncoding._borrowed(capi.lib().n2_field_encoding(self._h), self)
 
     def param_offsets(self):
         o = (C.c_uint32 * 5)()

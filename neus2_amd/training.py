@@ -228,6 +228,12 @@ class Trainer:
     def _stream(self):
         return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
+    def encoding(self):
+        """The field's grid encoding (m_nerf_network->encoding(), src/testbed.cu:2643-2646): set_progressive /
+        set_max_level live there; every step tells it the number of steps taken so far."""
+        from .tcnn_api import GridEncoding
+        return GridEncoding._borrowed(capi.lib().n2_field_encoding(self._field), self)
+
     def set_parameters(self, master_np):
         self.master.copy_(torch.from_numpy(np.ascontiguousarray(master_np, np.float32)).to(self.master.device))
         check(capi.lib().n2_trainer_sync_params(self._h, self._stream()), "n2_trainer_sync_params")

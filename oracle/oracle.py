@@ -117,6 +117,33 @@ class Grid:
         return grad, out, din
 
 
+def level_mask(n_levels, n_points, max_level=1.0, valid_levels=None, n_features=2):
+    """bool [n_levels, n_points], True where a level is switched OFF.  tcnn's grid kernels (NVlabs tiny-cuda-nn
+    include/tiny-cuda-nn/encodings/grid.h, kernel_grid: "max_level = (max_level * num_grid_features) /
+    N_FEATURES_PER_LEVEL; if (level >= max_level + 1e-3f) -> zeros"), driven from src/testbed.cu:1861-1866 (global
+    fraction) and src/testbed_nerf.cu:1305, 1440-1444, 3837-3843 (one fraction per point); ``valid_levels`` adds the
+    progressive cut level >= valid_levels."""
+    frac = np.broadcast_to(np.asarray(max_level, np.float32), (n_points,))
+    limit = (frac * np.float32(n_levels * n_features)) / np.float32(n_features)
+    lv = np.arange(n_levels, dtype=np.float32)[:, None]
+    off = lv >= (limit[None, :] + np.float32(1e-3))
+    if valid_levels is not None:
+        off = off | (np.arange(n_levels)[:, None] >= valid_levels)
+    return off
+
+
+def progressive_levels(n_levels, base_valid_level_scale, valid_level_scale, base_training_step, step):
+    """Levels in use at a training step under the encoding keys of configs/nerf/base.json:36-38.  PARITY UNPINNED:
+    the arithmetic is in the tcnn fork the reference tree does not hold; this is the reading this build adopted
+    (fraction = base + scale * (step // base_training_step), floor(fraction * n_levels + 1e-3) clamped to
+    [1, n_levels]; the 1e-3 keeps a fraction that reaches 1 up to rounding from losing the last level)."""
+    if base_training_step == 0:
+        return n_levels
+    frac = np.float32(base_valid_level_scale) + np.float32(valid_level_scale) * np.float32(step // base_training_step)
+    lv = np.float32(frac) * np.float32(n_levels) + np.float32(1e-3)
+    return int(min(n_levels, max(1, int(np.floor(lv))))) if lv < n_levels else n_levels
+
+
 class Mlp:
     def __init__(self, in_width, width, n_hidden, out_width):
         self.in_w, self.width, self.n_hidden, self.out_w = in_width, width, n_hidden, out_width

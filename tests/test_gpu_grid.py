@@ -281,3 +281,88 @@ def test_sorted_scatter_path(oracle, kind):
     gg.backward(None, d_xyz, d_dy, mode=GRAD_OVERWRITE)
     got = host(dg)
     assert (got[ref1 == 0] == 0).all()
+
+
+def _level_tols(og, n):
+    return [RTOL * max(1.0, np.sqrt(8.0 * n / max(1, int(og.entries[l])))) for l in range(og.n_levels)]
+
+
+@pytest.mark.parametrize("kind", ["global", "per_point", "progressive"])
+@pytest.mark.parametrize("bucketed", [False, True])
+def test_level_mask(setup, oracle, kind, bucketed):
+    """Switched-off levels: zero features and dy_dx, no gradient, zero dL_ddLdy rows; everything else as unmasked.
+    Expected values = the oracle on inputs whose switched-off (level, point) rows are zeroed."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE
+    og, gg, params, d_params, d_grads = setup
+    n = 3 * 4096 + 40 if bucketed else 3000
+    rng = np.random.default_rng(77)
+    xyz = rng.random((3, n), dtype=np.float32)
+    dy = q16(rng.standard_normal((32, n)))
+    g2 = q16(rng.standard_normal((32, n)) * 0.1)
+    v = (rng.standard_normal((3, n)) * 1e-3).astype(np.float32)
+    keep = None
+    try:
+        if bucketed:
+            assert gg.reserve_scatter_workspace(1 << 14)
+        if kind == "global":
+            gg.set_max_level(0.5)
+            assert gg.active_levels() == 9
+            off = oracle.level_mask(16, n, 0.5)
+        elif kind == "per_point":
+            frac = (rng.random(n) * 2).astype(np.float32)  # the reference draws random_val * 2 per ray
+            keep = dev(frac)
+            gg.set_max_level_gpu(keep)
+            off = oracle.level_mask(16, n, frac)
+            assert 0.2 < off.mean() < 0.4
+        else:
+            gg.set_progressive(0.2, 0.02, 100)
+            gg.set_training_step(1234)
+            want = oracle.progressive_levels(16, 0.2, 0.02, 100, 1234)
+            assert gg.active_levels() == want == 7
+            off = oracle.level_mask(16, n, 1.0, valid_levels=want)
+        off_rows = np.repeat(off, 2, axis=0)
+        ref_y, ref_j = og.forward(params, xyz, want_dy_dx=True)
+        ref_y[off_rows] = 0
+        ref_j[off_rows] = 0
+        d_xyz = dev(xyz)
+        y, ctx = gg.forward(d_xyz, prepare_input_gradients=True)
+        assert_close(host(y), ref_y, what="masked grid output")
+        assert_close(host(ctx), ref_j, rtol=1e-4, what="masked dy_dx")
+        assert (host(y)[off_rows] == 0).all() and (host(ctx)[off_rows] == 0).all()
+        dy_m, g2_m = dy.copy(), g2.copy()
+        dy_m[off_rows] = 0
+        g2_m[off_rows] = 0
+        ref1, ref_dx = og.backward(params, xyz, dy_m)
+        ref, ref_out, _ = og.backward_backward_input(params, xyz, v, g2_m, grad=ref1.copy(), want_dinput=False)
+        ref_out[off_rows] = 0
+        d_grads.fill_(5.0)
+        dx = gg.backward(ctx, d_xyz, dev(dy, torch.float16), want_input_grad=True, mode=GRAD_OVERWRITE)
+        assert_close(host(dx), ref_dx, rtol=1e-4, what="masked dL_dx")
+        got1 = host(d_grads)
+        d_grads.fill_(5.0)
+        out = gg.backward_fused(d_xyz, dev(dy, torch.float16), dev(v), dev(g2, torch.float16), mode=GRAD_OVERWRITE)
+        got = host(d_grads)
+        assert_close(host(out), ref_out, what="masked dL_ddLdy")
+        assert (host(out)[off_rows] == 0).all()
+        for l, tol in enumerate(_level_tols(og, n)):
+            a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+            for g, r, what in ((got1, ref1, "first order"), (got, ref, "fused")):
+                if np.abs(r[a:b]).max() == 0:
+                    assert (g[a:b] == 0).all(), (what, l)  # a level nobody uses: Overwrite leaves zeros
+                else:
+                    assert rel_l2(g[a:b], r[a:b]) < tol, (what, l, rel_l2(g[a:b], r[a:b]), tol)
+        # the second-order kernel that also returns dL_dx
+        out2, din = gg.backward_backward_input(d_xyz, dev(v), dev(g2, torch.float16), want_dL_ddLdy=True, want_dL_dx=True,
+                                               mode=GRAD_OVERWRITE)
+        _, _, ref_din = og.backward_backward_input(params, xyz, v, g2_m)
+        assert_close(host(out2), ref_out, what="masked dL_ddLdy (dL_dx variant)")
+        assert_close(host(din), ref_din, rtol=1e-3, what="masked second-order dL_dx")
+    finally:
+        gg.set_max_level(1.0)
+        gg.set_max_level_gpu(None)
+        gg.set_progressive(1.0, 0.0, 0)
+        if bucketed:
+            from neus2_amd import capi
+            import ctypes as C
+            capi.lib().n2_grid_set_workspace(gg._h, None, C.c_uint64(0), C.c_uint32(0))
+    assert gg.active_levels() == 16

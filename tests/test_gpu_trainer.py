@@ -146,3 +146,28 @@ def test_samples_generated_ahead_give_the_same_steps():
         assert abs(a["loss"] - b["loss"]) <= 0.01 * abs(a["loss"]) + 1e-6
     assert cos_sim(m_a - m_a.mean(), m_b - m_b.mean()) > 0.999
     assert np.abs(m_a - m_b).max() < 2e-2
+
+
+def test_progressive_level_mask_follows_the_step_count(oracle):
+    """With the progressive keys set, every step tells the encoding how many steps were taken before it: the levels
+    not yet switched on receive exactly zero gradient, the others do receive some."""
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    cams = scene.cameras_on_sphere(8, 96)
+    T = 4096
+    tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=2048, max_samples=16 * T, background=(1.0, 1.0, 1.0)))
+    tr.set_scene(pack_cameras(cams), len(cams), dev(scene.render_sphere_images(cams)), dev(scene.sphere_bitfield()))
+    tr.initialize_params(seed=5, sdf_mlp_weights=None)
+    enc = tr.encoding()
+    enc.set_progressive(0.25, 0.125, 2)          # 4 levels, two more every 2 steps
+    _, _, entries, offset = enc.level_table()
+    g0 = tr.offsets[2]
+    for step in range(5):
+        tr.step(n_rays=300, n_inference=16 * T, seed=step)
+        want = oracle.progressive_levels(16, 0.25, 0.125, 2, step)
+        assert enc.active_levels() == want == 4 + 2 * (step // 2)
+        g = host(tr.grads)[g0:g0 + 2 * int(offset[-1])]
+        assert np.abs(g[:2 * int(offset[want])]).max() > 0
+        assert (g[2 * int(offset[want]):] == 0).all()
+    enc.set_progressive(1.0, 0.0, 0)
+    assert enc.active_levels() == 16

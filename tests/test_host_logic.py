@@ -99,3 +99,26 @@ def test_ema_oracle_closed_forms(oracle):
         k = np.arange(1, t + 1)
         want = ((1 - decay) * decay ** (t - k)[:, None] * ws[:t].astype(np.float64)).sum(0) / (1 - decay ** t)
         np.testing.assert_allclose(tmp, want, rtol=1e-5, atol=1e-6)
+
+
+def test_level_mask_closed_forms(oracle):
+    """tcnn's cut: level >= fraction * n_levels + 1e-3, so a level EQUAL to the limit stays on.  Fractions 0, 1/2, 1
+    and > 1 on 16 and 14 levels."""
+    m = oracle.level_mask(16, 1, 1.0)
+    assert not m.any()
+    assert oracle.level_mask(16, 1, 0.5)[:, 0].tolist() == [False] * 9 + [True] * 7
+    assert oracle.level_mask(16, 1, 0.0)[:, 0].tolist() == [False] + [True] * 15     # level 0 survives: 0 < 0 + 1e-3
+    assert not oracle.level_mask(14, 1, 1.7).any()
+    assert oracle.level_mask(14, 1, 0.25)[:, 0].sum() == 10                           # limit 3.5: levels 0..3 stay
+    per_point = oracle.level_mask(16, 3, np.array([0.0, 0.5, 2.0], np.float32))
+    assert per_point.sum(0).tolist() == [15, 7, 0]
+    assert oracle.level_mask(16, 2, 1.0, valid_levels=3).sum(0).tolist() == [13, 13]
+
+
+def test_progressive_levels_schedule(oracle):
+    """base.json: 14 levels, base 0.2, +0.02 per 100 steps -> 2 levels at the start, all 14 from step 4000 on."""
+    f = lambda step: oracle.progressive_levels(14, 0.2, 0.02, 100, step)
+    assert f(0) == 2 and f(99) == 2 and f(100) == 3 and f(4000) == 14 and f(10 ** 6) == 14
+    steps = [f(s) for s in range(0, 5000, 100)]
+    assert steps == sorted(steps)
+    assert oracle.progressive_levels(16, 0.2, 0.02, 0, 5) == 16   # base_training_step 0: off
