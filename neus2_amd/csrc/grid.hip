@@ -436,9 +436,12 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bbi_kernel(N2LevelTable tab, 
 // Accumulation is fp32 until the single rounding to fp16 at the store, which
 // also removes the rounding drift of chained fp16 atomics.
 // ----------------------------------------------------------------------------
-constexpr uint32_t BKT_ENTRIES = 8192;   // entries per bucket: 64 KiB of fp32 pairs in LDS
-constexpr uint32_t BKT_SHIFT = 13;
-constexpr uint32_t BKT_MAX = 64;         // buckets per level (entries <= 2^19)
+#ifndef N2_BKT_SHIFT
+#define N2_BKT_SHIFT 12
+#endif
+constexpr uint32_t BKT_SHIFT = N2_BKT_SHIFT;           // 4096 entries per bucket: a 64 KiB accumulator image, two reduce workgroups per CU
+constexpr uint32_t BKT_ENTRIES = 1u << BKT_SHIFT;
+constexpr uint32_t BKT_MAX = (1u << 19) >> BKT_SHIFT;  // buckets per level (entries <= 2^19)
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
 constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
 constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: two workgroups (2 x 64 KiB staging) keep 4 waves on every SIMD
@@ -596,16 +599,21 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 		}
 	}
 	__syncthreads();
-	if (threadIdx.x < 64) {  // one wave scans the 64 counters
-		const uint32_t c = hist[threadIdx.x];
-		uint32_t s = c;
+	if (threadIdx.x < 64) {  // one wave scans the counters, BKT_MAX / 64 consecutive ones per lane
+		constexpr uint32_t PER = BKT_MAX / 64;
+		uint32_t c[PER], s = 0;
+#pragma unroll
+		for (uint32_t q = 0; q < PER; ++q) { c[q] = hist[threadIdx.x * PER + q]; s += c[q]; }
+		const uint32_t own = s;
 #pragma unroll
 		for (int o = 1; o < 64; o <<= 1) {
 			const uint32_t u = __shfl_up(s, o);
 			if ((int)threadIdx.x >= o) s += u;
 		}
-		prefix[threadIdx.x] = s - c;
-		if (threadIdx.x == 63) prefix[64] = s;
+		uint32_t run = s - own;
+#pragma unroll
+		for (uint32_t q = 0; q < PER; ++q) { prefix[threadIdx.x * PER + q] = run; run += c[q]; }
+		if (threadIdx.x == 63) prefix[BKT_MAX] = s;
 	}
 	__syncthreads();
 #pragma unroll
@@ -619,7 +627,7 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 		}
 	}
 	__syncthreads();
-	const uint32_t total = prefix[64];
+	const uint32_t total = prefix[BKT_MAX];
 	uint2* out = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
 	for (uint32_t t = threadIdx.x; t < total; t += BIN_BLOCK) out[t] = staging[t];
 	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
@@ -629,9 +637,12 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 // ~5.5 (64-bit) lanes per clock.  The reduce therefore accumulates in 64-bit fixed point: a record holds
 // fp16 values, i.e. multiples of 2^-24 below 2^16, so value * 2^32 is an exact integer below 2^48 and the
 // sum of a whole bucket stays far inside 64 bits.  The accumulation is exact and independent of order.
-constexpr uint32_t RED_BLOCK = 1024;              // 16 waves; the 128 KiB table allows one workgroup per CU
-constexpr uint32_t RED_CHUNK = 2048;              // tiles whose runs are gathered per pass
-constexpr uint32_t RED_PER_THREAD = RED_CHUNK / RED_BLOCK;
+constexpr uint32_t RED_BLOCK = 1024;              // 16 waves; two workgroups share a CU
+constexpr uint32_t RED_ITEMS = (BKT_SHIFT == 13) ? 4 : 2;  // items a wave has in flight per fetch
+constexpr uint32_t ITEM_SHIFT = 7;                // a run is cut into items of 128 records
+constexpr uint32_t ITEM_RECORDS = 1u << ITEM_SHIFT;
+constexpr uint32_t ITEM_LOADS = ITEM_RECORDS / 64;  // loads per lane and item
+constexpr uint32_t ITEM_CAP = 2048;               // items listed in LDS at a time
 constexpr float FIX_SCALE = 4294967296.0f;        // 2^32
 
 // x * 2^32 as a two's complement 64-bit integer, for |x| < 2^31 with at most 24 significant bits (any fp16 value):
@@ -644,13 +655,16 @@ __device__ __forceinline__ unsigned long long to_fixed(float x) {
 }
 __device__ __forceinline__ float from_fixed(unsigned long long q) { return (float)((double)(long long)q * (1.0 / 4294967296.0)); }
 
-__global__ void __launch_bounds__(RED_BLOCK) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
-                                                                const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
-                                                                __half2* __restrict__ grads, int accumulate) {
-	__shared__ unsigned long long acc[2 * BKT_ENTRIES];  // 128 KiB
-	__shared__ uint32_t run_src[RED_CHUNK];               // index of the run's first record in `records`
-	__shared__ uint16_t run_len[RED_CHUNK];
-	__shared__ uint32_t item_pos[RED_CHUNK + 1];          // exclusive prefix of the runs' item counts
+// Every thread owns the bucket's run of one tile.  The runs are cut into items, the items of all runs are numbered
+// consecutively (block scan of the item counts) and listed in LDS (first record, record count), ITEM_CAP at a time:
+// a wave then finds an item's records with one LDS read instead of searching the runs' prefix sums, whose chain of
+// dependent LDS reads was most of this kernel's time.
+__global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
+                                                                   const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
+                                                                   __half2* __restrict__ grads, int accumulate) {
+	__shared__ unsigned long long acc[2 * BKT_ENTRIES];
+	__shared__ uint32_t item_src[ITEM_CAP];  // index of the item's first record in the level's records
+	__shared__ uint8_t item_n[ITEM_CAP];     // its record count - 1
 	__shared__ uint32_t wave_tot[RED_BLOCK / 64];
 	// which (level, bucket, group) is this workgroup?
 	uint32_t level = 0;
@@ -658,95 +672,90 @@ __global__ void __launch_bounds__(RED_BLOCK) grid_reduce_kernel(N2LevelTable tab
 	const uint32_t local = blockIdx.x - plan.wg_begin[level];
 	const uint32_t G = plan.groups[level];
 	const uint32_t bucket = local / G, group = local - bucket * G;
-	for (uint32_t e = threadIdx.x; e < 2 * BKT_ENTRIES; e += RED_BLOCK) acc[e] = 0ull;
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
 	const uint32_t my_tiles = (tiles > group) ? (tiles - group + G - 1) / G : 0;  // tiles group, group + G, ...
 	const size_t level_tile0 = (size_t)level * tiles;
 	const uint2* base = records + level_tile0 * BIN_RECORDS;
-	for (uint32_t c0 = 0; c0 < my_tiles; c0 += RED_CHUNK) {
-		__syncthreads();
-		// every thread fetches the bucket's run bounds of 4 tiles (independent loads); a run is cut into items
-		// of 128 records and the items of all runs are numbered consecutively (block scan of the item counts)
-		uint32_t cnt[RED_PER_THREAD], sum = 0;
-#pragma unroll
-		for (uint32_t j = 0; j < RED_PER_THREAD; ++j) {
-			const uint32_t k = threadIdx.x * RED_PER_THREAD + j, t = c0 + k;
-			cnt[j] = 0;
-			if (t < my_tiles) {
-				const size_t tile = level_tile0 + group + (size_t)t * G;
-				const uint16_t* off = offsets + tile * (BKT_MAX + 1) + bucket;
-				const uint32_t begin = off[0], end = off[1];
-				run_src[k] = (uint32_t)((tile - level_tile0) * BIN_RECORDS) + begin;
-				run_len[k] = (uint16_t)(end - begin);
-				cnt[j] = (end - begin + 127u) >> 7;
-			}
-			sum += cnt[j];
+	for (uint32_t c0 = 0; c0 < my_tiles || c0 == 0; c0 += RED_BLOCK) {
+		// this thread's run (the load is in flight while the accumulators are cleared)
+		uint32_t src = 0, len = 0;
+		const uint32_t t = c0 + threadIdx.x;
+		if (t < my_tiles) {
+			const size_t tile = level_tile0 + group + (size_t)t * G;
+			const uint16_t* off = offsets + tile * (BKT_MAX + 1) + bucket;
+			const uint32_t begin = off[0], end = off[1];
+			src = (uint32_t)((tile - level_tile0) * BIN_RECORDS) + begin;
+			len = end - begin;
 		}
-		uint32_t incl = sum;
+		if (c0 == 0) {
+			for (uint32_t e = threadIdx.x; e < 2 * BKT_ENTRIES; e += RED_BLOCK) acc[e] = 0ull;
+		}
+		const uint32_t cnt = (len + ITEM_RECORDS - 1u) >> ITEM_SHIFT;
+		uint32_t incl = cnt;
 #pragma unroll
 		for (int o = 1; o < 64; o <<= 1) {
 			const uint32_t u = __shfl_up(incl, o);
 			if ((int)lane >= o) incl += u;
 		}
+		__syncthreads();  // the previous chunk's items are done with wave_tot and the item list
 		if (lane == 63) wave_tot[wave] = incl;
 		__syncthreads();
-		uint32_t run = incl - sum;
-		for (uint32_t w = 0; w < wave; ++w) run += wave_tot[w];
-#pragma unroll
-		for (uint32_t j = 0; j < RED_PER_THREAD; ++j) {
-			item_pos[threadIdx.x * RED_PER_THREAD + j] = run;
-			run += cnt[j];
+		uint32_t first = incl - cnt, n_items = 0;  // number of this thread's first item; items of the chunk
+		for (uint32_t w = 0; w < RED_BLOCK / 64; ++w) {
+			const uint32_t tot = wave_tot[w];
+			if (w < wave) first += tot;
+			n_items += tot;
 		}
-		if (threadIdx.x == RED_BLOCK - 1) item_pos[RED_CHUNK] = run;
-		__syncthreads();
-		const uint32_t n_items = item_pos[RED_CHUNK];
-		// a wave takes 4 items at a time (8 independent 8-byte loads per lane); the loads of the next 4 items are
-		// issued before the current ones are accumulated
-		auto fetch = [&](uint32_t i0, uint2 (&rec)[8], uint32_t& okmask) {
-			okmask = 0;
+		for (uint32_t w0 = 0; w0 < n_items; w0 += ITEM_CAP) {
+			if (w0 > 0) __syncthreads();  // the previous window has been read
+			// list this thread's items that fall into the window [w0, w0 + ITEM_CAP)
+			for (uint32_t i = (first < w0) ? w0 - first : 0u; i < cnt && first + i < w0 + ITEM_CAP; ++i) {
+				const uint32_t rest = len - (i << ITEM_SHIFT);
+				item_src[first + i - w0] = src + (i << ITEM_SHIFT);
+				item_n[first + i - w0] = (uint8_t)((rest < ITEM_RECORDS ? rest : ITEM_RECORDS) - 1u);
+			}
+			__syncthreads();
+			const uint32_t n_win = (n_items - w0 < ITEM_CAP) ? n_items - w0 : ITEM_CAP;
+			// a wave takes RED_ITEMS items at a time; the loads of its next items are issued before the current ones
+			// are accumulated
+			auto fetch = [&](uint32_t i0, uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t& okmask) {
+				okmask = 0;
 #pragma unroll
-			for (uint32_t j = 0; j < 4; ++j) {
-				const uint32_t it = i0 + j;
-				uint32_t src = 0, n = 0, t0 = 0;
-				if (it < n_items) {
-					uint32_t lo = 0, hi = RED_CHUNK;  // last run k with item_pos[k] <= it
+				for (uint32_t j = 0; j < RED_ITEMS; ++j) {
+					const uint32_t it = i0 + j;
+					uint32_t s0 = 0, n = 0;
+					if (it < n_win) { s0 = item_src[it]; n = (uint32_t)item_n[it] + 1u; }
 #pragma unroll
-					for (int step = 0; step < 11; ++step) {
-						const uint32_t mid = (lo + hi) >> 1;
-						if (item_pos[mid] <= it) lo = mid; else hi = mid;
+					for (uint32_t h = 0; h < ITEM_LOADS; ++h) {
+						const uint32_t r = h * 64 + lane;
+						const bool ok = r < n;
+						okmask |= (ok ? 1u : 0u) << (ITEM_LOADS * j + h);
+						rec[ITEM_LOADS * j + h] = ok ? base[(size_t)s0 + r] : make_uint2(0u, 0u);
 					}
-					src = run_src[lo]; n = run_len[lo]; t0 = (it - item_pos[lo]) << 7;
 				}
+			};
+			constexpr uint32_t STRIDE = (RED_BLOCK / 64) * RED_ITEMS;
+			uint2 cur[ITEM_LOADS * RED_ITEMS], nxt[ITEM_LOADS * RED_ITEMS];
+			uint32_t cur_ok = 0, nxt_ok = 0;
+			uint32_t i0 = wave * RED_ITEMS;
+			if (i0 < n_win) fetch(i0, cur, cur_ok);
+			for (; i0 < n_win; i0 += STRIDE) {
+				const bool more = i0 + STRIDE < n_win;
+				if (more) fetch(i0 + STRIDE, nxt, nxt_ok);
 #pragma unroll
-				for (uint32_t h = 0; h < 2; ++h) {
-					const uint32_t t = t0 + h * 64 + lane;
-					const bool ok = t < n;
-					okmask |= (ok ? 1u : 0u) << (2 * j + h);
-					rec[2 * j + h] = ok ? base[(size_t)src + t] : make_uint2(0u, 0u);
+				for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) {
+					if (cur_ok & (1u << q)) {
+						const __half2 hh = *reinterpret_cast<const __half2*>(&cur[q].y);
+						const float2 f = __half22float2(hh);
+						atomicAdd(&acc[2 * cur[q].x], to_fixed(f.x));  // LDS integer atomics
+						atomicAdd(&acc[2 * cur[q].x + 1], to_fixed(f.y));
+					}
 				}
-			}
-		};
-		constexpr uint32_t STRIDE = (RED_BLOCK / 64) * 4;
-		uint2 cur[8], nxt[8];
-		uint32_t cur_ok = 0, nxt_ok = 0;
-		uint32_t i0 = wave * 4;
-		if (i0 < n_items) fetch(i0, cur, cur_ok);
-		for (; i0 < n_items; i0 += STRIDE) {
-			const bool more = i0 + STRIDE < n_items;
-			if (more) fetch(i0 + STRIDE, nxt, nxt_ok);
+				if (more) {
 #pragma unroll
-			for (uint32_t q = 0; q < 8; ++q) {
-				if (cur_ok & (1u << q)) {
-					const __half2 hh = *reinterpret_cast<const __half2*>(&cur[q].y);
-					const float2 f = __half22float2(hh);
-					atomicAdd(&acc[2 * cur[q].x], to_fixed(f.x));  // LDS integer atomics
-					atomicAdd(&acc[2 * cur[q].x + 1], to_fixed(f.y));
+					for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) cur[q] = nxt[q];
+					cur_ok = nxt_ok;
 				}
-			}
-			if (more) {
-#pragma unroll
-				for (uint32_t q = 0; q < 8; ++q) cur[q] = nxt[q];
-				cur_ok = nxt_ok;
 			}
 		}
 	}
