@@ -478,23 +478,33 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
 	}
 	const __half2* P = params + tab.offset[level];
 	float o0 = 0.f, o1 = 0.f;
+	// Corner k = i + 2 j + 4 l has weight X_i Y_j Z_l and signs (sx_i, sy_j, sz_l).  Its record is
+	//   a X Y Z + c (v0 sx Y Z + v1 sy X Z + v2 sz X Y)  =  (Y Z) (a X + c v0 sx) + (c X) (v1 sy Z + v2 sz Y),
+	// so the eight corners share two x terms per feature and four (y, z) terms.
+	const float X[2] = {1.f - p.w[0], p.w[0]}, Y[2] = {1.f - p.w[1], p.w[1]}, Z[2] = {1.f - p.w[2], p.w[2]};
+	float Pyz[4], Qyz[4], A0[2], A1[2], B0[2] = {0.f, 0.f}, B1[2] = {0.f, 0.f};
+#pragma unroll
+	for (uint32_t jl = 0; jl < 4; ++jl) {
+		const uint32_t j = jl & 1u, l = jl >> 1;
+		Pyz[jl] = Y[j] * Z[l];
+		Qyz[jl] = SECOND ? (j ? v1 : -v1) * Z[l] + (l ? v2 : -v2) * Y[j] : 0.f;
+	}
+#pragma unroll
+	for (uint32_t ix = 0; ix < 2; ++ix) {
+		const float sv = ix ? v0 : -v0;
+		A0[ix] = FIRST ? fmaf(a0, X[ix], c0 * sv) : c0 * sv;
+		A1[ix] = FIRST ? fmaf(a1, X[ix], c1 * sv) : c1 * sv;
+		if (SECOND) { B0[ix] = c0 * X[ix]; B1[ix] = c1 * X[ix]; }
+	}
 #pragma unroll
 	for (uint32_t k = 0; k < 8; ++k) {
-		const float w0 = (k & 1u) ? p.w[0] : 1.f - p.w[0];
-		const float w1 = (k & 2u) ? p.w[1] : 1.f - p.w[1];
-		const float w2 = (k & 4u) ? p.w[2] : 1.f - p.w[2];
-		float r0 = 0.f, r1 = 0.f;
-		if (FIRST) {
-			const float wt = w0 * w1 * w2;
-			r0 = a0 * wt;
-			r1 = a1 * wt;
-		}
+		const uint32_t ix = k & 1u, jl = k >> 1;
+		float r0 = Pyz[jl] * A0[ix], r1 = Pyz[jl] * A1[ix];
 		if (SECOND) {
-			const float s0 = (k & 1u) ? 1.f : -1.f, s1 = (k & 2u) ? 1.f : -1.f, s2 = (k & 4u) ? 1.f : -1.f;
-			const float coef = v0 * s0 * w1 * w2 + v1 * s1 * w0 * w2 + v2 * s2 * w0 * w1;
-			r0 = fmaf(c0, coef, r0);
-			r1 = fmaf(c1, coef, r1);
+			r0 = fmaf(B0[ix], Qyz[jl], r0);
+			r1 = fmaf(B1[ix], Qyz[jl], r1);
 			if (WANT_OUT) {
+				const float coef = fmaf(ix ? v0 : -v0, Pyz[jl], X[ix] * Qyz[jl]);
 				const float2 val = __half22float2(P[e[k]]);
 				o0 = fmaf(coef, val.x, o0);
 				o1 = fmaf(coef, val.y, o1);
@@ -576,11 +586,10 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 			const uint32_t depth = lane - start;  // lanes of the run below this one
 #define N2_SCAN_STEP(D)                                               \
 			{                                                         \
-				const bool take = depth >= D;                         \
+				const float take = depth >= D ? 1.f : 0.f;            \
 				_Pragma("unroll") for (uint32_t k = 0; k < 8; ++k) {  \
-					const float t0 = n2_row_shr<D>(r0[k]), t1 = n2_row_shr<D>(r1[k]); \
-					r0[k] += take ? t0 : 0.f;                         \
-					r1[k] += take ? t1 : 0.f;                         \
+					r0[k] = fmaf(n2_row_shr<D>(r0[k]), take, r0[k]);  \
+					r1[k] = fmaf(n2_row_shr<D>(r1[k]), take, r1[k]);  \
 				}                                                     \
 			}
 			N2_SCAN_STEP(1) N2_SCAN_STEP(2) N2_SCAN_STEP(4) N2_SCAN_STEP(8)
