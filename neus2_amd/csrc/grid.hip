@@ -543,10 +543,12 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
                                                               uint32_t dim_stride, const __half* __restrict__ dL_dy,
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
                                                               const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
-                                                              uint2* __restrict__ records, uint16_t* __restrict__ offsets) {
+                                                              uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
+                                                              uint16_t* __restrict__ offsets) {
 	__shared__ uint32_t hist[BKT_MAX];
 	__shared__ uint32_t prefix[BKT_MAX + 1];
-	__shared__ uint2 staging[BIN_RECORDS];
+	__shared__ __align__(16) uint32_t stage_val[BIN_RECORDS];  // sorted records: packed half2 value ...
+	__shared__ __align__(16) uint16_t stage_key[BIN_RECORDS];  // ... and entry within its bucket
 	const uint32_t level = first_level + blockIdx.x / tiles, tile = blockIdx.x % tiles;
 	const uint32_t lane = threadIdx.x & 63u;
 	if (threadIdx.x < BKT_MAX) hist[threadIdx.x] = 0;
@@ -631,14 +633,22 @@ __global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, u
 		for (uint32_t k = 0; k < 8; ++k) {
 			if (re[8 * j + k] != REC_SKIP) {
 				const uint32_t e = re[8 * j + k] & 0x7FFFFu, rank = re[8 * j + k] >> 19;
-				staging[prefix[e >> BKT_SHIFT] + rank] = make_uint2(e & (BKT_ENTRIES - 1u), rv[8 * j + k]);
+				const uint32_t pos = prefix[e >> BKT_SHIFT] + rank;
+				stage_val[pos] = rv[8 * j + k];
+				stage_key[pos] = (uint16_t)(e & (BKT_ENTRIES - 1u));
 			}
 		}
 	}
 	__syncthreads();
 	const uint32_t total = prefix[BKT_MAX];
-	uint2* out = records + ((size_t)level * tiles + tile) * BIN_RECORDS;
-	for (uint32_t t = threadIdx.x; t < total; t += BIN_BLOCK) out[t] = staging[t];
+	// 16 bytes per lane; the last store of each array may run past `total` inside the tile's own slot, which nobody reads
+	const size_t slot = ((size_t)level * tiles + tile) * BIN_RECORDS;
+	uint4* out_val = reinterpret_cast<uint4*>(rec_vals + slot);
+	uint4* out_key = reinterpret_cast<uint4*>(rec_keys + slot);
+	const uint4* sv = reinterpret_cast<const uint4*>(stage_val);
+	const uint4* sk = reinterpret_cast<const uint4*>(stage_key);
+	for (uint32_t t = threadIdx.x; 4 * t < total; t += BIN_BLOCK) out_val[t] = sv[t];
+	for (uint32_t t = threadIdx.x; 8 * t < total; t += BIN_BLOCK) out_key[t] = sk[t];
 	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
 }
 
@@ -669,7 +679,8 @@ __device__ __forceinline__ float from_fixed(unsigned long long q) { return (floa
 // a wave then finds an item's records with one LDS read instead of searching the runs' prefix sums, whose chain of
 // dependent LDS reads was most of this kernel's time.
 __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
-                                                                   const uint2* __restrict__ records, const uint16_t* __restrict__ offsets,
+                                                                   const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
+                                                                   const uint16_t* __restrict__ offsets,
                                                                    __half2* __restrict__ grads, int accumulate) {
 	__shared__ unsigned long long acc[2 * BKT_ENTRIES];
 	__shared__ uint32_t item_src[ITEM_CAP];  // index of the item's first record in the level's records
@@ -684,7 +695,8 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
 	const uint32_t my_tiles = (tiles > group) ? (tiles - group + G - 1) / G : 0;  // tiles group, group + G, ...
 	const size_t level_tile0 = (size_t)level * tiles;
-	const uint2* base = records + level_tile0 * BIN_RECORDS;
+	const uint32_t* base_val = rec_vals + level_tile0 * BIN_RECORDS;
+	const uint16_t* base_key = rec_keys + level_tile0 * BIN_RECORDS;
 	for (uint32_t c0 = 0; c0 < my_tiles || c0 == 0; c0 += RED_BLOCK) {
 		// this thread's run (the load is in flight while the accumulators are cleared)
 		uint32_t src = 0, len = 0;
@@ -739,7 +751,7 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 						const uint32_t r = h * 64 + lane;
 						const bool ok = r < n;
 						okmask |= (ok ? 1u : 0u) << (ITEM_LOADS * j + h);
-						rec[ITEM_LOADS * j + h] = ok ? base[(size_t)s0 + r] : make_uint2(0u, 0u);
+						rec[ITEM_LOADS * j + h] = ok ? make_uint2(base_key[(size_t)s0 + r], base_val[(size_t)s0 + r]) : make_uint2(0u, 0u);
 					}
 				}
 			};
@@ -1056,7 +1068,7 @@ static bool bucket_supported(const n2_grid_t* grid) {
 }
 static uint64_t bucket_ws_bytes(const n2_grid_t* grid, uint32_t max_points) {
 	const uint64_t tiles = n_bin_tiles(max_points), L = grid->tab.n_levels;
-	const uint64_t rec = L * tiles * BIN_RECORDS * sizeof(uint2);
+	const uint64_t rec = L * tiles * BIN_RECORDS * (sizeof(uint32_t) + sizeof(uint16_t));
 	const uint64_t off = (L * tiles * (BKT_MAX + 1) * sizeof(uint16_t) + 255) / 256 * 256;
 	return rec + off;
 }
@@ -1100,11 +1112,14 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
 	const dim3 bd(BIN_BLOCK);
-	uint2* records = reinterpret_cast<uint2*>(grid->ws);
-	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + (uint64_t)L * tiles * BIN_RECORDS * sizeof(uint2));
+	// workspace: packed half2 values of all records, then their 16-bit keys, then the tiles' bucket offsets
+	const uint64_t n_rec = (uint64_t)L * tiles * BIN_RECORDS;
+	uint32_t* rec_vals = reinterpret_cast<uint32_t*>(grid->ws);
+	uint16_t* rec_keys = reinterpret_cast<uint16_t*>(grid->ws + n_rec * sizeof(uint32_t));
+	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + n_rec * (sizeof(uint32_t) + sizeof(uint16_t)));
 	const dim3 gd(tiles * L);
 #define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
-                                                                   grid->params, dL_ddLdy, records, offsets)
+                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
 	else if (second && out) LAUNCH(false, true, true);
@@ -1124,7 +1139,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	}
 	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
 	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; }
-	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, records, offsets, grid->grads, accumulate ? 1 : 0);
+	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, rec_vals, rec_keys, offsets, grid->grads, accumulate ? 1 : 0);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
