@@ -538,7 +538,7 @@ __device__ __forceinline__ float n2_row_shr(float x) {
 constexpr uint32_t REC_SKIP = 0xFFFFFFFFu;
 
 template <bool FIRST, bool SECOND, bool WANT_OUT>
-__global__ void __launch_bounds__(BIN_BLOCK) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
+__global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
                                                               const float* __restrict__ xyz, uint32_t point_stride,
                                                               uint32_t dim_stride, const __half* __restrict__ dL_dy,
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
