@@ -9,9 +9,23 @@
 typedef _Float16 hf;
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float loss_scale, const n2_adam_config& c, float g16,
-                                         float& w, float& m1, float& m2, uint32_t& t) {
-	float g = g16 / loss_scale;
+// Bias correction sqrt(1 - beta2^t) / (1 - beta1^t) for t < ADAM_TABLE, computed once per (beta1, beta2) by
+// adam_table_kernel.  Two powf per parameter made the step kernel ALU bound; a (mostly uniform) table read costs nothing.
+constexpr uint32_t ADAM_TABLE = 4096;
+__device__ float g_adam_bias[ADAM_TABLE];
+
+__device__ __forceinline__ float adam_bias(float beta1, float beta2, uint32_t t) {
+	return sqrtf(1.f - powf(beta2, (float)t)) / (1.f - powf(beta1, (float)t));
+}
+__global__ void __launch_bounds__(256) adam_table_kernel(float beta1, float beta2) {
+	const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+	if (t < ADAM_TABLE) g_adam_bias[t] = adam_bias(beta1, beta2, t);
+}
+
+// inv_loss_scale > 0: loss_scale is a power of two and multiplying by its reciprocal is the exact division
+__device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
+                                         const n2_adam_config& c, float g16, float& w, float& m1, float& m2, uint32_t& t) {
+	float g = inv_loss_scale > 0.f ? g16 * inv_loss_scale : g16 / loss_scale;
 	if (i >= n_matrix) {
 		if (g == 0.f) return false;
 	} else {
@@ -21,12 +35,14 @@ __device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float lo
 	m1 = c.beta1 * m1 + (1.f - c.beta1) * g;
 	m2 = c.beta2 * m2 + (1.f - c.beta2) * gs;
 	t += 1u;
-	const float lr = c.learning_rate * sqrtf(1.f - powf(c.beta2, (float)t)) / (1.f - powf(c.beta1, (float)t));
+	// beyond the table the factor is exactly 1 once both powers have underflowed (saturated), else it is computed
+	const float bias = t < ADAM_TABLE ? g_adam_bias[t] : (saturated ? 1.f : adam_bias(c.beta1, c.beta2, t));
+	const float lr = c.learning_rate * bias;
 	w -= lr * m1 / (sqrtf(m2) + c.epsilon);
 	return true;
 }
 
-__global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale,
+__global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
                                                         float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
                                                         float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps) {
 	const uint32_t q = blockIdx.x * 256 + threadIdx.x;
@@ -41,10 +57,10 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		float4 b = *reinterpret_cast<float4*>(m2 + i0);
 		uint4 t = *reinterpret_cast<uint4*>(steps + i0);
 		bool any = false;
-		any |= adam_one(i0 + 0, n_matrix, loss_scale, c, (float)g[0], w.x, a.x, b.x, t.x);
-		any |= adam_one(i0 + 1, n_matrix, loss_scale, c, (float)g[1], w.y, a.y, b.y, t.y);
-		any |= adam_one(i0 + 2, n_matrix, loss_scale, c, (float)g[2], w.z, a.z, b.z, t.z);
-		any |= adam_one(i0 + 3, n_matrix, loss_scale, c, (float)g[3], w.w, a.w, b.w, t.w);
+		any |= adam_one(i0 + 0, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[0], w.x, a.x, b.x, t.x);
+		any |= adam_one(i0 + 1, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[1], w.y, a.y, b.y, t.y);
+		any |= adam_one(i0 + 2, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[2], w.z, a.z, b.z, t.z);
+		any |= adam_one(i0 + 3, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[3], w.w, a.w, b.w, t.w);
 		if (!any) return;
 		*reinterpret_cast<float4*>(master + i0) = w;
 		*reinterpret_cast<float4*>(m1 + i0) = a;
@@ -55,7 +71,7 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		for (uint32_t i = i0; i < n; ++i) {
 			float w = master[i], a = m1[i], b = m2[i];
 			uint32_t t = steps[i];
-			if (adam_one(i, n_matrix, loss_scale, c, (float)grads[i], w, a, b, t)) {
+			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)grads[i], w, a, b, t)) {
 				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
 			}
 		}
@@ -76,8 +92,26 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 8 == 0 && reinterpret_cast<uintptr_t>(d_gradients) % 8 == 0,
 	           "n2_adam_step: fp16 buffers must be 8-byte aligned");
 	const uint32_t quads = (n_params + 3) / 4;
-	N2ProfScope prof(N2_PROF_ADAM, n2_stream(stream));
-	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(*config, n_params, n_matrix_params, loss_scale,
+	hipStream_t s = n2_stream(stream);
+	// the bias-correction table of this device holds the factors of one (beta1, beta2) pair; calls with other
+	// betas rebuild it on their stream (calls on different streams with different betas must not overlap)
+	struct Built { bool valid = false; float beta1 = 0.f, beta2 = 0.f; };
+	static Built built[64];
+	int dev = 0;
+	N2_HIP(hipGetDevice(&dev));
+	N2_REQUIRE(dev >= 0 && dev < 64, "n2_adam_step: device index %d not supported", dev);
+	if (!built[dev].valid || built[dev].beta1 != config->beta1 || built[dev].beta2 != config->beta2) {
+		adam_table_kernel<<<dim3(ADAM_TABLE / 256), dim3(256), 0, s>>>(config->beta1, config->beta2);
+		N2_LAUNCH_CHECK();
+		built[dev].valid = true; built[dev].beta1 = config->beta1; built[dev].beta2 = config->beta2;
+	}
+	// 1 - beta^t == 1 in fp32 for every t past the table?
+	const double small = std::ldexp(1.0, -26);
+	const int saturated = (std::pow((double)config->beta1, (double)ADAM_TABLE) < small && std::pow((double)config->beta2, (double)ADAM_TABLE) < small) ? 1 : 0;
+	int exp2 = 0;
+	const float inv_loss_scale = (std::frexp(loss_scale, &exp2) == 0.5f && exp2 > -120 && exp2 < 120) ? 1.f / loss_scale : 0.f;
+	N2ProfScope prof(N2_PROF_ADAM, s);
+	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated,
 		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
