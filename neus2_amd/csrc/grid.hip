@@ -50,8 +50,8 @@ __device__ __forceinline__ void n2_locate(float x, float scale, float& w, uint32
 // Level mask of tcnn's grid encoding: the limit is (max_level * n_output_features) / n_features_per_level in fp32
 // and a level is off when level >= limit + 1e-3; the progressive mask adds level >= valid_levels.
 __device__ __forceinline__ bool n2_level_masked(const N2LevelTable& tab, uint32_t level, uint32_t i) {
-	const float fraction = tab.max_level_gpu ? tab.max_level_gpu[i] : tab.max_level;
-	const float limit = (fraction * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
+	if (tab.max_level_gpu == nullptr) return level >= tab.active_levels;  // uniform: the host has applied both rules
+	const float limit = (tab.max_level_gpu[i] * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
 	return (float)level >= limit + 1e-3f || level >= tab.valid_levels;
 }
 
@@ -657,7 +657,7 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 // fp16 values, i.e. multiples of 2^-24 below 2^16, so value * 2^32 is an exact integer below 2^48 and the
 // sum of a whole bucket stays far inside 64 bits.  The accumulation is exact and independent of order.
 constexpr uint32_t RED_BLOCK = 1024;              // 16 waves; two workgroups share a CU
-constexpr uint32_t RED_ITEMS = (BKT_SHIFT == 13) ? 4 : 2;  // items a wave has in flight per fetch
+constexpr uint32_t RED_ITEMS = 2;                 // items a wave has in flight per fetch
 constexpr uint32_t ITEM_SHIFT = 7;                // a run is cut into items of 128 records
 constexpr uint32_t ITEM_RECORDS = 1u << ITEM_SHIFT;
 constexpr uint32_t ITEM_LOADS = ITEM_RECORDS / 64;  // loads per lane and item
@@ -737,8 +737,7 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 			}
 			__syncthreads();
 			const uint32_t n_win = (n_items - w0 < ITEM_CAP) ? n_items - w0 : ITEM_CAP;
-			// a wave takes RED_ITEMS items at a time; the loads of its next items are issued before the current ones
-			// are accumulated
+			// a wave takes RED_ITEMS items at a time
 			auto fetch = [&](uint32_t i0, uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t& okmask) {
 				okmask = 0;
 #pragma unroll
@@ -751,31 +750,43 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 						const uint32_t r = h * 64 + lane;
 						const bool ok = r < n;
 						okmask |= (ok ? 1u : 0u) << (ITEM_LOADS * j + h);
-						rec[ITEM_LOADS * j + h] = ok ? make_uint2(base_key[(size_t)s0 + r], base_val[(size_t)s0 + r]) : make_uint2(0u, 0u);
+						// lanes past the end of the run read the level's first record instead (and ignore it): with every
+						// load issued unconditionally the compiler can count them, and waits for the CURRENT items only
+						// while the next ones are in flight
+						const size_t at = ok ? (size_t)s0 + r : 0;
+						rec[ITEM_LOADS * j + h] = make_uint2(base_key[at], base_val[at]);
 					}
 				}
 			};
 			constexpr uint32_t STRIDE = (RED_BLOCK / 64) * RED_ITEMS;
-			uint2 cur[ITEM_LOADS * RED_ITEMS], nxt[ITEM_LOADS * RED_ITEMS];
-			uint32_t cur_ok = 0, nxt_ok = 0;
-			uint32_t i0 = wave * RED_ITEMS;
-			if (i0 < n_win) fetch(i0, cur, cur_ok);
-			for (; i0 < n_win; i0 += STRIDE) {
-				const bool more = i0 + STRIDE < n_win;
-				if (more) fetch(i0 + STRIDE, nxt, nxt_ok);
+			auto accumulate = [&](const uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t okmask) {
 #pragma unroll
 				for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) {
-					if (cur_ok & (1u << q)) {
-						const __half2 hh = *reinterpret_cast<const __half2*>(&cur[q].y);
+					if (okmask & (1u << q)) {
+						const __half2 hh = *reinterpret_cast<const __half2*>(&rec[q].y);
 						const float2 f = __half22float2(hh);
-						atomicAdd(&acc[2 * cur[q].x], to_fixed(f.x));  // LDS integer atomics
-						atomicAdd(&acc[2 * cur[q].x + 1], to_fixed(f.y));
+						atomicAdd(&acc[2 * rec[q].x], to_fixed(f.x));  // LDS integer atomics
+						atomicAdd(&acc[2 * rec[q].x + 1], to_fixed(f.y));
 					}
 				}
-				if (more) {
-#pragma unroll
-					for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) cur[q] = nxt[q];
-					cur_ok = nxt_ok;
+			};
+			// Two register sets take turns: while one is accumulated the loads of the other are in flight.  Every fetch
+			// issues the same number of loads (items past the end read the first record and are ignored) and no set is
+			// ever copied, so each wait covers exactly the set that is about to be used.
+			uint2 ra[ITEM_LOADS * RED_ITEMS], rb[ITEM_LOADS * RED_ITEMS];
+			uint32_t ok_a = 0, ok_b = 0;
+			uint32_t i0 = wave * RED_ITEMS;
+			if (i0 < n_win) {
+				fetch(i0, ra, ok_a);
+				for (;;) {
+					fetch(i0 + STRIDE, rb, ok_b);
+					accumulate(ra, ok_a);
+					i0 += STRIDE;
+					if (i0 >= n_win) break;
+					fetch(i0 + STRIDE, ra, ok_a);
+					accumulate(rb, ok_b);
+					i0 += STRIDE;
+					if (i0 >= n_win) break;
 				}
 			}
 		}
@@ -834,6 +845,7 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->tab.max_level = 1.0f;
 	g->tab.max_level_gpu = nullptr;
 	g->tab.valid_levels = n_levels;
+	g->tab.active_levels = n_levels;
 	g->base_valid_level_scale = 1.0f;
 	g->valid_level_scale = 0.0f;
 	g->base_training_step = 0;
@@ -899,10 +911,19 @@ N2_API int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs) {
 	return N2_OK;
 }
 
+// levels in use under the global settings, with the device predicate's arithmetic
+static uint32_t count_active_levels(const N2LevelTable& tab) {
+	const float limit = (tab.max_level * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
+	uint32_t n = 0;
+	while (n < tab.n_levels && n < tab.valid_levels && !((float)n >= limit + 1e-3f)) ++n;  // both rules cut a suffix of the levels
+	return n;
+}
+
 N2_API int n2_grid_set_max_level(n2_grid_t* grid, float max_level) {
 	N2_REQUIRE(grid != nullptr, "n2_grid_set_max_level: grid is null");
 	N2_REQUIRE(max_level >= 0.f && max_level <= 1000.f, "n2_grid_set_max_level: max_level %g outside [0, 1000]", (double)max_level);
 	grid->tab.max_level = max_level;
+	grid->tab.active_levels = count_active_levels(grid->tab);
 	return N2_OK;
 }
 
@@ -919,6 +940,7 @@ N2_API int n2_grid_set_progressive(n2_grid_t* grid, float base_valid_level_scale
 	grid->valid_level_scale = valid_level_scale;
 	grid->base_training_step = base_training_step;
 	if (base_training_step == 0) grid->tab.valid_levels = grid->tab.n_levels;
+	grid->tab.active_levels = count_active_levels(grid->tab);
 	return N2_OK;
 }
 
@@ -933,18 +955,11 @@ N2_API int n2_grid_set_training_step(n2_grid_t* grid, uint32_t training_step) {
 	uint32_t n = levels >= (float)grid->tab.n_levels ? grid->tab.n_levels : (uint32_t)levels;
 	if (n < 1) n = 1;
 	grid->tab.valid_levels = n;
+	grid->tab.active_levels = count_active_levels(grid->tab);
 	return N2_OK;
 }
 
-N2_API uint32_t n2_grid_active_levels(const n2_grid_t* grid) {
-	if (!grid) return 0;
-	uint32_t n = 0;
-	const N2LevelTable& tab = grid->tab;
-	const float limit = (tab.max_level * (float)(tab.n_levels * tab.n_features)) / (float)tab.n_features;
-	for (uint32_t l = 0; l < tab.n_levels; ++l)
-		if (!((float)l >= limit + 1e-3f || l >= tab.valid_levels)) ++n;
-	return n;
-}
+N2_API uint32_t n2_grid_active_levels(const n2_grid_t* grid) { return grid ? grid->tab.active_levels : 0; }
 
 N2_API int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients) {
 	N2_REQUIRE(grid != nullptr, "n2_grid_set_params: grid is null");

@@ -56,6 +56,7 @@ struct N2LevelTable {
 	float max_level;               // fraction of the levels in use, 1 = all
 	const float* max_level_gpu;    // per point, or null
 	uint32_t valid_levels;         // progressive training: number of levels switched on so far
+	uint32_t active_levels;        // levels in use under max_level and valid_levels (kept up to date by the setters)
 	uint32_t n_features;
 };
 
