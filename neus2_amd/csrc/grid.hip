@@ -31,6 +31,9 @@ struct n2_grid {
 	unsigned char* ws;
 	uint64_t ws_bytes;
 	uint32_t ws_max_points;
+	// part of the gradient buffer the next bucketed scatter clears in its bin kernel (OVERWRITE, levels that add with atomics)
+	uint4* zero_begin;
+	uint32_t zero_count;  // in 16-byte units
 };
 
 // ----------------------------------------------------------------------------
@@ -544,7 +547,9 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
                                                               const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
                                                               uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
-                                                              uint16_t* __restrict__ offsets) {
+                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count) {
+	// part of the gradient buffer that the reduce kernel will add to with atomics: cleared here, one 16-byte store per thread
+	for (uint32_t z = blockIdx.x * BIN_BLOCK + threadIdx.x; z < zero_count; z += gridDim.x * BIN_BLOCK) zero_begin[z] = make_uint4(0u, 0u, 0u, 0u);
 	__shared__ uint32_t hist[BKT_MAX];
 	__shared__ uint32_t prefix[BKT_MAX + 1];
 	__shared__ __align__(16) uint32_t stage_val[BIN_RECORDS];  // sorted records: packed half2 value ...
@@ -881,6 +886,8 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->ws = nullptr;
 	g->ws_bytes = 0;
 	g->ws_max_points = 0;
+	g->zero_begin = nullptr;
+	g->zero_count = 0;
 	*out = g;
 	return N2_OK;
 }
@@ -1055,6 +1062,8 @@ static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_
 // clearing beforehand.
 static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2_grad_mode mode, uint32_t n_points) {
 	N2_REQUIRE(mode == N2_GRAD_IGNORE || mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "%s: bad gradient mode %d", fn, (int)mode);
+	grid->zero_begin = nullptr;
+	grid->zero_count = 0;
 	if (mode == N2_GRAD_IGNORE) return N2_OK;
 	N2_REQUIRE(grid->grads != nullptr, "%s: gradient mode %d needs a gradient buffer (n2_grid_set_params)", fn, (int)mode);
 	if (mode != N2_GRAD_OVERWRITE) return N2_OK;
@@ -1068,9 +1077,12 @@ static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2
 		}
 	}
 	if (first == 0xFFFFFFFFu) return N2_OK;
-	// one fill over the span of those levels (they are the coarse, small ones): 16-byte aligned because every level holds a multiple of 8 entries
+	// the span of those levels (they are the coarse, small ones) is cleared by the bin kernel, which runs to completion
+	// before the reduce kernel adds to it; 16-byte aligned because every level holds a multiple of 8 entries
 	const size_t begin = (size_t)grid->tab.offset[first] * sizeof(__half2), end = (size_t)grid->tab.offset[last + 1] * sizeof(__half2);
-	return n2_fill_zero_u32(stream, reinterpret_cast<unsigned char*>(grid->grads) + begin, end - begin);
+	grid->zero_begin = reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(grid->grads) + begin);
+	grid->zero_count = (uint32_t)((end - begin) / 16);
+	return N2_OK;
 }
 
 static inline uint32_t n_pair_tiles(uint32_t n_points) { return (n_points + PAIR_POINTS - 1) / PAIR_POINTS; }
@@ -1133,8 +1145,12 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	uint16_t* rec_keys = reinterpret_cast<uint16_t*>(grid->ws + n_rec * sizeof(uint32_t));
 	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + n_rec * (sizeof(uint32_t) + sizeof(uint16_t)));
 	const dim3 gd(tiles * L);
+	uint4* zero_begin = grid->zero_begin;
+	const uint32_t zero_count = grid->zero_count;
+	grid->zero_begin = nullptr;
+	grid->zero_count = 0;
 #define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
-                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets)
+                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, zero_begin, zero_count)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
 	else if (second && out) LAUNCH(false, true, true);
