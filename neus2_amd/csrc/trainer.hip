@@ -130,18 +130,16 @@ __global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, co
 // output gradients, fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916) and, in the last workgroup, sum the
 // per-ray losses of the live rays and publish the sample set's counters.
 __global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, const uint32_t* __restrict__ n_in_ptr, hf* __restrict__ dloss,
-                                                                   float* __restrict__ coords, uint32_t blocks_f16, uint32_t blocks_f32,
-                                                                   const uint32_t* __restrict__ set_counters, uint32_t max_rays,
+                                                                   float* __restrict__ coords, const uint32_t* __restrict__ set_counters, uint32_t max_rays,
                                                                    const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
 	const uint32_t n_in = *n_in_ptr;
-	if (blockIdx.x < blocks_f16) {
-		const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, lim = (size_t)n_in * 16;
-		if (n_in == 0 || i < lim || i >= (size_t)T * 16) return;
-		dloss[i] = (hf)((float)dloss[i % lim] * (float)n_in / (float)T);
-	} else if (blockIdx.x < blocks_f16 + blocks_f32) {
-		const size_t i = (size_t)(blockIdx.x - blocks_f16) * 256 + threadIdx.x, lim = (size_t)n_in * 7;
-		if (n_in == 0 || i < lim || i >= (size_t)T * 7) return;
-		coords[i] = coords[i % lim];
+	if (blockIdx.x + 1 < gridDim.x) {
+		// the padding is usually a small tail of the batch: the workgroups stride over it instead of covering all of T
+		if (n_in == 0 || n_in >= T) return;
+		const size_t stride = (size_t)(gridDim.x - 1) * 256, first = (size_t)blockIdx.x * 256 + threadIdx.x;
+		const size_t lim16 = (size_t)n_in * 16, lim7 = (size_t)n_in * 7;
+		for (size_t i = lim16 + first; i < (size_t)T * 16; i += stride) dloss[i] = (hf)((float)dloss[i % lim16] * (float)n_in / (float)T);
+		for (size_t i = lim7 + first; i < (size_t)T * 7; i += stride) coords[i] = coords[i % lim7];
 	} else {
 		__shared__ float part[4];
 		const uint32_t n = min(set_counters[0], max_rays);
@@ -333,9 +331,10 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	                               set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
 	                               t->ws_composite, t->ws_composite_bytes)) return rc;
 	// pad the compacted batch to exactly T samples; loss sum and counters
-	const uint32_t blocks_f16 = (uint32_t)(((size_t)T * 16 + 255) / 256), blocks_f32 = (uint32_t)(((size_t)T * 7 + 255) / 256);
-	trainer_finish_batch_kernel<<<dim3(blocks_f16 + blocks_f32 + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, blocks_f16,
-	                                                                                  blocks_f32, ray_counter, n_rays, t->ray_loss, t->counters);
+	uint32_t pad_blocks = (uint32_t)(((size_t)T * 16 + 255) / 256);
+	if (pad_blocks > 512) pad_blocks = 512;
+	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, ray_counter, n_rays,
+	                                                                     t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
 	// forward + backward on the compacted batch, then the optimiser
 	if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
