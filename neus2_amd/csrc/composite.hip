@@ -93,13 +93,14 @@ constexpr int CB = 256;  // 4 rays per workgroup
 
 __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uint32_t n_rays, const uint32_t* __restrict__ ray_counter,
                                                                const uint32_t* __restrict__ numsteps, const hf* __restrict__ net_out,
-                                                               const float* __restrict__ coords, RayScratch* __restrict__ scratch) {
+                                                               const float* __restrict__ coords, RayScratch* __restrict__ scratch,
+                                                               uint32_t* __restrict__ kept_of) {
 	const int lane = threadIdx.x & 63;
 	const uint32_t ray = blockIdx.x * (CB / 64) + (threadIdx.x >> 6);
 	if (ray >= n_rays) return;
 	const uint32_t live = ray_counter ? min(*ray_counter, n_rays) : n_rays;
 	if (ray >= live) {
-		if (lane == 0) scratch[ray] = RayScratch{{0.f, 0.f, 0.f}, 0u};
+		if (lane == 0) { scratch[ray] = RayScratch{{0.f, 0.f, 0.f}, 0u}; kept_of[ray] = 0u; }
 		return;
 	}
 	const uint32_t n = numsteps[2 * ray], base = numsteps[2 * ray + 1];
@@ -130,53 +131,37 @@ __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uin
 		if (n_proc < 64) break;
 	}
 	if (kept == n) { r0 += T * c.bg[0]; r1 += T * c.bg[1]; r2 += T * c.bg[2]; }
-	if (lane == 0) scratch[ray] = RayScratch{{r0, r1, r2}, kept};
-}
-
-// exclusive scan of kept counts in ray order, one workgroup; also applies the budget clamp
-__global__ void __launch_bounds__(1024) composite_scan_kernel(uint32_t n_rays, uint32_t max_compacted, const RayScratch* __restrict__ scratch,
-                                                              uint32_t* __restrict__ cbase, uint32_t* __restrict__ ckept,
-                                                              uint32_t* __restrict__ counter) {
-	__shared__ uint32_t wave_tot[16];
-	__shared__ uint32_t carry_s;
-	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	if (threadIdx.x == 0) carry_s = 0;
-	__syncthreads();
-	for (uint32_t r0 = 0; r0 < n_rays; r0 += 1024) {
-		const uint32_t r = r0 + threadIdx.x;
-		const uint32_t k = r < n_rays ? scratch[r].kept : 0u;
-		uint32_t v = k;
-#pragma unroll
-		for (int o = 1; o < 64; o <<= 1) {
-			const uint32_t u = __shfl_up(v, o);
-			if (lane >= o) v += u;
-		}
-		if (lane == 63) wave_tot[wave] = v;
-		__syncthreads();
-		uint32_t before = carry_s;
-		for (int w = 0; w < wave; ++w) before += wave_tot[w];
-		const uint32_t excl = before + v - k;
-		if (r < n_rays) {
-			cbase[r] = excl;
-			ckept[r] = min(max_compacted - min(max_compacted, excl), k);
-		}
-		__syncthreads();
-		if (threadIdx.x == 1023) carry_s = excl + k;
-		__syncthreads();
-	}
-	if (threadIdx.x == 0) *counter = carry_s;
+	if (lane == 0) { scratch[ray] = RayScratch{{r0, r1, r2}, kept}; kept_of[ray] = kept; }
 }
 
 __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, uint32_t n_rays, uint32_t* __restrict__ numsteps,
                                                                 const hf* __restrict__ net_out, const float* __restrict__ coords,
                                                                 const float* __restrict__ rgb_target, const RayScratch* __restrict__ scratch,
-                                                                const uint32_t* __restrict__ cbase, const uint32_t* __restrict__ ckept,
-                                                                float* __restrict__ coords_out, hf* __restrict__ dloss, float* __restrict__ loss) {
-	const int lane = threadIdx.x & 63;
-	const uint32_t ray = blockIdx.x * (CB / 64) + (threadIdx.x >> 6);
+                                                                const uint32_t* __restrict__ kept_of, uint32_t max_compacted,
+                                                                uint32_t* __restrict__ counter, float* __restrict__ coords_out,
+                                                                hf* __restrict__ dloss, float* __restrict__ loss) {
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	// Where this workgroup's rays start in the compacted batch: the kept samples of all rays before them, in ray order
+	// (deterministic).  Every workgroup adds up the counts of its predecessors itself: a few KiB of L2 reads each
+	// instead of a scan kernel in between.
+	__shared__ uint32_t part[CB / 64];
+	const uint32_t first = blockIdx.x * (CB / 64);
+	uint32_t before = 0;
+	for (uint32_t r = threadIdx.x; r < first; r += CB) before += kept_of[r];
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
+	if (lane == 0) part[wave] = before;
+	__syncthreads();
+	const uint32_t ray = first + wave;
 	if (ray >= n_rays) return;
+	uint32_t cb = 0;
+#pragma unroll
+	for (int w = 0; w < CB / 64; ++w) cb += part[w];
+	for (int w = 0; w < wave; ++w) cb += kept_of[first + w];
+	const uint32_t kept = kept_of[ray];
+	const uint32_t m = min(max_compacted - min(max_compacted, cb), kept);  // the batch holds max_compacted samples
+	if (ray == n_rays - 1 && lane == 0) *counter = cb + kept;
 	const uint32_t base = numsteps[2 * ray + 1];
-	const uint32_t m = ckept[ray], cb = cbase[ray];
 	const RayScratch rs = scratch[ray];
 	// Huber(0.1)/5 per channel
 	float grad[3], lsum = 0.f;
@@ -305,17 +290,14 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
 	c.max_step = c.min_step * 128.f;       // * 2^(NERF_CASCADES-1), unwarp_dt :617-620
 	unsigned char* w = reinterpret_cast<unsigned char*>(d_workspace);
 	RayScratch* scratch = reinterpret_cast<RayScratch*>(w);
-	uint32_t* cbase = reinterpret_cast<uint32_t*>(w + up256(sizeof(RayScratch) * (uint64_t)n_rays));
-	uint32_t* ckept = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(cbase) + up256(4ull * n_rays));
+	uint32_t* kept_of = reinterpret_cast<uint32_t*>(w + up256(sizeof(RayScratch) * (uint64_t)n_rays));
 	const dim3 grid((n_rays + CB / 64 - 1) / (CB / 64)), block(CB);
 	const hf* out = reinterpret_cast<const hf*>(d_network_output);
 	N2ProfScope prof(N2_PROF_COMPOSITE, s);
-	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch);
+	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch, kept_of);
 	N2_LAUNCH_CHECK();
-	composite_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples_compacted, scratch, cbase, ckept, d_compacted_counter);
-	N2_LAUNCH_CHECK();
-	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, cbase, ckept,
-	                                                 d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss);
+	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, kept_of, max_samples_compacted,
+	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
