@@ -221,6 +221,12 @@ int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, ui
 int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                     const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode);
 
+/* n2_mlp_backward that uses only the first n_rows rows of dL_doutput and takes the others as zero.  The reference
+ * extracts the three colour rows of dL_doutput into a zero-padded matrix before the colour net's backward
+ * (nerf_network.h:338-340); this call reads them in place. */
+int n2_mlp_backward_rows(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n, const n2_half* d_dL_doutput,
+                         n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode);
+
 /* DifferentiableObject::input_gradient(stream, dim, input, d_dinput): gradient of output
  * row `dim` w.r.t. the input, i.e. backward with dL_doutput = e_dim and no parameter
  * gradients.  The reference builds e_0 by hand and calls backward with Ignore to get the

@@ -37,7 +37,6 @@ struct n2_field {
 	hf* d_sdf_in;      // [sdf_in_w][N]
 	float* v;          // [3][N]  dL / d normal
 	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
-	hf* dL_drgb;       // [N][16]
 	float* var_acc;    // [4]
 	void* ws_sdf;
 	void* ws_rgb;
@@ -142,22 +141,19 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 	o[10] = (hf)c[6];
 }
 
-// dL_drgb = rows 0..2 of dL_doutput (rest zero); variance gradient = sum of row 7
-// (workgroup reduction, then one atomic per 1024 samples: same-address atomics serialise).
+// After the colour net's backward: the SDF output also receives dL_doutput row 3 directly (the density path); the
+// variance gradient is the sum of row 7 (workgroup reduction, then one atomic per 1024 samples: same-address atomics
+// serialise).
 constexpr uint32_t PREP_BLOCK = 1024;
-__global__ void __launch_bounds__(PREP_BLOCK) field_backward_prep_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ dL_drgb,
-                                                                         float* __restrict__ var_acc) {
+__global__ void __launch_bounds__(PREP_BLOCK) field_direct_gradients_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ d_sdf_out_row0,
+                                                                            float* __restrict__ var_acc) {
 	__shared__ float part[PREP_BLOCK / 64];
 	const uint32_t i = blockIdx.x * PREP_BLOCK + threadIdx.x;
 	float s = 0.f;
 	if (i < N) {
-		const hf* src = dL_dout + (size_t)i * 16;
 		typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-		const half8 in = *reinterpret_cast<const half8*>(src);
-		half8 lo = {in[0], in[1], in[2], (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
-		half8 hi = {(hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0, (hf)0};
-		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16) = lo;
-		*reinterpret_cast<half8*>(dL_drgb + (size_t)i * 16 + 8) = hi;
+		const half8 in = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16);
+		d_sdf_out_row0[i] = d_sdf_out_row0[i] + in[3];
 		s = (float)in[7];
 	}
 #pragma unroll
@@ -169,12 +165,6 @@ __global__ void __launch_bounds__(PREP_BLOCK) field_backward_prep_kernel(uint32_
 		for (uint32_t w = 0; w < PREP_BLOCK / 64; ++w) t += part[w];
 		if (t != 0.f) atomicAdd(var_acc, t);
 	}
-}
-
-__global__ void __launch_bounds__(FB) field_add_density_gradient_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ d_sdf_out_row0) {
-	const uint32_t i = blockIdx.x * FB + threadIdx.x;
-	if (i >= N) return;
-	d_sdf_out_row0[i] = d_sdf_out_row0[i] + dL_dout[(size_t)i * 16 + 3];
 }
 
 // v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
@@ -288,7 +278,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, dL_drgb, var_acc, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_acc, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -308,7 +298,6 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
 	c.v = take(12ull * n);
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
-	c.dL_drgb = take(32ull * n);
 	c.var_acc = take(16);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
@@ -342,7 +331,6 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->d_sdf_in = reinterpret_cast<hf*>(b + c.d_sdf_in);
 	f->v = reinterpret_cast<float*>(b + c.v);
 	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
-	f->dL_drgb = reinterpret_cast<hf*>(b + c.dL_drgb);
 	f->var_acc = reinterpret_cast<float*>(b + c.var_acc);
 	f->ws_sdf = b + c.ws_sdf;
 	f->ws_rgb = b + c.ws_rgb;
@@ -397,13 +385,11 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0, "n2_field_backward: d_dL_doutput must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
 	const hf* dL = reinterpret_cast<const hf*>(d_dL_doutput);
+	// colour net: only rows 0..2 of dL_doutput belong to it
+	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
+	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
 	// (the variance accumulator was cleared by the forward of this batch)
-	field_backward_prep_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->dL_drgb, f->var_acc);
-	N2_LAUNCH_CHECK();
-	// colour net
-	if (int rc = n2_mlp_backward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, reinterpret_cast<const n2_half*>(f->dL_drgb),
-	                             N2_LAYOUT_AOS, reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
-	field_add_density_gradient_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, dL, f->d_rgb_in);
+	field_direct_gradients_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->d_rgb_in, f->var_acc);
 	N2_LAUNCH_CHECK();
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient
 	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),

@@ -155,7 +155,9 @@ __device__ __forceinline__ float16v zero16() {
 __device__ __forceinline__ int drow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 
 // 16-row operand (network output gradient) as B operand of both tiles, K = 16
-__device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N, uint32_t col, int g, bool aos, int unit_row, half8& t0, half8& t1) {
+// rows >= n_rows of the operand count as zero (n_rows = 16: all rows are read)
+__device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N, uint32_t col, int g, bool aos, int unit_row, int n_rows, half8& t0,
+                                             half8& t1) {
 	if (unit_row >= 0) {
 		// dL_dy = e_{unit_row} for every sample: nothing is read
 #pragma unroll
@@ -165,6 +167,11 @@ __device__ __forceinline__ void outgrad_frag(const hf* __restrict__ dY, size_t N
 		t1 = *reinterpret_cast<const half8*>(dY + (size_t)(col + 1) * MLP_OUT + 8 * g);
 	} else {
 		bfrag_soa(dY, (uint32_t)N, 8u * g * (uint32_t)N + col, 0, MLP_OUT, t0, t1);
+	}
+	if (unit_row < 0 && n_rows < MLP_OUT) {
+#pragma unroll
+		for (int e = 0; e < 8; ++e)
+			if (8 * g + e >= n_rows) { t0[e] = (hf)0; t1[e] = (hf)0; }
 	}
 }
 
@@ -462,7 +469,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_backward_kernel(const hf* __
 		const uint32_t off4 = 4u * g * N + col;
 		half8 xp[2][IC], dyp[2];
 		load_input<IC>(X, N, col, g, xp);
-		outgrad_frag(dY, N, col, g, dy_aos != 0, unit_row, dyp[0], dyp[1]);
+		outgrad_frag(dY, N, col, g, (dy_aos & 1) != 0, unit_row, dy_aos >> 8, dyp[0], dyp[1]);
 		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
 		constexpr int DX_TILES = WANT_DW ? 1 : IN_MT;  // with two roles each computes one row tile of dL_dx
 		half8 dx_keep[DX_TILES][2];                    // tile 0's rows until tile 1's are known (sample-pair stores)
@@ -606,7 +613,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_bbi_kernel(const hf* __restr
 		half8 xp[2][IC], vp[2][IC], gp[2];
 		load_input<IC>(X, N, col, g, xp);
 		load_input<IC>(V, N, col, g, vp);
-		outgrad_frag(G, N, col, g, false, unit_row, gp[0], gp[1]);
+		outgrad_frag(G, N, col, g, false, unit_row, MLP_OUT, gp[0], gp[1]);
 		if (!valid) {
 			gp[0] = zero8(); gp[1] = zero8();
 #pragma unroll
@@ -915,7 +922,7 @@ static int allow_lds(K kernel, size_t bytes) {
 // unit_row >= 0: dL_doutput is the constant e_{unit_row} and d_dL_doutput is not read
 static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                              const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode,
-                             n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA) {
+                             n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA, uint32_t dy_rows = MLP_OUT) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
@@ -934,7 +941,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	const hf* X = reinterpret_cast<const hf*>(d_input);
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
-	const int aos = dL_layout == N2_LAYOUT_AOS ? 1 : 0;
+	const int aos = (dL_layout == N2_LAYOUT_AOS ? 1 : 0) | ((int)dy_rows << 8);  // layout flag and the number of rows in use
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 #define LAUNCH(IC, NH, DX, DW)                                                                                      \
 	do {                                                                                                            \
@@ -977,6 +984,12 @@ N2_API int n2_mlp_forward_and_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, 
 N2_API int n2_mlp_backward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                            const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput, n2_grad_mode mode) {
 	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode);
+}
+
+N2_API int n2_mlp_backward_rows(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n, const n2_half* d_dL_doutput,
+                                n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode) {
+	N2_REQUIRE(n_rows >= 1 && n_rows <= (uint32_t)MLP_OUT, "n2_mlp_backward_rows: n_rows %u outside [1, %d]", n_rows, MLP_OUT);
+	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows);
 }
 
 N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
