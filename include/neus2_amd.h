@@ -318,6 +318,14 @@ int n2_field_set_workspace(n2_field_t* field, void* d_workspace, uint64_t n_byte
  * The forward context stays in the workspace until the next forward. */
 int n2_field_forward(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, n2_half* d_output);
 
+/* Makes the samples d_source_index[0 .. n) of the last n2_field_forward (over n_source samples) the batch that the next
+ * n2_field_backward differentiates: their saved activations are gathered instead of being computed again.  The
+ * result is bit-identical to n2_field_forward on those samples' coordinates followed by n2_field_backward, because
+ * every sample is evaluated independently of its batch.  n <= the workspace's backward capacity; indices may repeat.
+ * No counterpart in the reference, which runs the network a second time on the compacted batch
+ * (src/testbed_nerf.cu:3919-3936). */
+int n2_field_select(n2_field_t* field, n2_stream_t stream, const uint32_t* d_source_index, uint32_t n_source, uint32_t n);
+
 /* NerfNetwork::backward_impl, nerf_network.h:317-588, for the batch of the last forward.
  *  d_dL_doutput   fp16 N x 16 (AoS): rows 0..2 colour, 3 sdf, 4..6 eikonal (divided here by
  *                 ek_batch_size), 7 variance, 8..10 gradient w.r.t. the normal through cos
@@ -405,6 +413,15 @@ int n2_composite_loss(n2_stream_t stream, const n2_composite_config* config, uin
                       const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
                       uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
                       float* d_loss, void* d_workspace, uint64_t workspace_bytes);
+/* n2_composite_loss that also writes, for every compacted sample, the index of the marched sample it is
+ * (d_source_index: uint32 [max_samples_compacted], may be NULL).  No counterpart in the reference, whose step evaluates
+ * the network a second time on the compacted coordinates; with the index the saved activations of the first evaluation
+ * can be selected instead (n2_field_select). */
+int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* config, uint32_t n_rays,
+                              const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                              const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                              uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                              float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes);
 
 /* tcnn fill_rollover / fill_rollover_and_rescale, src/testbed_nerf.cu:3908-3916: pad a compacted
  * batch of *d_n_in rows to n_total rows by wrapping around; the fp16 variant scales the wrapped
@@ -482,6 +499,10 @@ typedef struct n2_trainer_config {
 	                                   (or from streams the caller orders against each other). */
 	float ema_decay;                /* 0: plain Adam.  In (0, 1): the Ema wrapper of configs/nerf/base.json:5-7 (0.95) keeps a
 	                                   bias-corrected moving average of the fp16 weights as the inference parameters */
+	uint32_t recompute_training_forward; /* non-zero: the field is evaluated a second time on the compacted batch, as the
+	                                   reference does (src/testbed_nerf.cu:3919-3936).  0: the activations that the first
+	                                   evaluation saved are selected for the compacted samples (n2_field_select); the
+	                                   gradients are bit-identical either way */
 } n2_trainer_config;
 
 /* All device memory a trainer uses (parameters, optimiser state, every temporary) lives in one

@@ -45,7 +45,8 @@ class TrainerConfig(C.Structure):
     """struct n2_trainer_config"""
     _fields_ = [("field", FieldConfig), ("adam", AdamConfig), ("composite", CompositeConfig),
                 ("target_batch_size", C.c_uint32), ("max_rays_per_batch", C.c_uint32), ("max_samples", C.c_uint32),
-                ("loss_scale", C.c_float), ("prefetch_samples", C.c_uint32), ("ema_decay", C.c_float)]
+                ("loss_scale", C.c_float), ("prefetch_samples", C.c_uint32), ("ema_decay", C.c_float),
+                ("recompute_training_forward", C.c_uint32)]
 
 
 class TrainerOptimizerBuffers(C.Structure):

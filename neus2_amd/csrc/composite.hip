@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
                                                                 const float* __restrict__ rgb_target, const RayScratch* __restrict__ scratch,
                                                                 const uint32_t* __restrict__ kept_of, uint32_t max_compacted,
                                                                 uint32_t* __restrict__ counter, float* __restrict__ coords_out,
-                                                                hf* __restrict__ dloss, float* __restrict__ loss) {
+                                                                hf* __restrict__ dloss, float* __restrict__ loss, uint32_t* __restrict__ source_index) {
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 	// Where this workgroup's rays start in the compacted batch: the kept samples of all rays before them, in ray order
 	// (deterministic).  Every workgroup adds up the counts of its predecessors itself: a few KiB of L2 reads each
@@ -241,6 +241,7 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 			float* co = coords_out + ((size_t)cb + s) * 7;
 #pragma unroll
 			for (int k = 0; k < 7; ++k) co[k] = ci[k];
+			if (source_index) source_index[cb + s] = base + s;  // which marched sample this compacted sample is
 		}
 		T = __shfl(Ta, 63);
 		p0 = __shfl(q0, 63); p1 = __shfl(q1, 63); p2 = __shfl(q2, 63);
@@ -271,6 +272,16 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
                              const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
                              uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
                              float* d_loss, void* d_workspace, uint64_t workspace_bytes) {
+	return n2_composite_loss_indexed(stream, cfg, n_rays, d_ray_counter, d_numsteps, d_network_output, d_coords, d_rgb_target,
+	                                 max_samples_compacted, d_compacted_counter, d_coords_compacted, d_dloss_doutput, d_loss, nullptr,
+	                                 d_workspace, workspace_bytes);
+}
+
+N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
+                                     const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                                     const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                                     uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                                     float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes) {
 	N2_REQUIRE(cfg != nullptr, "n2_composite_loss: config is null");
 	N2_REQUIRE(d_compacted_counter != nullptr, "n2_composite_loss: d_compacted_counter is null");
 	hipStream_t s = n2_stream(stream);
@@ -297,7 +308,7 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
 	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch, kept_of);
 	N2_LAUNCH_CHECK();
 	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, kept_of, max_samples_compacted,
-	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss);
+	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss, d_source_index);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -38,6 +38,14 @@ struct n2_field {
 	float* v;          // [3][N]  dL / d normal
 	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
 	float* var_acc;    // [4]
+	// a selection of the last forward's samples (n2_field_select), read by the backward instead of the rows above
+	hf* sel_sdf_in;       // [sdf_in_w][n]
+	hf* sel_rgb_in;       // [48][n]
+	hf* sel_dsdf_denc;    // [enc_w][n]  rows 3 .. 3 + enc_w of dsdf_din
+	float* sel_xyz;       // [3][n]
+	uint32_t* sel_index;  // [n]
+	uint32_t last_n;      // samples of the last forward
+	uint32_t sel_n;       // samples selected (0: the backward reads the forward's own rows)
 	void* ws_sdf;
 	void* ws_rgb;
 	void* ws_grid;
@@ -174,10 +182,13 @@ __global__ void __launch_bounds__(PREP_BLOCK) field_direct_gradients_kernel(uint
 __global__ void __launch_bounds__(FB) field_second_order_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, const hf* __restrict__ d_rgb_in,
                                                                      const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
                                                                      float* __restrict__ v, hf* __restrict__ d_density_in,
-                                                                     const float* __restrict__ var_acc, hf* __restrict__ var_grad, int accumulate) {
+                                                                     const float* __restrict__ var_acc, hf* __restrict__ var_grad, int accumulate,
+                                                                     const uint32_t* __restrict__ src_index, uint32_t n_src) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + var_acc[0]) : (hf)var_acc[0];
 	if (i >= N) return;
+	// the Jacobian rows are those of the forward: of sample src_index[i] among n_src when a selection is active
+	const size_t js = src_index ? src_index[i] : i, jn = src_index ? n_src : N;
 	const hf* g = dL_dout + (size_t)i * 16;
 	float vv[3];
 #pragma unroll
@@ -190,10 +201,60 @@ __global__ void __launch_bounds__(FB) field_second_order_prep_kernel(uint32_t N,
 		d_density_in[(size_t)d * N + i] = (hf)x;
 	}
 	for (uint32_t r = 0; r < enc_w; ++r) {
-		const float* j = dy_dx + ((size_t)r * N + i) * 3;
+		const float* j = dy_dx + ((size_t)r * jn + js) * 3;
 		d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
 	}
 	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
+}
+
+// out[r][j] = in[r][index[j]] for the rows the backward reads; blockIdx.y picks a group of 8 fp16 rows (SDF-net input,
+// colour-net input, encoding rows of d sdf / d input) or, last, the three fp32 position rows.  Two samples per thread so
+// that the stores move pairs.
+__global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n_src, const uint32_t* __restrict__ index, uint32_t sdf_in_w,
+                                                          uint32_t rgb_in_w, uint32_t enc_w, const hf* __restrict__ sdf_in,
+                                                          const hf* __restrict__ rgb_in, const hf* __restrict__ dsdf_din,
+                                                          const float* __restrict__ xyz, hf* __restrict__ o_sdf_in, hf* __restrict__ o_rgb_in,
+                                                          hf* __restrict__ o_denc, float* __restrict__ o_xyz, uint32_t* __restrict__ o_index) {
+	typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+	const uint32_t j = (blockIdx.x * FB + threadIdx.x) * 2;
+	if (j >= n) return;
+	const bool two = j + 1 < n;
+	const uint32_t s0 = min(index[j], n_src - 1u), s1 = two ? min(index[j + 1], n_src - 1u) : s0;
+	const uint32_t groups_a = (sdf_in_w + 7) / 8, groups_b = (rgb_in_w + 7) / 8, groups_c = (enc_w + 7) / 8;
+	uint32_t g = blockIdx.y, rows;  // rows of this group (the last group of a matrix may be short)
+	const hf* in;
+	hf* out;
+	if (g < groups_a) { in = sdf_in + (size_t)g * 8 * n_src; out = o_sdf_in + (size_t)g * 8 * n; rows = min(8u, sdf_in_w - g * 8); }
+	else if ((g -= groups_a) < groups_b) { in = rgb_in + (size_t)g * 8 * n_src; out = o_rgb_in + (size_t)g * 8 * n; rows = min(8u, rgb_in_w - g * 8); }
+	else if ((g -= groups_b) < groups_c) { in = dsdf_din + (size_t)(3 + g * 8) * n_src; out = o_denc + (size_t)g * 8 * n; rows = min(8u, enc_w - g * 8); }
+	else {
+#pragma unroll
+		for (int d = 0; d < 3; ++d) {
+			o_xyz[(size_t)d * n + j] = xyz[(size_t)d * n_src + s0];
+			if (two) o_xyz[(size_t)d * n + j + 1] = xyz[(size_t)d * n_src + s1];
+		}
+		o_index[j] = s0;
+		if (two) o_index[j + 1] = s1;
+		return;
+	}
+	hf a[8], b[8];
+#pragma unroll
+	for (uint32_t r = 0; r < 8; ++r) {
+		if (r < rows) { a[r] = in[(size_t)r * n_src + s0]; b[r] = in[(size_t)r * n_src + s1]; }
+	}
+	if (two && (n & 1u) == 0) {
+#pragma unroll
+		for (uint32_t r = 0; r < 8; ++r)
+			if (r < rows) *reinterpret_cast<half2v*>(out + (size_t)r * n + j) = half2v{a[r], b[r]};
+	} else {
+#pragma unroll
+		for (uint32_t r = 0; r < 8; ++r) {
+			if (r < rows) {
+				out[(size_t)r * n + j] = a[r];
+				if (two) out[(size_t)r * n + j + 1] = b[r];
+			}
+		}
+	}
 }
 
 __global__ void __launch_bounds__(FB) field_add_bias_kernel(uint32_t N, hf bias, hf* __restrict__ row0) {
@@ -278,7 +339,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_acc, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_acc, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -299,6 +360,11 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.v = take(12ull * n);
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
 	c.var_acc = take(16);
+	c.sel_sdf_in = take(2ull * f->sdf_in_w * n);
+	c.sel_rgb_in = take(2ull * f->rgb_in_w * n);
+	c.sel_dsdf_denc = take(2ull * f->enc_w * n);
+	c.sel_xyz = take(12ull * n);
+	c.sel_index = take(4ull * n);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
 	c.ws_grid = take(n2_grid_workspace_bytes(f->grid, (uint32_t)nbw));
@@ -332,6 +398,13 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->v = reinterpret_cast<float*>(b + c.v);
 	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
 	f->var_acc = reinterpret_cast<float*>(b + c.var_acc);
+	f->sel_sdf_in = reinterpret_cast<hf*>(b + c.sel_sdf_in);
+	f->sel_rgb_in = reinterpret_cast<hf*>(b + c.sel_rgb_in);
+	f->sel_dsdf_denc = reinterpret_cast<hf*>(b + c.sel_dsdf_denc);
+	f->sel_xyz = reinterpret_cast<float*>(b + c.sel_xyz);
+	f->sel_index = reinterpret_cast<uint32_t*>(b + c.sel_index);
+	f->last_n = 0;
+	f->sel_n = 0;
 	f->ws_sdf = b + c.ws_sdf;
 	f->ws_rgb = b + c.ws_rgb;
 	f->ws_grid = b + c.ws_grid;
@@ -358,6 +431,8 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	N2_REQUIRE(d_coords != nullptr && d_output != nullptr, "n2_field_forward: null buffer");
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "n2_field_forward: d_output must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
+	f->last_n = n;
+	f->sel_n = 0;
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
@@ -385,30 +460,53 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0, "n2_field_backward: d_dL_doutput must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
 	const hf* dL = reinterpret_cast<const hf*>(d_dL_doutput);
+	// the saved activations: those of the last forward, or the samples n2_field_select picked from them
+	const bool sel = f->sel_n != 0;
+	N2_REQUIRE(n == (sel ? f->sel_n : f->last_n), "n2_field_backward: batch %u, but the last %s was over %u samples", n,
+	           sel ? "n2_field_select" : "n2_field_forward", sel ? f->sel_n : f->last_n);
+	const hf* sdf_in = sel ? f->sel_sdf_in : f->sdf_in;
+	const hf* rgb_in = sel ? f->sel_rgb_in : f->rgb_in;
+	const hf* dsdf_denc = sel ? f->sel_dsdf_denc : f->dsdf_din + (size_t)3 * n;
+	const float* xyz = sel ? f->sel_xyz : f->xyz;
 	// colour net: only rows 0..2 of dL_doutput belong to it
-	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
+	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
 	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
 	// (the variance accumulator was cleared by the forward of this batch)
 	field_direct_gradients_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->d_rgb_in, f->var_acc);
 	N2_LAUNCH_CHECK();
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient
-	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
+	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
 	                             N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), mode)) return rc;
 	// dL/dnormal and the variance gradient
 	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
 	                                                             f->d_density_in, f->var_acc, f->grads + f->off_var,
-	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0, sel ? f->sel_index : nullptr, f->last_n);
 	N2_LAUNCH_CHECK();
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)
-	if (int rc = n2_grid_backward_fused(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
-	                                    reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n), nullptr, mode)) return rc;
+	if (int rc = n2_grid_backward_fused(f->grid, stream, xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
+	                                    reinterpret_cast<const n2_half*>(dsdf_denc), nullptr, mode)) return rc;
 	// second order through the SDF net
-	if (int rc = n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n,
+	if (int rc = n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n,
 	                                            reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
 	// pending: one launch sums them
 	return n2_mlp_reduce_deferred(f->rgb, f->sdf, stream);
+}
+
+N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_source_index, uint32_t n_source, uint32_t n) {
+	if (int rc = check_field(f, "n2_field_select", n)) return rc;
+	N2_REQUIRE(n <= f->max_batch_bwd, "n2_field_select: batch %u exceeds the workspace's backward capacity %u", n, f->max_batch_bwd);
+	N2_REQUIRE(n_source == f->last_n && n_source > 0, "n2_field_select: n_source %u, but the last n2_field_forward was over %u samples", n_source,
+	           f->last_n);
+	N2_REQUIRE(n > 0 && d_source_index != nullptr, "n2_field_select: empty selection");
+	const uint32_t groups = (f->sdf_in_w + 7) / 8 + (f->rgb_in_w + 7) / 8 + (f->enc_w + 7) / 8 + 1;
+	field_select_kernel<<<dim3((n + 2 * FB - 1) / (2 * FB), groups), dim3(FB), 0, n2_stream(stream)>>>(
+		n, n_source, d_source_index, f->sdf_in_w, f->rgb_in_w, f->enc_w, f->sdf_in, f->rgb_in, f->dsdf_din, f->xyz, f->sel_sdf_in, f->sel_rgb_in,
+		f->sel_dsdf_denc, f->sel_xyz, f->sel_index);
+	N2_LAUNCH_CHECK();
+	f->sel_n = n;
+	return N2_OK;
 }
 
 static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n,

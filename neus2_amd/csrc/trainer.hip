@@ -39,6 +39,7 @@ struct n2_trainer {
 	hf* mlp_out;              // [max(max_samples, target)][16]
 	hf* dloss;                // [target][16]
 	float* coords_compacted;  // [target][7]
+	uint32_t* src_index;      // [target] marched sample behind every compacted sample
 	float* ray_loss;          // [max_rays]
 	uint32_t* counters;       // [0] live rays, [1] marched samples, [2] compacted samples (+ [4] as float: loss)
 	void* ws_composite;
@@ -59,7 +60,7 @@ struct n2_trainer {
 };
 
 struct TrainerCarve {
-	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], mlp_out, dloss, coords_compacted, numsteps[2], ray_indices[2], rgb_target[2],
+	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], mlp_out, dloss, coords_compacted, src_index, numsteps[2], ray_indices[2], rgb_target[2],
 		set_counters[2], ray_loss, counters, ws_sampler[2], ws_composite, ws_field, total;
 };
 
@@ -85,6 +86,7 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	c.mlp_out = take(32 * (S > T ? S : T));
 	c.dloss = take(32 * T);
 	c.coords_compacted = take(28 * T);
+	c.src_index = take(4 * T);
 	for (int i = 0; i < 2; ++i) {
 		c.numsteps[i] = take(8 * R);
 		c.ray_indices[i] = take(4 * R);
@@ -130,7 +132,8 @@ __global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, co
 // output gradients, fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916) and, in the last workgroup, sum the
 // per-ray losses of the live rays and publish the sample set's counters.
 __global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, const uint32_t* __restrict__ n_in_ptr, hf* __restrict__ dloss,
-                                                                   float* __restrict__ coords, const uint32_t* __restrict__ set_counters, uint32_t max_rays,
+                                                                   float* __restrict__ coords, uint32_t* __restrict__ src_index,
+                                                                   const uint32_t* __restrict__ set_counters, uint32_t max_rays,
                                                                    const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
 	const uint32_t n_in = *n_in_ptr;
 	if (blockIdx.x + 1 < gridDim.x) {
@@ -140,6 +143,7 @@ __global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, c
 		const size_t lim16 = (size_t)n_in * 16, lim7 = (size_t)n_in * 7;
 		for (size_t i = lim16 + first; i < (size_t)T * 16; i += stride) dloss[i] = (hf)((float)dloss[i % lim16] * (float)n_in / (float)T);
 		for (size_t i = lim7 + first; i < (size_t)T * 7; i += stride) coords[i] = coords[i % lim7];
+		for (size_t i = n_in + first; i < T; i += stride) src_index[i] = src_index[i % n_in];
 	} else {
 		__shared__ float part[4];
 		const uint32_t n = min(set_counters[0], max_rays);
@@ -201,6 +205,7 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->mlp_out = reinterpret_cast<hf*>(b + c.mlp_out);
 	t->dloss = reinterpret_cast<hf*>(b + c.dloss);
 	t->coords_compacted = reinterpret_cast<float*>(b + c.coords_compacted);
+	t->src_index = reinterpret_cast<uint32_t*>(b + c.src_index);
 	t->ray_loss = reinterpret_cast<float*>(b + c.ray_loss);
 	t->counters = reinterpret_cast<uint32_t*>(b + c.counters);
 	t->ws_sampler_bytes = c.ws_sampler[1] - c.ws_sampler[0];
@@ -327,17 +332,23 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	n2_composite_config cc = t->cfg.composite;
 	cc.n_rays_norm = n_rays;
 	cc.loss_scale = t->cfg.loss_scale;
-	if (int rc = n2_composite_loss(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
-	                               set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss), t->ray_loss,
-	                               t->ws_composite, t->ws_composite_bytes)) return rc;
+	if (int rc = n2_composite_loss_indexed(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
+	                                       set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss),
+	                                       t->ray_loss, t->src_index, t->ws_composite, t->ws_composite_bytes)) return rc;
 	// pad the compacted batch to exactly T samples; loss sum and counters
 	uint32_t pad_blocks = (uint32_t)(((size_t)T * 16 + 255) / 256);
 	if (pad_blocks > 512) pad_blocks = 512;
-	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, ray_counter, n_rays,
+	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, t->src_index, ray_counter, n_rays,
 	                                                                     t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
-	// forward + backward on the compacted batch, then the optimiser
-	if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	// forward + backward on the compacted batch, then the optimiser.  Every compacted sample is one of the marched
+	// samples the field has just been evaluated on: unless asked to run the field again, the activations saved for it
+	// are selected instead (the same values, a fraction of the work).
+	if (t->cfg.recompute_training_forward) {
+		if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	} else {
+		if (int rc = n2_field_select(t->field, stream, t->src_index, n_inference, T)) return rc;
+	}
 	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
 	if (int rc = n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
 	                          reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps)) return rc;

@@ -19,7 +19,8 @@ def next_multiple(x, m):
 
 def default_config(target_batch_size=1 << 18, max_rays_per_batch=1 << 16, max_samples=None, n_levels=16,
                    log2_hashmap_size=19, base_resolution=16, per_level_scale=1.447, ek_loss_weight=0.01,
-                   background=(1.0, 1.0, 1.0), learning_rate=1e-3, prefetch_samples=True, ema_decay=0.0):
+                   background=(1.0, 1.0, 1.0), learning_rate=1e-3, prefetch_samples=True, ema_decay=0.0,
+                   recompute_training_forward=False):
     """configs/nerf/base.json, with the level count / growth factor BASELINE's configs fix."""
     if max_samples is None:
         max_samples = 16 * target_batch_size  # src/testbed_nerf.cu:3719
@@ -33,6 +34,8 @@ def default_config(target_batch_size=1 << 18, max_rays_per_batch=1 << 16, max_sa
     cfg.loss_scale = 128.0
     cfg.prefetch_samples = 1 if prefetch_samples else 0
     cfg.ema_decay = ema_decay  # configs/nerf/base.json:5-7 wraps Adam in Ema(0.95); 0 leaves plain Adam
+    # False: the compacted batch re-uses the activations of the step's first field evaluation (bit-identical gradients)
+    cfg.recompute_training_forward = 1 if recompute_training_forward else 0
     return cfg
 
 

@@ -171,3 +171,33 @@ def test_progressive_level_mask_follows_the_step_count(oracle):
         assert (g[2 * int(offset[want]):] == 0).all()
     enc.set_progressive(1.0, 0.0, 0)
     assert enc.active_levels() == 16
+
+
+def test_selected_activations_give_the_same_steps_as_a_second_forward():
+    """The step can evaluate the field again on the compacted batch (as the reference does) or select the activations
+    its first evaluation saved: parameters, optimiser state and counters agree bit for bit after several steps, also
+    when the batch is padded by roll-over and when rays are cut by the batch limit."""
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    cams = scene.cameras_on_sphere(6, 64)
+    d_cams, d_rgba, d_bits = pack_cameras(cams), dev(scene.render_sphere_images(cams)), dev(scene.sphere_bitfield())
+    T = 4096
+    plan = [(60, 0), (60, 1), (200, 2), (200, 3), (33, 4)]  # few rays: roll-over padding; many: the batch limit cuts rays
+    runs = []
+    for recompute in (True, False):
+        tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=512, max_samples=16 * T, recompute_training_forward=recompute))
+        tr.set_scene(d_cams, len(cams), d_rgba, d_bits)
+        tr.initialize_params(seed=5, sdf_mlp_weights=None)
+        seen = []
+        for n_rays, seed in plan:
+            tr.step(n_rays=n_rays, n_inference=16 * T, seed=seed)
+            seen.append((tr.read_counters(), tr.grads.clone()))
+        runs.append((seen, tr.master.clone()))
+    (a, ma), (b, mb) = runs
+    kinds = set()
+    for (ca, ga), (cb, gb) in zip(a, b):
+        assert ca == cb
+        assert torch.equal(ga, gb)
+        kinds.add("padded" if ca["compacted"] < T else "cut" if ca["compacted"] > T else "exact")
+    assert {"padded", "cut"} <= kinds
+    assert torch.equal(ma, mb)

@@ -56,7 +56,7 @@ def test_trainer_config_struct_matches_header():
     from neus2_amd import capi
     assert ctypes.sizeof(capi.FieldConfig) == 32 and ctypes.sizeof(capi.AdamConfig) == 20
     assert ctypes.sizeof(capi.CompositeConfig) == 28 and ctypes.sizeof(capi.Camera) == 80
-    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 24
+    assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 28
     assert ctypes.sizeof(capi.OccupancyBuffers) == 6 * 8 + 3 * 4 + 4 + 2 * 8 and ctypes.sizeof(capi.TrainerOptimizerBuffers) == 5 * 8 + 8
     L = capi.lib()
     cfg = capi.TrainerConfig()
