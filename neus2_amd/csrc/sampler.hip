@@ -12,6 +12,9 @@
 
 constexpr float STEP = 1.73205080757f / 1024.f;  // STEPSIZE(), src/testbed_nerf.cu:51-53
 constexpr uint32_t GRIDSIZE = 128, MARCH_STEPS = 1024;
+// One lane per ray: a few thousand lanes that mostly wait for memory.  Small workgroups spread them over many CUs (packed
+// onto a few CUs the rays slow each other down by a fifth and the generator no longer hides behind a training step).
+constexpr uint32_t SAMPLER_BLOCK = 128;
 
 __device__ __forceinline__ uint32_t hash_u32(uint32_t seed, uint32_t ctr) {
 	uint32_t x = ctr * 747796405u + seed * 2891336453u + 1u;
@@ -108,41 +111,54 @@ __device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint3
 	return r;
 }
 
-template <bool EMIT>
-__device__ __forceinline__ uint32_t march(const RaySetup& r, const uint8_t* __restrict__ bitfield, float* __restrict__ coords, uint32_t max_emit) {
-	uint32_t j = 0;
+// The march of one ray, as the reference writes it: t_0 = startt, every visited step adds STEP to t; at an occupied
+// step a sample is emitted, at an empty one the steps below t + to_next_voxel(pos) are skipped without being looked at;
+// the ray ends at the first visited step outside the unit cube or after MARCH_STEPS samples.  Every visited step costs
+// a dependent read of the bitfield, so the walk is done ONCE: it returns the number of samples and records which
+// steps (counted in additions of STEP) emitted one, as a bit mask of MASK_WORDS words kept word-major
+// (mask[word * n_rays + ray]).  The coordinates are written later from the mask, without touching the bitfield.
+// A ray inside the unit cube is at most sqrt(3) long, i.e. MARCH_STEPS steps plus the start jitter.
+constexpr uint32_t MASK_WORDS = 34, MASK_BITS = MASK_WORDS * 32;
+
+__device__ __forceinline__ uint32_t march_and_mark(const RaySetup& r, const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ mask,
+                                                   uint32_t ray, uint32_t n_rays) {
+	uint32_t j = 0, k = 0, word = 0, widx = 0;
 	float t = r.startt;
-	const uint32_t limit = EMIT ? max_emit : MARCH_STEPS;
-	while (j < limit) {
+	while (j < MARCH_STEPS && k < MASK_BITS) {
 		float pos[3];
 #pragma unroll
-		for (int k = 0; k < 3; ++k) pos[k] = __fmaf_rn(t, r.dir[k], r.o[k]);
+		for (int d = 0; d < 3; ++d) pos[d] = __fmaf_rn(t, r.dir[d], r.o[d]);
 		if (!(pos[0] >= 0.f && pos[0] <= 1.f && pos[1] >= 0.f && pos[1] <= 1.f && pos[2] >= 0.f && pos[2] <= 1.f)) break;
 		if (occupied(bitfield, pos)) {
-			if (EMIT) {
-				float* c = coords + (size_t)j * 7;
-				c[0] = pos[0]; c[1] = pos[1]; c[2] = pos[2];
-				c[3] = 0.0f;
-#pragma unroll
-				for (int k = 0; k < 3; ++k) c[4 + k] = (r.dir[k] + 1.0f) * 0.5f;
+			while ((k >> 5) != widx) {  // words that are complete
+				mask[(size_t)widx * n_rays + ray] = word;
+				word = 0;
+				++widx;
 			}
+			word |= 1u << (k & 31u);
 			++j;
 			t += STEP;
+			++k;
 		} else {
 			const float t_target = t + to_next_voxel(pos, r.dir, r.idir);
-			do { t += STEP; } while (t < t_target);
+			do { t += STEP; ++k; } while (t < t_target);
 		}
+	}
+	for (; widx < MASK_WORDS; ++widx) {
+		mask[(size_t)widx * n_rays + ray] = word;
+		word = 0;
 	}
 	return j;
 }
 
-__global__ void __launch_bounds__(128) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+__global__ void __launch_bounds__(SAMPLER_BLOCK) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                             uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
-                                                            const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts) {
-	const uint32_t i = blockIdx.x * 128 + threadIdx.x;
+                                                            const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts,
+                                                            uint32_t* __restrict__ mask) {
+	const uint32_t i = blockIdx.x * SAMPLER_BLOCK + threadIdx.x;
 	if (i >= n_rays) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
-	counts[i] = r.alive ? march<false>(r, bitfield, nullptr, 0) : 0u;
+	counts[i] = r.alive ? march_and_mark(r, bitfield, mask, i, n_rays) : 0u;
 }
 
 // base[i] = exclusive sum of counts; slot[i] = rank among rays that have samples and fit the budget
@@ -184,29 +200,51 @@ __global__ void __launch_bounds__(1024) sampler_scan_kernel(uint32_t n_rays, uin
 	if (threadIdx.x == 0) { *ray_counter = carry_b; *sample_counter = carry_a; }
 }
 
-__global__ void __launch_bounds__(128) sampler_emit_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+// Coordinates of the samples the march marked: step k of a ray lies at startt + k additions of STEP (the same
+// additions the march made), so the walk is replayed on t alone.
+__global__ void __launch_bounds__(SAMPLER_BLOCK) sampler_emit_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                            uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
-                                                           const uint8_t* __restrict__ bitfield, const uint32_t* __restrict__ counts,
+                                                           const uint32_t* __restrict__ mask, const uint32_t* __restrict__ counts,
                                                            const uint32_t* __restrict__ base, const uint32_t* __restrict__ slot,
                                                            uint32_t* __restrict__ ray_indices, uint32_t* __restrict__ numsteps,
                                                            float* __restrict__ rgb_target, float* __restrict__ coords) {
-	const uint32_t i = blockIdx.x * 128 + threadIdx.x;
+	const uint32_t i = blockIdx.x * SAMPLER_BLOCK + threadIdx.x;
 	if (i >= n_rays) return;
 	const uint32_t s = slot[i];
 	if (s == 0xFFFFFFFFu) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
+	const uint32_t n = counts[i];
 	ray_indices[s] = i;
-	numsteps[2 * s] = counts[i];
+	numsteps[2 * s] = n;
 	numsteps[2 * s + 1] = base[i];
 	rgb_target[(size_t)s * 3 + 0] = r.target[0];
 	rgb_target[(size_t)s * 3 + 1] = r.target[1];
 	rgb_target[(size_t)s * 3 + 2] = r.target[2];
-	march<true>(r, bitfield, coords + (size_t)base[i] * 7, counts[i]);
+	float* c = coords + (size_t)base[i] * 7;
+	const float d0 = (r.dir[0] + 1.0f) * 0.5f, d1 = (r.dir[1] + 1.0f) * 0.5f, d2 = (r.dir[2] + 1.0f) * 0.5f;
+	float t = r.startt;
+	uint32_t j = 0;
+	for (uint32_t w = 0; w < MASK_WORDS && j < n; ++w) {
+		uint32_t bits = mask[(size_t)w * n_rays + i];
+		for (uint32_t b = 0; b < 32u; ++b) {
+			if (bits & 1u) {
+				c[0] = __fmaf_rn(t, r.dir[0], r.o[0]);
+				c[1] = __fmaf_rn(t, r.dir[1], r.o[1]);
+				c[2] = __fmaf_rn(t, r.dir[2], r.o[2]);
+				c[3] = 0.0f;
+				c[4] = d0; c[5] = d1; c[6] = d2;
+				c += 7;
+				++j;
+			}
+			bits >>= 1;
+			t += STEP;
+		}
+	}
 }
 
 static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
 
-N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays); }
+N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays) + up256(4ull * MASK_WORDS * max_rays); }
 
 N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
                                         const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
@@ -230,15 +268,16 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	uint32_t* counts = reinterpret_cast<uint32_t*>(w);
 	uint32_t* base = reinterpret_cast<uint32_t*>(w + up256(4ull * n_rays));
 	uint32_t* slot = reinterpret_cast<uint32_t*>(w + 2 * up256(4ull * n_rays));
-	const dim3 grid((n_rays + 127) / 128), block(128);
+	uint32_t* mask = reinterpret_cast<uint32_t*>(w + 3 * up256(4ull * n_rays));
+	const dim3 grid((n_rays + SAMPLER_BLOCK - 1) / SAMPLER_BLOCK), block(SAMPLER_BLOCK);
 	N2ProfScope prof(N2_PROF_SAMPLER, s);
 	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                            background[2], d_bitfield, counts);
+	                                            background[2], d_bitfield, counts, mask);
 	N2_LAUNCH_CHECK();
 	sampler_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples, counts, base, slot, d_ray_counter, d_sample_counter);
 	N2_LAUNCH_CHECK();
 	sampler_emit_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                           background[2], d_bitfield, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
+	                                           background[2], mask, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
