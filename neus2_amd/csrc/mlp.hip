@@ -444,8 +444,13 @@ struct GradAcc {
 // ----------------------------------------------------------------------------
 // WANT_Y: the forward output is written as well (the recomputed hidden activations are at hand): forward and input
 // gradient of the SDF net in one pass over its input.
+// Register cap: amdgpu_num_vgpr counts half of the unified vector registers on this part, so 120 means 240.  Two of
+// these waves then leave 32 of a SIMD's 512 registers free, enough for one small wave of another kernel: with the
+// 248 the compiler takes by itself, a CU that holds a single wave of the sample generator (which runs beside the
+// training step on its own stream) could start only one of these workgroups at a time, and the colour net's backward
+// took 67 us instead of 46.
 template <int IC, int NH, bool WANT_DX, bool WANT_DW, bool WANT_Y = false>
-__global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
+__global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(120))) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
                                                                     const hf* __restrict__ dY, int dy_aos, int unit_row,
                                                                     hf* __restrict__ dX, float* __restrict__ partials,
                                                                     hf* __restrict__ Y = nullptr, int y_aos = 0) {
