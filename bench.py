@@ -300,6 +300,8 @@ def run_lattice_workload(args):
     xyz = xyz.view(3, use, CH).permute(1, 0, 2).contiguous()  # [chunk][3][CH]
     del idx
 
+    net.encoding().set_point_order(True)  # x-fastest lattice points, as Testbed::get_density_on_grid produces them
+
     def chunk(k):
         k %= use
         return net.sdf(xyz[k])

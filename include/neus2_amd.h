@@ -81,6 +81,12 @@ int n2_grid_level_table(const n2_grid_t* grid, float* scale, uint32_t* resolutio
  * Results do not depend on it. */
 int n2_grid_set_level_costs(n2_grid_t* grid, const float* costs);
 
+/* Hint for n2_grid_forward calls without dy_dx: non-zero says that the points of the following calls come in lattice
+ * order (neighbouring points in neighbouring cells, as in Testbed::get_density_on_grid, src/testbed_nerf.cu:4082-4133).
+ * Such calls are served by a kernel with one lane per point, which is faster when the gathers hit cached lines; values
+ * agree with the default kernel's up to fp32 summation order.  Off by default. */
+int n2_grid_set_point_order(n2_grid_t* grid, int lattice_order);
+
 /* Level mask of the grid encoding.
  *  - n2_grid_set_max_level: GridEncoding::set_max_level as driven by Testbed::set_max_level (src/testbed.cu:1861-1866,
  *    2618): max_level is the fraction of the levels in use, 1 = all.  Level l is switched off when

@@ -31,6 +31,7 @@ struct n2_grid {
 	unsigned char* ws;
 	uint64_t ws_bytes;
 	uint32_t ws_max_points;
+	bool lattice_order;  // points of the next forwards come in lattice order (n2_grid_set_point_order)
 	// part of the gradient buffer the next bucketed scatter clears in its bin kernel (OVERWRITE, levels that add with atomics)
 	uint4* zero_begin;
 	uint32_t zero_count;  // in 16-byte units
@@ -204,6 +205,52 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_forward_kernel(N2LevelTable t
 	const uint32_t i = tile * FWD_POINTS + (threadIdx.x >> 1), b = threadIdx.x & 1u;
 	if (i >= N) return;  // both lanes of a pair share i, so pairs leave together
 #define CALL(M) grid_forward_pair<M, WANT_DYDX>(tab, level, i, b, N, xyz, point_stride, dim_stride, params, out, dy_dx)
+	N2_DISPATCH_MODE(tab.mode[level], CALL)
+#undef CALL
+}
+
+// One lane per (point, level): eight gathers and one fused multiply-add chain per feature.  For points that arrive
+// in lattice order (neighbouring lanes in neighbouring cells) the gathers hit lines the wave has just fetched and
+// the kernel is bound by instruction issue, where the lane pairs of the kernel above cost twice the lanes.
+template <uint32_t MODE>
+__device__ __forceinline__ void grid_forward_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
+                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                                   const __half2* __restrict__ params, __half* __restrict__ out) {
+	const size_t row = (size_t)level * 2;
+	if (n2_level_masked(tab, level, i)) {
+		out[row * N + i] = __float2half_rn(0.f);
+		out[(row + 1) * N + i] = __float2half_rn(0.f);
+		return;
+	}
+	const __half2* P = params + tab.offset[level];
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, tab.scale[level]);
+	uint32_t e[8];
+	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
+	float2 v[8];
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) v[k] = __half22float2(P[e[k]]);
+	float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+	for (uint32_t k = 0; k < 8; ++k) {
+		const float wt = n2_corner_weight(p, k);
+		a0 = fmaf(wt, v[k].x, a0);
+		a1 = fmaf(wt, v[k].y, a1);
+	}
+	out[row * N + i] = __float2half_rn(a0);
+	out[(row + 1) * N + i] = __float2half_rn(a1);
+}
+
+__global__ void __launch_bounds__(GRID_BLOCK) grid_forward_point_kernel(N2LevelTable tab, uint32_t N, uint32_t tiles,
+                                                                        const float* __restrict__ xyz, uint32_t point_stride,
+                                                                        uint32_t dim_stride, const __half2* __restrict__ params,
+                                                                        __half* __restrict__ out) {
+	// level-major workgroup ids, dealt round-robin over the XCDs: every XCD sees an eighth of the tiles of every level.
+	// (Giving whole levels to an XCD, as the scattered-point kernel does, makes every XCD stream all positions and
+	// nearly doubles the time of a lattice chunk: with coherent points the tables' hot lines fit every L2 anyway.)
+	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
+	const uint32_t i = tile * GRID_BLOCK + threadIdx.x;
+	if (i >= N) return;
+#define CALL(M) grid_forward_point<M>(tab, level, i, N, xyz, point_stride, dim_stride, params, out)
 	N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
 }
@@ -888,6 +935,7 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->ws_max_points = 0;
 	g->zero_begin = nullptr;
 	g->zero_count = 0;
+	g->lattice_order = false;
 	*out = g;
 	return N2_OK;
 }
@@ -968,6 +1016,12 @@ N2_API int n2_grid_set_training_step(n2_grid_t* grid, uint32_t training_step) {
 
 N2_API uint32_t n2_grid_active_levels(const n2_grid_t* grid) { return grid ? grid->tab.active_levels : 0; }
 
+N2_API int n2_grid_set_point_order(n2_grid_t* grid, int lattice_order) {
+	N2_REQUIRE(grid != nullptr, "n2_grid_set_point_order: grid is null");
+	grid->lattice_order = lattice_order != 0;
+	return N2_OK;
+}
+
 N2_API int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients) {
 	N2_REQUIRE(grid != nullptr, "n2_grid_set_params: grid is null");
 	N2_REQUIRE(d_params != nullptr, "n2_grid_set_params: d_params is null");
@@ -1027,10 +1081,18 @@ N2_API int n2_grid_forward(n2_grid_t* grid, n2_stream_t stream, const float* d_x
 	if (int rc = check_batch(grid, "n2_grid_forward", d_xyz, point_stride, dim_stride, n_points)) return rc;
 	if (n_points == 0) return N2_OK;
 	N2_REQUIRE(d_out != nullptr, "n2_grid_forward: d_out is null");
-	const uint32_t tiles = (n_points + FWD_POINTS - 1) / FWD_POINTS;
 	N2XcdPlan plan;
-	const dim3 grid_dim(make_xcd_plan(grid, tiles, plan) * N_XCD), block(GRID_BLOCK);
 	N2ProfScope prof(N2_PROF_GRID_FORWARD, n2_stream(stream));
+	if (grid->lattice_order && !d_dy_dx) {
+		const uint32_t tiles = n_tiles(n_points);
+		const dim3 grid_dim(tiles * grid->tab.n_levels);
+		grid_forward_point_kernel<<<grid_dim, dim3(GRID_BLOCK), 0, n2_stream(stream)>>>(grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride,
+			grid->params, reinterpret_cast<__half*>(d_out));
+		N2_LAUNCH_CHECK();
+		return N2_OK;
+	}
+	const uint32_t tiles = (n_points + FWD_POINTS - 1) / FWD_POINTS;
+	const dim3 grid_dim(make_xcd_plan(grid, tiles, plan) * N_XCD), block(GRID_BLOCK);
 	if (d_dy_dx) {
 		grid_forward_kernel<true><<<grid_dim, block, 0, n2_stream(stream)>>>(grid->tab, plan, n_points, tiles, d_xyz, point_stride,
 			dim_stride, grid->params, reinterpret_cast<__half*>(d_out), d_dy_dx);

@@ -423,13 +423,17 @@ N2_API int n2_density_on_grid(n2_field_t* field, n2_stream_t stream, const uint3
 	g.rx = res[0]; g.ry = res[1]; g.rz = res[2]; g.thresh = 0.f;
 	// here scale is the aabb's extent (the division by the resolution is part of the position formula)
 	for (int d = 0; d < 3; ++d) { g.scale[d] = aabb_max[d] - aabb_min[d]; g.offset[d] = aabb_min[d]; }
-	for (uint64_t first = 0; first < n; first += chunk) {
+	// lattice points arrive x fastest: neighbouring lanes in neighbouring cells
+	n2_grid_set_point_order(n2_field_encoding(field), 1);
+	int rc = N2_OK;
+	for (uint64_t first = 0; first < n && rc == N2_OK; first += chunk) {
 		const uint32_t m = (uint32_t)((n - first < chunk) ? n - first : chunk), m8 = (m + 7) / 8 * 8;
 		mc_lattice_positions_kernel<<<mgrid(m8), dim3(MC_BLOCK), 0, s>>>(g, first, m, m8, positions);
-		N2_LAUNCH_CHECK();
-		if (int rc = n2_field_sdf(field, stream, positions, 3, 1, m8, reinterpret_cast<n2_half*>(mlp_out))) return rc;
-		mc_widen_kernel<<<mgrid(m), dim3(MC_BLOCK), 0, s>>>(m, mlp_out, d_density + first);
-		N2_LAUNCH_CHECK();
+		rc = n2_field_sdf(field, stream, positions, 3, 1, m8, reinterpret_cast<n2_half*>(mlp_out));
+		if (rc == N2_OK) mc_widen_kernel<<<mgrid(m), dim3(MC_BLOCK), 0, s>>>(m, mlp_out, d_density + first);
 	}
+	n2_grid_set_point_order(n2_field_encoding(field), 0);
+	if (rc != N2_OK) return rc;
+	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

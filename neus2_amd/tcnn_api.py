@@ -91,6 +91,10 @@ class GridEncoding:
         check(capi.lib().n2_grid_set_params(self._h, ptr(params), ptr(gradients)), "n2_grid_set_params")
         self._params, self._grads = params, gradients
 
+    def set_point_order(self, lattice_order):
+        """Hint for forwards without dy_dx: True when the points come in lattice order (get_density_on_grid)."""
+        check(capi.lib().n2_grid_set_point_order(self._h, C.c_int(1 if lattice_order else 0)), "n2_grid_set_point_order")
+
     def set_max_level(self, value):
         """Fraction of the levels in use (GridEncoding::set_max_level, src/testbed.cu:1861-1866); 1 = all."""
         check(capi.lib().n2_grid_set_max_level(self._h, C.c_float(value)), "n2_grid_set_max_level")
