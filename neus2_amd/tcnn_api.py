@@ -271,6 +271,16 @@ class FullyFusedMLP:
               "n2_mlp_input_gradient")
         return d
 
+    def backward_rows(self, x, dL_dy, n_rows, dL_layout=LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE):
+        """backward() that uses only the first n_rows rows of dL_dy and takes the others as zero (n2_mlp_backward_rows)."""
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        _check_half(dL_dy, (n, 16) if dL_layout == LAYOUT_AOS else (16, n), "dL_doutput")
+        dx = torch.empty((self.input_width(), n), dtype=torch.float16, device=x.device) if want_input_grad else None
+        check(capi.lib().n2_mlp_backward_rows(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(dL_dy), C.c_int(dL_layout),
+                                              C.c_uint32(n_rows), ptr(dx), C.c_int(mode)), "n2_mlp_backward_rows")
+        return dx
+
     def forward_and_input_gradient(self, x, dim=0, out_layout=LAYOUT_SOA, out=None):
         """forward and input_gradient(dim) in one pass over the input: (y, d output[dim] / d input)."""
         n = x.shape[1]
@@ -380,6 +390,14 @@ class NerfNetwork:
         check(capi.lib().n2_field_backward(self._h, _stream(), ptr(coords), C.c_uint32(n), ptr(dL_doutput),
                                            C.c_uint32(n if ek_batch_size is None else ek_batch_size), C.c_int(mode)),
               "n2_field_backward")
+
+    def select(self, source_index, n_source):
+        """Makes the samples source_index (uint32/int32 CUDA tensor) of the last forward, which ran over n_source
+        samples, the batch of the next backward (n2_field_select); backward is then called with their coordinates."""
+        if source_index.dtype not in (torch.int32, torch.uint32) or not source_index.is_cuda or not source_index.is_contiguous():
+            raise N2Error("source_index must be a contiguous 32-bit integer CUDA tensor")
+        check(capi.lib().n2_field_select(self._h, _stream(), ptr(source_index), C.c_uint32(n_source), C.c_uint32(source_index.numel())),
+              "n2_field_select")
 
     def _sdf(self, fn, xyz):
         x, ps, ds, n = _positions(xyz)

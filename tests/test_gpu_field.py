@@ -140,3 +140,33 @@ def test_field_errors(oracle):
     with pytest.raises(N2Error, match="multiple of 8"):
         gf.forward(torch.rand((12, 7), device="cuda"))
     assert gf.forward(torch.rand((0, 7), device="cuda")).shape == (0, 16)
+
+
+def test_select_equals_forward_on_the_selected_samples(oracle):
+    """n2_field_select: backward over samples picked from the last forward (with repeats and gaps, odd and even counts)
+    gives exactly the gradients of a forward over those samples' coordinates followed by the same backward."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, N2Error
+    of, gf, p, dp, dg, rng = make(oracle, seed=6)
+    n_src = 6000
+    coords = rand_coords(rng, n_src)
+    d_coords = dev(coords)
+    for n in (4096, 5000):  # (smaller batches scatter with fp16 atomics, whose order of arrival is not reproducible)
+        idx = np.sort(rng.integers(0, n_src, n)).astype(np.int32)
+        idx[-40:] = idx[:40]  # roll-over style repeats, out of order
+        dL = q16(rng.standard_normal((n, 16)) * np.array([.1, .1, .1, .1, 3, 3, 3, .1, .003, .003, .003, 0, 0, 0, 0, 0]))
+        d_dL = dev(dL, torch.float16)
+        sub = dev(coords[idx])
+        gf.forward(sub)
+        dg.fill_(3.0)
+        gf.backward(sub, d_dL, ek_batch_size=n, mode=GRAD_OVERWRITE)
+        want = dg.clone()
+        gf.forward(d_coords)
+        gf.select(dev(idx, torch.int32), n_src)
+        dg.fill_(3.0)  # (the three spare variance slots are never written)
+        gf.backward(sub, d_dL, ek_batch_size=n, mode=GRAD_OVERWRITE)
+        assert torch.equal(dg, want), n
+    # the batch of a backward must be the selection (or the forward) that precedes it
+    with pytest.raises(N2Error):
+        gf.backward(d_coords, dev(q16(rng.standard_normal((n_src, 16))), torch.float16), ek_batch_size=n_src)
+    with pytest.raises(N2Error):
+        gf.select(dev(idx, torch.int32), n_src + 8)

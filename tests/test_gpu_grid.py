@@ -366,3 +366,28 @@ def test_level_mask(setup, oracle, kind, bucketed):
             import ctypes as C
             capi.lib().n2_grid_set_workspace(gg._h, None, C.c_uint64(0), C.c_uint32(0))
     assert gg.active_levels() == 16
+
+
+def test_lattice_order_forward(setup):
+    """The one-lane-per-point forward that n2_grid_set_point_order selects for lattice-ordered inference: same values as
+    the oracle (and as the default kernel up to fp32 summation order), also with a level mask and ragged sizes."""
+    og, gg, params, d_params, d_grads = setup
+    r = 40
+    z, y, x = np.meshgrid(np.arange(r), np.arange(r), np.arange(r), indexing="ij")
+    xyz = (np.stack([x, y, z]).reshape(3, -1)[:, :r ** 3 - 13] / np.float32(r)).astype(np.float32)
+    ref = og.forward(params, xyz)
+    try:
+        gg.set_point_order(True)
+        y1, _ = gg.forward(dev(xyz))
+        assert_close(host(y1), ref, what="lattice-order forward")
+        gg.set_max_level(0.25)
+        y2, _ = gg.forward(dev(xyz))
+        ref2 = ref.copy()
+        ref2[10:] = 0  # limit 4: levels 0..4 stay
+        assert_close(host(y2), ref2, what="lattice-order forward, masked")
+        assert (host(y2)[10:] == 0).all()
+    finally:
+        gg.set_point_order(False)
+        gg.set_max_level(1.0)
+    y0, _ = gg.forward(dev(xyz))
+    assert rel_l2(host(y1), host(y0)) < 1e-3

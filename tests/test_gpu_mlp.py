@@ -206,3 +206,21 @@ def test_deferred_reduction_sums_pending_passes_in_one_launch(oracle):
     gm.reduce_deferred()
     assert_grad_close(host(dG), 2 * ref1 + ref2, what="accumulate through a deferred reduction")
     gm.set_deferred_reduction(False)
+
+
+@pytest.mark.parametrize("layout", ["soa", "aos"])
+def test_backward_rows_equals_backward_of_the_zero_padded_gradient(oracle, layout):
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, LAYOUT_AOS, LAYOUT_SOA
+    om, gm, W, dW, dG, rng = make(oracle, 48, 2, 21)
+    n = 4096 + 136
+    x = dev(q16(rng.standard_normal((48, n))), torch.float16)
+    dy = q16(rng.standard_normal((16, n)))
+    padded = dy.copy()
+    padded[3:] = 0
+    lay = LAYOUT_AOS if layout == "aos" else LAYOUT_SOA
+    shape = (lambda a: np.ascontiguousarray(a.T)) if layout == "aos" else (lambda a: a)
+    dx_ref = gm.backward(x, dev(shape(padded), torch.float16), lay, mode=GRAD_OVERWRITE)
+    g_ref = dG.clone()
+    dG.fill_(2.0)
+    dx = gm.backward_rows(x, dev(shape(dy), torch.float16), 3, lay, mode=GRAD_OVERWRITE)
+    assert torch.equal(dx, dx_ref) and torch.equal(dG, g_ref)
