@@ -734,6 +734,9 @@ int n2_profile_enable(int enable);
 /* Restricts the timing to the ids whose bit (1 << id) is set (default: all).  An event pair costs a few microseconds of
  * stream time, so a benchmark that times whole steps selects only the kernel it reports on. */
 int n2_profile_select(uint32_t id_mask);
+/* Time only every `every`-th launch of each selected id (1: all).  An event pair costs a few microseconds of stream time,
+ * so a benchmark that times a kernel inside its own timed region samples it. */
+int n2_profile_set_period(uint32_t every);
 /* Waits for all recorded events; total milliseconds and launch count per id since the last reset. */
 int n2_profile_read(n2_prof_id id, float* total_ms, uint32_t* launches);
 int n2_profile_reset(void);

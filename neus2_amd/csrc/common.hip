@@ -53,6 +53,8 @@ namespace {
 struct ProfState {
 	bool enabled = false;
 	uint32_t mask = 0xFFFFFFFFu;                  // ids that are timed while enabled
+	uint32_t period = 1;                          // every period-th launch of an id is timed
+	uint32_t seen[N2_PROF_COUNT] = {};
 	std::vector<hipEvent_t> pool;                 // recycled events
 	std::vector<hipEvent_t> pending[N2_PROF_COUNT];  // begin/end pairs, not yet read
 	float total_ms[N2_PROF_COUNT] = {};
@@ -89,6 +91,7 @@ void prof_collect(int id) {
 
 void n2_prof_begin(int id, hipStream_t stream) {
 	if (!g_prof.enabled || !((g_prof.mask >> id) & 1u)) return;
+	if (g_prof.seen[id]++ % g_prof.period != 0) return;
 	hipEvent_t e = prof_take();
 	if (!e) return;
 	(void)hipEventRecord(e, stream);
@@ -113,6 +116,13 @@ N2_API int n2_profile_enable(int enable) {
 
 N2_API int n2_profile_select(uint32_t id_mask) {
 	g_prof.mask = id_mask;
+	return N2_OK;
+}
+
+N2_API int n2_profile_set_period(uint32_t every) {
+	N2_REQUIRE(every >= 1, "n2_profile_set_period: the period must be at least 1");
+	g_prof.period = every;
+	for (int id = 0; id < N2_PROF_COUNT; ++id) g_prof.seen[id] = 0;
 	return N2_OK;
 }
 
