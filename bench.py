@@ -153,6 +153,15 @@ def run_step_workload(args):
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
+    # MFMA side of the metric: algorithmic flops of every MLP kernel of a step (SDF net 48-64-16: forward 8192 + input
+    # gradient 8192 per marched sample, backward 24576 + second order 14336 per batch sample; colour net 48-64-64-16:
+    # forward 16384 per marched sample, backward with the recomputed forward 47104 per batch sample) over their summed
+    # durations from the untimed per-kernel pass
+    mlp_flops = n_inf * (8192 + 8192 + 16384) + TARGET * (24576 + 14336 + 47104)
+    mlp_ms = sum(kernels[k]["ms_per_step"] for k in ("mlp_forward", "mlp_backward", "mlp_second_order") if k in kernels)
+    mfma = {"kernels": "mlp_forward + mlp_backward + mlp_second_order (all MLP launches of a step)", "algorithmic_flops_per_step": mlp_flops,
+            "ms_per_step": mlp_ms, "achieved_tflops": mlp_flops / (mlp_ms * 1e-3) / 1e12 if mlp_ms else None, "peak_tflops": MFMA_PEAK_TFLOPS,
+            "frac": mlp_flops / (mlp_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS if mlp_ms else None}
     result = {
         "metric": "SDF train samples/sec @2^18 batch (1 GPU)",
         "value": args.steps * TARGET / elapsed,
@@ -172,6 +181,7 @@ def run_step_workload(args):
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated; recorded from profiles/)",
                      "algorithmic_bytes_per_sample": STEP_ALGO_BYTES[dom], "samples_per_launch": per_launch,
                      "avg_launch_us": kernels[dom]["avg_us"], "timed_launches": dom_n},
+        "mfma": mfma,
         "kernels": kernels,
         "kernels_note": "grid_backward_params is timed with HIP events inside the timed region (every fourth step's launch); the other entries come from a "
                         "second, untimed pass of the same steps with every listed kernel bracketed by events",
