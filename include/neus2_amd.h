@@ -266,6 +266,19 @@ int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, const n2_h
                                    const n2_half* d_dL_ddLdinput, const n2_half* d_dL_doutput,
                                    n2_half* d_dL_ddLdoutput, n2_grad_mode mode);
 
+/* Network::backward(..., mode) followed by Network::backward_backward_input(..., nullptr, nullptr, Accumulate) on the
+ * same input, as NerfNetwork::backward_impl calls them on the SDF net (nerf_network.h:402 and :560-571), in one pass:
+ * both sets of weight gradients have the same shape and are summed in the same accumulators.  The parameter
+ * gradients equal those of the two calls up to fp32 summation order.  One hidden layer only.
+ *  d_dL_doutput         fp16 16 x N in dL_layout (first-order output gradient)
+ *  d_dL_dinput          fp16 SoA in_width x N (first-order input gradient, written)
+ *  d_dL_ddLdinput       fp16 SoA in_width x N
+ *  d_second_dL_doutput  the dL_doutput of the second-order call: fp16 SoA 16 x N, or NULL for the constant e_0
+ *  mode                 OVERWRITE or ACCUMULATE */
+int n2_mlp_backward_and_second_order(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                                     const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
+                                     const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode);
+
 /* ------------------------------------------------------------------------
  * The NeuS field: NerfNetwork<__half> (include/neural-graphics-primitives/nerf_network.h),
  * static scene (delta network off, src/testbed.cu:2695-2697).  Composes the hash grid, the

@@ -241,6 +241,19 @@ public:
 		                                     dL_ddLdoutput ? dL_ddLdoutput->data() : nullptr, (n2_grad_mode)mode),
 		      "FullyFusedMLP::backward_backward_input");
 	}
+	// backward(mode) and backward_backward_input(nullptr, nullptr, Accumulate) of the same input in one pass
+	// (nerf_network.h:402 and :560-571 on the SDF net).  second_dL_doutput == nullptr: e_0.
+	void backward_and_second_order(stream_t stream, const GPUMatrixDynamic<half_t>& input, const GPUMatrixDynamic<half_t>& dL_doutput,
+	                               GPUMatrixDynamic<half_t>& dL_dinput, const GPUMatrixDynamic<half_t>& dL_ddLdinput,
+	                               const GPUMatrixDynamic<half_t>* second_dL_doutput = nullptr, GradientMode mode = GradientMode::Overwrite) {
+		detail::require_soa(input, input_width(), input.n(), "FullyFusedMLP input");
+		detail::require_soa(dL_dinput, input_width(), input.n(), "FullyFusedMLP::backward_and_second_order dL_dinput");
+		detail::require_soa(dL_ddLdinput, input_width(), input.n(), "FullyFusedMLP::backward_and_second_order dL_ddLdinput");
+		if (second_dL_doutput) detail::require_soa(*second_dL_doutput, output_width(), input.n(), "FullyFusedMLP::backward_and_second_order second dL_doutput");
+		check(n2_mlp_backward_and_second_order(m_mlp, stream, input.data(), input.n(), dL_doutput.data(), out_layout(dL_doutput, input.n()),
+		                                       dL_dinput.data(), dL_ddLdinput.data(), second_dL_doutput ? second_dL_doutput->data() : nullptr,
+		                                       (n2_grad_mode)mode), "FullyFusedMLP::backward_and_second_order");
+	}
 
 private:
 	n2_layout out_layout(const GPUMatrixDynamic<half_t>& mat, uint32_t n) const {

@@ -37,7 +37,7 @@ struct n2_field {
 	hf* d_sdf_in;      // [sdf_in_w][N]
 	float* v;          // [3][N]  dL / d normal
 	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
-	float* var_acc;    // [4]
+	float* var_part;    // one partial sum of the variance gradient per workgroup of the backward's preparation kernel
 	// a selection of the last forward's samples (n2_field_select), read by the backward instead of the rows above
 	hf* sel_sdf_in;       // [sdf_in_w][n]
 	hf* sel_rgb_in;       // [48][n]
@@ -133,10 +133,9 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 // 11..15 keep what the colour net wrote.
 __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __restrict__ coords, uint32_t N, const hf* __restrict__ sdf_out,
                                                                  hf bias, const float* __restrict__ normal, const hf* __restrict__ variance,
-                                                                 hf* __restrict__ output, float* __restrict__ var_acc) {
+                                                                 hf* __restrict__ output) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
-	if (i == 0) var_acc[0] = 0.f;  // the backward of this batch accumulates the variance gradient here
 	hf* o = output + (size_t)i * 16;
 	const float* c = coords + (size_t)i * 7;
 	o[3] = sdf_out[i] + bias;
@@ -149,20 +148,46 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 	o[10] = (hf)c[6];
 }
 
-// After the colour net's backward: the SDF output also receives dL_doutput row 3 directly (the density path); the
-// variance gradient is the sum of row 7 (workgroup reduction, then one atomic per 1024 samples: same-address atomics
-// serialise).
-constexpr uint32_t PREP_BLOCK = 1024;
-__global__ void __launch_bounds__(PREP_BLOCK) field_direct_gradients_kernel(uint32_t N, const hf* __restrict__ dL_dout, hf* __restrict__ d_sdf_out_row0,
-                                                                            float* __restrict__ var_acc) {
-	__shared__ float part[PREP_BLOCK / 64];
-	const uint32_t i = blockIdx.x * PREP_BLOCK + threadIdx.x;
+// After the colour net's backward, one pass over the samples prepares everything the SDF net's and the grid's
+// backward read:
+//  * the SDF output also receives dL_doutput row 3 directly (the density path): added to row 0 of the colour net's
+//    input gradient, which is the SDF net's output gradient;
+//  * v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
+//  * second-order MLP input rows 0..2 = half(v), rows 3 .. 3+enc_w = dy_dx v (the encoding's
+//    backward_backward_input output dL_ddLdoutput, taken from the Jacobian the forward stored instead of
+//    gathering the table again), rows [3 + enc_w, sdf_in_w) = 0;
+//  * the variance gradient is the sum of row 7: every workgroup leaves its partial sum in var_part[blockIdx.x] and
+//    field_variance_gradient_kernel adds them up in a fixed order.
+__global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, hf* __restrict__ d_rgb_in,
+                                                                 const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
+                                                                 float* __restrict__ v, hf* __restrict__ d_density_in,
+                                                                 float* __restrict__ var_part, const uint32_t* __restrict__ src_index,
+                                                                 uint32_t n_src) {
+	typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+	__shared__ float part[FB / 64];
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	float s = 0.f;
 	if (i < N) {
-		typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-		const half8 in = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16);
-		d_sdf_out_row0[i] = d_sdf_out_row0[i] + in[3];
-		s = (float)in[7];
+		// the Jacobian rows are those of the forward: of sample src_index[i] among n_src when a selection is active
+		const size_t js = src_index ? src_index[i] : i, jn = src_index ? n_src : N;
+		const half8 lo = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16), hi = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16 + 8);
+		d_rgb_in[i] = d_rgb_in[i] + lo[3];
+		s = (float)lo[7];
+		float vv[3];
+#pragma unroll
+		for (int d = 0; d < 3; ++d) {
+			float x = (float)d_rgb_in[(size_t)(35 + d) * N + i];
+			x += (float)lo[4 + d] / ek_batch;
+			x += (float)hi[d];
+			vv[d] = x;
+			v[(size_t)d * N + i] = x;
+			d_density_in[(size_t)d * N + i] = (hf)x;
+		}
+		for (uint32_t r = 0; r < enc_w; ++r) {
+			const float* j = dy_dx + ((size_t)r * jn + js) * 3;
+			d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
+		}
+		for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
 	}
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -170,41 +195,29 @@ __global__ void __launch_bounds__(PREP_BLOCK) field_direct_gradients_kernel(uint
 	__syncthreads();
 	if (threadIdx.x == 0) {
 		float t = 0.f;
-		for (uint32_t w = 0; w < PREP_BLOCK / 64; ++w) t += part[w];
-		if (t != 0.f) atomicAdd(var_acc, t);
+		for (uint32_t w = 0; w < FB / 64; ++w) t += part[w];
+		var_part[blockIdx.x] = t;
 	}
 }
 
-// v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
-// second-order MLP input rows 0..2 = half(v), rows 3 .. 3+enc_w = dy_dx v (the encoding's
-// backward_backward_input output dL_ddLdoutput, taken from the Jacobian the forward stored instead of
-// gathering the table again), rows [3 + enc_w, sdf_in_w) = 0; variance gradient written.
-__global__ void __launch_bounds__(FB) field_second_order_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, const hf* __restrict__ d_rgb_in,
-                                                                     const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
-                                                                     float* __restrict__ v, hf* __restrict__ d_density_in,
-                                                                     const float* __restrict__ var_acc, hf* __restrict__ var_grad, int accumulate,
-                                                                     const uint32_t* __restrict__ src_index, uint32_t n_src) {
-	const uint32_t i = blockIdx.x * FB + threadIdx.x;
-	if (i == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + var_acc[0]) : (hf)var_acc[0];
-	if (i >= N) return;
-	// the Jacobian rows are those of the forward: of sample src_index[i] among n_src when a selection is active
-	const size_t js = src_index ? src_index[i] : i, jn = src_index ? n_src : N;
-	const hf* g = dL_dout + (size_t)i * 16;
-	float vv[3];
+// var_grad = [var_grad +] sum of the n_parts partial sums: one workgroup, fixed order.  1024 lanes, so that a 2^18 batch
+// is one load per lane (the kernel is nothing but memory latency).
+constexpr uint32_t VB = 1024;
+__global__ void __launch_bounds__(VB) field_variance_gradient_kernel(const float* __restrict__ var_part, uint32_t n_parts, hf* __restrict__ var_grad,
+                                                                     int accumulate) {
+	__shared__ float part[VB / 64];
+	float s = 0.f;
+	for (uint32_t i = threadIdx.x; i < n_parts; i += VB) s += var_part[i];
 #pragma unroll
-	for (int d = 0; d < 3; ++d) {
-		float x = (float)d_rgb_in[(size_t)(35 + d) * N + i];
-		x += (float)g[4 + d] / ek_batch;
-		x += (float)g[8 + d];
-		vv[d] = x;
-		v[(size_t)d * N + i] = x;
-		d_density_in[(size_t)d * N + i] = (hf)x;
+	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if (threadIdx.x < 64) {
+		float t = threadIdx.x < VB / 64 ? part[threadIdx.x] : 0.f;
+#pragma unroll
+		for (int o = 8; o > 0; o >>= 1) t += __shfl_xor(t, o);
+		if (threadIdx.x == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + t) : (hf)t;
 	}
-	for (uint32_t r = 0; r < enc_w; ++r) {
-		const float* j = dy_dx + ((size_t)r * jn + js) * 3;
-		d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
-	}
-	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
 }
 
 // out[r][j] = in[r][index[j]] for the rows the backward reads; blockIdx.y picks a group of 8 fp16 rows (SDF-net input,
@@ -339,7 +352,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_acc, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -359,7 +372,7 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
 	c.v = take(12ull * n);
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
-	c.var_acc = take(16);
+	c.var_part = take(4ull * ((n + FB - 1) / FB + 1));
 	c.sel_sdf_in = take(2ull * f->sdf_in_w * n);
 	c.sel_rgb_in = take(2ull * f->rgb_in_w * n);
 	c.sel_dsdf_denc = take(2ull * f->enc_w * n);
@@ -397,7 +410,7 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->d_sdf_in = reinterpret_cast<hf*>(b + c.d_sdf_in);
 	f->v = reinterpret_cast<float*>(b + c.v);
 	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
-	f->var_acc = reinterpret_cast<float*>(b + c.var_acc);
+	f->var_part = reinterpret_cast<float*>(b + c.var_part);
 	f->sel_sdf_in = reinterpret_cast<hf*>(b + c.sel_sdf_in);
 	f->sel_rgb_in = reinterpret_cast<hf*>(b + c.sel_rgb_in);
 	f->sel_dsdf_denc = reinterpret_cast<hf*>(b + c.sel_dsdf_denc);
@@ -443,7 +456,7 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_mlp_forward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_output, N2_LAYOUT_AOS, nullptr)) return rc;
 	field_finish_output_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->rgb_in, (hf)f->sdf_bias, f->normal, f->params + f->off_var,
-	                                                         reinterpret_cast<hf*>(d_output), f->var_acc);
+	                                                         reinterpret_cast<hf*>(d_output));
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
@@ -471,24 +484,21 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	// colour net: only rows 0..2 of dL_doutput belong to it
 	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
 	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
-	// (the variance accumulator was cleared by the forward of this batch)
-	field_direct_gradients_kernel<<<dim3((n + PREP_BLOCK - 1) / PREP_BLOCK), dim3(PREP_BLOCK), 0, s>>>(n, dL, f->d_rgb_in, f->var_acc);
+	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
+	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
+	                                                         f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n);
 	N2_LAUNCH_CHECK();
-	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient
-	if (int rc = n2_mlp_backward(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
-	                             N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), mode)) return rc;
-	// dL/dnormal and the variance gradient
-	field_second_order_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-	                                                             f->d_density_in, f->var_acc, f->grads + f->off_var,
-	                                                             mode == N2_GRAD_ACCUMULATE ? 1 : 0, sel ? f->sel_index : nullptr, f->last_n);
+	field_variance_gradient_kernel<<<dim3(1), dim3(VB), 0, s>>>(f->var_part, fgrid(n).x, f->grads + f->off_var, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();
+	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient; the second-order pass through the
+	// net (the reference's backward_backward_input with Accumulate) rides along
+	if (int rc = n2_mlp_backward_and_second_order(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
+	                                              N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), reinterpret_cast<const n2_half*>(f->d_density_in),
+	                                              nullptr, mode)) return rc;
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)
 	if (int rc = n2_grid_backward_fused(f->grid, stream, xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
 	                                    reinterpret_cast<const n2_half*>(dsdf_denc), nullptr, mode)) return rc;
-	// second order through the SDF net
-	if (int rc = n2_mlp_backward_backward_input(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n,
-	                                            reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, nullptr, N2_GRAD_ACCUMULATE)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
 	// pending: one launch sums them
 	return n2_mlp_reduce_deferred(f->rgb, f->sdf, stream);

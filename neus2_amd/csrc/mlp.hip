@@ -449,11 +449,18 @@ struct GradAcc {
 // 248 the compiler takes by itself, a CU that holds a single wave of the sample generator (which runs beside the
 // training step on its own stream) could start only one of these workgroups at a time, and the colour net's backward
 // took 67 us instead of 46.
-template <int IC, int NH, bool WANT_DX, bool WANT_DW, bool WANT_Y = false>
+// SECOND (one hidden layer, with WANT_DW): the second-order pass of mlp_bbi_kernel rides along.  Its weight gradients
+//   dW_0 += (m * W_out^T g) v^T,  dW_out += g (m * W_0 v)^T
+// have the shape of the first-order ones, so they go into the same accumulators: the pass costs its own MFMAs but
+// shares the input loads, the activation mask, the fragment set-up and the slab of partial sums.
+template <int IC, int NH, bool WANT_DX, bool WANT_DW, bool WANT_Y = false, bool SECOND = false>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(120))) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
                                                                     const hf* __restrict__ dY, int dy_aos, int unit_row,
                                                                     hf* __restrict__ dX, float* __restrict__ partials,
-                                                                    hf* __restrict__ Y = nullptr, int y_aos = 0) {
+                                                                    hf* __restrict__ Y = nullptr, int y_aos = 0,
+                                                                    const hf* __restrict__ V = nullptr, const hf* __restrict__ G2 = nullptr,
+                                                                    int unit_row2 = -1) {
+	static_assert(!SECOND || (NH == 1 && WANT_DW), "the second-order pass needs one hidden layer and weight gradients");
 	using M = FragMap<IC, NH>;
 	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT, ROLES = WANT_DW ? 2 : 1;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
@@ -476,6 +483,16 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 		load_input<IC>(X, N, col, g, xp);
 		outgrad_frag(dY, N, col, g, (dy_aos & 1) != 0, unit_row, dy_aos >> 8, dyp[0], dyp[1]);
 		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
+		half8 vp[2][IC], gp[2];
+		if (SECOND) {
+			load_input<IC>(V, N, col, g, vp);
+			outgrad_frag(G2, N, col, g, false, unit_row2, MLP_OUT, gp[0], gp[1]);
+			if (!valid) {
+				gp[0] = zero8(); gp[1] = zero8();
+#pragma unroll
+				for (int c = 0; c < IC; ++c) { vp[0][c] = zero8(); vp[1][c] = zero8(); }
+			}
+		}
 		constexpr int DX_TILES = WANT_DW ? 1 : IN_MT;  // with two roles each computes one row tile of dL_dx
 		half8 dx_keep[DX_TILES][2];                    // tile 0's rows until tile 1's are known (sample-pair stores)
 		half4 y_keep[2];
@@ -516,6 +533,26 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 				acc.gWo = N2_MFMA(dyN[0], hN[0], acc.gWo);
 				acc.gWo = N2_MFMA(dyN[1], hN[1], acc.gWo);
 				mask_pack(N2_MFMA(dy, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], dhN[0], dhN[1]);
+				if (SECOND) {  // hN is the hidden layer itself here: its sign is the mask m
+					half8 v[IC], aN[2], bN[2], gN[2];
+					split_pairs<IC>(vp, t, v);
+					const half8 gg = gp[t];
+					float16v a = zero16();
+#pragma unroll
+					for (int c = 0; c < IC; ++c) a = N2_MFMA(v[c], frag(F, M::W0 + role * IC + c, lane), a);
+					mask_pack(a, hN[0], hN[1], aN[0], aN[1]);
+					mask_pack(N2_MFMA(gg, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], bN[0], bN[1]);
+					plain_pack(N2_MFMA(gg, frag(F, M::ID, lane), zero16()), gN[0], gN[1]);
+					acc.gWo = N2_MFMA(gN[0], aN[0], acc.gWo);
+					acc.gWo = N2_MFMA(gN[1], aN[1], acc.gWo);
+#pragma unroll
+					for (int nt = 0; nt < IN_MT; ++nt) {
+						half8 vN[2];
+						input_N<IC, NH>(F, lane, nt, v, vN);
+						acc.gW0[nt] = N2_MFMA(bN[0], vN[0], acc.gW0[nt]);
+						acc.gW0[nt] = N2_MFMA(bN[1], vN[1], acc.gW0[nt]);
+					}
+				}
 			}
 #pragma unroll
 			for (int mt = 0; mt < 2; ++mt)
@@ -1002,6 +1039,52 @@ N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim
 	N2_REQUIRE(dim < (uint32_t)MLP_OUT, "n2_mlp_input_gradient: output dimension %u out of range", dim);
 	N2_REQUIRE(d_dinput != nullptr || n == 0, "n2_mlp_input_gradient: d_dinput is null");
 	return mlp_backward_impl(mlp, stream, d_input, n, nullptr, N2_LAYOUT_SOA, (int)dim, d_dinput, N2_GRAD_IGNORE);
+}
+
+N2_API int n2_mlp_backward_and_second_order(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
+                                            const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
+                                            const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode) {
+	const char* fn = "n2_mlp_backward_and_second_order";
+	if (int rc = check_mlp_batch(mlp, fn, d_input, n)) return rc;
+	if (int rc = check_grad_mode(mlp, fn, mode)) return rc;
+	N2_REQUIRE(mode != N2_GRAD_IGNORE, "%s: the merged pass exists for its weight gradients (mode must be OVERWRITE or ACCUMULATE)", fn);
+	if (mlp->n_hidden != 1) {
+		n2_set_error("%s: implemented for one hidden layer (got %u)", fn, mlp->n_hidden);
+		return N2_ERR_UNSUPPORTED;
+	}
+	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "%s: bad layout %d", fn, (int)dL_layout);
+	N2_REQUIRE((d_dL_doutput != nullptr && d_dL_dinput != nullptr && d_dL_ddLdinput != nullptr) || n == 0,
+	           "%s: d_dL_doutput, d_dL_dinput and d_dL_ddLdinput are required", fn);
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_dL_doutput) % 16 == 0 && reinterpret_cast<uintptr_t>(d_dL_dinput) % 16 == 0 &&
+	           reinterpret_cast<uintptr_t>(d_dL_ddLdinput) % 16 == 0 && reinterpret_cast<uintptr_t>(d_second_dL_doutput) % 16 == 0,
+	           "%s: buffers must be 16-byte aligned", fn);
+	hipStream_t s = n2_stream(stream);
+	if (n == 0) {
+		if (mode == N2_GRAD_OVERWRITE) return n2_fill_zero_u32(s, mlp->grads, mlp->n_params * sizeof(hf));
+		return N2_OK;
+	}
+	const uint32_t blocks = stream_grid(n, 2);
+	if (int rc = check_pending(mlp, fn, blocks, mode)) return rc;
+	const int aos = (dL_layout == N2_LAYOUT_AOS ? 1 : 0) | (MLP_OUT << 8);
+	const int unit_row2 = d_second_dL_doutput == nullptr ? 0 : -1;
+	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
+	switch (mlp->in_w / 16) {
+#define CASE(IC)                                                                                                           \
+	case IC: {                                                                                                             \
+		const size_t lds = frag_bytes(FragMap<IC, 1>::COUNT);                                                              \
+		if (int rc = allow_lds(mlp_backward_kernel<IC, 1, true, true, false, true>, lds)) return rc;                       \
+		mlp_backward_kernel<IC, 1, true, true, false, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,        \
+			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, -1,                   \
+			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), nullptr, 0, reinterpret_cast<const hf*>(d_dL_ddLdinput),  \
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2);                                                  \
+		break;                                                                                                             \
+	}
+		CASE(1) CASE(2) CASE(3) CASE(4)
+#undef CASE
+		default: n2_set_error("mlp: unsupported shape"); return N2_ERR_UNSUPPORTED;
+	}
+	N2_LAUNCH_CHECK();
+	return reduce_partials(mlp, s, blocks, mode);
 }
 
 N2_API int n2_mlp_backward_backward_input(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,

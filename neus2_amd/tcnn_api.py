@@ -313,6 +313,22 @@ class FullyFusedMLP:
               "n2_mlp_backward_backward_input")
         return o
 
+    def backward_and_second_order(self, x, dL_dy, dL_ddLdinput, second_dL_doutput=None, dL_layout=LAYOUT_SOA, mode=GRAD_OVERWRITE):
+        """backward(mode) followed by backward_backward_input(Accumulate) in one pass over the input (one hidden
+        layer).  Returns dL_dx of the first-order pass."""
+        n = x.shape[1]
+        _check_half(x, (self.input_width(), n), "mlp input")
+        _check_half(dL_dy, (n, 16) if dL_layout == LAYOUT_AOS else (16, n), "dL_doutput")
+        _check_half(dL_ddLdinput, (self.input_width(), n), "dL_ddLdinput")
+        if second_dL_doutput is not None:
+            _check_half(second_dL_doutput, (16, n), "second dL_doutput")
+        dx = torch.empty((self.input_width(), n), dtype=torch.float16, device=x.device)
+        check(capi.lib().n2_mlp_backward_and_second_order(self._h, _stream(), ptr(x), C.c_uint32(n), ptr(dL_dy),
+                                                          C.c_int(dL_layout), ptr(dx), ptr(dL_ddLdinput),
+                                                          ptr(second_dL_doutput), C.c_int(mode)),
+              "n2_mlp_backward_and_second_order")
+        return dx
+
 
 class NerfNetwork:
     """NerfNetwork<__half> of the reference (nerf_network.h), static scene: grid + SDF MLP +

@@ -224,3 +224,57 @@ def test_backward_rows_equals_backward_of_the_zero_padded_gradient(oracle, layou
     dG.fill_(2.0)
     dx = gm.backward_rows(x, dev(shape(dy), torch.float16), 3, lay, mode=GRAD_OVERWRITE)
     assert torch.equal(dx, dx_ref) and torch.equal(dG, g_ref)
+
+
+@pytest.mark.parametrize("in_w", [48, 32, 16, 64])
+@pytest.mark.parametrize("unit", [True, False])
+def test_backward_and_second_order_equals_the_two_calls(oracle, in_w, unit):
+    """The SDF net's first-order backward and its second-order pass (nerf_network.h:402 and :560-571) in one launch:
+    the input gradient is that of backward, the weight gradients are the sum of both passes, against the oracle and
+    against the two separate calls."""
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_OVERWRITE, LAYOUT_AOS, LAYOUT_SOA
+    om, gm, W, dW, dG, rng = make(oracle, in_w, 1, 31)
+    n = 8192 + 72
+    x = q16(rng.standard_normal((in_w, n)))
+    dy = q16(rng.standard_normal((16, n)))
+    v = q16(rng.standard_normal((in_w, n)))
+    g = np.zeros((16, n), np.float32)
+    if unit:
+        g[0] = 1
+    else:
+        g[:] = q16(rng.standard_normal((16, n)))
+    _, h = om.forward(W, x, round_hidden=True)
+    ref_dx, ref1 = om.backward(W, x, h, dy)
+    ref2, _ = om.backward_backward_input(W, h, v, g)
+    dx_, ddy, dv = dev(x, torch.float16), dev(dy, torch.float16), dev(v, torch.float16)
+    dg = None if unit else dev(g, torch.float16)
+    # the two calls
+    dx_two = gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE)
+    gm.backward_backward_input(dx_, dv, dg, mode=GRAD_ACCUMULATE)
+    two = host(dG)
+    # one launch
+    dG.fill_(5.0)
+    dx_one = gm.backward_and_second_order(dx_, ddy, dv, dg, mode=GRAD_OVERWRITE)
+    one = host(dG)
+    assert torch.equal(dx_one, dx_two)
+    assert_close(host(dx_one), ref_dx, what="dL_dinput", outlier_frac=FLIP)
+    assert_grad_close(one, ref1 + ref2, what="first + second order weight gradients")
+    assert rel_l2(one, two) < 1e-3  # the same sums in another order, each rounded to fp16 once
+    # AoS first-order gradient, Accumulate on top of what is there
+    base = q16(rng.standard_normal(om.n_params))
+    dG.copy_(dev(base, torch.float16))
+    dx_aos = gm.backward_and_second_order(dx_, ddy.t().contiguous(), dv, dg, dL_layout=LAYOUT_AOS, mode=GRAD_ACCUMULATE)
+    assert torch.equal(dx_aos, dx_one)
+    assert_grad_close(host(dG), base + ref1 + ref2, what="accumulated first + second order weight gradients")
+
+
+def test_backward_and_second_order_errors(oracle):
+    from neus2_amd.tcnn_api import GRAD_IGNORE, FullyFusedMLP, N2Error
+    om, gm, W, dW, dG, rng = make(oracle, 48, 1, 32)
+    x = dev(q16(rng.standard_normal((48, 256))), torch.float16)
+    dy = dev(q16(rng.standard_normal((16, 256))), torch.float16)
+    with pytest.raises(N2Error, match="OVERWRITE or ACCUMULATE"):
+        gm.backward_and_second_order(x, dy, x, mode=GRAD_IGNORE)
+    om2, gm2, *_ = make(oracle, 48, 2, 33)
+    with pytest.raises(N2Error, match="one hidden layer"):
+        gm2.backward_and_second_order(x, dy, x)
