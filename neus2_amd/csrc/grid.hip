@@ -492,6 +492,7 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bbi_kernel(N2LevelTable tab, 
 constexpr uint32_t BKT_SHIFT = N2_BKT_SHIFT;           // 4096 entries per bucket: a 64 KiB accumulator image, two reduce workgroups per CU
 constexpr uint32_t BKT_ENTRIES = 1u << BKT_SHIFT;
 constexpr uint32_t BKT_MAX = (1u << 19) >> BKT_SHIFT;  // buckets per level (entries <= 2^19)
+constexpr uint32_t PAIR_MAX_CELL = BKT_ENTRIES - 2u;  // pair records (grid_bin_kernel): x + 1 <= BKT_ENTRIES - 1
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
 constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
 constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: two workgroups (2 x 64 KiB staging) keep 4 waves on every SIMD
@@ -503,7 +504,7 @@ struct N2BucketPlan {
 	uint32_t groups[N2_MAX_LEVELS];        // tile groups per bucket
 };
 
-template <uint32_t MODE, bool FIRST, bool SECOND, bool WANT_OUT>
+template <uint32_t MODE, bool FIRST, bool SECOND, bool WANT_OUT, bool CLAMP_X>
 __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t level, uint32_t i, uint32_t N,
                                                const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
                                                const __half* __restrict__ dL_dy, const float* __restrict__ v,
@@ -511,7 +512,8 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
                                                __half* __restrict__ dL_ddLdy, uint32_t* e_out, float* r0_out, float* r1_out,
                                                uint32_t* cell) {
 	const float scale = tab.scale[level];
-	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	if (CLAMP_X) p.c[0] = min(p.c[0], PAIR_MAX_CELL);  // pair records: x + 1 stays inside the bucket's index bits
 	cell[0] = p.c[0]; cell[1] = p.c[1]; cell[2] = p.c[2];
 	uint32_t e[8];
 	n2_corner_entries<MODE>(p, tab.entries[level], tab.resolution[level], e);
@@ -587,26 +589,25 @@ __device__ __forceinline__ float n2_row_shr(float x) {
 }
 constexpr uint32_t REC_SKIP = 0xFFFFFFFFu;
 
-template <bool FIRST, bool SECOND, bool WANT_OUT>
-__global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
-                                                              const float* __restrict__ xyz, uint32_t point_stride,
-                                                              uint32_t dim_stride, const __half* __restrict__ dL_dy,
-                                                              const float* __restrict__ v, const __half* __restrict__ g2,
-                                                              const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
-                                                              uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
-                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count) {
-	// part of the gradient buffer that the reduce kernel will add to with atomics: cleared here, one 16-byte store per thread
-	for (uint32_t z = blockIdx.x * BIN_BLOCK + threadIdx.x; z < zero_count; z += gridDim.x * BIN_BLOCK) zero_begin[z] = make_uint4(0u, 0u, 0u, 0u);
-	__shared__ uint32_t hist[BKT_MAX];
-	__shared__ uint32_t prefix[BKT_MAX + 1];
-	__shared__ __align__(16) uint32_t stage_val[BIN_RECORDS];  // sorted records: packed half2 value ...
-	__shared__ __align__(16) uint16_t stage_key[BIN_RECORDS];  // ... and entry within its bucket
-	const uint32_t level = first_level + blockIdx.x / tiles, tile = blockIdx.x % tiles;
+// Pair records.  On a hashed level the entry of corner (x, y, z) is (x ^ y P1 ^ z P2) & (T - 1); while x + 1 stays below
+// the bucket size, x only reaches the bits below BKT_SHIFT: the two x-neighbours of a (y, z) corner pair always share a
+// bucket, and their places in it differ by x ^ (x + 1) = 2^(t+1) - 1, t = number of trailing one bits of x.  Such levels
+// (pair_levels in the level table) sort and store ONE record per pair: both packed values (8 bytes) and a 16-bit key,
+// entry of the x corner within the bucket | t << BKT_SHIFT.  Half the counter updates, prefix look-ups and staging
+// stores here, half the key traffic and decoding in the reduce kernel.  Points outside the unit cube could carry an x
+// beyond that range: their cell is clamped for the records (the dense levels clamp such points too).
+
+template <bool FIRST, bool SECOND, bool WANT_OUT, bool PAIR>
+__device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uint32_t level, const uint32_t tile, uint32_t N, uint32_t tiles,
+                                              const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
+                                              const __half* __restrict__ dL_dy, const float* __restrict__ v, const __half* __restrict__ g2,
+                                              const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
+                                              uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys, uint16_t* __restrict__ offsets,
+                                              uint32_t* hist, uint32_t* prefix, uint32_t* stage_val, uint16_t* stage_key) {
+	constexpr uint32_t R = PAIR ? 4 : 8;  // sorted records per point
 	const uint32_t lane = threadIdx.x & 63u;
-	if (threadIdx.x < BKT_MAX) hist[threadIdx.x] = 0;
-	__syncthreads();
 	// records of this thread: entry | rank << 19 after the counting step (REC_SKIP: merged into a later lane)
-	uint32_t re[BIN_PER_THREAD * 8], rv[BIN_PER_THREAD * 8];
+	uint32_t re[BIN_PER_THREAD * R], rv[BIN_PER_THREAD * 8], tcode[BIN_PER_THREAD];
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
 		const uint32_t i = tile * BIN_POINTS + j * BIN_BLOCK + threadIdx.x;
@@ -623,9 +624,13 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 #pragma unroll
 		for (uint32_t k = 0; k < 8; ++k) { e[k] = 0; r0[k] = 0.f; r1[k] = 0.f; }
 		if (valid) {
-#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell)
-			N2_DISPATCH_MODE(tab.mode[level], CALL)
+			if (PAIR) {
+				grid_bin_point<N2_LEVEL_HASH, FIRST, SECOND, WANT_OUT, true>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell);
+			} else {
+#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT, false>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell)
+				N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
+			}
 		}
 		// runs of equal cells among the wave's 64 consecutive points
 		const uint32_t up_x = __shfl_up(cell[0], 1), up_y = __shfl_up(cell[1], 1), up_z = __shfl_up(cell[2], 1);
@@ -649,14 +654,17 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 			N2_SCAN_STEP(1) N2_SCAN_STEP(2) N2_SCAN_STEP(4) N2_SCAN_STEP(8)
 #undef N2_SCAN_STEP
 		}
+		if (PAIR) tcode[j] = ((uint32_t)__popc((e[0] ^ e[1]) & (BKT_ENTRIES - 1u)) - 1u) << BKT_SHIFT;
 #pragma unroll
 		for (uint32_t k = 0; k < 8; ++k) {
-			uint32_t rec = REC_SKIP;
-			if (emit) {
-				const uint32_t rank = atomicAdd(&hist[e[k] >> BKT_SHIFT], 1u);
-				rec = e[k] | (rank << 19);
+			if (!PAIR || (k & 1u) == 0) {
+				uint32_t rec = REC_SKIP;
+				if (emit) {
+					const uint32_t rank = atomicAdd(&hist[e[k] >> BKT_SHIFT], 1u);
+					rec = e[k] | (rank << 19);
+				}
+				re[R * j + (PAIR ? k >> 1 : k)] = rec;
 			}
-			re[8 * j + k] = rec;
 			const __half2 h = __floats2half2_rn(r0[k], r1[k]);
 			rv[8 * j + k] = *reinterpret_cast<const uint32_t*>(&h);
 		}
@@ -682,12 +690,17 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 #pragma unroll
 	for (uint32_t j = 0; j < BIN_PER_THREAD; ++j) {
 #pragma unroll
-		for (uint32_t k = 0; k < 8; ++k) {
-			if (re[8 * j + k] != REC_SKIP) {
-				const uint32_t e = re[8 * j + k] & 0x7FFFFu, rank = re[8 * j + k] >> 19;
+		for (uint32_t k = 0; k < R; ++k) {
+			if (re[R * j + k] != REC_SKIP) {
+				const uint32_t e = re[R * j + k] & 0x7FFFFu, rank = re[R * j + k] >> 19;
 				const uint32_t pos = prefix[e >> BKT_SHIFT] + rank;
-				stage_val[pos] = rv[8 * j + k];
-				stage_key[pos] = (uint16_t)(e & (BKT_ENTRIES - 1u));
+				if (PAIR) {
+					reinterpret_cast<uint2*>(stage_val)[pos] = make_uint2(rv[8 * j + 2 * k], rv[8 * j + 2 * k + 1]);
+					stage_key[pos] = (uint16_t)((e & (BKT_ENTRIES - 1u)) | tcode[j]);
+				} else {
+					stage_val[pos] = rv[8 * j + k];
+					stage_key[pos] = (uint16_t)(e & (BKT_ENTRIES - 1u));
+				}
 			}
 		}
 	}
@@ -699,9 +712,34 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 	uint4* out_key = reinterpret_cast<uint4*>(rec_keys + slot);
 	const uint4* sv = reinterpret_cast<const uint4*>(stage_val);
 	const uint4* sk = reinterpret_cast<const uint4*>(stage_key);
-	for (uint32_t t = threadIdx.x; 4 * t < total; t += BIN_BLOCK) out_val[t] = sv[t];
+	for (uint32_t t = threadIdx.x; (PAIR ? 2 : 4) * t < total; t += BIN_BLOCK) out_val[t] = sv[t];
 	for (uint32_t t = threadIdx.x; 8 * t < total; t += BIN_BLOCK) out_key[t] = sk[t];
 	if (threadIdx.x <= BKT_MAX) offsets[((size_t)level * tiles + tile) * (BKT_MAX + 1) + threadIdx.x] = (uint16_t)prefix[threadIdx.x];
+}
+
+template <bool FIRST, bool SECOND, bool WANT_OUT>
+__global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab, uint32_t first_level, uint32_t N, uint32_t tiles,
+                                                              const float* __restrict__ xyz, uint32_t point_stride,
+                                                              uint32_t dim_stride, const __half* __restrict__ dL_dy,
+                                                              const float* __restrict__ v, const __half* __restrict__ g2,
+                                                              const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
+                                                              uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
+                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count) {
+	// part of the gradient buffer that the reduce kernel will add to with atomics: cleared here, one 16-byte store per thread
+	for (uint32_t z = blockIdx.x * BIN_BLOCK + threadIdx.x; z < zero_count; z += gridDim.x * BIN_BLOCK) zero_begin[z] = make_uint4(0u, 0u, 0u, 0u);
+	__shared__ uint32_t hist[BKT_MAX];
+	__shared__ uint32_t prefix[BKT_MAX + 1];
+	__shared__ __align__(16) uint32_t stage_val[BIN_RECORDS];  // sorted records: packed half2 value (a pair of them on pair levels) ...
+	__shared__ __align__(16) uint16_t stage_key[BIN_RECORDS];  // ... and entry within its bucket
+	const uint32_t level = first_level + blockIdx.x / tiles, tile = blockIdx.x % tiles;
+	if (threadIdx.x < BKT_MAX) hist[threadIdx.x] = 0;
+	__syncthreads();
+	if ((tab.pair_levels >> level) & 1u)
+		grid_bin_tile<FIRST, SECOND, WANT_OUT, true>(tab, level, tile, N, tiles, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, rec_vals,
+		                                             rec_keys, offsets, hist, prefix, stage_val, stage_key);
+	else
+		grid_bin_tile<FIRST, SECOND, WANT_OUT, false>(tab, level, tile, N, tiles, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, rec_vals,
+		                                              rec_keys, offsets, hist, prefix, stage_val, stage_key);
 }
 
 // LDS float atomics retire about one lane every three clocks on this part, integer ones at ~9 (32-bit) and
@@ -726,24 +764,24 @@ __device__ __forceinline__ unsigned long long to_fixed(float x) {
 }
 __device__ __forceinline__ float from_fixed(unsigned long long q) { return (float)((double)(long long)q * (1.0 / 4294967296.0)); }
 
+// Pair levels: an item is 16 pair records and a wave's load covers four items, one per 16 lanes (a bucket's run in a tile
+// is about 32 pair records: whole-wave items would leave half the lanes idle).
+constexpr uint32_t PITEM_SHIFT = 4;
+constexpr uint32_t PITEM_RECORDS = 1u << PITEM_SHIFT;
+constexpr uint32_t PITEM_PER_LOAD = 64 / PITEM_RECORDS;
+constexpr uint32_t P_LOADS = 4;  // loads per lane in flight per register set
+
 // Every thread owns the bucket's run of one tile.  The runs are cut into items, the items of all runs are numbered
 // consecutively (block scan of the item counts) and listed in LDS (first record, record count), ITEM_CAP at a time:
 // a wave then finds an item's records with one LDS read instead of searching the runs' prefix sums, whose chain of
 // dependent LDS reads was most of this kernel's time.
-__global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
-                                                                   const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
-                                                                   const uint16_t* __restrict__ offsets,
-                                                                   __half2* __restrict__ grads, int accumulate) {
-	__shared__ unsigned long long acc[2 * BKT_ENTRIES];
-	__shared__ uint32_t item_src[ITEM_CAP];  // index of the item's first record in the level's records
-	__shared__ uint8_t item_n[ITEM_CAP];     // its record count - 1
-	__shared__ uint32_t wave_tot[RED_BLOCK / 64];
-	// which (level, bucket, group) is this workgroup?
-	uint32_t level = 0;
-	while (blockIdx.x >= plan.wg_begin[level + 1]) ++level;
-	const uint32_t local = blockIdx.x - plan.wg_begin[level];
-	const uint32_t G = plan.groups[level];
-	const uint32_t bucket = local / G, group = local - bucket * G;
+template <bool PAIR>
+__device__ __forceinline__ void grid_reduce_runs(const uint32_t tiles, const uint32_t level, const uint32_t bucket, const uint32_t group,
+                                                 const uint32_t G, const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
+                                                 const uint16_t* __restrict__ offsets, unsigned long long* acc, uint32_t* item_src,
+                                                 uint8_t* item_n, uint32_t* wave_tot) {
+	constexpr uint32_t SHIFT = PAIR ? PITEM_SHIFT : ITEM_SHIFT, RECS = 1u << SHIFT;
+	constexpr uint32_t TILE_RECS = PAIR ? BIN_RECORDS / 2 : BIN_RECORDS;  // records in a tile's slot of the value array
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
 	const uint32_t my_tiles = (tiles > group) ? (tiles - group + G - 1) / G : 0;  // tiles group, group + G, ...
 	const size_t level_tile0 = (size_t)level * tiles;
@@ -757,13 +795,13 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 			const size_t tile = level_tile0 + group + (size_t)t * G;
 			const uint16_t* off = offsets + tile * (BKT_MAX + 1) + bucket;
 			const uint32_t begin = off[0], end = off[1];
-			src = (uint32_t)((tile - level_tile0) * BIN_RECORDS) + begin;
+			src = (uint32_t)((tile - level_tile0) * TILE_RECS) + begin;
 			len = end - begin;
 		}
 		if (c0 == 0) {
 			for (uint32_t e = threadIdx.x; e < 2 * BKT_ENTRIES; e += RED_BLOCK) acc[e] = 0ull;
 		}
-		const uint32_t cnt = (len + ITEM_RECORDS - 1u) >> ITEM_SHIFT;
+		const uint32_t cnt = (len + RECS - 1u) >> SHIFT;
 		uint32_t incl = cnt;
 #pragma unroll
 		for (int o = 1; o < 64; o <<= 1) {
@@ -783,73 +821,148 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 			if (w0 > 0) __syncthreads();  // the previous window has been read
 			// list this thread's items that fall into the window [w0, w0 + ITEM_CAP)
 			for (uint32_t i = (first < w0) ? w0 - first : 0u; i < cnt && first + i < w0 + ITEM_CAP; ++i) {
-				const uint32_t rest = len - (i << ITEM_SHIFT);
-				item_src[first + i - w0] = src + (i << ITEM_SHIFT);
-				item_n[first + i - w0] = (uint8_t)((rest < ITEM_RECORDS ? rest : ITEM_RECORDS) - 1u);
+				const uint32_t rest = len - (i << SHIFT);
+				item_src[first + i - w0] = src + (i << SHIFT);
+				item_n[first + i - w0] = (uint8_t)((rest < RECS ? rest : RECS) - 1u);
 			}
 			__syncthreads();
 			const uint32_t n_win = (n_items - w0 < ITEM_CAP) ? n_items - w0 : ITEM_CAP;
-			// a wave takes RED_ITEMS items at a time
-			auto fetch = [&](uint32_t i0, uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t& okmask) {
-				okmask = 0;
+			if constexpr (PAIR) {
+				const uint2* base_val2 = reinterpret_cast<const uint2*>(base_val);
+				const uint32_t r = lane & (PITEM_RECORDS - 1u), sub = lane >> PITEM_SHIFT;
+				// Lanes past the end of an item read the level's first record instead (and ignore it): with every load issued
+				// unconditionally the compiler can count them, and waits for the CURRENT set only while the next is in flight.
+				auto fetch = [&](uint32_t i0, uint2 (&val)[P_LOADS], uint32_t (&key)[P_LOADS], uint32_t& okmask) {
+					okmask = 0;
 #pragma unroll
-				for (uint32_t j = 0; j < RED_ITEMS; ++j) {
-					const uint32_t it = i0 + j;
-					uint32_t s0 = 0, n = 0;
-					if (it < n_win) { s0 = item_src[it]; n = (uint32_t)item_n[it] + 1u; }
-#pragma unroll
-					for (uint32_t h = 0; h < ITEM_LOADS; ++h) {
-						const uint32_t r = h * 64 + lane;
+					for (uint32_t h = 0; h < P_LOADS; ++h) {
+						const uint32_t it = i0 + PITEM_PER_LOAD * h + sub;
+						uint32_t s0 = 0, n = 0;
+						if (it < n_win) { s0 = item_src[it]; n = (uint32_t)item_n[it] + 1u; }
 						const bool ok = r < n;
-						okmask |= (ok ? 1u : 0u) << (ITEM_LOADS * j + h);
-						// lanes past the end of the run read the level's first record instead (and ignore it): with every
-						// load issued unconditionally the compiler can count them, and waits for the CURRENT items only
-						// while the next ones are in flight
-						const size_t at = ok ? (size_t)s0 + r : 0;
-						rec[ITEM_LOADS * j + h] = make_uint2(base_key[at], base_val[at]);
+						okmask |= (ok ? 1u : 0u) << h;
+						const uint32_t at = ok ? s0 + r : 0u;
+						val[h] = base_val2[at];
+						key[h] = base_key[at + (at & ~(TILE_RECS - 1u))];  // a tile's key slot is twice as long as its pair records
 					}
-				}
-			};
-			constexpr uint32_t STRIDE = (RED_BLOCK / 64) * RED_ITEMS;
-			auto accumulate = [&](const uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t okmask) {
+				};
+				auto accumulate = [&](const uint2 (&val)[P_LOADS], const uint32_t (&key)[P_LOADS], uint32_t okmask) {
 #pragma unroll
-				for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) {
-					if (okmask & (1u << q)) {
-						const __half2 hh = *reinterpret_cast<const __half2*>(&rec[q].y);
-						const float2 f = __half22float2(hh);
-						atomicAdd(&acc[2 * rec[q].x], to_fixed(f.x));  // LDS integer atomics
-						atomicAdd(&acc[2 * rec[q].x + 1], to_fixed(f.y));
+					for (uint32_t q = 0; q < P_LOADS; ++q) {
+						if (okmask & (1u << q)) {
+							const uint32_t a1 = key[q] & (BKT_ENTRIES - 1u);
+							const uint32_t a2 = a1 ^ ((2u << (key[q] >> BKT_SHIFT)) - 1u);  // the x + 1 corner: x ^ (x + 1) = 2^(t+1) - 1
+							const float2 f = __half22float2(*reinterpret_cast<const __half2*>(&val[q].x));
+							const float2 g = __half22float2(*reinterpret_cast<const __half2*>(&val[q].y));
+							atomicAdd(&acc[a1], to_fixed(f.x));  // LDS integer atomics
+							atomicAdd(&acc[BKT_ENTRIES + a1], to_fixed(f.y));
+							atomicAdd(&acc[a2], to_fixed(g.x));
+							atomicAdd(&acc[BKT_ENTRIES + a2], to_fixed(g.y));
+						}
+					}
+				};
+				constexpr uint32_t PER_WAVE = PITEM_PER_LOAD * P_LOADS, STRIDE = (RED_BLOCK / 64) * PER_WAVE;
+				uint2 va[P_LOADS], vb[P_LOADS];
+				uint32_t ka[P_LOADS], kb[P_LOADS], ok_a = 0, ok_b = 0;
+				uint32_t i0 = wave * PER_WAVE;
+				if (i0 < n_win) {
+					fetch(i0, va, ka, ok_a);
+					for (;;) {
+						fetch(i0 + STRIDE, vb, kb, ok_b);
+						accumulate(va, ka, ok_a);
+						i0 += STRIDE;
+						if (i0 >= n_win) break;
+						fetch(i0 + STRIDE, va, ka, ok_a);
+						accumulate(vb, kb, ok_b);
+						i0 += STRIDE;
+						if (i0 >= n_win) break;
 					}
 				}
-			};
-			// Two register sets take turns: while one is accumulated the loads of the other are in flight.  Every fetch
-			// issues the same number of loads (items past the end read the first record and are ignored) and no set is
-			// ever copied, so each wait covers exactly the set that is about to be used.
-			uint2 ra[ITEM_LOADS * RED_ITEMS], rb[ITEM_LOADS * RED_ITEMS];
-			uint32_t ok_a = 0, ok_b = 0;
-			uint32_t i0 = wave * RED_ITEMS;
-			if (i0 < n_win) {
-				fetch(i0, ra, ok_a);
-				for (;;) {
-					fetch(i0 + STRIDE, rb, ok_b);
-					accumulate(ra, ok_a);
-					i0 += STRIDE;
-					if (i0 >= n_win) break;
-					fetch(i0 + STRIDE, ra, ok_a);
-					accumulate(rb, ok_b);
-					i0 += STRIDE;
-					if (i0 >= n_win) break;
+			} else {
+				// a wave takes RED_ITEMS items at a time
+				auto fetch = [&](uint32_t i0, uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t& okmask) {
+					okmask = 0;
+#pragma unroll
+					for (uint32_t j = 0; j < RED_ITEMS; ++j) {
+						const uint32_t it = i0 + j;
+						uint32_t s0 = 0, n = 0;
+						if (it < n_win) { s0 = item_src[it]; n = (uint32_t)item_n[it] + 1u; }
+#pragma unroll
+						for (uint32_t h = 0; h < ITEM_LOADS; ++h) {
+							const uint32_t r = h * 64 + lane;
+							const bool ok = r < n;
+							okmask |= (ok ? 1u : 0u) << (ITEM_LOADS * j + h);
+							// lanes past the end of the run read the level's first record instead (and ignore it): with every
+							// load issued unconditionally the compiler can count them, and waits for the CURRENT items only
+							// while the next ones are in flight
+							const size_t at = ok ? (size_t)s0 + r : 0;
+							rec[ITEM_LOADS * j + h] = make_uint2(base_key[at], base_val[at]);
+						}
+					}
+				};
+				constexpr uint32_t STRIDE = (RED_BLOCK / 64) * RED_ITEMS;
+				auto accumulate = [&](const uint2 (&rec)[ITEM_LOADS * RED_ITEMS], uint32_t okmask) {
+#pragma unroll
+					for (uint32_t q = 0; q < ITEM_LOADS * RED_ITEMS; ++q) {
+						if (okmask & (1u << q)) {
+							const __half2 hh = *reinterpret_cast<const __half2*>(&rec[q].y);
+							const float2 f = __half22float2(hh);
+							atomicAdd(&acc[rec[q].x], to_fixed(f.x));  // LDS integer atomics
+							atomicAdd(&acc[BKT_ENTRIES + rec[q].x], to_fixed(f.y));
+						}
+					}
+				};
+				// Two register sets take turns: while one is accumulated the loads of the other are in flight.  Every fetch
+				// issues the same number of loads (items past the end read the first record and are ignored) and no set is
+				// ever copied, so each wait covers exactly the set that is about to be used.
+				uint2 ra[ITEM_LOADS * RED_ITEMS], rb[ITEM_LOADS * RED_ITEMS];
+				uint32_t ok_a = 0, ok_b = 0;
+				uint32_t i0 = wave * RED_ITEMS;
+				if (i0 < n_win) {
+					fetch(i0, ra, ok_a);
+					for (;;) {
+						fetch(i0 + STRIDE, rb, ok_b);
+						accumulate(ra, ok_a);
+						i0 += STRIDE;
+						if (i0 >= n_win) break;
+						fetch(i0 + STRIDE, ra, ok_a);
+						accumulate(rb, ok_b);
+						i0 += STRIDE;
+						if (i0 >= n_win) break;
+					}
 				}
 			}
 		}
 	}
+}
+
+__global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
+                                                                   const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
+                                                                   const uint16_t* __restrict__ offsets,
+                                                                   __half2* __restrict__ grads, int accumulate) {
+	// one plane per feature: lanes of a wave's atomic then spread over all bank pairs (entry-major pairs of features would
+	// leave every other pair unused)
+	__shared__ unsigned long long acc[2 * BKT_ENTRIES];
+	__shared__ uint32_t item_src[ITEM_CAP];  // index of the item's first record in the level's records
+	__shared__ uint8_t item_n[ITEM_CAP];     // its record count - 1
+	__shared__ uint32_t wave_tot[RED_BLOCK / 64];
+	// which (level, bucket, group) is this workgroup?
+	uint32_t level = 0;
+	while (blockIdx.x >= plan.wg_begin[level + 1]) ++level;
+	const uint32_t local = blockIdx.x - plan.wg_begin[level];
+	const uint32_t G = plan.groups[level];
+	const uint32_t bucket = local / G, group = local - bucket * G;
+	if ((tab.pair_levels >> level) & 1u)
+		grid_reduce_runs<true>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot);
+	else
+		grid_reduce_runs<false>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot);
 	__syncthreads();
 	const uint32_t entries = tab.entries[level];
 	__half2* Gd = grads + tab.offset[level];
 	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) {
 		const uint32_t idx = bucket * BKT_ENTRIES + e;
 		if (idx >= entries) break;
-		const float ax = from_fixed(acc[2 * e]), ay = from_fixed(acc[2 * e + 1]);
+		const float ax = from_fixed(acc[e]), ay = from_fixed(acc[BKT_ENTRIES + e]);
 		if (G > 1) {
 			// several tile groups fold into the same entries (coarse levels only)
 			if (ax != 0.f || ay != 0.f) unsafeAtomicAdd(&Gd[idx], __floats2half2_rn(ax, ay));
@@ -898,6 +1011,7 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->tab.max_level_gpu = nullptr;
 	g->tab.valid_levels = n_levels;
 	g->tab.active_levels = n_levels;
+	g->tab.pair_levels = 0;
 	g->base_valid_level_scale = 1.0f;
 	g->valid_level_scale = 0.0f;
 	g->base_training_step = 0;
@@ -919,6 +1033,8 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 		g->tab.mode[l] = level_mode(res, n);
 		// hashed levels gather from all over their table; the dense ones mostly hit lines their neighbours fetched
 		g->level_cost[l] = (g->tab.mode[l] == N2_LEVEL_HASH || g->tab.mode[l] == N2_LEVEL_HASH_MOD) ? 1.0f : 0.6f;
+		// pair records in the bucketed scatter: x and x + 1 must stay below the bucket size (see grid_bin_kernel)
+		if (g->tab.mode[l] == N2_LEVEL_HASH && res <= PAIR_MAX_CELL + 1u && n >= BKT_ENTRIES) g->tab.pair_levels |= 1u << l;
 		off += n;
 	}
 	if (off * n_features_per_level > 0x7FFFFFFFull) {

@@ -58,6 +58,8 @@ struct N2LevelTable {
 	uint32_t valid_levels;         // progressive training: number of levels switched on so far
 	uint32_t active_levels;        // levels in use under max_level and valid_levels (kept up to date by the setters)
 	uint32_t n_features;
+	// bit l set: level l's bucketed scatter writes one record per PAIR of x-neighbour corners (see grid_bin_kernel)
+	uint32_t pair_levels;
 };
 
 static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
