@@ -283,6 +283,48 @@ def test_sorted_scatter_path(oracle, kind):
     assert (got[ref1 == 0] == 0).all()
 
 
+def test_sorted_scatter_pair_records_edge_cells(oracle):
+    """Hashed levels sort one record per pair of x-neighbour corners; the second corner's place in the bucket is the
+    first one's xor 2^(t+1) - 1, t = trailing one bits of the cell's x.  Cells whose x ends in 0 .. 11 one bits (the
+    longest carries a 12-bit index can take), the first and the last cell of every level, against the oracle; and points
+    outside the unit cube that carry a zero gradient change nothing."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding
+    og = oracle.Grid(CFG["n_levels"], CFG["log2_hashmap_size"], CFG["base_resolution"], CFG["per_level_scale"])
+    gg = GridEncoding(**CFG)
+    rng = np.random.default_rng(41)
+    params = q16(rng.uniform(-1, 1, og.n_params))
+    dp = dev(params, torch.float16)
+    dg = torch.zeros_like(dp)
+    gg.set_params(dp, dg)
+    n = 2 * 4096 + 264
+    assert gg.reserve_scatter_workspace(1 << 14)
+    xyz = rng.random((3, n), dtype=np.float32)
+    # x coordinates in the middle of cells 2^k - 1 (k = 0 .. 11), 0 and res - 2 of the finest levels
+    j = 0
+    for level in (15, 14, 11, 8, 5):
+        scale = float(og.scale[level])
+        res = int(og.resolution[level])
+        for cell in [0, res - 2] + [(1 << k) - 1 for k in range(13) if (1 << k) - 1 <= res - 2]:
+            for rep in range(4):
+                xyz[0, j] = np.float32((cell + 0.1 + 0.2 * rep) / scale)
+                j += 1
+    assert j < 4096
+    dy = q16(rng.standard_normal((32, n)))
+    stray = slice(n - 200, n)
+    xyz[:, stray] = rng.uniform(-3, 4, (3, 200)).astype(np.float32)
+    xyz[0, n - 200:n - 100] = rng.uniform(1.001, 40, 100).astype(np.float32)  # cells beyond the 12 index bits
+    dy[:, stray] = 0
+    inside = slice(0, n - 200)
+    ref, _ = og.backward(params, np.ascontiguousarray(xyz[:, inside]), np.ascontiguousarray(dy[:, inside]), want_dx=False)
+    dg.fill_(9.0)
+    gg.backward(None, dev(xyz), dev(dy, torch.float16), mode=GRAD_OVERWRITE)
+    got = host(dg)
+    for l in range(16):
+        a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+        assert rel_l2(got[a:b], ref[a:b]) < RTOL, (l, rel_l2(got[a:b], ref[a:b]))
+    assert (got[ref == 0] == 0).all()
+
+
 def _level_tols(og, n):
     return [RTOL * max(1.0, np.sqrt(8.0 * n / max(1, int(og.entries[l])))) for l in range(og.n_levels)]
 
