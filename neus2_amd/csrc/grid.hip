@@ -951,7 +951,13 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 	while (blockIdx.x >= plan.wg_begin[level + 1]) ++level;
 	const uint32_t local = blockIdx.x - plan.wg_begin[level];
 	const uint32_t G = plan.groups[level];
-	const uint32_t bucket = local / G, group = local - bucket * G;
+	uint32_t bucket = local / G;
+	const uint32_t group = local - bucket * G;
+	// A tile's runs for neighbouring buckets meet inside a 128-byte line, which both buckets' workgroups fetch.  Workgroup
+	// ids are dealt round-robin over the XCDs: XCD x takes the x-th eighth of the level's buckets, in order, so that both
+	// fetches of such a line go through the same L2 at about the same time.
+	const uint32_t nb = plan.n_buckets[level];
+	if (G == 1 && nb % N_XCD == 0) bucket = (blockIdx.x % N_XCD) * (nb / N_XCD) + local / N_XCD;
 	if ((tab.pair_levels >> level) & 1u)
 		grid_reduce_runs<true>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot);
 	else
