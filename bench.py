@@ -34,8 +34,8 @@ COLOUR_BACKWARD_FLOPS = 14336 + 16384 + 16384
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 # HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
 # (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
-# scatter pair = bin (48.4 + 158.3 MiB) + reduce (210.8 + 24.0 MiB); forward = 82.3 + 115.2 MiB
-STEP_TRAFFIC_BYTES = {"grid_backward_params": int(441.5 * 2**20), "grid_forward": int(197.5 * 2**20)}
+# scatter pair = bin (43.2 + 105.9 MiB) + reduce (110.9 + 24.0 MiB); forward = 82.3 + 115.2 MiB
+STEP_TRAFFIC_BYTES = {"grid_backward_params": int(283.9 * 2**20), "grid_forward": int(197.6 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8}
 
