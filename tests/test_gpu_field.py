@@ -91,6 +91,8 @@ def test_backward_full_config(oracle):
     got2 = host(dg)
     assert rel_l2(got2[:of.off_grid], 2 * ref[:of.off_grid]) < 3 * RTOL
     assert rel_l2(got2[of.off_grid:of.off_var], 2 * ref[of.off_grid:of.off_var]) < 2e-2
+    # ... the variance gradient too (every backward sums its own batch, nothing is left over from the first call)
+    assert abs(got2[of.off_var] - 2 * ref[of.off_var]) <= 2 * RTOL * abs(ref[of.off_var]) + 0.1, (got2[of.off_var], ref[of.off_var])
 
 
 def test_backward_reference_14_level_config(oracle):
