@@ -180,6 +180,39 @@ def test_other_table_shapes(oracle, cfg):
     assert rel_l2(host(dg), ref_grad) < 2e-2
 
 
+@pytest.mark.parametrize("cfg", [(6, 12, 4, 1.6), (5, 4, 2, 1.5), (8, 14, 4, 2.0), (14, 19, 16, 1.4472692012786865),
+                                 (16, 19, 32, 1.4472692012786865), (4, 21, 512, 1.9)])
+def test_sorted_scatter_other_table_shapes(oracle, cfg):
+    """The bucketed scatter on other tables: one bucket per level (2^12 entries), four buckets (2^14: no multiple of the
+    8 XCDs), tiny tables with a true modulo, the 14-level config, hashed levels whose resolution exceeds the 12 index bits
+    a pair record relies on (base 32: 5646 and 8170 cells, one record per corner there), and a table too large for the
+    bucket plan (2^21 entries: falls back to the atomic scatter)."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding
+    og = oracle.Grid(*cfg)
+    gg = GridEncoding(n_levels=cfg[0], log2_hashmap_size=cfg[1], base_resolution=cfg[2], per_level_scale=cfg[3])
+    rng = np.random.default_rng(23)
+    params = q16(rng.uniform(-1, 1, og.n_params))
+    dp = dev(params, torch.float16)
+    dg = torch.zeros_like(dp)
+    gg.set_params(dp, dg)
+    n = 3 * 4096 + 13 * 8
+    assert gg.reserve_scatter_workspace(1 << 14) == (cfg[1] <= 19)
+    xyz = rng.random((3, n), dtype=np.float32)
+    dy = q16(rng.standard_normal((og.n_out, n)))
+    g2 = q16(rng.standard_normal((og.n_out, n)) * 0.1)
+    v = (rng.standard_normal((3, n)) * 1e-3).astype(np.float32)
+    ref1, _ = og.backward(params, xyz, dy, want_dx=False)
+    ref, _, _ = og.backward_backward_input(params, xyz, v, g2, grad=ref1.copy(), want_dinput=False)
+    dg.fill_(7.0)
+    gg.backward_fused(dev(xyz), dev(dy, torch.float16), dev(v), dev(g2, torch.float16), want_dL_ddLdy=False, mode=GRAD_OVERWRITE)
+    got = host(dg)
+    for l in range(cfg[0]):
+        a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+        k = 8.0 * n / max(1, int(og.entries[l]))
+        tol = RTOL * (1.0 if cfg[1] <= 19 else max(1.0, np.sqrt(k)))  # the atomic fallback adds in fp16
+        assert rel_l2(got[a:b], ref[a:b]) < tol, (l, rel_l2(got[a:b], ref[a:b]), tol)
+
+
 def test_errors_are_reported_not_launched():
     from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding, N2Error
     gg = GridEncoding(**CFG)
