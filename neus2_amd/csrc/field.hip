@@ -26,6 +26,9 @@ struct n2_field {
 	unsigned char* ws;
 	uint64_t ws_bytes;
 	uint32_t max_batch, max_batch_bwd;
+	// Batch size for which the padding rows of each input-side matrix of the two networks hold zeros (0: not known).
+	// The matrices are rows x N with N the batch size of the call, so the padding rows move when N changes.
+	struct { uint32_t sdf_in, rgb_in, sel_sdf_in, sel_rgb_in, d_density_in; } pad_n;
 	// carved from the workspace
 	hf* sdf_in;        // [sdf_in_w][N]
 	float* xyz;        // [3][N]  positions of the last forward, row per coordinate (the grid kernels read each row 16 times)
@@ -52,15 +55,16 @@ struct n2_field {
 };
 
 constexpr uint32_t FB = 256;
+constexpr uint32_t RGB_IN_ROWS = 38;  // colour net input: 16 SDF-net outputs, 16 SH, xyz, normal (padded to 48)
 
 // ----------------------------------------------------------------------------
 // glue kernels
 // ----------------------------------------------------------------------------
-// rows 0..2 = half(x) - half(0.5) (computed in half precision like the reference's
-// (T)pos - (T)0.5f), rows [3 + enc_w, sdf_in_w) = 0.
+// rows 0..2 = half(x) - half(0.5) (computed in half precision like the reference's (T)pos - (T)0.5f).  The padding rows
+// [3 + enc_w, sdf_in_w) are zero as in the reference, but not written here: they are cleared once per batch size
+// (zero_padding below) and nothing writes them afterwards.
 __global__ void __launch_bounds__(FB) field_pack_sdf_input_kernel(const float* __restrict__ xyz, uint32_t ps, uint32_t ds, uint32_t N,
-                                                                  hf* __restrict__ sdf_in, uint32_t enc_w, uint32_t sdf_in_w,
-                                                                  float* __restrict__ xyz_rows) {
+                                                                  hf* __restrict__ sdf_in, float* __restrict__ xyz_rows) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
 	const float* q = xyz + (size_t)i * ps;
@@ -70,7 +74,6 @@ __global__ void __launch_bounds__(FB) field_pack_sdf_input_kernel(const float* _
 		sdf_in[(size_t)d * N + i] = (hf)x - (hf)0.5f;
 		xyz_rows[(size_t)d * N + i] = x;
 	}
-	for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) sdf_in[(size_t)r * N + i] = (hf)0;
 }
 
 __device__ __forceinline__ void sh4_eval(float x, float y, float z, float* o) {
@@ -94,7 +97,7 @@ __device__ __forceinline__ void sh4_eval(float x, float y, float z, float* o) {
 }
 
 // normal = dy_dx^T dsdf_din[3..3+enc_w) + dsdf_din[0..3); then the colour net's input rows
-// 16..31 (SH of the direction), 32..34 (xyz), 35..37 (normal), 38..47 (zero).
+// 16..31 (SH of the direction), 32..34 (xyz), 35..37 (normal); the padding rows 38..47 stay zero (zero_padding).
 __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float* __restrict__ coords, uint32_t N, uint32_t enc_w,
                                                                      const hf* __restrict__ dsdf_din, const float* __restrict__ dy_dx,
                                                                      float* __restrict__ normal, hf* __restrict__ rgb_in) {
@@ -125,8 +128,6 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 	rgb_in[(size_t)35 * N + i] = (hf)n0;
 	rgb_in[(size_t)36 * N + i] = (hf)n1;
 	rgb_in[(size_t)37 * N + i] = (hf)n2;
-#pragma unroll
-	for (int k = 38; k < 48; ++k) rgb_in[(size_t)k * N + i] = (hf)0;
 }
 
 // output rows 3 (sdf + bias), 4..6 (normal), 7 (variance), 8..10 (direction); rows 0..2 and
@@ -155,10 +156,10 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 //  * v = dL/dnormal = colour-net input gradient rows 35..37 + eikonal rows 4..6 / batch + cos rows 8..10;
 //  * second-order MLP input rows 0..2 = half(v), rows 3 .. 3+enc_w = dy_dx v (the encoding's
 //    backward_backward_input output dL_ddLdoutput, taken from the Jacobian the forward stored instead of
-//    gathering the table again), rows [3 + enc_w, sdf_in_w) = 0;
+//    gathering the table again); the padding rows above stay zero (zero_padding);
 //  * the variance gradient is the sum of row 7: every workgroup leaves its partial sum in var_part[blockIdx.x] and
 //    field_variance_gradient_kernel adds them up in a fixed order.
-__global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uint32_t enc_w, uint32_t sdf_in_w, hf* __restrict__ d_rgb_in,
+__global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uint32_t enc_w, hf* __restrict__ d_rgb_in,
                                                                  const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
                                                                  float* __restrict__ v, hf* __restrict__ d_density_in,
                                                                  float* __restrict__ var_part, const uint32_t* __restrict__ src_index,
@@ -187,7 +188,6 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 			const float* j = dy_dx + ((size_t)r * jn + js) * 3;
 			d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
 		}
-		for (uint32_t r = 3 + enc_w; r < sdf_in_w; ++r) d_density_in[(size_t)r * N + i] = (hf)0;
 	}
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -223,8 +223,8 @@ __global__ void __launch_bounds__(VB) field_variance_gradient_kernel(const float
 // out[r][j] = in[r][index[j]] for the rows the backward reads; blockIdx.y picks a group of 8 fp16 rows (SDF-net input,
 // colour-net input, encoding rows of d sdf / d input) or, last, the three fp32 position rows.  Two samples per thread so
 // that the stores move pairs.
-__global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n_src, const uint32_t* __restrict__ index, uint32_t sdf_in_w,
-                                                          uint32_t rgb_in_w, uint32_t enc_w, const hf* __restrict__ sdf_in,
+__global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n_src, const uint32_t* __restrict__ index, uint32_t sdf_rows,
+                                                          uint32_t rgb_rows, uint32_t enc_w, const hf* __restrict__ sdf_in,
                                                           const hf* __restrict__ rgb_in, const hf* __restrict__ dsdf_din,
                                                           const float* __restrict__ xyz, hf* __restrict__ o_sdf_in, hf* __restrict__ o_rgb_in,
                                                           hf* __restrict__ o_denc, float* __restrict__ o_xyz, uint32_t* __restrict__ o_index) {
@@ -233,12 +233,12 @@ __global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n
 	if (j >= n) return;
 	const bool two = j + 1 < n;
 	const uint32_t s0 = min(index[j], n_src - 1u), s1 = two ? min(index[j + 1], n_src - 1u) : s0;
-	const uint32_t groups_a = (sdf_in_w + 7) / 8, groups_b = (rgb_in_w + 7) / 8, groups_c = (enc_w + 7) / 8;
+	const uint32_t groups_a = (sdf_rows + 7) / 8, groups_b = (rgb_rows + 7) / 8, groups_c = (enc_w + 7) / 8;
 	uint32_t g = blockIdx.y, rows;  // rows of this group (the last group of a matrix may be short)
 	const hf* in;
 	hf* out;
-	if (g < groups_a) { in = sdf_in + (size_t)g * 8 * n_src; out = o_sdf_in + (size_t)g * 8 * n; rows = min(8u, sdf_in_w - g * 8); }
-	else if ((g -= groups_a) < groups_b) { in = rgb_in + (size_t)g * 8 * n_src; out = o_rgb_in + (size_t)g * 8 * n; rows = min(8u, rgb_in_w - g * 8); }
+	if (g < groups_a) { in = sdf_in + (size_t)g * 8 * n_src; out = o_sdf_in + (size_t)g * 8 * n; rows = min(8u, sdf_rows - g * 8); }
+	else if ((g -= groups_a) < groups_b) { in = rgb_in + (size_t)g * 8 * n_src; out = o_rgb_in + (size_t)g * 8 * n; rows = min(8u, rgb_rows - g * 8); }
 	else if ((g -= groups_b) < groups_c) { in = dsdf_din + (size_t)(3 + g * 8) * n_src; out = o_denc + (size_t)g * 8 * n; rows = min(8u, enc_w - g * 8); }
 	else {
 #pragma unroll
@@ -418,6 +418,7 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->sel_index = reinterpret_cast<uint32_t*>(b + c.sel_index);
 	f->last_n = 0;
 	f->sel_n = 0;
+	f->pad_n = {0, 0, 0, 0, 0};
 	f->ws_sdf = b + c.ws_sdf;
 	f->ws_rgb = b + c.ws_rgb;
 	f->ws_grid = b + c.ws_grid;
@@ -438,6 +439,15 @@ static int check_field(const n2_field_t* f, const char* fn, uint32_t n) {
 
 static inline dim3 fgrid(uint32_t n) { return dim3((n + FB - 1) / FB); }
 
+// Rows [first_row, n_rows) of the rows x n matrix m are padding: the networks read them and they must be zero.  No kernel
+// writes them, so they are cleared when the batch size (the row pitch) differs from the one they were last cleared for.
+static int zero_padding(hipStream_t s, hf* m, uint32_t first_row, uint32_t n_rows, uint32_t n, uint32_t& cleared_for) {
+	if (cleared_for == n || first_row >= n_rows) return N2_OK;
+	if (int rc = n2_fill_zero_u32(s, m + (size_t)first_row * n, (size_t)(n_rows - first_row) * n * sizeof(hf))) return rc;
+	cleared_for = n;
+	return N2_OK;
+}
+
 N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, n2_half* d_output) {
 	if (int rc = check_field(f, "n2_field_forward", n)) return rc;
 	if (n == 0) return N2_OK;
@@ -446,7 +456,9 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	hipStream_t s = n2_stream(stream);
 	f->last_n = n;
 	f->sel_n = 0;
-	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
+	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
+	if (int rc = zero_padding(s, f->rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.rgb_in)) return rc;
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
 	// SDF net forward (into rows 0..15 of the colour net's input) and d sdf / d input in one pass over the input
@@ -485,7 +497,8 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
 	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
 	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
-	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->sdf_in_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
+	if (int rc = zero_padding(s, f->d_density_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.d_density_in)) return rc;
+	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
 	                                                         f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n);
 	N2_LAUNCH_CHECK();
 	field_variance_gradient_kernel<<<dim3(1), dim3(VB), 0, s>>>(f->var_part, fgrid(n).x, f->grads + f->off_var, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
@@ -510,9 +523,12 @@ N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_
 	N2_REQUIRE(n_source == f->last_n && n_source > 0, "n2_field_select: n_source %u, but the last n2_field_forward was over %u samples", n_source,
 	           f->last_n);
 	N2_REQUIRE(n > 0 && d_source_index != nullptr, "n2_field_select: empty selection");
-	const uint32_t groups = (f->sdf_in_w + 7) / 8 + (f->rgb_in_w + 7) / 8 + (f->enc_w + 7) / 8 + 1;
+	const uint32_t sdf_rows = 3 + f->enc_w;  // the padding rows above are not copied: they are zero on both sides
+	if (int rc = zero_padding(n2_stream(stream), f->sel_sdf_in, sdf_rows, f->sdf_in_w, n, f->pad_n.sel_sdf_in)) return rc;
+	if (int rc = zero_padding(n2_stream(stream), f->sel_rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.sel_rgb_in)) return rc;
+	const uint32_t groups = (sdf_rows + 7) / 8 + (RGB_IN_ROWS + 7) / 8 + (f->enc_w + 7) / 8 + 1;
 	field_select_kernel<<<dim3((n + 2 * FB - 1) / (2 * FB), groups), dim3(FB), 0, n2_stream(stream)>>>(
-		n, n_source, d_source_index, f->sdf_in_w, f->rgb_in_w, f->enc_w, f->sdf_in, f->rgb_in, f->dsdf_din, f->xyz, f->sel_sdf_in, f->sel_rgb_in,
+		n, n_source, d_source_index, sdf_rows, RGB_IN_ROWS, f->enc_w, f->sdf_in, f->rgb_in, f->dsdf_din, f->xyz, f->sel_sdf_in, f->sel_rgb_in,
 		f->sel_dsdf_denc, f->sel_xyz, f->sel_index);
 	N2_LAUNCH_CHECK();
 	f->sel_n = n;
@@ -527,7 +543,8 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	N2_REQUIRE(ps >= 1 && ds >= 1, "%s: strides must be >= 1", fn);
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "%s: d_output must be 16-byte aligned", fn);
 	hipStream_t s = n2_stream(stream);
-	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->enc_w, f->sdf_in_w, f->xyz);
+	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
+	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), nullptr)) return rc;
 	if (int rc = n2_mlp_forward(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n, d_output, N2_LAYOUT_SOA, nullptr)) return rc;

@@ -172,3 +172,38 @@ def test_select_equals_forward_on_the_selected_samples(oracle):
         gf.backward(d_coords, dev(q16(rng.standard_normal((n_src, 16))), torch.float16), ek_batch_size=n_src)
     with pytest.raises(N2Error):
         gf.select(dev(idx, torch.int32), n_src + 8)
+
+
+def test_padding_rows_follow_the_batch_size(oracle):
+    """The inputs of the two networks are padded to 48 rows; the padding rows are cleared once per batch size and never
+    written again.  Starting from a workspace full of NaNs, batches of changing sizes (the rows move with the row pitch),
+    the SDF-only path and a backward through a selection all agree with the oracle."""
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE
+    of, gf, p, dp, dg, rng = make(oracle, seed=11)
+    gf.reserve(8192)
+    gf._ws.fill_(0xFF)  # every fp16 of the workspace is a NaN
+    for n in (4096, 2048, 8192, 4096):
+        coords = rand_coords(rng, n)
+        ref, ctx = of.forward(p, coords)
+        out = host(gf.forward(dev(coords))).T
+        assert np.isfinite(out[:11]).all(), n
+        assert_close(out[:11], ref[:11], what=f"field output at n={n}", outlier_frac=FLIP)
+        xyz = np.ascontiguousarray(coords[: n // 2, :3])
+        sdf = host(gf.sdf(dev(xyz)))
+        assert np.isfinite(sdf[0]).all()
+        assert_close(sdf[0], of.sdf_values(p, xyz.T.copy())[0], what=f"sdf at n={n // 2}", outlier_frac=FLIP)
+    # a backward through a selection of half the last batch
+    n = 4096
+    coords = rand_coords(rng, n)
+    gf.forward(dev(coords))
+    pick = np.sort(rng.choice(n, n // 2, replace=False)).astype(np.int32)
+    gf.select(torch.from_numpy(pick).cuda(), n)
+    dL = q16(rng.standard_normal((16, n // 2)) * np.array([.1, .1, .1, .1, 3, 3, 3, .1, .003, .003, .003, 0, 0, 0, 0, 0])[:, None])
+    sub = np.ascontiguousarray(coords[pick])
+    _, ctx = of.forward(p, sub)
+    ref = of.backward(p, ctx, dL, ek_batch_size=n // 2)
+    gf.backward(dev(sub), dev(np.ascontiguousarray(dL.T), torch.float16), ek_batch_size=n // 2, mode=GRAD_OVERWRITE)
+    got = host(dg)
+    assert np.isfinite(got).all()
+    assert_grad_close(got[of.off_sdf:of.off_rgb], ref[of.off_sdf:of.off_rgb], what="SDF MLP gradients", rtol=2 * RTOL)
+    assert_grad_close(got[of.off_rgb:of.off_grid], ref[of.off_rgb:of.off_grid], what="colour MLP gradients", rtol=2 * RTOL)
