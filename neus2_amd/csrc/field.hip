@@ -35,7 +35,6 @@ struct n2_field {
 	hf* rgb_in;        // [48][N]
 	float* dy_dx;      // [enc_w][N][3]
 	hf* dsdf_din;      // [sdf_in_w][N]  d sdf / d (SDF net input)
-	float* normal;     // [3][N]
 	hf* d_rgb_in;      // [48][N]
 	hf* d_sdf_in;      // [sdf_in_w][N]
 	float* v;          // [3][N]  dL / d normal
@@ -100,7 +99,7 @@ __device__ __forceinline__ void sh4_eval(float x, float y, float z, float* o) {
 // 16..31 (SH of the direction), 32..34 (xyz), 35..37 (normal); the padding rows 38..47 stay zero (zero_padding).
 __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float* __restrict__ coords, uint32_t N, uint32_t enc_w,
                                                                      const hf* __restrict__ dsdf_din, const float* __restrict__ dy_dx,
-                                                                     float* __restrict__ normal, hf* __restrict__ rgb_in) {
+                                                                     hf* __restrict__ rgb_in) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
 	float n0 = 0.f, n1 = 0.f, n2 = 0.f;
@@ -114,9 +113,6 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 	n0 += (float)dsdf_din[i];
 	n1 += (float)dsdf_din[(size_t)N + i];
 	n2 += (float)dsdf_din[(size_t)2 * N + i];
-	normal[i] = n0;
-	normal[(size_t)N + i] = n1;
-	normal[(size_t)2 * N + i] = n2;
 	const float* c = coords + (size_t)i * 7;
 	float sh[16];
 	sh4_eval(c[4] * 2.f - 1.f, c[5] * 2.f - 1.f, c[6] * 2.f - 1.f, sh);
@@ -131,18 +127,18 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 }
 
 // output rows 3 (sdf + bias), 4..6 (normal), 7 (variance), 8..10 (direction); rows 0..2 and
-// 11..15 keep what the colour net wrote.
-__global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __restrict__ coords, uint32_t N, const hf* __restrict__ sdf_out,
-                                                                 hf bias, const float* __restrict__ normal, const hf* __restrict__ variance,
-                                                                 hf* __restrict__ output) {
+// 11..15 keep what the colour net wrote.  The SDF and the normal are taken from the colour net's input (rows 0 and
+// 35..37), where they already stand in half precision.
+__global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __restrict__ coords, uint32_t N, const hf* __restrict__ rgb_in,
+                                                                 hf bias, const hf* __restrict__ variance, hf* __restrict__ output) {
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
 	hf* o = output + (size_t)i * 16;
 	const float* c = coords + (size_t)i * 7;
-	o[3] = sdf_out[i] + bias;
-	o[4] = (hf)normal[i];
-	o[5] = (hf)normal[(size_t)N + i];
-	o[6] = (hf)normal[(size_t)2 * N + i];
+	o[3] = rgb_in[i] + bias;
+	o[4] = rgb_in[(size_t)35 * N + i];
+	o[5] = rgb_in[(size_t)36 * N + i];
+	o[6] = rgb_in[(size_t)37 * N + i];
 	o[7] = variance[0];
 	o[8] = (hf)c[4];
 	o[9] = (hf)c[5];
@@ -352,7 +348,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, normal, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -366,7 +362,6 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.rgb_in = take(2ull * f->rgb_in_w * n);
 	c.dy_dx = take(12ull * f->enc_w * n);
 	c.dsdf_din = take(2ull * f->sdf_in_w * n);
-	c.normal = take(12ull * n);
 	n = nbw;
 	c.d_rgb_in = take(2ull * f->rgb_in_w * n);
 	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
@@ -405,7 +400,6 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->rgb_in = reinterpret_cast<hf*>(b + c.rgb_in);
 	f->dy_dx = reinterpret_cast<float*>(b + c.dy_dx);
 	f->dsdf_din = reinterpret_cast<hf*>(b + c.dsdf_din);
-	f->normal = reinterpret_cast<float*>(b + c.normal);
 	f->d_rgb_in = reinterpret_cast<hf*>(b + c.d_rgb_in);
 	f->d_sdf_in = reinterpret_cast<hf*>(b + c.d_sdf_in);
 	f->v = reinterpret_cast<float*>(b + c.v);
@@ -464,10 +458,10 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	// SDF net forward (into rows 0..15 of the colour net's input) and d sdf / d input in one pass over the input
 	if (int rc = n2_mlp_forward_and_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
 	                                               reinterpret_cast<n2_half*>(f->rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->dsdf_din))) return rc;
-	field_normals_rgb_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->enc_w, f->dsdf_din, f->dy_dx, f->normal, f->rgb_in);
+	field_normals_rgb_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->enc_w, f->dsdf_din, f->dy_dx, f->rgb_in);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_mlp_forward(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n, d_output, N2_LAYOUT_AOS, nullptr)) return rc;
-	field_finish_output_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->rgb_in, (hf)f->sdf_bias, f->normal, f->params + f->off_var,
+	field_finish_output_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->rgb_in, (hf)f->sdf_bias, f->params + f->off_var,
 	                                                         reinterpret_cast<hf*>(d_output));
 	N2_LAUNCH_CHECK();
 	return N2_OK;
