@@ -323,7 +323,10 @@ int n2_field_set_params(n2_field_t* field, const n2_half* d_params, n2_half* d_g
  * the grid's dy_dx context, input gradients and the MLP weight-gradient slabs.
  * max_batch bounds forward / sdf / density calls, max_batch_backward (<= max_batch) the batches
  * that are also run backward: the training step runs the forward over every marched sample
- * (up to 16 x 2^18) but the backward only over the compacted 2^18 (src/testbed_nerf.cu:3840, 3931-3932). */
+ * (up to 16 x 2^18) but the backward only over the compacted 2^18 (src/testbed_nerf.cu:3840, 3931-3932).
+ * The workspace belongs to the field until another one is set: between calls it keeps the activations a backward or a
+ * selection reads and the zero padding rows of the networks' inputs, which are cleared once per batch size and not
+ * in every call; do not write to it. */
 uint64_t n2_field_workspace_bytes(const n2_field_t* field, uint32_t max_batch, uint32_t max_batch_backward);
 int n2_field_set_workspace(n2_field_t* field, void* d_workspace, uint64_t n_bytes, uint32_t max_batch,
                            uint32_t max_batch_backward);
