@@ -493,6 +493,7 @@ constexpr uint32_t BKT_SHIFT = N2_BKT_SHIFT;           // 4096 entries per bucke
 constexpr uint32_t BKT_ENTRIES = 1u << BKT_SHIFT;
 constexpr uint32_t BKT_MAX = (1u << 19) >> BKT_SHIFT;  // buckets per level (entries <= 2^19)
 constexpr uint32_t PAIR_MAX_CELL = BKT_ENTRIES - 2u;  // pair records (grid_bin_kernel): x + 1 <= BKT_ENTRIES - 1
+static_assert(BKT_SHIFT <= 12, "a pair record's 16-bit key holds the entry within the bucket and four bits of carry length");
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
 constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
 constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: two workgroups (2 x 64 KiB staging) keep 4 waves on every SIMD
