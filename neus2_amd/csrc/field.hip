@@ -103,7 +103,26 @@ __global__ void __launch_bounds__(FB) field_normals_rgb_input_kernel(const float
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	if (i >= N) return;
 	float n0 = 0.f, n1 = 0.f, n2 = 0.f;
-	for (uint32_t k = 0; k < enc_w; ++k) {
+	// eight rows' loads are issued before the first is used: the kernel is a stream of 14 bytes per lane and row, and one
+	// row in flight per lane leaves it waiting on memory latency
+	constexpr uint32_t U = 8;
+	uint32_t k = 0;
+	for (; k + U <= enc_w; k += U) {
+		float g[U], j[U][3];
+#pragma unroll
+		for (uint32_t u = 0; u < U; ++u) {
+			g[u] = (float)dsdf_din[(size_t)(3 + k + u) * N + i];
+			const float* q = dy_dx + ((size_t)(k + u) * N + i) * 3;
+			j[u][0] = q[0]; j[u][1] = q[1]; j[u][2] = q[2];
+		}
+#pragma unroll
+		for (uint32_t u = 0; u < U; ++u) {
+			n0 = fmaf(g[u], j[u][0], n0);
+			n1 = fmaf(g[u], j[u][1], n1);
+			n2 = fmaf(g[u], j[u][2], n2);
+		}
+	}
+	for (; k < enc_w; ++k) {
 		const float g = (float)dsdf_din[(size_t)(3 + k) * N + i];
 		const float* j = dy_dx + ((size_t)k * N + i) * 3;
 		n0 = fmaf(g, j[0], n0);
@@ -180,7 +199,20 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 			v[(size_t)d * N + i] = x;
 			d_density_in[(size_t)d * N + i] = (hf)x;
 		}
-		for (uint32_t r = 0; r < enc_w; ++r) {
+		// eight rows' loads in flight per lane (see the normals kernel)
+		constexpr uint32_t U = 8;
+		uint32_t r = 0;
+		for (; r + U <= enc_w; r += U) {
+			float j[U][3];
+#pragma unroll
+			for (uint32_t u = 0; u < U; ++u) {
+				const float* q = dy_dx + ((size_t)(r + u) * jn + js) * 3;
+				j[u][0] = q[0]; j[u][1] = q[1]; j[u][2] = q[2];
+			}
+#pragma unroll
+			for (uint32_t u = 0; u < U; ++u) d_density_in[(size_t)(3 + r + u) * N + i] = (hf)(j[u][0] * vv[0] + j[u][1] * vv[1] + j[u][2] * vv[2]);
+		}
+		for (; r < enc_w; ++r) {
 			const float* j = dy_dx + ((size_t)r * jn + js) * 3;
 			d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
 		}
