@@ -147,7 +147,18 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 	__shared__ uint32_t part[CB / 64];
 	const uint32_t first = blockIdx.x * (CB / 64);
 	uint32_t before = 0;
-	for (uint32_t r = threadIdx.x; r < first; r += CB) before += kept_of[r];
+	// eight loads in flight per lane: the last workgroups add up thousands of counts, and one dependent L2 round trip per
+	// CB of them was most of this kernel's duration
+	for (uint32_t r0 = 0; r0 < first; r0 += 8 * CB) {
+		uint32_t v[8];
+#pragma unroll
+		for (uint32_t u = 0; u < 8; ++u) {
+			const uint32_t r = r0 + u * CB + threadIdx.x;
+			v[u] = r < first ? kept_of[r] : 0u;
+		}
+#pragma unroll
+		for (uint32_t u = 0; u < 8; ++u) before += v[u];
+	}
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
 	if (lane == 0) part[wave] = before;
