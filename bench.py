@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload step|grid|sdf|lattice|occupancy|mesh] [--no-cpu-baseline]
 
-A step is one full static NeuS2 training step (BASELINE config 4) on a synthetic scene: an analytic sphere of
+A step is one full static NeuS2 training step (configuration 4 of BASELINE.json) on a synthetic scene: an analytic sphere of
 radius 0.3, Lambertian-textured, seen by 64 cameras at 512x512 on a sphere of radius 2; rays are marched through a
 128^3 occupancy bitfield and compacted to 2^18 samples; hash grid + SDF MLP + colour MLP forward, first- and
 second-order backward, compositing and Adam, all on the GPU.  Prints ONE JSON line.
@@ -192,7 +192,7 @@ def run_step_workload(args):
 
 
 def run_grid_workload(args):
-    """BASELINE configs[1]: hash-grid encoding only, forward + backward on 2^18 uniform points."""
+    """Configuration 2 of BASELINE.json: hash-grid encoding only, forward + backward on 2^18 uniform points."""
     import torch
     from neus2_amd import capi
     from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding
@@ -237,7 +237,7 @@ def run_grid_workload(args):
 
 
 def run_sdf_workload(args):
-    """BASELINE configs[2]: grid + SDF MLP with the eikonal second-order path on 2^18 uniform points: forward,
+    """Configuration 3 of BASELINE.json: grid + SDF MLP with the eikonal second-order path on 2^18 uniform points: forward,
     normals, backward of mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 through the encoding and the MLP weights."""
     import numpy as np
     import torch
@@ -291,7 +291,7 @@ def run_sdf_workload(args):
 
 
 def run_lattice_workload(args):
-    """BASELINE configs[4]: SDF inference for mesh extraction (hash grid + SDF MLP forward, fp16) over the 512^3
+    """Configuration 5 of BASELINE.json: SDF inference for mesh extraction (hash grid + SDF MLP forward, fp16) over the 512^3
     lattice p = (i, j, k) / 512, in chunks of 2^22 points; a step is one chunk, chunks are visited in order."""
     import numpy as np
     import torch
@@ -412,7 +412,7 @@ def run_occupancy_workload(args):
 
 
 def run_mesh_workload(args):
-    """The consumer of BASELINE configs[4]: marching cubes over the 512^3 SDF lattice (count, prefix sums, vertices, faces,
+    """The consumer of configuration 5 of BASELINE.json: marching cubes over the 512^3 SDF lattice (count, prefix sums, vertices, faces,
     normals).  The lattice is evaluated once, untimed (that part is `--workload lattice`); a step is one full extraction."""
     import numpy as np
     import torch

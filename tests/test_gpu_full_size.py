@@ -42,7 +42,7 @@ def level_slices(og):
 
 
 def test_grid_forward_2p18_against_oracle(grid):
-    """BASELINE's grid-only configuration: 2^18 uniform points, every value and derivative against the oracle."""
+    """The benchmark's grid-only configuration: 2^18 uniform points, every value and derivative against the oracle."""
     og, gg, params, dg, xyz, dy, rng = grid
     ref_y, ref_j = og.forward(params, xyz, want_dy_dx=True)
     y, ctx = gg.forward(dev(xyz), prepare_input_gradients=True)
@@ -81,7 +81,7 @@ def test_grid_scatter_2p18_against_oracle_and_checksums(grid):
 
 
 def test_field_step_2p18_against_oracle(oracle):
-    """BASELINE's SDF-net configuration at 2^18 samples: forward, normals, first- and second-order backward of the whole
+    """The benchmark's SDF-net configuration at 2^18 samples: forward, normals, first- and second-order backward of the whole
     field against the oracle's field."""
     from neus2_amd.tcnn_api import GRAD_OVERWRITE, NerfNetwork
     from oracle.field import Field
@@ -119,7 +119,7 @@ def test_field_step_2p18_against_oracle(oracle):
 
 
 def test_lattice_512_chunks_and_subsample(oracle):
-    """BASELINE's mesh-inference configuration: the SDF over the 512^3 lattice in 2^22-point chunks.  A random subsample
+    """The benchmark's mesh-inference configuration: the SDF over the 512^3 lattice in 2^22-point chunks.  A random subsample
     is compared with the oracle; cutting the lattice into other chunk sizes gives the same bits."""
     from neus2_amd.mesh import density_on_grid
     from neus2_amd.tcnn_api import NerfNetwork

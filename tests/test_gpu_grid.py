@@ -25,7 +25,7 @@ def setup(oracle):
 
 
 def test_config1_indices_bit_exact(setup):
-    """BASELINE config 1: 2^14 points U[0,1)^3, seed 0: every corner index of every level identical."""
+    """The benchmark's plumbing configuration: 2^14 points U[0,1)^3, seed 0: every corner index of every level identical."""
     og, gg, *_ = setup
     xyz = np.random.default_rng(0).random((3, 1 << 14), dtype=np.float32)
     ref, _ = og.indices(xyz)
