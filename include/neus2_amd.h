@@ -445,6 +445,22 @@ int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* con
                               uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
                               float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes);
 
+/* n2_composite_loss_indexed without a workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-ray scratch (composited colour and kept-sample count of every ray, 24 bytes per ray) lives in an array inside
+ * the library's device image, 1.5 MiB that each GPU the library runs on holds until the process ends; the call
+ * allocates and frees nothing.  n_rays above N2_COMPOSITE_STATIC_MAX_RAYS is rejected with N2_ERR_INVALID_ARGUMENT.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or host threads
+ * without ordering between them) race; calls ordered on one stream are safe.  Nothing in the array has to start at
+ * zero: the forward kernel writes every ray's slot below n_rays before the backward kernel reads it.  Results are
+ * bit-identical to n2_composite_loss_indexed's. */
+#define N2_COMPOSITE_STATIC_MAX_RAYS 65536u
+int n2_composite_loss_static(n2_stream_t stream, const n2_composite_config* config, uint32_t n_rays,
+                             const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                             const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                             uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                             float* d_loss, uint32_t* d_source_index);
+
 /* tcnn fill_rollover / fill_rollover_and_rescale, src/testbed_nerf.cu:3908-3916: pad a compacted
  * batch of *d_n_in rows to n_total rows by wrapping around; the fp16 variant scales the wrapped
  * copies by n_in/n_total.  No-op when *d_n_in is 0 or >= n_total. */

@@ -9,6 +9,8 @@
 // ray order, backward (gradients and compacted coordinates).
 #include "n2_common.h"
 
+#include <mutex>
+
 typedef _Float16 hf;
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
@@ -286,6 +288,48 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
 	return n2_composite_loss_indexed(stream, cfg, n_rays, d_ray_counter, d_numsteps, d_network_output, d_coords, d_rgb_target,
 	                                 max_samples_compacted, d_compacted_counter, d_coords_compacted, d_dloss_doutput, d_loss, nullptr,
 	                                 d_workspace, workspace_bytes);
+}
+
+// Scratch of n2_composite_loss_static: per-ray colour and kept counts for up to N2_COMPOSITE_STATIC_MAX_RAYS rays, held
+// by every GPU the library runs on until the process ends.  In host code the array's name stands for the symbol only;
+// the device address of each GPU's copy is looked up once per device (static_scratch) and that pointer is what the
+// kernels receive.
+constexpr uint32_t STATIC_MAX_RAYS = N2_COMPOSITE_STATIC_MAX_RAYS;
+constexpr uint64_t STATIC_BYTES = (sizeof(RayScratch) * (uint64_t)STATIC_MAX_RAYS + 255) / 256 * 256 + 2 * ((4ull * STATIC_MAX_RAYS + 255) / 256 * 256);
+static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static std::mutex g_static_lock;
+static void* g_static_ptr[STATIC_MAX_DEVICES] = {};
+
+// device address of the current device's copy of `scratch` (looked up on the first call on that device)
+static int static_scratch(void** out) {
+	int device = -1;
+	N2_HIP(hipGetDevice(&device));
+	N2_REQUIRE(device >= 0 && device < STATIC_MAX_DEVICES, "n2_composite_loss_static: device ordinal %d outside [0, %d)", device, STATIC_MAX_DEVICES);
+	std::lock_guard<std::mutex> guard(g_static_lock);
+	if (g_static_ptr[device] == nullptr) {
+		void* p = nullptr;
+		N2_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+		N2_REQUIRE(p != nullptr && reinterpret_cast<uintptr_t>(p) % 256 == 0, "n2_composite_loss_static: bad address for the scratch array");
+		g_static_ptr[device] = p;
+	}
+	*out = g_static_ptr[device];
+	return N2_OK;
+}
+
+N2_API int n2_composite_loss_static(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
+                                    const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                                    const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                                    uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                                    float* d_loss, uint32_t* d_source_index) {
+	N2_REQUIRE(n_rays <= STATIC_MAX_RAYS, "n2_composite_loss_static: %u rays exceed the static scratch's maximum of %u (use n2_composite_loss_indexed with a workspace)",
+	           n_rays, STATIC_MAX_RAYS);
+	void* ws = nullptr;
+	if (int rc = static_scratch(&ws)) return rc;
+	return n2_composite_loss_indexed(stream, cfg, n_rays, d_ray_counter, d_numsteps, d_network_output, d_coords, d_rgb_target,
+	                                 max_samples_compacted, d_compacted_counter, d_coords_compacted, d_dloss_doutput, d_loss, d_source_index,
+	                                 ws, STATIC_BYTES);
 }
 
 N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
