@@ -315,6 +315,13 @@ uint32_t n2_field_n_params(const n2_field_t* field);
  * (NerfNetwork::layer_sizes, nerf_network.h:902-990). */
 int n2_field_param_offsets(const n2_field_t* field, uint32_t offsets[5]);
 
+/* Tuning switch without a counterpart in the reference.  On (the default): n2_field_forward, n2_field_sdf and
+ * n2_field_density run as ONE kernel each (grid gather, both networks and the row bookkeeping fused) whenever the
+ * configuration allows it: at most 16 levels with power-of-two hash tables, one hidden layer in the SDF net, two in the
+ * colour net, no per-point level mask.  Off, or for other configurations: the same results from separate grid, network
+ * and element-wise kernels (values agree within fp32 summation order). */
+int n2_field_set_fused(n2_field_t* field, int enable);
+
 /* NerfNetwork::set_params, nerf_network.h:728-772 (fp16 params and gradients, n_params each). */
 int n2_field_set_params(n2_field_t* field, const n2_half* d_params, n2_half* d_gradients);
 
@@ -759,7 +766,8 @@ typedef enum n2_prof_id {
 	N2_PROF_COMPOSITE = 6,
 	N2_PROF_SAMPLER = 7,
 	N2_PROF_ADAM = 8,
-	N2_PROF_COUNT = 9
+	N2_PROF_FIELD_FORWARD = 9, /* the fused forward kernels of the field (grid + networks in one launch) */
+	N2_PROF_COUNT = 10
 } n2_prof_id;
 
 int n2_profile_enable(int enable);

@@ -51,6 +51,7 @@ struct n2_field {
 	void* ws_sdf;
 	void* ws_rgb;
 	void* ws_grid;
+	bool fused;  // forward passes go through the fused kernels where the configuration allows (n2_field_set_fused)
 };
 
 constexpr uint32_t FB = 256;
@@ -341,6 +342,7 @@ N2_API int n2_field_create(const n2_field_config* cfg, n2_field_t** out) {
 		return rc;
 	}
 	f->sdf_bias = cfg->sdf_bias;
+	f->fused = true;
 	f->off_sdf = 0;
 	f->off_rgb = n2_mlp_n_params(f->sdf);
 	f->off_grid = f->off_rgb + n2_mlp_n_params(f->rgb);
@@ -359,6 +361,12 @@ N2_API void n2_field_destroy(n2_field_t* f) {
 }
 
 N2_API n2_grid_t* n2_field_encoding(n2_field_t* field) { return field ? field->grid : nullptr; }
+
+N2_API int n2_field_set_fused(n2_field_t* field, int enable) {
+	N2_REQUIRE(field != nullptr, "n2_field_set_fused: field is null");
+	field->fused = enable != 0;
+	return N2_OK;
+}
 N2_API uint32_t n2_field_n_params(const n2_field_t* f) { return f ? f->n_params : 0; }
 
 N2_API int n2_field_param_offsets(const n2_field_t* f, uint32_t offsets[5]) {
@@ -465,6 +473,22 @@ static int check_field(const n2_field_t* f, const char* fn, uint32_t n) {
 
 static inline dim3 fgrid(uint32_t n) { return dim3((n + FB - 1) / FB); }
 
+static N2FusedNets fused_nets(const n2_field_t* f) {
+	N2FusedNets nets;
+	nets.tab = n2_grid_table(f->grid);
+	nets.table = n2_grid_params(f->grid);
+	nets.sdf_w = reinterpret_cast<const n2_half*>(f->params + f->off_sdf);
+	nets.rgb_w = reinterpret_cast<const n2_half*>(f->params + f->off_rgb);
+	nets.variance = reinterpret_cast<const n2_half*>(f->params + f->off_var);
+	nets.sdf_in_w = f->sdf_in_w;
+	nets.sdf_bias = f->sdf_bias;
+	return nets;
+}
+// the level mask can change between calls (n2_grid_set_max_level_gpu), so the check is made per call
+static bool fused_ok(const n2_field_t* f) {
+	return n2_fused_supported(*n2_grid_table(f->grid), n2_mlp_hidden_layers(f->sdf), n2_mlp_hidden_layers(f->rgb));
+}
+
 // Rows [first_row, n_rows) of the rows x n matrix m are padding: the networks read them and they must be zero.  No kernel
 // writes them, so they are cleared when the batch size (the row pitch) differs from the one they were last cleared for.
 static int zero_padding(hipStream_t s, hf* m, uint32_t first_row, uint32_t n_rows, uint32_t n, uint32_t& cleared_for) {
@@ -484,6 +508,11 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	f->sel_n = 0;
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	if (int rc = zero_padding(s, f->rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.rgb_in)) return rc;
+	if (f->fused && fused_ok(f)) {
+		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+		return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx,
+		                              reinterpret_cast<n2_half*>(f->dsdf_din), reinterpret_cast<n2_half*>(f->rgb_in), d_output);
+	}
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
@@ -569,6 +598,10 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	N2_REQUIRE(ps >= 1 && ds >= 1, "%s: strides must be >= 1", fn);
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "%s: d_output must be 16-byte aligned", fn);
 	hipStream_t s = n2_stream(stream);
+	if (f->fused && fused_ok(f)) {
+		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, d_output, nullptr, density);
+	}
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();

@@ -62,6 +62,34 @@ struct N2LevelTable {
 	uint32_t pair_levels;
 };
 
+// What the fused field kernels need of a field's parts: the grid's level table and parameters, the weights of the two
+// networks, the variance parameter.  Filled by the field from its sub-objects.
+struct N2FusedNets {
+	const N2LevelTable* tab;
+	const __half2* table;
+	const n2_half* sdf_w;
+	const n2_half* rgb_w;
+	const n2_half* variance;
+	uint32_t sdf_in_w;
+	float sdf_bias;
+};
+const N2LevelTable* n2_grid_table(const n2_grid_t* grid);
+const __half2* n2_grid_params(const n2_grid_t* grid);
+bool n2_grid_lattice_order(const n2_grid_t* grid);
+const n2_half* n2_mlp_params(const n2_mlp_t* mlp);
+uint32_t n2_mlp_hidden_layers(const n2_mlp_t* mlp);
+
+// The fused forward serves grids of at most 16 levels with two features whose levels are dense or hashed with a
+// power-of-two table, one hidden layer in the SDF net and two in the colour net, without per-point level masks.
+bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uint32_t rgb_hidden_layers);
+// NerfNetwork::forward_impl in one kernel: writes the network inputs, the Jacobian of the encoding, d sdf / d input
+// (SoA, n columns) and the [n][16] output.
+int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
+                           float* dy_dx, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output);
+// NerfNetwork::sdf / density in one kernel: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
+int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
+                       float* d_row0, bool density);
+
 static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // Zero-fill with a kernel (safe to record into HIP graphs, unlike memset nodes).
