@@ -9,6 +9,7 @@
 // writes rows 3..34 of the MLP's second-order input), which leaves three glue
 // kernels in the forward and three in the backward.
 #include "n2_common.h"
+#include "grid_device.h"
 
 #include <new>
 
@@ -33,7 +34,7 @@ struct n2_field {
 	hf* sdf_in;        // [sdf_in_w][N]
 	float* xyz;        // [3][N]  positions of the last forward, row per coordinate (the grid kernels read each row 16 times)
 	hf* rgb_in;        // [48][N]
-	float* dy_dx;      // [enc_w][N][3]
+	float* dy_dx;      // [enc_w][N][3] fp32, or (slopes_saved) 16-byte slope blocks [levels][N] without the levels' scale factors
 	hf* dsdf_din;      // [sdf_in_w][N]  d sdf / d (SDF net input)
 	hf* d_rgb_in;      // [48][N]
 	hf* d_sdf_in;      // [sdf_in_w][N]
@@ -52,6 +53,7 @@ struct n2_field {
 	void* ws_rgb;
 	void* ws_grid;
 	bool fused;  // forward passes go through the fused kernels where the configuration allows (n2_field_set_fused)
+	bool slopes_saved;  // the last forward left the encoding's Jacobian as fp16 slopes (fused forward), not as fp32 dy_dx
 };
 
 constexpr uint32_t FB = 256;
@@ -175,11 +177,15 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 //    gathering the table again); the padding rows above stay zero (zero_padding);
 //  * the variance gradient is the sum of row 7: every workgroup leaves its partial sum in var_part[blockIdx.x] and
 //    field_variance_gradient_kernel adds them up in a fixed order.
+struct LevelScales { float s[16]; };
+// SLOPES: the Jacobian comes as the fused forward stores it, 16 bytes per level and sample [level][n_src] without the level's scale factor
+// (scales.s[level] multiplies it back in); else as the grid encoding's fp32 dy_dx [enc_w][n_src][3].
+template <bool SLOPES>
 __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uint32_t enc_w, hf* __restrict__ d_rgb_in,
                                                                  const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
                                                                  float* __restrict__ v, hf* __restrict__ d_density_in,
                                                                  float* __restrict__ var_part, const uint32_t* __restrict__ src_index,
-                                                                 uint32_t n_src) {
+                                                                 uint32_t n_src, LevelScales scales) {
 	typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 	__shared__ float part[FB / 64];
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
@@ -200,6 +206,27 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 			v[(size_t)d * N + i] = x;
 			d_density_in[(size_t)d * N + i] = (hf)x;
 		}
+		if (SLOPES) {
+			const uint4* slopes = reinterpret_cast<const uint4*>(dy_dx);
+			constexpr uint32_t U = 8;  // eight levels' loads in flight per lane
+			for (uint32_t l0 = 0; 2 * l0 < enc_w; l0 += U) {
+				uint4 q[U];
+#pragma unroll
+				for (uint32_t u = 0; u < U; ++u) {
+					const uint32_t l = 2 * (l0 + u) < enc_w ? l0 + u : l0;
+					q[u] = slopes[(size_t)l * jn + js];
+				}
+#pragma unroll
+				for (uint32_t u = 0; u < U; ++u) {
+					if (2 * (l0 + u) < enc_w) {
+						float m[6];
+						const float unit = n2_slopes_unpack(q[u], m) * scales.s[l0 + u];
+						d_density_in[(size_t)(3 + 2 * (l0 + u)) * N + i] = (hf)((m[0] * vv[0] + m[1] * vv[1] + m[2] * vv[2]) * unit);
+						d_density_in[(size_t)(4 + 2 * (l0 + u)) * N + i] = (hf)((m[3] * vv[0] + m[4] * vv[1] + m[5] * vv[2]) * unit);
+					}
+				}
+			}
+		} else {
 		// eight rows' loads in flight per lane (see the normals kernel)
 		constexpr uint32_t U = 8;
 		uint32_t r = 0;
@@ -216,6 +243,7 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 		for (; r < enc_w; ++r) {
 			const float* j = dy_dx + ((size_t)r * jn + js) * 3;
 			d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
+		}
 		}
 	}
 #pragma unroll
@@ -508,7 +536,8 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	f->sel_n = 0;
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	if (int rc = zero_padding(s, f->rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.rgb_in)) return rc;
-	if (f->fused && fused_ok(f)) {
+	f->slopes_saved = f->fused && fused_ok(f);
+	if (f->slopes_saved) {
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
 		return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx,
 		                              reinterpret_cast<n2_half*>(f->dsdf_din), reinterpret_cast<n2_half*>(f->rgb_in), d_output);
@@ -553,8 +582,14 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
 	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
 	if (int rc = zero_padding(s, f->d_density_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.d_density_in)) return rc;
-	field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-	                                                         f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n);
+	LevelScales scales{};
+	for (uint32_t l = 0; l < 16 && 2 * l < f->enc_w; ++l) scales.s[l] = n2_grid_table(f->grid)->scale[l];
+	if (f->slopes_saved)
+		field_backward_prep_kernel<true><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
+		                                                               f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n, scales);
+	else
+		field_backward_prep_kernel<false><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
+		                                                                f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n, scales);
 	N2_LAUNCH_CHECK();
 	field_variance_gradient_kernel<<<dim3(1), dim3(VB), 0, s>>>(f->var_part, fgrid(n).x, f->grads + f->off_var, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 	N2_LAUNCH_CHECK();

@@ -1,20 +1,27 @@
-// Fused forward of the NeuS field for gfx950: one kernel takes a tile of samples through the 16 grid levels, the
-// SDF net (forward and the gradient of its first output w.r.t. its input), the normal, the direction encoding, the
-// colour net and the output rows (counterpart of NerfNetwork::forward_impl, nerf_network.h:132-315, and of
-// NerfNetwork::sdf / density, :643-726).  Nothing travels through memory between those stages; what the kernel
-// writes is what the backward pass reads (network inputs, the encoding's Jacobian, d sdf / d encoding) and the
-// 16 output rows.
+// Fused forward of the NeuS field for gfx950 (counterpart of NerfNetwork::forward_impl, nerf_network.h:132-315, and of
+// NerfNetwork::sdf / density, :643-726).
 //
-// Layout.  A wave takes 32 consecutive samples per pass, one 32-column MFMA tile: lane (n, g), n = lane % 32,
-// g = lane / 32, works for sample b0 + n.  In the MFMA layouts (see mlp_device.h) lane (n, g)
+// Training forward = two kernels.
+//  * field_gather_kernel walks the grid LEVEL-MAJOR (one workgroup = one level x 256 samples, all workgroups of a
+//    level next to each other in time), so that the level being read (<= 2 MiB) stays resident in every L2; a
+//    sample-major walk touches all 24 MiB of tables at once and three of five L2 requests miss.  It writes the
+//    features into the SDF net's input rows and the level's slopes (the Jacobian of the encoding without the level's
+//    scale factor) as a 16-byte block-float per sample and level (n2_slopes_pack), against 24 bytes of fp32.
+//  * field_fused_forward_kernel then takes 32 samples per wave through everything else without touching memory in
+//    between: SDF net forward, the gradient of its first output w.r.t. its input, the normal (that gradient contracted
+//    with the slopes), the direction encoding, the colour net and the 16 output rows.
+// Inference (sdf / density) is the second kernel alone with the gather inside it: positions that arrive in lattice or
+// near-lattice order hit cached lines whatever the order of the levels.
+//
+// Layout of the network kernel.  Lane (n, g), n = lane % 32, g = lane / 32, works for sample b0 + n.  In the MFMA
+// layouts (see mlp_device.h) lane (n, g)
 // holds, of a B operand in chained order, the rows {16c + 4g + 0..3, 16c + 8 + 4g + 0..3} of chunk c, and of a D tile
 // the rows {8q + 4g + 0..3}, q = 0..3.  With the encoding's features as rows 0..31 of the SDF net's input (row
 // 2 l + f for feature f of level l; the three centred coordinates follow as rows 32..34) both sets are the levels
 //     l(j, g) = 4 (j / 2) + 2 g + j % 2,   j = 0..7,
-// so a lane gathers exactly those eight levels for its sample: the features land in its B operand registers,
+// so a lane loads (or gathers) exactly those eight levels of its sample: the features are its B operand registers,
 // the rows of d sdf / d encoding come back to it in the D tile of the input-gradient product, and the contraction
-// with the Jacobian it kept in registers (normal = J^T g) is lane-local up to one exchange between the two halves
-// of the wave.  The permutation of the input rows is folded into the weight fragments, which are built once per
+// with the slopes it holds (normal = J^T g) is lane-local up to one exchange between the two halves of the wave.  The permutation of the input rows is folded into the weight fragments, which are built once per
 // workgroup in LDS.
 #include "n2_common.h"
 
@@ -60,7 +67,7 @@ struct FusedArgs {
 	// full field: what the backward pass reads, and the output
 	hf* sdf_in;             // [sdf_in_w][N]  rows 0..2 centred coordinates, 3.. features
 	float* xyz_rows;        // [3][N]
-	float* dy_dx;           // [enc_w][N][3]
+	uint4* slopes;          // [n_levels][N]: d feature / d position of each level (2 x 3 values, see n2_slopes_pack), without the level's scale
 	hf* dsdf_din;           // [sdf_in_w][N]
 	hf* rgb_in;             // [48][N]
 	hf* output;             // [N][16]
@@ -249,10 +256,53 @@ __device__ __forceinline__ void sh4(float x, float y, float z, float* o) {
 }
 
 // ----------------------------------------------------------------------------
-// the kernel: a wave takes 32 samples per pass, lane (n, g) works for sample b0 + n on the levels l(j, g)
+// level-major gather: features into the SDF net's input rows, slopes as fp16
 // ----------------------------------------------------------------------------
-template <bool FULL>
+constexpr uint32_t FG_BLOCK = 256;
+
+__global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
+	const uint32_t level = blockIdx.x / tiles, i = (blockIdx.x - level * tiles) * FG_BLOCK + threadIdx.x;
+	const uint32_t N = a.N;
+	if (i >= N) return;
+	const float* q = a.coords + (size_t)i * 7;
+	const float p[3] = {q[0], q[1], q[2]};
+	if (level == 0) {
+#pragma unroll
+		for (int d = 0; d < 3; ++d) {
+			a.sdf_in[(size_t)d * N + i] = (hf)p[d] - (hf)0.5f;
+			a.xyz_rows[(size_t)d * N + i] = p[d];
+		}
+	}
+	float feat[2] = {0.f, 0.f}, J[2][3] = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+	if (level < a.lv.active_levels) {  // a switched-off level: zero features, zero slopes
+		LaneLevel L;
+		L.scale = a.lv.scale[level]; L.res = a.lv.res[level]; L.entries = a.lv.entries[level]; L.offset = a.lv.offset[level];
+		L.hashed = (a.lv.hash_mask >> level) & 1u;
+		Item it;
+		uint32_t c[3], boff[8];
+#pragma unroll
+		for (int d = 0; d < 3; ++d) n2_locate(p[d], L.scale, it.w[d], c[d]);
+		it.scale = 1.f;  // slopes are stored without the level's scale factor
+		if (L.hashed) corner_offsets<1>(L, c, boff);
+		else corner_offsets<0>(L, c, boff);
+		const char* base = reinterpret_cast<const char*>(a.table);
+#pragma unroll
+		for (int k = 0; k < 8; ++k) it.raw[k] = *reinterpret_cast<const uint32_t*>(base + boff[k]);
+		item_finish<true>(it, feat, J);
+	}
+	a.sdf_in[(size_t)(3 + 2 * level) * N + i] = (hf)feat[0];
+	a.sdf_in[(size_t)(4 + 2 * level) * N + i] = (hf)feat[1];
+	const float six[6] = {J[0][0], J[0][1], J[0][2], J[1][0], J[1][1], J[1][2]};
+	a.slopes[(size_t)level * N + i] = n2_slopes_pack(six);
+}
+
+// ----------------------------------------------------------------------------
+// the network kernel: a wave takes 32 samples per pass, lane (n, g) works for sample b0 + n on the levels l(j, g).
+// GATHER: the features come from the table (inference); else from the rows the gather kernel wrote.
+// ----------------------------------------------------------------------------
+template <bool FULL, bool GATHER>
 __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const FusedArgs a) {
+	static_assert(FULL != GATHER, "the full forward reads the gather kernel's rows, inference gathers itself");
 	extern __shared__ __align__(16) unsigned char smem[];
 	hf* F = reinterpret_cast<hf*>(smem);
 	uint4* LV = reinterpret_cast<uint4*>(smem + (size_t)(FULL ? FF_COUNT : FF_SDF_COUNT) * 1024);
@@ -267,28 +317,22 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 		const uint32_t col_raw = tile * 32u + n;
 		const bool valid = col_raw < N;
 		const uint32_t col = valid ? col_raw : N - 1u;
-		// position (and direction) of the lane's sample
+		half8 xs[3];               // SDF net input, B operands
 		float p[3], dir[3] = {0.f, 0.f, 0.f};
-		if (FULL) {
-			const float* q = a.coords + (size_t)col * 7;
-#pragma unroll
-			for (int d = 0; d < 3; ++d) { p[d] = q[d]; dir[d] = q[4 + d]; }
-		} else {
+		uint4 slope[8];            // FULL: the slopes of the lane's 8 levels as stored
+		if (GATHER) {
 			const float* q = a.pos + (size_t)col * a.ps;
 #pragma unroll
 			for (int d = 0; d < 3; ++d) p[d] = q[(size_t)d * a.ds];
-		}
-		// ---- gather: the lane's 8 levels, the next level's loads in flight while one is finished ----
-		half8 xs[3];        // SDF net input, B operands
-		float Jm[8][2][3];  // [step][feature][dimension]
-		{
+			// the lane's 8 levels, the next level's loads in flight while one is finished
 			Item cur, nxt;
+			float unused[2][3];
 			item_fetch<0>(LV, hash_mask, active, a.table, g, p, cur);
 #define FF_STEP(J)                                                                           \
 			if (J < 7) item_fetch<(J < 7 ? J + 1 : 0)>(LV, hash_mask, active, a.table, g, p, nxt); \
 			{                                                                                \
 				float feat[2];                                                               \
-				item_finish<FULL>(cur, feat, Jm[J]);                                         \
+				item_finish<false>(cur, feat, unused);                                       \
 				xs[J >> 2][2 * (J & 3)] = (hf)feat[0];                                       \
 				xs[J >> 2][2 * (J & 3) + 1] = (hf)feat[1];                                   \
 			}                                                                                \
@@ -296,34 +340,24 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 			__builtin_amdgcn_sched_barrier(0);
 			FF_STEP(0) FF_STEP(1) FF_STEP(2) FF_STEP(3) FF_STEP(4) FF_STEP(5) FF_STEP(6) FF_STEP(7)
 #undef FF_STEP
-			xs[2] = zero8();
-			if (g == 0) {
+		} else {
+			const float* q = a.coords + (size_t)col * 7;
 #pragma unroll
-				for (int d = 0; d < 3; ++d) xs[2][d] = (hf)p[d] - (hf)0.5f;
-			}
-		}
-		if (FULL && valid) {
-			// what the backward pass reads of the encoding: features, Jacobian, positions
+			for (int d = 0; d < 3; ++d) { p[d] = q[d]; dir[d] = q[4 + d]; }
 #pragma unroll
 			for (int j = 0; j < 8; ++j) {
 				const uint32_t level = 4u * (j >> 1) + 2u * g + (j & 1);
-				if (2u * level < a.enc_w) {
-#pragma unroll
-					for (int f = 0; f < 2; ++f) {
-						const size_t row = 2u * level + f;
-						a.sdf_in[(3 + row) * N + col] = xs[j >> 2][2 * (j & 3) + f];
-						float* q = a.dy_dx + (row * N + col) * 3;
-						q[0] = Jm[j][f][0]; q[1] = Jm[j][f][1]; q[2] = Jm[j][f][2];
-					}
-				}
+				// levels the grid does not have read level 0's rows and are ignored (their weights are zero)
+				const uint32_t lr = 2u * level < a.enc_w ? level : 0u;
+				xs[j >> 2][2 * (j & 3)] = a.sdf_in[(size_t)(3 + 2 * lr) * N + col];
+				xs[j >> 2][2 * (j & 3) + 1] = a.sdf_in[(size_t)(4 + 2 * lr) * N + col];
+				slope[j] = a.slopes[(size_t)lr * N + col];
 			}
-			if (g == 0) {
+		}
+		xs[2] = zero8();
+		if (g == 0) {
 #pragma unroll
-				for (int d = 0; d < 3; ++d) {
-					a.sdf_in[(size_t)d * N + col] = xs[2][d];
-					a.xyz_rows[(size_t)d * N + col] = p[d];
-				}
-			}
+			for (int d = 0; d < 3; ++d) xs[2][d] = (hf)p[d] - (hf)0.5f;
 		}
 		const size_t off4 = (size_t)4u * g * N + col;
 		// ---- SDF net ----
@@ -377,10 +411,14 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 #pragma unroll
 		for (int d = 0; d < 3; ++d) nrm[d] = g == 0 ? (float)gx[d] : 0.f;
 #pragma unroll
-		for (int r = 0; r < 16; ++r) {
-			const float gv = (float)(r < 8 ? g_lo[r] : g_hi[r - 8]);
+		for (int j = 0; j < 8; ++j) {
+			const uint32_t level = 4u * (j >> 1) + 2u * g + (j & 1);
+			const float sc = 2u * level < a.enc_w ? __uint_as_float(LV[level].x) : 0.f;
+			float q[6];
+			const float unit = n2_slopes_unpack(slope[j], q) * sc;
+			const float g0 = (float)(j < 4 ? g_lo[2 * j] : g_hi[2 * j - 8]) * unit, g1 = (float)(j < 4 ? g_lo[2 * j + 1] : g_hi[2 * j - 7]) * unit;
 #pragma unroll
-			for (int d = 0; d < 3; ++d) nrm[d] = fmaf(gv, Jm[r >> 1][r & 1][d], nrm[d]);
+			for (int d = 0; d < 3; ++d) nrm[d] = fmaf(g0, q[d], fmaf(g1, q[3 + d], nrm[d]));
 		}
 #pragma unroll
 		for (int d = 0; d < 3; ++d) nrm[d] += __shfl_xor(nrm[d], 32);
@@ -495,16 +533,19 @@ static FusedArgs fused_base(const N2FusedNets& nets, uint32_t n) {
 }
 
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           float* dy_dx, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output) {
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output) {
 	FusedArgs a = fused_base(nets, n);
 	a.coords = d_coords;
 	a.sdf_in = reinterpret_cast<hf*>(sdf_in);
 	a.xyz_rows = xyz_rows;
-	a.dy_dx = dy_dx;
+	a.slopes = reinterpret_cast<uint4*>(slopes);
 	a.dsdf_din = reinterpret_cast<hf*>(dsdf_din);
 	a.rgb_in = reinterpret_cast<hf*>(rgb_in);
 	a.output = reinterpret_cast<hf*>(d_output);
-	field_fused_forward_kernel<true><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT), s>>>(a);
+	const uint32_t tiles = (n + FG_BLOCK - 1) / FG_BLOCK;
+	field_gather_kernel<<<dim3(tiles * nets.tab->n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
+	N2_LAUNCH_CHECK();
+	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
@@ -516,7 +557,7 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 	a.sdf_out = reinterpret_cast<hf*>(d_out_soa);
 	a.row0 = d_row0;
 	a.density = density ? 1 : 0;
-	field_fused_forward_kernel<false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
+	field_fused_forward_kernel<false, true><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -43,3 +43,44 @@ __device__ __forceinline__ uint32_t n2_entry(uint32_t entries, uint32_t res, uin
 	}
 }
 
+
+// ----------------------------------------------------------------------------
+// Slopes of one (sample, level): the six values d feature_f / d x_d (before the level's scale factor) as one 16-byte
+// block-float: 20-bit signed mantissas q_0..q_5 and a shared exponent e (value_i = q_i * 2^(e - 19), |value_i| < 2^e).
+// The contraction of the slopes with a gradient then carries an error of 2^-20 of the largest slope, where fp16 storage
+// (2^-11 of every slope) shows in the normals; fp32 storage takes 24 bytes.
+//   word 0: q0 | q1 << 20     word 1: q1 >> 12 | q2 << 8 | q3 << 28     word 2: q3 >> 4 | q4 << 16
+//   word 3: q4 >> 16 | q5 << 4 | e << 24
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ uint4 n2_slopes_pack(const float (&v)[6]) {
+	float m = 0.f;
+#pragma unroll
+	for (int i = 0; i < 6; ++i) m = fmaxf(m, fabsf(v[i]));
+	int e = 0;
+	(void)frexpf(m, &e);  // m = f * 2^e with f in [0.5, 1); 0 for m = 0
+	e = min(max(e, -100), 100);
+	uint32_t q[6];
+#pragma unroll
+	for (int i = 0; i < 6; ++i) {
+		int x = (int)rintf(ldexpf(v[i], 19 - e));
+		x = min(max(x, -524287), 524287);
+		q[i] = (uint32_t)x & 0xFFFFFu;
+	}
+	uint4 w;
+	w.x = q[0] | (q[1] << 20);
+	w.y = (q[1] >> 12) | (q[2] << 8) | (q[3] << 28);
+	w.z = (q[3] >> 4) | (q[4] << 16);
+	w.w = (q[4] >> 16) | (q[5] << 4) | ((uint32_t)e << 24);
+	return w;
+}
+// mantissas as floats and the factor 2^(e - 19) they share
+__device__ __forceinline__ float n2_slopes_unpack(const uint4 w, float (&q)[6]) {
+	auto sext20 = [](uint32_t x) { return (float)((int32_t)(x << 12) >> 12); };
+	q[0] = sext20(w.x);
+	q[1] = sext20((w.x >> 20) | (w.y << 12));
+	q[2] = sext20(w.y >> 8);
+	q[3] = sext20((w.y >> 28) | (w.z << 4));
+	q[4] = sext20((w.z >> 16) | (w.w << 16));
+	q[5] = sext20(w.w >> 4);
+	return ldexpf(1.f, ((int32_t)w.w >> 24) - 19);
+}

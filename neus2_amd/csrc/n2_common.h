@@ -82,10 +82,11 @@ uint32_t n2_mlp_hidden_layers(const n2_mlp_t* mlp);
 // The fused forward serves grids of at most 16 levels with two features whose levels are dense or hashed with a
 // power-of-two table, one hidden layer in the SDF net and two in the colour net, without per-point level masks.
 bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uint32_t rgb_hidden_layers);
-// NerfNetwork::forward_impl in one kernel: writes the network inputs, the Jacobian of the encoding, d sdf / d input
-// (SoA, n columns) and the [n][16] output.
+// NerfNetwork::forward_impl as a level-major gather kernel plus one kernel for everything behind it: writes the network
+// inputs and d sdf / d input (SoA, n columns), the slopes of the encoding (16 bytes per level and sample, [n_levels][n]:
+// d feature / d position without the level's scale factor, n2_slopes_pack) and the [n][16] output.
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           float* dy_dx, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output);
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output);
 // NerfNetwork::sdf / density in one kernel: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
                        float* d_row0, bool density);
