@@ -1,7 +1,6 @@
 // Training-sample generator: pixel pick, ray / unit-cube intersection and the
-// march through the occupancy bitfield.  One thread per ray (a ray is a serial,
-// data-dependent walk); three kernels: count steps, exclusive scan in ray order,
-// emit coordinates.
+// march through the occupancy bitfield.  One wave per ray (see march_wave); three
+// kernels: march and count, exclusive scan in ray order, emit coordinates.
 //
 // Sample positions are part of the bit-exact contract with the CPU oracle, so
 // floating-point contraction is switched off for this file and every fused
@@ -12,10 +11,6 @@
 
 constexpr float STEP = 1.73205080757f / 1024.f;  // STEPSIZE(), src/testbed_nerf.cu:51-53
 constexpr uint32_t GRIDSIZE = 128, MARCH_STEPS = 1024;
-// One lane per ray: a few thousand lanes that mostly wait for memory.  Small workgroups spread them over many CUs (packed
-// onto a few CUs the rays slow each other down by a fifth and the generator no longer hides behind a training step).
-constexpr uint32_t SAMPLER_BLOCK = 128;
-
 __device__ __forceinline__ uint32_t hash_u32(uint32_t seed, uint32_t ctr) {
 	uint32_t x = ctr * 747796405u + seed * 2891336453u + 1u;
 	x = ((x >> ((x >> 28) + 4u)) ^ x) * 277803737u;
@@ -113,52 +108,102 @@ __device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint3
 
 // The march of one ray, as the reference writes it: t_0 = startt, every visited step adds STEP to t; at an occupied
 // step a sample is emitted, at an empty one the steps below t + to_next_voxel(pos) are skipped without being looked at;
-// the ray ends at the first visited step outside the unit cube or after MARCH_STEPS samples.  Every visited step costs
-// a dependent read of the bitfield, so the walk is done ONCE: it returns the number of samples and records which
-// steps (counted in additions of STEP) emitted one, as a bit mask of MASK_WORDS words kept word-major
-// (mask[word * n_rays + ray]).  The coordinates are written later from the mask, without touching the bitfield.
-// A ray inside the unit cube is at most sqrt(3) long, i.e. MARCH_STEPS steps plus the start jitter.
-constexpr uint32_t MASK_WORDS = 34, MASK_BITS = MASK_WORDS * 32;
+// the ray ends at the first visited step outside the unit cube or after MARCH_STEPS samples.  One lane per ray makes
+// that a chain of dependent bitfield reads (0.4 us per step, a few thousand lanes on the whole GPU).  Here a WAVE owns a
+// ray and looks at 64 consecutive steps at once: every lane forms its own t, position, occupancy bit and skip target
+// with the serial form's arithmetic, and the wave then replays the serial decisions on the ballots (which steps are
+// visited, which emit, where the ray ends).  The result is the serial one bit for bit; the bitfield latency is paid
+// once per 64 steps.  The march runs once: it records which steps emitted (64 bits per window) and the t of every
+// window's first step; the coordinates are written afterwards from those, without touching the bitfield.
+constexpr uint32_t WINDOWS = 17;                      // 1088 steps: a ray inside the unit cube is at most sqrt(3) long,
+constexpr uint32_t MASK_BITS = WINDOWS * 64;          // i.e. MARCH_STEPS steps plus the start jitter
+constexpr uint32_t RAYS_PER_BLOCK = 4;                // one wave per ray
 
-__device__ __forceinline__ uint32_t march_and_mark(const RaySetup& r, const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ mask,
-                                                   uint32_t ray, uint32_t n_rays) {
-	uint32_t j = 0, k = 0, word = 0, widx = 0;
-	float t = r.startt;
-	while (j < MARCH_STEPS && k < MASK_BITS) {
+// t of this lane's step: t_first plus `lane` additions of STEP, one at a time like the serial march.  Inside a binade
+// [2^e, 2^(e+1)) every such addition moves t by the same amount d_e = (2^e + STEP) - 2^e: t is a multiple of the
+// binade's ulp and STEP's remainder below that ulp rounds the same way each time (STEP has no tie in any binade
+// above 2^-8), so t_k = t_0 + k d_e exactly, as long as the binade is not left.  64 steps are shorter than any binade
+// from 2^-3 up, so a window crosses at most one boundary: the lanes behind it continue from the one real addition that
+// crosses it with the next binade's increment.  Below 2^-3 (a camera inside the volume) the additions are done one by one.
+// Must be called by all 64 lanes.
+__device__ __forceinline__ float window_t(float t_first, uint32_t lane) {
+	if (!(t_first >= 0.125f && t_first < 1e30f)) {
+		float t = t_first;
+		for (uint32_t a = 0; a < lane; ++a) t += STEP;
+		return t;
+	}
+	const float lo = __uint_as_float(__float_as_uint(t_first) & 0x7F800000u), hi = lo + lo;
+	const float d1 = (lo + STEP) - lo, d2 = (hi + STEP) - hi;
+	const float x = __fmaf_rn((float)lane, d1, t_first);  // exact below hi; at or above hi only the comparison is used
+	const unsigned long long below = __ballot(x < hi);     // lanes 0 .. kc-1 (lane 0 always)
+	const uint32_t kc = (uint32_t)__popcll(below);
+	if (kc == 64u) return x;
+	const float t_cross = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)kc - 1)) + STEP;
+	return lane < kc ? x : __fmaf_rn((float)(lane - kc), d2, t_cross);
+}
+
+// Returns the number of samples; mask[2 w], mask[2 w + 1]: which steps of window w emitted; t_first[w]: t of its first step.
+__device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ mask,
+                                               float* __restrict__ t_first_out) {
+	const uint32_t lane = threadIdx.x & 63u;
+	uint32_t j = 0;
+	float t_first = r.startt;  // t of the window's first step
+	float pending = -3.4e38f;  // steps with t below this are skipped (target of the last visited empty step)
+	for (uint32_t w = 0; w < WINDOWS; ++w) {
+		const float t = window_t(t_first, lane);
 		float pos[3];
 #pragma unroll
-		for (int d = 0; d < 3; ++d) pos[d] = __fmaf_rn(t, r.dir[d], r.o[d]);
-		if (!(pos[0] >= 0.f && pos[0] <= 1.f && pos[1] >= 0.f && pos[1] <= 1.f && pos[2] >= 0.f && pos[2] <= 1.f)) break;
-		if (occupied(bitfield, pos)) {
-			while ((k >> 5) != widx) {  // words that are complete
-				mask[(size_t)widx * n_rays + ray] = word;
-				word = 0;
-				++widx;
+		for (int k = 0; k < 3; ++k) pos[k] = __fmaf_rn(t, r.dir[k], r.o[k]);
+		const bool inside = pos[0] >= 0.f && pos[0] <= 1.f && pos[1] >= 0.f && pos[1] <= 1.f && pos[2] >= 0.f && pos[2] <= 1.f;
+		const bool occ = inside && occupied(bitfield, pos);
+		const float target = t + to_next_voxel(pos, r.dir, r.idir);
+		const unsigned long long m_inside = __ballot(inside), m_occ = __ballot(occ);
+		// replay the serial walk over this window (all values below are the same in every lane)
+		unsigned long long emit = 0;
+		bool done = false;
+		const unsigned long long reach = __ballot(t >= pending);  // steps not skipped by the pending target
+		uint32_t cur = reach ? (uint32_t)__ffsll((long long)reach) - 1u : 64u;
+		while (cur < 64u) {
+			if (!((m_inside >> cur) & 1ull)) { done = true; break; }
+			if ((m_occ >> cur) & 1ull) {
+				// a run of occupied steps: each emits and moves on by one step
+				const unsigned long long rest = ~(m_occ >> cur);
+				uint32_t run = rest ? (uint32_t)__ffsll((long long)rest) - 1u : 64u - cur;
+				if (run > 64u - cur) run = 64u - cur;
+				if (run > MARCH_STEPS - j) run = MARCH_STEPS - j;
+				emit |= (run == 64u ? ~0ull : ((1ull << run) - 1ull)) << cur;
+				j += run;
+				cur += run;
+				if (j >= MARCH_STEPS) { done = true; break; }
+			} else {
+				// an empty step: the next visited step is the first later one whose t reaches its target
+				pending = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(target), (int)cur));
+				const unsigned long long later = __ballot(t >= pending) & (cur == 63u ? 0ull : (~0ull << (cur + 1u)));
+				// the serial form always moves on by at least one step
+				cur = later ? (uint32_t)__ffsll((long long)later) - 1u : 64u;
 			}
-			word |= 1u << (k & 31u);
-			++j;
-			t += STEP;
-			++k;
-		} else {
-			const float t_target = t + to_next_voxel(pos, r.dir, r.idir);
-			do { t += STEP; ++k; } while (t < t_target);
 		}
-	}
-	for (; widx < MASK_WORDS; ++widx) {
-		mask[(size_t)widx * n_rays + ray] = word;
-		word = 0;
+		if (lane == 0) {
+			mask[2 * w] = (uint32_t)emit;
+			mask[2 * w + 1] = (uint32_t)(emit >> 32);
+			t_first_out[w] = t_first;
+		}
+		if (done) break;
+		// next window starts one step after this window's last one
+		t_first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 63)) + STEP;
 	}
 	return j;
 }
 
-__global__ void __launch_bounds__(SAMPLER_BLOCK) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+__global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                             uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
                                                             const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts,
-                                                            uint32_t* __restrict__ mask) {
-	const uint32_t i = blockIdx.x * SAMPLER_BLOCK + threadIdx.x;
+                                                            uint32_t* __restrict__ mask, float* __restrict__ t_first) {
+	const uint32_t i = blockIdx.x * RAYS_PER_BLOCK + (threadIdx.x >> 6);
 	if (i >= n_rays) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
-	counts[i] = r.alive ? march_and_mark(r, bitfield, mask, i, n_rays) : 0u;
+	const uint32_t n = r.alive ? march_wave(r, bitfield, mask + (size_t)i * 2 * WINDOWS, t_first + (size_t)i * WINDOWS) : 0u;
+	if ((threadIdx.x & 63u) == 0) counts[i] = n;
 }
 
 // base[i] = exclusive sum of counts; slot[i] = rank among rays that have samples and fit the budget
@@ -200,51 +245,51 @@ __global__ void __launch_bounds__(1024) sampler_scan_kernel(uint32_t n_rays, uin
 	if (threadIdx.x == 0) { *ray_counter = carry_b; *sample_counter = carry_a; }
 }
 
-// Coordinates of the samples the march marked: step k of a ray lies at startt + k additions of STEP (the same
-// additions the march made), so the walk is replayed on t alone.
-__global__ void __launch_bounds__(SAMPLER_BLOCK) sampler_emit_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
+// Coordinates of the samples the march marked, one wave per ray: lane l of window w is the step at t_first[w] plus l
+// additions of STEP, formed exactly as in the march.
+__global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_emit_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                            uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
-                                                           const uint32_t* __restrict__ mask, const uint32_t* __restrict__ counts,
+                                                           const uint32_t* __restrict__ mask, const float* __restrict__ t_first,
+                                                           const uint32_t* __restrict__ counts,
                                                            const uint32_t* __restrict__ base, const uint32_t* __restrict__ slot,
                                                            uint32_t* __restrict__ ray_indices, uint32_t* __restrict__ numsteps,
                                                            float* __restrict__ rgb_target, float* __restrict__ coords) {
-	const uint32_t i = blockIdx.x * SAMPLER_BLOCK + threadIdx.x;
+	const uint32_t i = blockIdx.x * RAYS_PER_BLOCK + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
 	if (i >= n_rays) return;
 	const uint32_t s = slot[i];
 	if (s == 0xFFFFFFFFu) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
-	const uint32_t n = counts[i];
-	ray_indices[s] = i;
-	numsteps[2 * s] = n;
-	numsteps[2 * s + 1] = base[i];
-	rgb_target[(size_t)s * 3 + 0] = r.target[0];
-	rgb_target[(size_t)s * 3 + 1] = r.target[1];
-	rgb_target[(size_t)s * 3 + 2] = r.target[2];
-	float* c = coords + (size_t)base[i] * 7;
+	const uint32_t n = counts[i], first = base[i];
+	if (lane == 0) {
+		ray_indices[s] = i;
+		numsteps[2 * s] = n;
+		numsteps[2 * s + 1] = first;
+		rgb_target[(size_t)s * 3 + 0] = r.target[0];
+		rgb_target[(size_t)s * 3 + 1] = r.target[1];
+		rgb_target[(size_t)s * 3 + 2] = r.target[2];
+	}
 	const float d0 = (r.dir[0] + 1.0f) * 0.5f, d1 = (r.dir[1] + 1.0f) * 0.5f, d2 = (r.dir[2] + 1.0f) * 0.5f;
-	float t = r.startt;
+	const uint32_t* m = mask + (size_t)i * 2 * WINDOWS;
 	uint32_t j = 0;
-	for (uint32_t w = 0; w < MASK_WORDS && j < n; ++w) {
-		uint32_t bits = mask[(size_t)w * n_rays + i];
-		for (uint32_t b = 0; b < 32u; ++b) {
-			if (bits & 1u) {
-				c[0] = __fmaf_rn(t, r.dir[0], r.o[0]);
-				c[1] = __fmaf_rn(t, r.dir[1], r.o[1]);
-				c[2] = __fmaf_rn(t, r.dir[2], r.o[2]);
-				c[3] = 0.0f;
-				c[4] = d0; c[5] = d1; c[6] = d2;
-				c += 7;
-				++j;
-			}
-			bits >>= 1;
-			t += STEP;
+	for (uint32_t w = 0; w < WINDOWS && j < n; ++w) {
+		const unsigned long long bits = (unsigned long long)m[2 * w] | ((unsigned long long)m[2 * w + 1] << 32);
+		if (bits == 0ull) continue;  // uniform: the whole wave skips the window
+		const float t = window_t(t_first[(size_t)i * WINDOWS + w], lane);
+		if ((bits >> lane) & 1ull) {
+			float* c = coords + (size_t)(first + j + (uint32_t)__popcll(bits & ((1ull << lane) - 1ull))) * 7;
+			c[0] = __fmaf_rn(t, r.dir[0], r.o[0]);
+			c[1] = __fmaf_rn(t, r.dir[1], r.o[1]);
+			c[2] = __fmaf_rn(t, r.dir[2], r.o[2]);
+			c[3] = 0.0f;
+			c[4] = d0; c[5] = d1; c[6] = d2;
 		}
+		j += (uint32_t)__popcll(bits);
 	}
 }
 
 static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
 
-N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays) + up256(4ull * MASK_WORDS * max_rays); }
+N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays) + 2 * up256(4ull * 2 * WINDOWS * max_rays); }
 
 N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
                                         const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
@@ -269,15 +314,16 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	uint32_t* base = reinterpret_cast<uint32_t*>(w + up256(4ull * n_rays));
 	uint32_t* slot = reinterpret_cast<uint32_t*>(w + 2 * up256(4ull * n_rays));
 	uint32_t* mask = reinterpret_cast<uint32_t*>(w + 3 * up256(4ull * n_rays));
-	const dim3 grid((n_rays + SAMPLER_BLOCK - 1) / SAMPLER_BLOCK), block(SAMPLER_BLOCK);
+	float* t_first = reinterpret_cast<float*>(w + 3 * up256(4ull * n_rays) + up256(4ull * 2 * WINDOWS * n_rays));
+	const dim3 grid((n_rays + RAYS_PER_BLOCK - 1) / RAYS_PER_BLOCK), block(64 * RAYS_PER_BLOCK);
 	N2ProfScope prof(N2_PROF_SAMPLER, s);
 	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                            background[2], d_bitfield, counts, mask);
+	                                            background[2], d_bitfield, counts, mask, t_first);
 	N2_LAUNCH_CHECK();
 	sampler_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples, counts, base, slot, d_ray_counter, d_sample_counter);
 	N2_LAUNCH_CHECK();
 	sampler_emit_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                           background[2], mask, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
+	                                           background[2], mask, t_first, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }
