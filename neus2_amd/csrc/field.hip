@@ -29,7 +29,7 @@ struct n2_field {
 	uint32_t max_batch, max_batch_bwd;
 	// Batch size for which the padding rows of each input-side matrix of the two networks hold zeros (0: not known).
 	// The matrices are rows x N with N the batch size of the call, so the padding rows move when N changes.
-	struct { uint32_t sdf_in, rgb_in, sel_sdf_in, sel_rgb_in, d_density_in; } pad_n;
+	struct { uint32_t sdf_in, rgb_in, d_density_in; } pad_n;
 	// carved from the workspace
 	hf* sdf_in;        // [sdf_in_w][N]
 	float* xyz;        // [3][N]  positions of the last forward, row per coordinate (the grid kernels read each row 16 times)
@@ -41,14 +41,10 @@ struct n2_field {
 	float* v;          // [3][N]  dL / d normal
 	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
 	float* var_part;    // one partial sum of the variance gradient per workgroup of the backward's preparation kernel
-	// a selection of the last forward's samples (n2_field_select), read by the backward instead of the rows above
-	hf* sel_sdf_in;       // [sdf_in_w][n]
-	hf* sel_rgb_in;       // [48][n]
-	hf* sel_dsdf_denc;    // [enc_w][n]  rows 3 .. 3 + enc_w of dsdf_din
-	float* sel_xyz;       // [3][n]
+	// a selection of the last forward's samples (n2_field_select): the backward reads the rows above through this index
 	uint32_t* sel_index;  // [n]
 	uint32_t last_n;      // samples of the last forward
-	uint32_t sel_n;       // samples selected (0: the backward reads the forward's own rows)
+	uint32_t sel_n;       // samples selected (0: the backward's batch is the forward's)
 	void* ws_sdf;
 	void* ws_rgb;
 	void* ws_grid;
@@ -277,54 +273,11 @@ __global__ void __launch_bounds__(VB) field_variance_gradient_kernel(const float
 	}
 }
 
-// out[r][j] = in[r][index[j]] for the rows the backward reads; blockIdx.y picks a group of 8 fp16 rows (SDF-net input,
-// colour-net input, encoding rows of d sdf / d input) or, last, the three fp32 position rows.  Two samples per thread so
-// that the stores move pairs.
-__global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n_src, const uint32_t* __restrict__ index, uint32_t sdf_rows,
-                                                          uint32_t rgb_rows, uint32_t enc_w, const hf* __restrict__ sdf_in,
-                                                          const hf* __restrict__ rgb_in, const hf* __restrict__ dsdf_din,
-                                                          const float* __restrict__ xyz, hf* __restrict__ o_sdf_in, hf* __restrict__ o_rgb_in,
-                                                          hf* __restrict__ o_denc, float* __restrict__ o_xyz, uint32_t* __restrict__ o_index) {
-	typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-	const uint32_t j = (blockIdx.x * FB + threadIdx.x) * 2;
-	if (j >= n) return;
-	const bool two = j + 1 < n;
-	const uint32_t s0 = min(index[j], n_src - 1u), s1 = two ? min(index[j + 1], n_src - 1u) : s0;
-	const uint32_t groups_a = (sdf_rows + 7) / 8, groups_b = (rgb_rows + 7) / 8, groups_c = (enc_w + 7) / 8;
-	uint32_t g = blockIdx.y, rows;  // rows of this group (the last group of a matrix may be short)
-	const hf* in;
-	hf* out;
-	if (g < groups_a) { in = sdf_in + (size_t)g * 8 * n_src; out = o_sdf_in + (size_t)g * 8 * n; rows = min(8u, sdf_rows - g * 8); }
-	else if ((g -= groups_a) < groups_b) { in = rgb_in + (size_t)g * 8 * n_src; out = o_rgb_in + (size_t)g * 8 * n; rows = min(8u, rgb_rows - g * 8); }
-	else if ((g -= groups_b) < groups_c) { in = dsdf_din + (size_t)(3 + g * 8) * n_src; out = o_denc + (size_t)g * 8 * n; rows = min(8u, enc_w - g * 8); }
-	else {
-#pragma unroll
-		for (int d = 0; d < 3; ++d) {
-			o_xyz[(size_t)d * n + j] = xyz[(size_t)d * n_src + s0];
-			if (two) o_xyz[(size_t)d * n + j + 1] = xyz[(size_t)d * n_src + s1];
-		}
-		o_index[j] = s0;
-		if (two) o_index[j + 1] = s1;
-		return;
-	}
-	hf a[8], b[8];
-#pragma unroll
-	for (uint32_t r = 0; r < 8; ++r) {
-		if (r < rows) { a[r] = in[(size_t)r * n_src + s0]; b[r] = in[(size_t)r * n_src + s1]; }
-	}
-	if (two && (n & 1u) == 0) {
-#pragma unroll
-		for (uint32_t r = 0; r < 8; ++r)
-			if (r < rows) *reinterpret_cast<half2v*>(out + (size_t)r * n + j) = half2v{a[r], b[r]};
-	} else {
-#pragma unroll
-		for (uint32_t r = 0; r < 8; ++r) {
-			if (r < rows) {
-				out[(size_t)r * n + j] = a[r];
-				if (two) out[(size_t)r * n + j + 1] = b[r];
-			}
-		}
-	}
+// The selection of a backward batch among the forward's samples: the index is copied (clamped into the forward's batch)
+// so that the caller's buffer is free again; the backward kernels read the saved rows through it.
+__global__ void __launch_bounds__(FB) field_select_kernel(uint32_t n, uint32_t n_src, const uint32_t* __restrict__ index, uint32_t* __restrict__ o_index) {
+	const uint32_t j = blockIdx.x * FB + threadIdx.x;
+	if (j < n) o_index[j] = min(index[j], n_src - 1u);
 }
 
 __global__ void __launch_bounds__(FB) field_add_bias_kernel(uint32_t N, hf bias, hf* __restrict__ row0) {
@@ -416,7 +369,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_sdf_in, sel_rgb_in, sel_dsdf_denc, sel_xyz, sel_index, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_index, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -436,10 +389,6 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.v = take(12ull * n);
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
 	c.var_part = take(4ull * ((n + FB - 1) / FB + 1));
-	c.sel_sdf_in = take(2ull * f->sdf_in_w * n);
-	c.sel_rgb_in = take(2ull * f->rgb_in_w * n);
-	c.sel_dsdf_denc = take(2ull * f->enc_w * n);
-	c.sel_xyz = take(12ull * n);
 	c.sel_index = take(4ull * n);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
@@ -473,14 +422,10 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->v = reinterpret_cast<float*>(b + c.v);
 	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
 	f->var_part = reinterpret_cast<float*>(b + c.var_part);
-	f->sel_sdf_in = reinterpret_cast<hf*>(b + c.sel_sdf_in);
-	f->sel_rgb_in = reinterpret_cast<hf*>(b + c.sel_rgb_in);
-	f->sel_dsdf_denc = reinterpret_cast<hf*>(b + c.sel_dsdf_denc);
-	f->sel_xyz = reinterpret_cast<float*>(b + c.sel_xyz);
 	f->sel_index = reinterpret_cast<uint32_t*>(b + c.sel_index);
 	f->last_n = 0;
 	f->sel_n = 0;
-	f->pad_n = {0, 0, 0, 0, 0};
+	f->pad_n = {0, 0, 0};
 	f->ws_sdf = b + c.ws_sdf;
 	f->ws_rgb = b + c.ws_rgb;
 	f->ws_grid = b + c.ws_grid;
@@ -573,13 +518,12 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	const bool sel = f->sel_n != 0;
 	N2_REQUIRE(n == (sel ? f->sel_n : f->last_n), "n2_field_backward: batch %u, but the last %s was over %u samples", n,
 	           sel ? "n2_field_select" : "n2_field_forward", sel ? f->sel_n : f->last_n);
-	const hf* sdf_in = sel ? f->sel_sdf_in : f->sdf_in;
-	const hf* rgb_in = sel ? f->sel_rgb_in : f->rgb_in;
-	const hf* dsdf_denc = sel ? f->sel_dsdf_denc : f->dsdf_din + (size_t)3 * n;
-	const float* xyz = sel ? f->sel_xyz : f->xyz;
+	// with a selection, sample i of the batch is column index[i] of the rows the forward saved over its n_src samples
+	const uint32_t* index = sel ? f->sel_index : nullptr;
+	const uint32_t n_src = f->last_n;
 	// colour net: only rows 0..2 of dL_doutput belong to it
-	if (int rc = n2_mlp_backward_rows(f->rgb, stream, reinterpret_cast<const n2_half*>(rgb_in), n, d_dL_doutput, N2_LAYOUT_AOS, 3,
-	                                  reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
+	if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
+	                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
 	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
 	if (int rc = zero_padding(s, f->d_density_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.d_density_in)) return rc;
 	LevelScales scales{};
@@ -595,13 +539,13 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_LAUNCH_CHECK();
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient; the second-order pass through the
 	// net (the reference's backward_backward_input with Accumulate) rides along
-	if (int rc = n2_mlp_backward_and_second_order(f->sdf, stream, reinterpret_cast<const n2_half*>(sdf_in), n, reinterpret_cast<const n2_half*>(f->d_rgb_in),
-	                                              N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in), reinterpret_cast<const n2_half*>(f->d_density_in),
-	                                              nullptr, mode)) return rc;
+	if (int rc = n2_mlp_backward_and_second_order_indexed(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n_src, index, n,
+	                                                      reinterpret_cast<const n2_half*>(f->d_rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in),
+	                                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, mode)) return rc;
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)
-	if (int rc = n2_grid_backward_fused(f->grid, stream, xyz, 1, n, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
-	                                    reinterpret_cast<const n2_half*>(dsdf_denc), nullptr, mode)) return rc;
+	if (int rc = n2_grid_backward_fused_indexed(f->grid, stream, f->xyz, n_src, index, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
+	                                            reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n_src), mode)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
 	// pending: one launch sums them
 	return n2_mlp_reduce_deferred(f->rgb, f->sdf, stream);
@@ -613,13 +557,7 @@ N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_
 	N2_REQUIRE(n_source == f->last_n && n_source > 0, "n2_field_select: n_source %u, but the last n2_field_forward was over %u samples", n_source,
 	           f->last_n);
 	N2_REQUIRE(n > 0 && d_source_index != nullptr, "n2_field_select: empty selection");
-	const uint32_t sdf_rows = 3 + f->enc_w;  // the padding rows above are not copied: they are zero on both sides
-	if (int rc = zero_padding(n2_stream(stream), f->sel_sdf_in, sdf_rows, f->sdf_in_w, n, f->pad_n.sel_sdf_in)) return rc;
-	if (int rc = zero_padding(n2_stream(stream), f->sel_rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.sel_rgb_in)) return rc;
-	const uint32_t groups = (sdf_rows + 7) / 8 + (RGB_IN_ROWS + 7) / 8 + (f->enc_w + 7) / 8 + 1;
-	field_select_kernel<<<dim3((n + 2 * FB - 1) / (2 * FB), groups), dim3(FB), 0, n2_stream(stream)>>>(
-		n, n_source, d_source_index, sdf_rows, RGB_IN_ROWS, f->enc_w, f->sdf_in, f->rgb_in, f->dsdf_din, f->xyz, f->sel_sdf_in, f->sel_rgb_in,
-		f->sel_dsdf_denc, f->sel_xyz, f->sel_index);
+	field_select_kernel<<<fgrid(n), dim3(FB), 0, n2_stream(stream)>>>(n, n_source, d_source_index, f->sel_index);
 	N2_LAUNCH_CHECK();
 	f->sel_n = n;
 	return N2_OK;

@@ -258,7 +258,8 @@ __device__ __forceinline__ void grid_scatter_pair(const N2LevelTable& tab, uint3
                                                   const float* __restrict__ xyz, uint32_t point_stride, uint32_t dim_stride,
                                                   const __half* __restrict__ dL_dy, const float* __restrict__ v,
                                                   const __half* __restrict__ g2, const __half2* __restrict__ params,
-                                                  __half2* __restrict__ grads, __half* __restrict__ dL_ddLdy) {
+                                                  __half2* __restrict__ grads, __half* __restrict__ dL_ddLdy, uint32_t xi, uint32_t Ng) {
+	// xi: where this point's position and g2 column stand (i itself unless the call reads them through an index); Ng: columns of g2
 	const float scale = tab.scale[level];
 	const uint32_t entries = tab.entries[level], res = tab.resolution[level];
 	const size_t row = (size_t)level * 2;
@@ -266,15 +267,15 @@ __device__ __forceinline__ void grid_scatter_pair(const N2LevelTable& tab, uint3
 		if (SECOND && WANT_OUT) dL_ddLdy[(row + b) * N + i] = __float2half_rn(0.f);
 		return;
 	}
-	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	const N2Point p = n2_load_point(xyz, point_stride, dim_stride, xi, scale);
 	float a0 = 0.f, a1 = 0.f, c0 = 0.f, c1 = 0.f, v0 = 0.f, v1 = 0.f, v2 = 0.f;
 	if (FIRST) {
 		a0 = __half2float(dL_dy[row * N + i]);
 		a1 = __half2float(dL_dy[(row + 1) * N + i]);
 	}
 	if (SECOND) {
-		c0 = __half2float(g2[row * N + i]);
-		c1 = __half2float(g2[(row + 1) * N + i]);
+		c0 = __half2float(g2[row * Ng + xi]);
+		c1 = __half2float(g2[(row + 1) * Ng + xi]);
 		v0 = v[i] * scale; v1 = v[(size_t)N + i] * scale; v2 = v[(size_t)2 * N + i] * scale;
 	}
 	const bool skip = !SECOND && a0 == 0.f && a1 == 0.f;  // nothing to add (both lanes of a pair agree)
@@ -321,12 +322,13 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_scatter_kernel(N2LevelTable t
                                                                   uint32_t dim_stride, const __half* __restrict__ dL_dy,
                                                                   const float* __restrict__ v, const __half* __restrict__ g2,
                                                                   const __half2* __restrict__ params, __half2* __restrict__ grads,
-                                                                  __half* __restrict__ dL_ddLdy) {
+                                                                  __half* __restrict__ dL_ddLdy, const uint32_t* __restrict__ index, uint32_t n_cols) {
 	const uint32_t level = blockIdx.x / tiles;
 	const uint32_t i = (blockIdx.x - level * tiles) * PAIR_POINTS + (threadIdx.x >> 1);
 	const uint32_t b = threadIdx.x & 1u;
 	if (i >= N) return;  // both lanes of a pair share i, so pairs leave together
-#define CALL(M) grid_scatter_pair<M, FIRST, SECOND, WANT_OUT>(tab, level, i, b, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, grads, dL_ddLdy)
+	const uint32_t xi = index ? min(index[i], n_cols - 1u) : i, Ng = index ? n_cols : N;
+#define CALL(M) grid_scatter_pair<M, FIRST, SECOND, WANT_OUT>(tab, level, i, b, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, grads, dL_ddLdy, xi, Ng)
 	N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
 }
@@ -472,9 +474,9 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
                                                const __half* __restrict__ dL_dy, const float* __restrict__ v,
                                                const __half* __restrict__ g2, const __half2* __restrict__ params,
                                                __half* __restrict__ dL_ddLdy, uint32_t* e_out, float* r0_out, float* r1_out,
-                                               uint32_t* cell) {
+                                               uint32_t* cell, uint32_t xi, uint32_t Ng) {
 	const float scale = tab.scale[level];
-	N2Point p = n2_load_point(xyz, point_stride, dim_stride, i, scale);
+	N2Point p = n2_load_point(xyz, point_stride, dim_stride, xi, scale);
 	if (CLAMP_X) p.c[0] = min(p.c[0], PAIR_MAX_CELL);  // pair records: x + 1 stays inside the bucket's index bits
 	cell[0] = p.c[0]; cell[1] = p.c[1]; cell[2] = p.c[2];
 	uint32_t e[8];
@@ -486,8 +488,8 @@ __device__ __forceinline__ void grid_bin_point(const N2LevelTable& tab, uint32_t
 		a1 = __half2float(dL_dy[(row + 1) * N + i]);
 	}
 	if (SECOND) {
-		c0 = __half2float(g2[row * N + i]);
-		c1 = __half2float(g2[(row + 1) * N + i]);
+		c0 = __half2float(g2[row * Ng + xi]);
+		c1 = __half2float(g2[(row + 1) * Ng + xi]);
 		v0 = v[i] * scale; v1 = v[(size_t)N + i] * scale; v2 = v[(size_t)2 * N + i] * scale;
 	}
 	const __half2* P = params + tab.offset[level];
@@ -565,7 +567,8 @@ __device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uin
                                               const __half* __restrict__ dL_dy, const float* __restrict__ v, const __half* __restrict__ g2,
                                               const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
                                               uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys, uint16_t* __restrict__ offsets,
-                                              uint32_t* hist, uint32_t* prefix, uint32_t* stage_val, uint16_t* stage_key) {
+                                              uint32_t* hist, uint32_t* prefix, uint32_t* stage_val, uint16_t* stage_key,
+                                              const uint32_t* __restrict__ index, uint32_t n_cols) {
 	constexpr uint32_t R = PAIR ? 4 : 8;  // sorted records per point
 	const uint32_t lane = threadIdx.x & 63u;
 	// records of this thread: entry | rank << 19 after the counting step (REC_SKIP: merged into a later lane)
@@ -586,10 +589,12 @@ __device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uin
 #pragma unroll
 		for (uint32_t k = 0; k < 8; ++k) { e[k] = 0; r0[k] = 0.f; r1[k] = 0.f; }
 		if (valid) {
+			// positions and g2 columns may be read through an index (see n2_grid_backward_fused_indexed)
+			const uint32_t xi = index ? min(index[i], n_cols - 1u) : i, Ng = index ? n_cols : N;
 			if (PAIR) {
-				grid_bin_point<N2_LEVEL_HASH, FIRST, SECOND, WANT_OUT, true>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell);
+				grid_bin_point<N2_LEVEL_HASH, FIRST, SECOND, WANT_OUT, true>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell, xi, Ng);
 			} else {
-#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT, false>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell)
+#define CALL(M) grid_bin_point<M, FIRST, SECOND, WANT_OUT, false>(tab, level, i, N, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, e, r0, r1, cell, xi, Ng)
 				N2_DISPATCH_MODE(tab.mode[level], CALL)
 #undef CALL
 			}
@@ -686,7 +691,8 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
                                                               const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
                                                               uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
-                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count) {
+                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count,
+                                                              const uint32_t* __restrict__ index, uint32_t n_cols) {
 	// part of the gradient buffer that the reduce kernel will add to with atomics: cleared here, one 16-byte store per thread
 	for (uint32_t z = blockIdx.x * BIN_BLOCK + threadIdx.x; z < zero_count; z += gridDim.x * BIN_BLOCK) zero_begin[z] = make_uint4(0u, 0u, 0u, 0u);
 	__shared__ uint32_t hist[BKT_MAX];
@@ -698,10 +704,10 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
 	__syncthreads();
 	if ((tab.pair_levels >> level) & 1u)
 		grid_bin_tile<FIRST, SECOND, WANT_OUT, true>(tab, level, tile, N, tiles, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, rec_vals,
-		                                             rec_keys, offsets, hist, prefix, stage_val, stage_key);
+		                                             rec_keys, offsets, hist, prefix, stage_val, stage_key, index, n_cols);
 	else
 		grid_bin_tile<FIRST, SECOND, WANT_OUT, false>(tab, level, tile, N, tiles, xyz, point_stride, dim_stride, dL_dy, v, g2, params, dL_ddLdy, rec_vals,
-		                                              rec_keys, offsets, hist, prefix, stage_val, stage_key);
+		                                              rec_keys, offsets, hist, prefix, stage_val, stage_key, index, n_cols);
 }
 
 // LDS float atomics retire about one lane every three clocks on this part, integer ones at ~9 (32-bit) and
@@ -1284,7 +1290,8 @@ N2_API int n2_grid_set_workspace(n2_grid_t* grid, void* d_workspace, uint64_t n_
 
 // Parameter gradients through the bin + reduce kernels.  The gradient buffer has been zeroed for OVERWRITE.
 static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
-                           const __half* dL_dy, const float* v, const __half* g2, __half* dL_ddLdy, bool accumulate) {
+                           const __half* dL_dy, const float* v, const __half* g2, __half* dL_ddLdy, bool accumulate,
+                           const uint32_t* index, uint32_t n_cols) {
 	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
 	const dim3 bd(BIN_BLOCK);
@@ -1299,7 +1306,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	grid->zero_begin = nullptr;
 	grid->zero_count = 0;
 #define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
-                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, zero_begin, zero_count)
+                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, zero_begin, zero_count, index, n_cols)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
 	else if (second && out) LAUNCH(false, true, true);
@@ -1326,14 +1333,15 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 
 // One scatter pass with any combination of first-order (dL_dy) and second-order (v, g2) terms.
 static int launch_scatter(n2_grid_t* grid, hipStream_t s, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n_points,
-                          const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy, bool accumulate) {
+                          const __half* dL_dy, const float* v, const __half* g2, __half2* grads, __half* dL_ddLdy, bool accumulate,
+                          const uint32_t* index = nullptr, uint32_t n_cols = 0) {
 	if (grads != nullptr && uses_bucketed(grid, n_points))
-		return launch_bucketed(grid, s, d_xyz, point_stride, dim_stride, n_points, dL_dy, v, g2, dL_ddLdy, accumulate);
+		return launch_bucketed(grid, s, d_xyz, point_stride, dim_stride, n_points, dL_dy, v, g2, dL_ddLdy, accumulate, index, n_cols);
 	const uint32_t tiles = n_pair_tiles(n_points);
 	const dim3 gd(tiles * grid->tab.n_levels), bd(GRID_BLOCK);
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
 #define LAUNCH(F, S, O) grid_scatter_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
-                                                                       grid->params, grads, dL_ddLdy)
+                                                                       grid->params, grads, dL_ddLdy, index, n_cols)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
 	else if (second && out) LAUNCH(false, true, true);
@@ -1380,6 +1388,22 @@ N2_API int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const flo
 	return launch_scatter(grid, s, d_xyz, point_stride, dim_stride, n_points, reinterpret_cast<const __half*>(d_dL_dy), d_dL_ddLdx,
 	                      reinterpret_cast<const __half*>(d_dL_dy_second), grid->grads, reinterpret_cast<__half*>(d_dL_ddLdy),
 	                      mode == N2_GRAD_ACCUMULATE);
+}
+
+int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz_rows, uint32_t n_cols, const uint32_t* d_index,
+                                   uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,
+                                   n2_grad_mode mode) {
+	if (d_index == nullptr) return n2_grid_backward_fused(grid, stream, d_xyz_rows, 1, n_points, n_points, d_dL_dy, d_dL_ddLdx, d_dL_dy_second, nullptr, mode);
+	if (int rc = check_batch(grid, "n2_grid_backward_fused", d_xyz_rows, 1, n_cols, n_points)) return rc;
+	N2_REQUIRE((d_dL_dy && d_dL_ddLdx && d_dL_dy_second) || n_points == 0, "n2_grid_backward_fused: d_dL_dy, d_dL_ddLdx and d_dL_dy_second are required");
+	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_grid_backward_fused: mode must be OVERWRITE or ACCUMULATE");
+	N2_REQUIRE(n_cols >= 1, "n2_grid_backward_fused: an indexed input needs at least one column");
+	hipStream_t s = n2_stream(stream);
+	if (int rc = prepare_grads(grid, "n2_grid_backward_fused", s, mode, n_points)) return rc;
+	if (n_points == 0) return N2_OK;
+	N2ProfScope prof(N2_PROF_GRID_BACKWARD_PARAMS, s);
+	return launch_scatter(grid, s, d_xyz_rows, 1, n_cols, n_points, reinterpret_cast<const __half*>(d_dL_dy), d_dL_ddLdx,
+	                      reinterpret_cast<const __half*>(d_dL_dy_second), grid->grads, nullptr, mode == N2_GRAD_ACCUMULATE, d_index, n_cols);
 }
 
 N2_API int n2_grid_backward_backward_input(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz,

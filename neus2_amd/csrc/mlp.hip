@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
                                                                     hf* __restrict__ dX, float* __restrict__ partials,
                                                                     hf* __restrict__ Y = nullptr, int y_aos = 0,
                                                                     const hf* __restrict__ V = nullptr, const hf* __restrict__ G2 = nullptr,
-                                                                    int unit_row2 = -1) {
+                                                                    int unit_row2 = -1, const uint32_t* __restrict__ x_index = nullptr, uint32_t x_cols = 0) {
 	static_assert(!SECOND || (NH == 1 && WANT_DW), "the second-order pass needs one hidden layer and weight gradients");
 	using M = FragMap<IC, NH>;
 	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT, ROLES = WANT_DW ? 2 : 1;
@@ -198,7 +198,9 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 		const uint32_t col = valid ? col_raw : N - 2;
 		const uint32_t off4 = 4u * g * N + col;
 		half8 xp[2][IC], dyp[2];
-		load_input<IC>(X, N, col, g, xp);
+		// x_index: sample i of the batch is column x_index[i] of X, which has x_cols columns (the other operands are indexed by i)
+		if (x_index) load_input_indexed<IC>(X, x_cols, min(x_index[col], x_cols - 1u), min(x_index[col + 1], x_cols - 1u), g, xp);
+		else load_input<IC>(X, N, col, g, xp);
 		outgrad_frag(dY, N, col, g, (dy_aos & 1) != 0, unit_row, dy_aos >> 8, dyp[0], dyp[1]);
 		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
 		half8 vp[2][IC], gp[2];
@@ -684,7 +686,8 @@ static int allow_lds(K kernel, size_t bytes) {
 // unit_row >= 0: dL_doutput is the constant e_{unit_row} and d_dL_doutput is not read
 static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                              const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode,
-                             n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA, uint32_t dy_rows = MLP_OUT) {
+                             n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA, uint32_t dy_rows = MLP_OUT,
+                             const uint32_t* x_index = nullptr, uint32_t x_cols = 0) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
@@ -709,7 +712,8 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	do {                                                                                                            \
 		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT); /* >= the fp32 parameter image laid over it */      \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
-		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, next_slabs(mlp)); \
+		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, next_slabs(mlp), \
+			nullptr, 0, nullptr, nullptr, -1, x_index, x_cols);                                                         \
 	} while (0)
 #define LAUNCH_Y(IC, NH)                                                                                            \
 	do {                                                                                                            \
@@ -754,6 +758,13 @@ N2_API int n2_mlp_backward_rows(n2_mlp_t* mlp, n2_stream_t stream, const n2_half
 	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows);
 }
 
+int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
+                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode) {
+	N2_REQUIRE(n_rows >= 1 && n_rows <= (uint32_t)MLP_OUT, "n2_mlp_backward_rows: n_rows %u outside [1, %d]", n_rows, MLP_OUT);
+	N2_REQUIRE(d_index == nullptr || n_cols >= 1, "n2_mlp_backward_rows: an indexed input needs at least one column");
+	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows, d_index, n_cols);
+}
+
 N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
                                  n2_half* d_dinput) {
 	N2_REQUIRE(dim < (uint32_t)MLP_OUT, "n2_mlp_input_gradient: output dimension %u out of range", dim);
@@ -764,7 +775,15 @@ N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim
 N2_API int n2_mlp_backward_and_second_order(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                                             const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode) {
+	return n2_mlp_backward_and_second_order_indexed(mlp, stream, d_input, 0, nullptr, n, d_dL_doutput, dL_layout, d_dL_dinput, d_dL_ddLdinput,
+	                                                d_second_dL_doutput, mode);
+}
+
+int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
+                                             uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
+                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode) {
 	const char* fn = "n2_mlp_backward_and_second_order";
+	N2_REQUIRE(d_index == nullptr || n_cols >= 1, "%s: an indexed input needs at least one column", fn);
 	if (int rc = check_mlp_batch(mlp, fn, d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, fn, mode)) return rc;
 	N2_REQUIRE(mode != N2_GRAD_IGNORE, "%s: the merged pass exists for its weight gradients (mode must be OVERWRITE or ACCUMULATE)", fn);
@@ -796,7 +815,7 @@ N2_API int n2_mlp_backward_and_second_order(n2_mlp_t* mlp, n2_stream_t stream, c
 		mlp_backward_kernel<IC, 1, true, true, false, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,        \
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, -1,                   \
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), nullptr, 0, reinterpret_cast<const hf*>(d_dL_ddLdinput),  \
-			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2);                                                  \
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);                                 \
 		break;                                                                                                             \
 	}
 		CASE(1) CASE(2) CASE(3) CASE(4)

@@ -161,6 +161,21 @@ __device__ __forceinline__ void load_input(const hf* __restrict__ X, size_t N, u
 	for (int c = 0; c < IC; ++c) bfrag_soa(X, (uint32_t)N, 8u * g * (uint32_t)N + col, c, 16 * IC, x[0][c], x[1][c]);
 }
 
+// the same operands when the wave's samples are columns s0 (tile 0) and s1 (tile 1) of a matrix with n_src columns:
+// the row part of every address is uniform (a scalar base), the lane part two 32-bit byte offsets
+template <int IC>
+__device__ __forceinline__ void load_input_indexed(const hf* __restrict__ X, uint32_t n_src, uint32_t s0, uint32_t s1, int g, half8 (&x)[2][IC]) {
+	const uint32_t b0 = (8u * g * n_src + s0) * 2u, b1 = (8u * g * n_src + s1) * 2u;
+#pragma unroll
+	for (int c = 0; c < IC; ++c)
+#pragma unroll
+		for (int e = 0; e < 8; ++e) {
+			const char* row = reinterpret_cast<const char*>(X + (size_t)(16 * c + e) * n_src);
+			x[0][c][e] = *reinterpret_cast<const hf*>(row + b0);
+			x[1][c][e] = *reinterpret_cast<const hf*>(row + b1);
+		}
+}
+
 // ----------------------------------------------------------------------------
 // Weight fragments in LDS.
 // A workgroup builds every MFMA operand the kernels need once, in "fragment

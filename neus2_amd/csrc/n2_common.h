@@ -91,6 +91,19 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
                        float* d_row0, bool density);
 
+// n2_mlp_backward_rows / n2_mlp_backward_and_second_order whose input is read through an index: sample i of the batch is
+// column d_index[i] of d_input, a matrix with n_cols columns (d_index null: column i of n columns).  Every other operand is
+// indexed by i.  The field's backward uses them to read the activations its forward saved for ALL marched samples.
+int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
+                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode);
+int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
+                                             uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
+                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode);
+// n2_grid_backward_fused whose positions (SoA 3 x n_cols) and d_dL_dy_second rows (n_cols columns) are read through d_index.
+int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz_rows, uint32_t n_cols, const uint32_t* d_index,
+                                   uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,
+                                   n2_grad_mode mode);
+
 static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // Zero-fill with a kernel (safe to record into HIP graphs, unlike memset nodes).

@@ -116,7 +116,7 @@ __device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint3
 // once per 64 steps.  The march runs once: it records which steps emitted (64 bits per window) and the t of every
 // window's first step; the coordinates are written afterwards from those, without touching the bitfield.
 constexpr uint32_t WINDOWS = 17;                      // 1088 steps: a ray inside the unit cube is at most sqrt(3) long,
-constexpr uint32_t MASK_BITS = WINDOWS * 64;          // i.e. MARCH_STEPS steps plus the start jitter
+                                                      // i.e. MARCH_STEPS steps plus the start jitter
 constexpr uint32_t RAYS_PER_BLOCK = 4;                // one wave per ray
 
 // t of this lane's step: t_first plus `lane` additions of STEP, one at a time like the serial march.  Inside a binade
