@@ -43,6 +43,7 @@ struct n2_field {
 	float* var_part;    // one partial sum of the variance gradient per workgroup of the backward's preparation kernel
 	// a selection of the last forward's samples (n2_field_select): the backward reads the rows above through this index
 	uint32_t* sel_index;  // [n]
+	const uint32_t* sel_use;  // the index in use: sel_index, or the caller's own buffer (n2_field_select_borrow)
 	uint32_t last_n;      // samples of the last forward
 	uint32_t sel_n;       // samples selected (0: the backward's batch is the forward's)
 	void* ws_sdf;
@@ -172,7 +173,7 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 //    backward_backward_input output dL_ddLdoutput, taken from the Jacobian the forward stored instead of
 //    gathering the table again); the padding rows above stay zero (zero_padding);
 //  * the variance gradient is the sum of row 7: every workgroup leaves its partial sum in var_part[blockIdx.x] and
-//    field_variance_gradient_kernel adds them up in a fixed order.
+//    the launch that reduces the networks' weight gradients adds them up in a fixed order.
 struct LevelScales { float s[16]; };
 // SLOPES: the Jacobian comes as the fused forward stores it, 16 bytes per level and sample [level][n_src] without the level's scale factor
 // (scales.s[level] multiplies it back in); else as the grid encoding's fp32 dy_dx [enc_w][n_src][3].
@@ -188,7 +189,7 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 	float s = 0.f;
 	if (i < N) {
 		// the Jacobian rows are those of the forward: of sample src_index[i] among n_src when a selection is active
-		const size_t js = src_index ? src_index[i] : i, jn = src_index ? n_src : N;
+		const size_t js = src_index ? min(src_index[i], n_src - 1u) : i, jn = src_index ? n_src : N;
 		const half8 lo = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16), hi = *reinterpret_cast<const half8*>(dL_dout + (size_t)i * 16 + 8);
 		d_rgb_in[i] = d_rgb_in[i] + lo[3];
 		s = (float)lo[7];
@@ -250,26 +251,6 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 		float t = 0.f;
 		for (uint32_t w = 0; w < FB / 64; ++w) t += part[w];
 		var_part[blockIdx.x] = t;
-	}
-}
-
-// var_grad = [var_grad +] sum of the n_parts partial sums: one workgroup, fixed order.  1024 lanes, so that a 2^18 batch
-// is one load per lane (the kernel is nothing but memory latency).
-constexpr uint32_t VB = 1024;
-__global__ void __launch_bounds__(VB) field_variance_gradient_kernel(const float* __restrict__ var_part, uint32_t n_parts, hf* __restrict__ var_grad,
-                                                                     int accumulate) {
-	__shared__ float part[VB / 64];
-	float s = 0.f;
-	for (uint32_t i = threadIdx.x; i < n_parts; i += VB) s += var_part[i];
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
-	__syncthreads();
-	if (threadIdx.x < 64) {
-		float t = threadIdx.x < VB / 64 ? part[threadIdx.x] : 0.f;
-#pragma unroll
-		for (int o = 8; o > 0; o >>= 1) t += __shfl_xor(t, o);
-		if (threadIdx.x == 0) var_grad[0] = accumulate ? (hf)((float)var_grad[0] + t) : (hf)t;
 	}
 }
 
@@ -519,7 +500,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	N2_REQUIRE(n == (sel ? f->sel_n : f->last_n), "n2_field_backward: batch %u, but the last %s was over %u samples", n,
 	           sel ? "n2_field_select" : "n2_field_forward", sel ? f->sel_n : f->last_n);
 	// with a selection, sample i of the batch is column index[i] of the rows the forward saved over its n_src samples
-	const uint32_t* index = sel ? f->sel_index : nullptr;
+	const uint32_t* index = sel ? f->sel_use : nullptr;
 	const uint32_t n_src = f->last_n;
 	// colour net: only rows 0..2 of dL_doutput belong to it
 	if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
@@ -530,12 +511,10 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	for (uint32_t l = 0; l < 16 && 2 * l < f->enc_w; ++l) scales.s[l] = n2_grid_table(f->grid)->scale[l];
 	if (f->slopes_saved)
 		field_backward_prep_kernel<true><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-		                                                               f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n, scales);
+		                                                               f->d_density_in, f->var_part, index, f->last_n, scales);
 	else
 		field_backward_prep_kernel<false><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-		                                                                f->d_density_in, f->var_part, sel ? f->sel_index : nullptr, f->last_n, scales);
-	N2_LAUNCH_CHECK();
-	field_variance_gradient_kernel<<<dim3(1), dim3(VB), 0, s>>>(f->var_part, fgrid(n).x, f->grads + f->off_var, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+		                                                                f->d_density_in, f->var_part, index, f->last_n, scales);
 	N2_LAUNCH_CHECK();
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient; the second-order pass through the
 	// net (the reference's backward_backward_input with Accumulate) rides along
@@ -547,8 +526,9 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	if (int rc = n2_grid_backward_fused_indexed(f->grid, stream, f->xyz, n_src, index, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
 	                                            reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n_src), mode)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
-	// pending: one launch sums them
-	return n2_mlp_reduce_deferred(f->rgb, f->sdf, stream);
+	// pending: one launch sums them, and with them the partial sums of the variance gradient
+	return n2_mlp_reduce_deferred_sum(f->rgb, f->sdf, stream, f->var_part, fgrid(n).x, reinterpret_cast<n2_half*>(f->grads + f->off_var),
+	                                  mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 }
 
 N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_source_index, uint32_t n_source, uint32_t n) {
@@ -560,6 +540,18 @@ N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_
 	field_select_kernel<<<fgrid(n), dim3(FB), 0, n2_stream(stream)>>>(n, n_source, d_source_index, f->sel_index);
 	N2_LAUNCH_CHECK();
 	f->sel_n = n;
+	f->sel_use = f->sel_index;
+	return N2_OK;
+}
+
+int n2_field_select_borrow(n2_field_t* f, const uint32_t* d_source_index, uint32_t n_source, uint32_t n) {
+	if (int rc = check_field(f, "n2_field_select", n)) return rc;
+	N2_REQUIRE(n <= f->max_batch_bwd, "n2_field_select: batch %u exceeds the workspace's backward capacity %u", n, f->max_batch_bwd);
+	N2_REQUIRE(n_source == f->last_n && n_source > 0, "n2_field_select: n_source %u, but the last n2_field_forward was over %u samples", n_source,
+	           f->last_n);
+	N2_REQUIRE(n > 0 && d_source_index != nullptr, "n2_field_select: empty selection");
+	f->sel_n = n;
+	f->sel_use = d_source_index;  // every kernel that reads through it clamps the entries into the forward's batch
 	return N2_OK;
 }
 

@@ -484,13 +484,27 @@ __global__ void __launch_bounds__(256) mlp_reduce_partials_kernel(const float* _
 	mlp_reduce_line(partials, n_slabs, n_params, grads, accumulate, blockIdx.x, fold);
 }
 
-// two parameter sets in one launch
+// two parameter sets in one launch; one more workgroup (when extra_n > 0) adds up extra_n floats in a fixed order into a
+// single fp16 value: the field's variance gradient rides along instead of taking a launch of its own
 __global__ void __launch_bounds__(256) mlp_reduce_two_kernel(const float* __restrict__ pa, uint32_t slabs_a, uint32_t params_a, hf* __restrict__ ga, int acc_a,
                                                              uint32_t blocks_a, const float* __restrict__ pb, uint32_t slabs_b, uint32_t params_b,
-                                                             hf* __restrict__ gb, int acc_b) {
+                                                             hf* __restrict__ gb, int acc_b, uint32_t blocks_b, const float* __restrict__ extra,
+                                                             uint32_t extra_n, hf* __restrict__ extra_out, int extra_acc) {
 	__shared__ float fold[32][33];
 	if (blockIdx.x < blocks_a) mlp_reduce_line(pa, slabs_a, params_a, ga, acc_a, blockIdx.x, fold);
-	else mlp_reduce_line(pb, slabs_b, params_b, gb, acc_b, blockIdx.x - blocks_a, fold);
+	else if (blockIdx.x < blocks_a + blocks_b) mlp_reduce_line(pb, slabs_b, params_b, gb, acc_b, blockIdx.x - blocks_a, fold);
+	else {
+		float s = 0.f;
+		for (uint32_t i = threadIdx.x; i < extra_n; i += 256) s += extra[i];
+#pragma unroll
+		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+		if ((threadIdx.x & 63) == 0) fold[0][threadIdx.x >> 6] = s;
+		__syncthreads();
+		if (threadIdx.x == 0) {
+			const float t = (fold[0][0] + fold[0][1]) + (fold[0][2] + fold[0][3]);
+			extra_out[0] = extra_acc ? (hf)((float)extra_out[0] + t) : (hf)t;
+		}
+	}
 }
 
 // ----------------------------------------------------------------------------
@@ -647,21 +661,30 @@ N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 	return N2_OK;
 }
 
-N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) {
+N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) { return n2_mlp_reduce_deferred_sum(a, b, stream, nullptr, 0, nullptr, 0); }
+
+int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate) {
 	N2_REQUIRE(a != nullptr, "n2_mlp_reduce_deferred: mlp is null");
 	hipStream_t s = n2_stream(stream);
 	if (b != nullptr && b->pending_slabs == 0) b = nullptr;
 	if (a->pending_slabs == 0) { a = b; b = nullptr; }
-	if (a == nullptr || a->pending_slabs == 0) return N2_OK;
+	if (a == nullptr || a->pending_slabs == 0 || (b == nullptr && n_parts > 0)) {
+		// nothing or one network pending: the sum, if any, goes alone
+		if (n_parts > 0) {
+			mlp_reduce_two_kernel<<<dim3(1), dim3(256), 0, s>>>(nullptr, 0, 0, nullptr, 0, 0, nullptr, 0, 0, nullptr, 0, 0, d_parts, n_parts, reinterpret_cast<hf*>(d_sum), accumulate);
+			N2_LAUNCH_CHECK();
+		}
+		if (a == nullptr || a->pending_slabs == 0) return N2_OK;
+	}
 	if (b == nullptr) {
 		const int rc = reduce_now(a, s, a->pending_slabs, a->pending_mode);
 		a->pending_slabs = 0;
 		return rc;
 	}
 	const uint32_t blocks_a = (a->n_params + 31) / 32, blocks_b = (b->n_params + 31) / 32;
-	mlp_reduce_two_kernel<<<dim3(blocks_a + blocks_b), dim3(256), 0, s>>>(a->workspace, a->pending_slabs, a->n_params, a->grads,
+	mlp_reduce_two_kernel<<<dim3(blocks_a + blocks_b + (n_parts > 0 ? 1u : 0u)), dim3(256), 0, s>>>(a->workspace, a->pending_slabs, a->n_params, a->grads,
 		a->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0, blocks_a, b->workspace, b->pending_slabs, b->n_params, b->grads,
-		b->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+		b->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0, blocks_b, d_parts, n_parts, reinterpret_cast<hf*>(d_sum), accumulate);
 	N2_LAUNCH_CHECK();
 	a->pending_slabs = 0;
 	b->pending_slabs = 0;

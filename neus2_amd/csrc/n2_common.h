@@ -99,6 +99,10 @@ int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_hal
 int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
                                              uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
                                              const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode);
+// n2_mlp_reduce_deferred that also adds up n_parts floats, in a fixed order, into one fp16 value ([+=] when accumulate)
+int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
+// n2_field_select without the copy of the index: d_source_index must stay valid and unchanged until the backward has run
+int n2_field_select_borrow(n2_field_t* field, const uint32_t* d_source_index, uint32_t n_source, uint32_t n);
 // n2_grid_backward_fused whose positions (SoA 3 x n_cols) and d_dL_dy_second rows (n_cols columns) are read through d_index.
 int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz_rows, uint32_t n_cols, const uint32_t* d_index,
                                    uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,

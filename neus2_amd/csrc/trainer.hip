@@ -347,7 +347,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	if (t->cfg.recompute_training_forward) {
 		if (int rc = n2_field_forward(t->field, stream, t->coords_compacted, T, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
 	} else {
-		if (int rc = n2_field_select(t->field, stream, t->src_index, n_inference, T)) return rc;
+		if (int rc = n2_field_select_borrow(t->field, t->src_index, n_inference, T)) return rc;
 	}
 	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
 	if (int rc = n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
