@@ -383,6 +383,8 @@ int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, 
  * Per parameter i:  g = grad/loss_scale;  i >= n_matrix_params and g == 0: skipped entirely;
  * i < n_matrix_params: g += l2_reg*w;  moments with beta1/beta2;  per-parameter step counter t;
  * w -= lr*sqrt(1-beta2^t)/(1-beta1^t) * m/(sqrt(v)+epsilon);  fp16 copy refreshed.
+ * The bias-correction factors come from a per-device table per (beta1, beta2); the first call with a new pair on a
+ * device builds it and waits for it on the host (the one exception to "calls never synchronise").
  * ---------------------------------------------------------------------- */
 typedef struct n2_adam_config {
 	float learning_rate; /* 1e-3 */
@@ -586,6 +588,18 @@ typedef struct n2_trainer_optimizer_buffers {
 } n2_trainer_optimizer_buffers;
 int n2_trainer_optimizer_state(n2_trainer_t* trainer, n2_trainer_optimizer_buffers* out);
 int n2_trainer_set_optimizer_steps(n2_trainer_t* trainer, uint32_t steps);
+/* The Ema wrapper's own step count (its bias correction 1 - decay^steps).  With ema_steps = 0 the moving average starts
+ * again from the current working parameters: the fp32 average and the fp16 inference copy are overwritten with them.
+ * Call it with 0 after parameters were loaded without Ema state (a snapshot without optimizer state, or
+ * n2_trainer_sync_params after writing the master weights), with the saved optimizer step count when the Ema weights
+ * were loaded too.  Without the wrapper (ema_decay 0) it only records the count. */
+int n2_trainer_restart_ema(n2_trainer_t* trainer, n2_stream_t stream, uint32_t ema_steps);
+/* Testbed::m_training_step: the number of training steps taken so far.  It is the clock of the encoding's progressive
+ * level mask (the reference sets it on the encoding at the top of Testbed::train, before the occupancy-grid update and the
+ * step, src/testbed.cu:2641-2647): this call also tells the encoding, so that an occupancy update that follows sees the
+ * mask of the step about to run.  n2_trainer_step uses it and adds one.  Set it after loading a snapshot (its
+ * training_step), whether or not the file holds optimizer state. */
+int n2_trainer_set_training_step(n2_trainer_t* trainer, uint32_t step);
 
 /* Call before the bitfield passed to n2_trainer_set_scene is rewritten in place (an occupancy-grid update): waits for a
  * sample generation that is running ahead on the trainer's own stream and discards it, so that the next step marches

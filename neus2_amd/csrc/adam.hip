@@ -5,26 +5,29 @@
 #include "n2_common.h"
 
 #include <cmath>
+#include <mutex>
 
 typedef _Float16 hf;
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 
 // Bias correction sqrt(1 - beta2^t) / (1 - beta1^t) for t < ADAM_TABLE, computed once per (beta1, beta2) by
 // adam_table_kernel.  Two powf per parameter made the step kernel ALU bound; a (mostly uniform) table read costs nothing.
-constexpr uint32_t ADAM_TABLE = 4096;
-__device__ float g_adam_bias[ADAM_TABLE];
+// A device holds ADAM_SLOTS such tables, one per pair of betas in use, so that optimisers with different betas (or on
+// different streams) never rewrite a table another one's step is reading.
+constexpr uint32_t ADAM_TABLE = 4096, ADAM_SLOTS = 4;
+__device__ float g_adam_bias[ADAM_SLOTS][ADAM_TABLE];
 
 __device__ __forceinline__ float adam_bias(float beta1, float beta2, uint32_t t) {
 	return sqrtf(1.f - powf(beta2, (float)t)) / (1.f - powf(beta1, (float)t));
 }
-__global__ void __launch_bounds__(256) adam_table_kernel(float beta1, float beta2) {
+__global__ void __launch_bounds__(256) adam_table_kernel(float beta1, float beta2, uint32_t slot) {
 	const uint32_t t = blockIdx.x * 256 + threadIdx.x;
-	if (t < ADAM_TABLE) g_adam_bias[t] = adam_bias(beta1, beta2, t);
+	if (t < ADAM_TABLE) g_adam_bias[slot][t] = adam_bias(beta1, beta2, t);
 }
 
 // inv_loss_scale > 0: loss_scale is a power of two and multiplying by its reciprocal is the exact division
 __device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
-                                         const n2_adam_config& c, float g16, float& w, float& m1, float& m2, uint32_t& t) {
+                                         const n2_adam_config& c, const float* __restrict__ table, float g16, float& w, float& m1, float& m2, uint32_t& t) {
 	float g = inv_loss_scale > 0.f ? g16 * inv_loss_scale : g16 / loss_scale;
 	if (i >= n_matrix) {
 		if (g == 0.f) return false;
@@ -36,18 +39,20 @@ __device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float lo
 	m2 = c.beta2 * m2 + (1.f - c.beta2) * gs;
 	t += 1u;
 	// beyond the table the factor is exactly 1 once both powers have underflowed (saturated), else it is computed
-	const float bias = t < ADAM_TABLE ? g_adam_bias[t] : (saturated ? 1.f : adam_bias(c.beta1, c.beta2, t));
+	const float bias = t < ADAM_TABLE ? table[t] : (saturated ? 1.f : adam_bias(c.beta1, c.beta2, t));
 	const float lr = c.learning_rate * bias;
 	w -= lr * m1 / (sqrtf(m2) + c.epsilon);
 	return true;
 }
 
 __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
-                                                        float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
+                                                        uint32_t slot, const uint32_t* __restrict__ gate, float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
                                                         float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps) {
 	const uint32_t q = blockIdx.x * 256 + threadIdx.x;
 	const uint32_t i0 = q * 4;
 	if (i0 >= n) return;
+	if (gate != nullptr && *gate == 0u) return;  // a step without samples leaves the parameters and the optimiser state alone
+	const float* table = g_adam_bias[slot];
 	if (i0 + 4 <= n) {
 		const half4 g = *reinterpret_cast<const half4*>(grads + i0);
 		const bool all_zero = g[0] == (hf)0 && g[1] == (hf)0 && g[2] == (hf)0 && g[3] == (hf)0;
@@ -57,10 +62,10 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		float4 b = *reinterpret_cast<float4*>(m2 + i0);
 		uint4 t = *reinterpret_cast<uint4*>(steps + i0);
 		bool any = false;
-		any |= adam_one(i0 + 0, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[0], w.x, a.x, b.x, t.x);
-		any |= adam_one(i0 + 1, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[1], w.y, a.y, b.y, t.y);
-		any |= adam_one(i0 + 2, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[2], w.z, a.z, b.z, t.z);
-		any |= adam_one(i0 + 3, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)g[3], w.w, a.w, b.w, t.w);
+		any |= adam_one(i0 + 0, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[0], w.x, a.x, b.x, t.x);
+		any |= adam_one(i0 + 1, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[1], w.y, a.y, b.y, t.y);
+		any |= adam_one(i0 + 2, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[2], w.z, a.z, b.z, t.z);
+		any |= adam_one(i0 + 3, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[3], w.w, a.w, b.w, t.w);
 		if (!any) return;
 		*reinterpret_cast<float4*>(master + i0) = w;
 		*reinterpret_cast<float4*>(m1 + i0) = a;
@@ -71,7 +76,7 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		for (uint32_t i = i0; i < n; ++i) {
 			float w = master[i], a = m1[i], b = m2[i];
 			uint32_t t = steps[i];
-			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, (float)grads[i], w, a, b, t)) {
+			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)grads[i], w, a, b, t)) {
 				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
 			}
 		}
@@ -81,6 +86,12 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                         float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
                         float* d_m2, uint32_t* d_steps) {
+	return n2_adam_step_gated(stream, config, n_params, n_matrix_params, loss_scale, d_master, d_params, d_gradients, d_m1, d_m2, d_steps, nullptr);
+}
+
+int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
+                       float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate) {
 	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
 	if (n_params == 0) return N2_OK;
 	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
@@ -93,17 +104,36 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 	           "n2_adam_step: fp16 buffers must be 8-byte aligned");
 	const uint32_t quads = (n_params + 3) / 4;
 	hipStream_t s = n2_stream(stream);
-	// the bias-correction table of this device holds the factors of one (beta1, beta2) pair; calls with other
-	// betas rebuild it on their stream (calls on different streams with different betas must not overlap)
-	struct Built { bool valid = false; float beta1 = 0.f, beta2 = 0.f; };
-	static Built built[64];
+	// The device's table for this pair of betas.  A new pair takes a free slot; its table is complete before any stream can
+	// read it (the host waits for the kernel that fills it, once per pair).  When all slots are taken the least recently
+	// used one is refilled after the whole device has gone idle, so that no step in flight still reads it.
+	struct Slot { bool valid = false; float beta1 = 0.f, beta2 = 0.f; uint64_t used = 0; };
+	static Slot slots[64][ADAM_SLOTS];
+	static uint64_t clock = 0;
+	static std::mutex lock;
 	int dev = 0;
 	N2_HIP(hipGetDevice(&dev));
 	N2_REQUIRE(dev >= 0 && dev < 64, "n2_adam_step: device index %d not supported", dev);
-	if (!built[dev].valid || built[dev].beta1 != config->beta1 || built[dev].beta2 != config->beta2) {
-		adam_table_kernel<<<dim3(ADAM_TABLE / 256), dim3(256), 0, s>>>(config->beta1, config->beta2);
-		N2_LAUNCH_CHECK();
-		built[dev].valid = true; built[dev].beta1 = config->beta1; built[dev].beta2 = config->beta2;
+	uint32_t slot = ADAM_SLOTS;
+	{
+		std::lock_guard<std::mutex> guard(lock);
+		for (uint32_t k = 0; k < ADAM_SLOTS && slot == ADAM_SLOTS; ++k)
+			if (slots[dev][k].valid && slots[dev][k].beta1 == config->beta1 && slots[dev][k].beta2 == config->beta2) slot = k;
+		uint32_t victim = 0;  // a free slot if there is one, else the least recently used
+		for (uint32_t k = 1; k < ADAM_SLOTS; ++k) {
+			const Slot &c = slots[dev][k], &v = slots[dev][victim];
+			if (v.valid && (!c.valid || c.used < v.used)) victim = k;
+		}
+		if (slot == ADAM_SLOTS) {
+			slot = victim;
+			if (slots[dev][slot].valid) N2_HIP(hipDeviceSynchronize());
+			slots[dev][slot].valid = false;
+			adam_table_kernel<<<dim3(ADAM_TABLE / 256), dim3(256), 0, s>>>(config->beta1, config->beta2, slot);
+			N2_LAUNCH_CHECK();
+			N2_HIP(hipStreamSynchronize(s));
+			slots[dev][slot].valid = true; slots[dev][slot].beta1 = config->beta1; slots[dev][slot].beta2 = config->beta2;
+		}
+		slots[dev][slot].used = ++clock;
 	}
 	// 1 - beta^t == 1 in fp32 for every t past the table?
 	const double small = std::ldexp(1.0, -26);
@@ -111,7 +141,7 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 	int exp2 = 0;
 	const float inv_loss_scale = (std::frexp(loss_scale, &exp2) == 0.5f && exp2 > -120 && exp2 < 120) ? 1.f / loss_scale : 0.f;
 	N2ProfScope prof(N2_PROF_ADAM, s);
-	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated,
+	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate,
 		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
 	N2_LAUNCH_CHECK();
 	return N2_OK;

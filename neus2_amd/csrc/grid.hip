@@ -28,6 +28,7 @@ struct n2_grid {
 	// progressive training (base_training_step 0: off)
 	float base_valid_level_scale, valid_level_scale;
 	uint32_t base_training_step;
+	uint32_t training_step;  // as last told by n2_grid_set_training_step
 	// optional scratch of the bucketed scatter
 	unsigned char* ws;
 	uint64_t ws_bytes;
@@ -989,6 +990,7 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->base_valid_level_scale = 1.0f;
 	g->valid_level_scale = 0.0f;
 	g->base_training_step = 0;
+	g->training_step = 0;
 	uint64_t off = 0;
 	const float log2_b = std::log2(per_level_scale);
 	for (uint32_t l = 0; l < n_levels; ++l) {
@@ -1087,9 +1089,8 @@ N2_API int n2_grid_set_progressive(n2_grid_t* grid, float base_valid_level_scale
 	grid->base_valid_level_scale = base_valid_level_scale;
 	grid->valid_level_scale = valid_level_scale;
 	grid->base_training_step = base_training_step;
-	if (base_training_step == 0) grid->tab.valid_levels = grid->tab.n_levels;
-	grid->tab.active_levels = count_active_levels(grid->tab);
-	return N2_OK;
+	// the levels in use follow from the keys and the training step last set
+	return n2_grid_set_training_step(grid, grid->training_step);
 }
 
 // levels in use at a training step: the fraction base + scale * (step / base_training_step), whole periods only,
@@ -1097,7 +1098,12 @@ N2_API int n2_grid_set_progressive(n2_grid_t* grid, float base_valid_level_scale
 // at least one level and at most all of them
 N2_API int n2_grid_set_training_step(n2_grid_t* grid, uint32_t training_step) {
 	N2_REQUIRE(grid != nullptr, "n2_grid_set_training_step: grid is null");
-	if (grid->base_training_step == 0) return N2_OK;
+	grid->training_step = training_step;
+	if (grid->base_training_step == 0) {
+		grid->tab.valid_levels = grid->tab.n_levels;
+		grid->tab.active_levels = count_active_levels(grid->tab);
+		return N2_OK;
+	}
 	const float fraction = grid->base_valid_level_scale + grid->valid_level_scale * (float)(training_step / grid->base_training_step);
 	const float levels = fraction * (float)grid->tab.n_levels + 1e-3f;
 	uint32_t n = levels >= (float)grid->tab.n_levels ? grid->tab.n_levels : (uint32_t)levels;

@@ -99,6 +99,10 @@ int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_hal
 int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
                                              uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
                                              const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode);
+// n2_adam_step that does nothing when *d_gate is zero on the device (d_gate null: always steps)
+int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
+                       float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate);
 // n2_mlp_reduce_deferred that also adds up n_parts floats, in a fixed order, into one fp16 value ([+=] when accumulate)
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
 // n2_field_select without the copy of the index: d_source_index must stay valid and unchanged until the backward has run

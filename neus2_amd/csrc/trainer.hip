@@ -27,6 +27,8 @@ struct n2_trainer {
 	float* ema_tmp;   // fp32 moving average of the fp16 weights (null without the Ema wrapper)
 	hf* ema;          // its fp16 copy: the inference parameters
 	uint32_t optimizer_steps;  // nested optimizer steps taken so far
+	uint32_t ema_steps;        // steps the moving average has taken since it was last (re)started
+	uint32_t training_step;    // m_training_step: steps taken so far, the clock of the encoding's progressive level mask
 	// per-step buffers; everything the sample generator writes exists twice
 	struct SampleSet {
 		float* coords;            // [max_samples][7]
@@ -194,6 +196,8 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->ema_tmp = cfg->ema_decay > 0.f ? reinterpret_cast<float*>(b + c.ema_tmp) : nullptr;
 	t->ema = cfg->ema_decay > 0.f ? reinterpret_cast<hf*>(b + c.ema) : nullptr;
 	t->optimizer_steps = 0;
+	t->ema_steps = 0;
+	t->training_step = 0;
 	for (int i = 0; i < 2; ++i) {
 		t->sets[i].coords = reinterpret_cast<float*>(b + c.coords[i]);
 		t->sets[i].numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps[i]);
@@ -290,8 +294,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	hipStream_t s = n2_stream(stream);
 	const uint32_t T = t->cfg.target_batch_size;
 	uint32_t* compacted_counter = t->counters + 2;
-	// progressive level mask: the encoding is told the number of steps taken so far before every step
-	if (int rc = n2_grid_set_training_step(n2_field_encoding(t->field), t->optimizer_steps)) return rc;
+	// progressive level mask: the encoding is told the number of training steps taken so far before every step
+	// (Testbed::train, src/testbed.cu:2641-2647)
+	if (int rc = n2_grid_set_training_step(n2_field_encoding(t->field), t->training_step)) return rc;
 	auto sample = [&](n2_trainer::SampleSet& set, hipStream_t on, uint32_t ray_base, uint32_t sd) {
 		// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
 		return n2_generate_training_samples(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,
@@ -350,11 +355,14 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		if (int rc = n2_field_select_borrow(t->field, t->src_index, n_inference, T)) return rc;
 	}
 	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
-	if (int rc = n2_adam_step(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                          reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps)) return rc;
+	// a step whose rays kept no sample (counter 2 is zero) must not apply the previous step's gradients again
+	if (int rc = n2_adam_step_gated(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
+	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter)) return rc;
 	t->optimizer_steps += 1;
+	t->training_step += 1;
 	if (t->ema) {
-		return n2_ema_step(stream, t->n_params, t->cfg.ema_decay, t->optimizer_steps, reinterpret_cast<const n2_half*>(t->params), t->ema_tmp,
+		t->ema_steps += 1;
+		return n2_ema_step(stream, t->n_params, t->cfg.ema_decay, t->ema_steps, reinterpret_cast<const n2_half*>(t->params), t->ema_tmp,
 		                   reinterpret_cast<n2_half*>(t->ema));
 	}
 	return N2_OK;
@@ -377,6 +385,26 @@ N2_API int n2_trainer_optimizer_state(n2_trainer_t* t, n2_trainer_optimizer_buff
 	out->optimizer_steps = t->optimizer_steps;
 	out->learning_rate = t->cfg.adam.learning_rate;
 	return N2_OK;
+}
+
+__global__ void __launch_bounds__(256) trainer_restart_ema_kernel(uint32_t n, const hf* __restrict__ params, float* __restrict__ tmp, hf* __restrict__ ema) {
+	const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+	if (i < n) { tmp[i] = (float)params[i]; ema[i] = params[i]; }
+}
+
+N2_API int n2_trainer_restart_ema(n2_trainer_t* t, n2_stream_t stream, uint32_t ema_steps) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_restart_ema: trainer is null");
+	t->ema_steps = ema_steps;
+	if (t->ema == nullptr || ema_steps != 0) return N2_OK;
+	trainer_restart_ema_kernel<<<dim3((t->n_params + 255) / 256), dim3(256), 0, n2_stream(stream)>>>(t->n_params, t->params, t->ema_tmp, t->ema);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API int n2_trainer_set_training_step(n2_trainer_t* t, uint32_t step) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_set_training_step: trainer is null");
+	t->training_step = step;
+	return n2_grid_set_training_step(n2_field_encoding(t->field), step);
 }
 
 N2_API int n2_trainer_set_optimizer_steps(n2_trainer_t* t, uint32_t steps) {

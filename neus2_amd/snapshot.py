@@ -128,7 +128,10 @@ def _stream():
 
 
 def save_snapshot(path, trainer, occupancy=None, config=None, include_optimizer_state=False, loss=0.0, aabb_scale=1):
-    """Testbed::save_snapshot(path, include_optimizer_state)."""
+    """Testbed::save_snapshot(path, include_optimizer_state).  ``params_binary`` holds the WORKING parameters (what
+    tcnn's Trainer::serialize stores and training continues from); with the Ema wrapper on, the averaged weights that
+    inference uses travel in the optimizer state (``include_optimizer_state=True``), and a file saved without it
+    restarts the average from the working parameters when it is loaded."""
     d = SnapshotDesc()
     blob = pack_config(config) if config else b""
     keep = C.create_string_buffer(blob, len(blob)) if blob else None
@@ -190,11 +193,18 @@ def load_snapshot(path, trainer, occupancy=None, load_optimizer_state=True):
         if with_opt:
             check(L.n2_trainer_set_optimizer_steps(trainer._h, C.c_uint32(info.optimizer_steps)), "n2_trainer_set_optimizer_steps")
             check(L.n2_trainer_set_learning_rate(trainer._h, C.c_float(info.learning_rate)), "n2_trainer_set_learning_rate")
-            if t.d_ema_weights:
-                trainer.inference_params.copy_(trainer.ema_weights.half())
+        if with_opt and t.d_ema_weights:
+            # the moving average continues: its fp16 copy (the inference parameters) follows from the fp32 weights
+            trainer.inference_params.copy_(trainer.ema_weights.half())
+            check(L.n2_trainer_restart_ema(trainer._h, _stream(), C.c_uint32(info.optimizer_steps)), "n2_trainer_restart_ema")
+        else:
+            # no Ema state came with the file: the average starts again from the loaded parameters, so that the
+            # inference parameters are the loaded ones and the next step does not blend a stale average into them
+            check(L.n2_trainer_restart_ema(trainer._h, _stream(), C.c_uint32(0)), "n2_trainer_restart_ema")
         if occupancy is not None and info.density_grid_cells:
             occupancy.update_bitfield()  # update_density_grid_mean_and_bitfield, src/testbed.cu:3225-3227
         trainer.step_index = info.training_step
+        check(L.n2_trainer_set_training_step(trainer._h, C.c_uint32(info.training_step)), "n2_trainer_set_training_step")
         trainer.budget.rays_per_batch = info.rays_per_batch or trainer.budget.rays_per_batch
         trainer.budget.measured_before_compaction = info.measured_batch_size_before_compaction
         trainer.budget.measured = info.measured_batch_size

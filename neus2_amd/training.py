@@ -267,6 +267,8 @@ class Trainer:
         occ = getattr(self, "occupancy", None)
         if occ is None:
             return None
+        # the encoding's level mask is that of the step about to run (src/testbed.cu:2641-2647)
+        check(capi.lib().n2_trainer_set_training_step(self._h, C.c_uint32(self.step_index)), "n2_trainer_set_training_step")
         plan = density_grid_update_plan(self.step_index, occ.n_cascades)
         if plan is None:
             return None
@@ -281,6 +283,7 @@ class Trainer:
         n_rays = self.budget.rays_per_batch if n_rays is None else n_rays
         n_inference = self.budget.n_inference() if n_inference is None else n_inference
         seed = self.step_index if seed is None else seed
+        check(capi.lib().n2_trainer_set_training_step(self._h, C.c_uint32(self.step_index)), "n2_trainer_set_training_step")
         check(capi.lib().n2_trainer_step(self._h, self._stream(), C.c_uint32(n_rays), C.c_uint32(n_inference),
                                          C.c_uint32(seed)), "n2_trainer_step")
         self.step_index += 1

@@ -117,3 +117,56 @@ def test_loads_files_of_another_writer_and_checks_shapes(tmp_path):
     p.write_bytes(msgpack.packb(doc, use_bin_type=True))
     with pytest.raises(capi.N2Error, match="cascades"):
         load_snapshot(p, tr, tr.occupancy)
+
+
+def test_params_only_resume_restores_level_mask_and_restarts_ema(tmp_path):
+    """A snapshot without optimizer state still carries the training step: the progressive level mask of a trainer
+    restored from it is that step's (not the first step's), the occupancy update that precedes the next step already sees
+    it, and the Ema average starts again from the loaded parameters."""
+    from neus2_amd.snapshot import load_snapshot, save_snapshot
+    tr = make_trainer(ema=0.9)
+    tr.encoding().set_progressive(0.25, 0.125, 2)  # 4 levels, two more every 2 steps
+    run_steps(tr, 5)
+    path = tmp_path / "params_only.msgpack"
+    save_snapshot(path, tr, tr.occupancy, config=CONFIG, include_optimizer_state=False)
+    tr2 = make_trainer(ema=0.9)
+    enc = tr2.encoding()
+    enc.set_progressive(0.25, 0.125, 2)
+    assert enc.active_levels() == 4                      # step 0
+    info = load_snapshot(path, tr2, tr2.occupancy)
+    assert info.training_step == 5 and not info.has_optimizer_state
+    assert enc.active_levels() == 4 + 2 * (5 // 2)       # restored from the file's training step
+    torch.testing.assert_close(tr2.params, tr.params, rtol=0, atol=0)
+    # the inference parameters are the loaded ones, not the fresh trainer's initial average
+    torch.testing.assert_close(tr2.inference_params, tr2.params, rtol=0, atol=0)
+    # the first Ema step after the restart reproduces the working weights (bias-corrected average of one sample)
+    tr2.training_prep()
+    assert enc.active_levels() == 8                      # the occupancy update of step 5 ran under step 5's mask
+    tr2.step(n_rays=256, n_inference=1 << 17)
+    torch.testing.assert_close(tr2.ema_weights, tr2.params.float(), rtol=1e-6, atol=1e-9)
+    assert enc.active_levels() == 8
+    tr2.training_prep()
+    assert enc.active_levels() == 4 + 2 * (6 // 2)       # step 6
+
+
+def test_ema_round_trip_with_optimizer_state(tmp_path):
+    """With the Ema wrapper on and the optimizer state in the file, working and averaged weights both come back and the
+    moving average continues from the saved step count."""
+    from neus2_amd.snapshot import load_snapshot, save_snapshot
+    tr = make_trainer(ema=0.9)
+    run_steps(tr, 3)
+    path = tmp_path / "ema.msgpack"
+    save_snapshot(path, tr, tr.occupancy, config=CONFIG, include_optimizer_state=True)
+    tr2 = make_trainer(ema=0.9)
+    info = load_snapshot(path, tr2, tr2.occupancy)
+    assert info.has_optimizer_state and info.has_ema_weights
+    torch.testing.assert_close(tr2.params, tr.params, rtol=0, atol=0)
+    torch.testing.assert_close(tr2.ema_weights, tr.ema_weights, rtol=0, atol=0)
+    torch.testing.assert_close(tr2.inference_params, tr.inference_params, rtol=0, atol=0)
+    assert not torch.equal(tr.inference_params, tr.params)   # the average is not the working copy
+    # the average continues with the saved step count: one more step on identical inputs moves both trainers' averages alike
+    load_snapshot(path, tr, tr.occupancy)
+    for t in (tr, tr2):
+        t.step(n_rays=256, n_inference=1 << 17, seed=99)
+    torch.testing.assert_close(tr2.ema_weights, tr.ema_weights, rtol=0, atol=0)
+    torch.testing.assert_close(tr2.inference_params, tr.inference_params, rtol=0, atol=0)

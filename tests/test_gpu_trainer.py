@@ -201,3 +201,27 @@ def test_selected_activations_give_the_same_steps_as_a_second_forward():
         kinds.add("padded" if ca["compacted"] < T else "cut" if ca["compacted"] > T else "exact")
     assert {"padded", "cut"} <= kinds
     assert torch.equal(ma, mb)
+
+
+def test_step_without_samples_changes_nothing(setup):
+    """No ray finds an occupied cell: the step generates no sample and must not apply the previous step's gradients
+    again (the reference stops training on an empty batch, src/testbed_nerf.cu:3536-3542)."""
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    _, cams, rgba, bits, T = setup
+    tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=2048, max_samples=16 * T))
+    empty = torch.zeros(bits.size, dtype=torch.uint8, device="cuda")
+    full = dev(bits)
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), full)
+    tr.initialize_params(seed=5, sdf_mlp_weights=None)
+    tr.step(n_rays=300, n_inference=16 * T, seed=3)          # an ordinary step first: gradients and moments exist
+    assert tr.read_counters()["compacted"] > 0
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), empty)
+    master, params = tr.master.clone(), tr.params.clone()
+    st = tr.optimizer_state()
+    m1 = tr._view(st.first_moments, tr.n_params, torch.float32).clone()
+    tr.step(n_rays=300, n_inference=16 * T, seed=4)
+    c = tr.read_counters()
+    assert c["samples"] == 0 and c["compacted"] == 0
+    assert torch.equal(tr.master, master) and torch.equal(tr.params, params)
+    assert torch.equal(tr._view(st.first_moments, tr.n_params, torch.float32), m1)
