@@ -614,6 +614,20 @@ int n2_trainer_invalidate_prefetch(n2_trainer_t* trainer);
  *  seed         seed of this step's random draws */
 int n2_trainer_step(n2_trainer_t* trainer, n2_stream_t stream, uint32_t n_rays, uint32_t n_inference, uint32_t seed);
 
+/* Device buffers of the last step, for inspection and tests (the reference keeps the same data in its arena allocation,
+ * src/testbed_nerf.cu:3723-3749): valid until the next step overwrites them. */
+typedef struct n2_trainer_step_view {
+	const float* coords;              /* [marched samples][7] of the step's sample set */
+	const uint32_t* numsteps;         /* [rays][2] after compositing: (kept samples, first compacted sample) per live ray */
+	const float* rgb_target;          /* [rays][3] */
+	const uint32_t* ray_indices;      /* [rays] */
+	const n2_half* network_output;    /* [n_inference][16] field output over the marched samples */
+	const float* coords_compacted;    /* [target_batch_size][7] after the roll-over */
+	const n2_half* dloss_doutput;     /* [target_batch_size][16] after the roll-over */
+	const uint32_t* source_index;     /* [target_batch_size] marched sample behind every compacted sample */
+} n2_trainer_step_view;
+int n2_trainer_last_step_view(n2_trainer_t* trainer, n2_trainer_step_view* out);
+
 /* Waits for the stream, then returns the last step's counters: live rays, marched samples, samples the
  * rays wanted to keep (before the clamp to target_batch_size), and the summed loss
  * (counters.update_after_training, src/testbed_nerf.cu:3406-3429). */

@@ -56,6 +56,13 @@ class TrainerOptimizerBuffers(C.Structure):
                 ("learning_rate", C.c_float)]
 
 
+class TrainerStepView(C.Structure):
+    """struct n2_trainer_step_view"""
+    _fields_ = [("coords", C.c_void_p), ("numsteps", C.c_void_p), ("rgb_target", C.c_void_p), ("ray_indices", C.c_void_p),
+                ("network_output", C.c_void_p), ("coords_compacted", C.c_void_p), ("dloss_doutput", C.c_void_p),
+                ("source_index", C.c_void_p)]
+
+
 class OccupancyBuffers(C.Structure):
     """struct n2_occupancy_buffers"""
     _fields_ = [("density_grid", C.c_void_p), ("density_grid_tmp", C.c_void_p), ("bitfield", C.c_void_p), ("mean", C.c_void_p),

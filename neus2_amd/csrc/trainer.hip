@@ -413,6 +413,20 @@ N2_API int n2_trainer_set_optimizer_steps(n2_trainer_t* t, uint32_t steps) {
 	return N2_OK;
 }
 
+N2_API int n2_trainer_last_step_view(n2_trainer_t* t, n2_trainer_step_view* out) {
+	N2_REQUIRE(t != nullptr && out != nullptr, "n2_trainer_last_step_view: null argument");
+	const n2_trainer::SampleSet& set = t->sets[t->last_set];
+	out->coords = set.coords;
+	out->numsteps = set.numsteps;
+	out->rgb_target = set.rgb_target;
+	out->ray_indices = set.ray_indices;
+	out->network_output = reinterpret_cast<const n2_half*>(t->mlp_out);
+	out->coords_compacted = t->coords_compacted;
+	out->dloss_doutput = reinterpret_cast<const n2_half*>(t->dloss);
+	out->source_index = t->src_index;
+	return N2_OK;
+}
+
 N2_API int n2_trainer_read_counters(n2_trainer_t* t, n2_stream_t stream, uint32_t* rays, uint32_t* samples, uint32_t* compacted, float* loss) {
 	N2_REQUIRE(t != nullptr, "n2_trainer_read_counters: trainer is null");
 	uint32_t host[8] = {};

@@ -312,6 +312,21 @@ class Trainer:
         s = self.optimizer_state()
         return None if not s.ema_weights else self._view(s.ema_weights, self.n_params, torch.float32)
 
+    def last_step(self, n_rays, n_samples, n_inference):
+        """Tensors (views into the workspace) of the last step's buffers: see n2_trainer_step_view.  n_rays / n_samples:
+        the step's live rays and marched samples (read_counters), n_inference: the forward batch it was called with."""
+        v = capi.TrainerStepView()
+        check(capi.lib().n2_trainer_last_step_view(self._h, C.byref(v)), "n2_trainer_last_step_view")
+        T = self.cfg.target_batch_size
+        return dict(coords=self._view(v.coords, n_samples * 7, torch.float32).view(-1, 7),
+                    numsteps=self._view(v.numsteps, n_rays * 2, torch.int32).view(-1, 2),
+                    rgb_target=self._view(v.rgb_target, n_rays * 3, torch.float32).view(-1, 3),
+                    ray_indices=self._view(v.ray_indices, n_rays, torch.int32),
+                    network_output=self._view(v.network_output, n_inference * 16, torch.float16).view(-1, 16),
+                    coords_compacted=self._view(v.coords_compacted, T * 7, torch.float32).view(-1, 7),
+                    dloss_doutput=self._view(v.dloss_doutput, T * 16, torch.float16).view(-1, 16),
+                    source_index=self._view(v.source_index, T, torch.int32))
+
     def read_counters(self):
         r, s, c, l = C.c_uint32(), C.c_uint32(), C.c_uint32(), C.c_float()
         check(capi.lib().n2_trainer_read_counters(self._h, self._stream(), C.byref(r), C.byref(s), C.byref(c), C.byref(l)),

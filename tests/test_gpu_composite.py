@@ -104,3 +104,16 @@ def test_empty(oracle):
     r = composite_loss(torch.zeros((0, 2), dtype=torch.int32, device="cuda"), torch.zeros((0, 16), dtype=torch.float16, device="cuda"),
                        torch.zeros((0, 7), device="cuda"), torch.zeros((0, 3), device="cuda"), 64)
     assert int(host(r["counter"])[0]) == 0
+
+
+def test_cos_anneal_ratio_below_one(oracle):
+    """cos_anneal_ratio < 1 blends the two cosine terms (nerf_network.h:1109-1118, src/testbed_nerf.cu:1583-1590)."""
+    rng = np.random.default_rng(8)
+    numsteps, out, coords, target = make_rays(rng, 1500, lo=1, hi=120, sharp=True)
+    results = {}
+    for ratio in (0.5, 0.0):
+        ref, got = run_both(oracle, numsteps, out, coords, target, 1 << 18, cos_anneal_ratio=ratio, ek_loss_weight=0.01)
+        compare(ref, got, numsteps, max_count_mismatch=1)
+        results[ratio] = ref["dloss"]
+    ref1 = oracle.composite_loss(numsteps, q16(out), coords, target, 1 << 18, cos_anneal_ratio=1.0, ek_loss_weight=0.01)
+    assert not np.allclose(results[0.5][:, 3], ref1["dloss"][:, 3])  # the ratio matters for these rays

@@ -79,7 +79,9 @@ def test_backward_full_config(oracle):
     assert_grad_close(got[of.off_sdf:of.off_rgb], ref[of.off_sdf:of.off_rgb], what="SDF MLP gradients (1st + 2nd order)",
                       rtol=2 * RTOL)
     assert_grad_close(got[of.off_rgb:of.off_grid], ref[of.off_rgb:of.off_grid], what="colour MLP gradients", rtol=2 * RTOL)
-    assert abs(got[of.off_var] - ref[of.off_var]) <= RTOL * abs(ref[of.off_var]) + 0.05, (got[of.off_var], ref[of.off_var])
+    # one fp16 rounding of a sum accumulated in fp32
+    var_floor = 1e-5 * float(np.abs(dL[7]).sum()) + 1e-6
+    assert abs(got[of.off_var] - ref[of.off_var]) <= RTOL * abs(ref[of.off_var]) + var_floor, (got[of.off_var], ref[of.off_var])
     for l in range(16):
         a = of.off_grid + 2 * int(of.grid.offset[l])
         b = of.off_grid + 2 * int(of.grid.offset[l + 1])
@@ -92,7 +94,7 @@ def test_backward_full_config(oracle):
     assert rel_l2(got2[:of.off_grid], 2 * ref[:of.off_grid]) < 3 * RTOL
     assert rel_l2(got2[of.off_grid:of.off_var], 2 * ref[of.off_grid:of.off_var]) < 2e-2
     # ... the variance gradient too (every backward sums its own batch, nothing is left over from the first call)
-    assert abs(got2[of.off_var] - 2 * ref[of.off_var]) <= 2 * RTOL * abs(ref[of.off_var]) + 0.1, (got2[of.off_var], ref[of.off_var])
+    assert abs(got2[of.off_var] - 2 * ref[of.off_var]) <= 3 * RTOL * abs(ref[of.off_var]) + 2 * var_floor, (got2[of.off_var], ref[of.off_var])
 
 
 def test_backward_reference_14_level_config(oracle):
@@ -207,3 +209,35 @@ def test_padding_rows_follow_the_batch_size(oracle):
     assert np.isfinite(got).all()
     assert_grad_close(got[of.off_sdf:of.off_rgb], ref[of.off_sdf:of.off_rgb], what="SDF MLP gradients", rtol=2 * RTOL)
     assert_grad_close(got[of.off_rgb:of.off_grid], ref[of.off_rgb:of.off_grid], what="colour MLP gradients", rtol=2 * RTOL)
+
+
+def test_direction_encoding_rows(oracle):
+    """The degree-4 spherical-harmonics rows of the colour net's input on their own: with every other input column of
+    the colour net's first layer zeroed, the output depends on the direction only through the 16 SH rows, and a net whose
+    hidden layers pass values through unchanged hands them to the output."""
+    from neus2_amd.tcnn_api import NerfNetwork
+    from oracle.field import Field
+    of, gf = Field(fp16=True), NerfNetwork()
+    rng = np.random.default_rng(4)
+    p = np.zeros(of.n_params, np.float32)
+    # colour net: W0 [64][48] picks SH row k (input column 16 + k) into neurons 2k (+) and 2k + 1 (-), the second layer is
+    # the identity, the output layer recombines relu(x) - relu(-x) = x for the first 16 SH values
+    W0 = np.zeros((64, 48), np.float32)
+    W1 = np.eye(64, dtype=np.float32)
+    Wo = np.zeros((16, 64), np.float32)
+    for k in range(16):
+        W0[2 * k, 16 + k], W0[2 * k + 1, 16 + k] = 1.0, -1.0
+        Wo[k, 2 * k], Wo[k, 2 * k + 1] = 1.0, -1.0
+    p[of.off_rgb:of.off_grid] = np.concatenate([W0.ravel(), W1.ravel(), Wo.ravel()])
+    p[of.off_sdf:of.off_rgb] = rng.standard_normal(of.off_rgb) * 0.1
+    p[of.off_grid:of.off_var] = rng.uniform(-0.1, 0.1, of.grid.n_params)
+    p = q16(p)
+    dp = dev(p, torch.float16)
+    gf.set_params(dp, torch.zeros_like(dp))
+    n = 4096
+    coords = rand_coords(rng, n)
+    out = host(gf.forward(dev(coords))).T
+    sh = oracle.sh4(np.ascontiguousarray(coords[:, 4:7].T))           # pinned by scipy.special.sph_harm_y
+    # rows 0..2 and 11..15 of the output are the colour net's own rows (3..10 are overwritten by sdf, normal, ...)
+    for r in (0, 1, 2, 11, 12, 13, 14, 15):
+        assert_close(out[r], q16(sh[r]), rtol=RTOL, what=f"SH row {r}", scale=1.0)
