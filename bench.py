@@ -280,8 +280,7 @@ def run_sdf_workload(args):
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "hash grid + SDF MLP 48-64-16, forward, normals, first and second order backward of "
-                                   "mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 (BASELINE configs[2]); 2^18 uniform points; element-wise "
-                                   "glue between the kernels runs in torch and is inside the wall clock",
+                                   "mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 (BASELINE configs[2]); 2^18 uniform points",
                        "batch": TARGET, "loss": float(loss), "kernel_ms_per_step": total},
             "roofline": {"kernel": "grid_backward_params (merged first+second order scatter)", "bound": "hbm", "achieved": achieved,
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,

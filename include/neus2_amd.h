@@ -376,6 +376,27 @@ int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, 
                      uint32_t dim_stride, uint32_t n, n2_half* d_output);
 
 /* ------------------------------------------------------------------------
+ * The SDF network trained on its own with the eikonal term (no colour branch): the element-wise steps that
+ * NerfNetwork performs between the encoding's and the network's calls, for a caller that composes
+ * n2_grid_* and n2_mlp_* itself (this repository's neus2_amd/sdf_net.py, BASELINE configuration 3):
+ *   n2_sdf_pack_input     rows 0..2 of the network input = (T)x - (T)0.5 and zero padding rows behind the encoding
+ *                         (fill_positions_view_with_fixed_offset, nerf_network.h:193-195, common_operation.cuh:186-199)
+ *   n2_sdf_eikonal_loss   d_normal_encoding holds the encoding's backward of rows 3.. of d sdf / d input (n2_grid_backward
+ *                         with d_dL_dx, nerf_network.h:230-234); the call writes d_normal = that + rows 0..2 of
+ *                         d sdf / d input (add_positions_view, :236-238; the two may be the same buffer), forms  loss = mean |sdf| + ek_weight mean (|normal| - 1)^2  and writes what the backward
+ *                         passes take: d_dL_doutput (fp16 SoA 16 x n: row 0 = sign(sdf) loss_scale / n), d_dL_dnormal
+ *                         (fp32 SoA 3 x n, times loss_scale) and rows 0..2 and the padding rows of the network's
+ *                         second-order input (fp16 SoA input_width x n, nerf_network.h:546-557; rows 3.. are the encoding's
+ *                         dL_ddLdoutput, written by n2_grid_backward_fused).  d_loss: one float.
+ * ---------------------------------------------------------------------- */
+int n2_sdf_pack_input(n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n,
+                      uint32_t encoding_width, uint32_t input_width, n2_half* d_input);
+uint64_t n2_sdf_eikonal_workspace_bytes(uint32_t n);
+int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding_width, uint32_t input_width, const n2_half* d_sdf_output,
+                        const n2_half* d_dsdf_dinput, const float* d_normal_encoding, float* d_normal, float ek_weight, float loss_scale, n2_half* d_dL_doutput,
+                        float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
  * Adam on fp32 master weights with an fp16 working copy: tcnn's Adam as the
  * trainer runs it, Trainer::optimizer_step(stream, LOSS_SCALE) at
  * src/testbed_nerf.cu:3498, hyper-parameters from configs/nerf/base.json:13-26

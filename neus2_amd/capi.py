@@ -115,6 +115,8 @@ def lib():
         _lib.n2_composite_workspace_bytes.argtypes = [C.c_uint32]
         _lib.n2_sampler_workspace_bytes.restype = C.c_uint64
         _lib.n2_sampler_workspace_bytes.argtypes = [C.c_uint32]
+        _lib.n2_sdf_eikonal_workspace_bytes.restype = C.c_uint64
+        _lib.n2_sdf_eikonal_workspace_bytes.argtypes = [C.c_uint32]
         _lib.n2_trainer_workspace_bytes.restype = C.c_uint64
         _lib.n2_trainer_workspace_bytes.argtypes = [C.c_void_p]
         _lib.n2_trainer_destroy.restype = None

@@ -555,6 +555,104 @@ int n2_field_select_borrow(n2_field_t* f, const uint32_t* d_source_index, uint32
 	return N2_OK;
 }
 
+// ----------------------------------------------------------------------------
+// The SDF network on its own with the eikonal term (no colour branch): the glue between the encoding's and the
+// network's kernels, i.e. what NerfNetwork does with small element-wise kernels at nerf_network.h:193-199 (input),
+// :230-238 (normal = encoding backward of d sdf / d encoding, plus the direct coordinate rows) and :546-557 (input of
+// the network's second-order pass), with the loss  mean |sdf| + w_ek mean (|normal| - 1)^2  in between.
+// ----------------------------------------------------------------------------
+__global__ void __launch_bounds__(FB) sdf_pack_input_kernel(const float* __restrict__ xyz, uint32_t ps, uint32_t ds, uint32_t N, uint32_t first_pad,
+                                                            uint32_t in_w, hf* __restrict__ input) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i >= N) return;
+	const float* q = xyz + (size_t)i * ps;
+#pragma unroll
+	for (int d = 0; d < 3; ++d) input[(size_t)d * N + i] = (hf)q[(size_t)d * ds] - (hf)0.5f;
+	for (uint32_t r = first_pad; r < in_w; ++r) input[(size_t)r * N + i] = (hf)0;
+}
+
+__global__ void __launch_bounds__(FB) sdf_eikonal_loss_kernel(uint32_t N, uint32_t first_pad, uint32_t in_w, const hf* __restrict__ sdf_out,
+                                                              const hf* __restrict__ g, const float* __restrict__ normal_enc, float* __restrict__ normal, float ek_weight, float scale,
+                                                              hf* __restrict__ dL_dy, float* __restrict__ v, hf* __restrict__ v_in,
+                                                              float* __restrict__ parts) {
+	__shared__ float part[FB / 64];
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	float term = 0.f;
+	if (i < N) {
+		const float sdf = (float)sdf_out[i];
+		float nrm[3], len2 = 0.f;
+#pragma unroll
+		for (int d = 0; d < 3; ++d) {
+			nrm[d] = normal_enc[(size_t)d * N + i] + (float)g[(size_t)d * N + i];  // add_positions_view: the direct coordinate rows
+			normal[(size_t)d * N + i] = nrm[d];
+			len2 = fmaf(nrm[d], nrm[d], len2);
+		}
+		const float len = fmaxf(sqrtf(len2), 1e-12f);
+		term = fabsf(sdf) + ek_weight * (len - 1.f) * (len - 1.f);
+		dL_dy[i] = (hf)((sdf > 0.f ? 1.f : sdf < 0.f ? -1.f : 0.f) * scale);
+		for (uint32_t r = 1; r < 16; ++r) dL_dy[(size_t)r * N + i] = (hf)0;
+		const float k = 2.f * ek_weight * (len - 1.f) / len * scale;
+#pragma unroll
+		for (int d = 0; d < 3; ++d) {
+			const float x = nrm[d] * k;  // d loss / d normal
+			v[(size_t)d * N + i] = x;
+			v_in[(size_t)d * N + i] = (hf)x;
+		}
+		for (uint32_t r = first_pad; r < in_w; ++r) v_in[(size_t)r * N + i] = (hf)0;
+	}
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) term += __shfl_xor(term, o);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = term;
+	__syncthreads();
+	if (threadIdx.x == 0) parts[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// loss = sum of the workgroups' partial sums / N, in a fixed order
+__global__ void __launch_bounds__(256) sdf_loss_sum_kernel(const float* __restrict__ parts, uint32_t n_parts, float inv_n, float* __restrict__ loss) {
+	__shared__ float part[4];
+	float s = 0.f;
+	for (uint32_t i = threadIdx.x; i < n_parts; i += 256) s += parts[i];
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if (threadIdx.x == 0) loss[0] = ((part[0] + part[1]) + (part[2] + part[3])) * inv_n;
+}
+
+N2_API int n2_sdf_pack_input(n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n, uint32_t encoding_width,
+                             uint32_t input_width, n2_half* d_input) {
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_xyz != nullptr && d_input != nullptr, "n2_sdf_pack_input: null buffer");
+	N2_REQUIRE(point_stride >= 1 && dim_stride >= 1, "n2_sdf_pack_input: strides must be >= 1");
+	N2_REQUIRE(input_width >= 3 + encoding_width && input_width <= 64, "n2_sdf_pack_input: input width %u does not hold 3 + %u rows", input_width, encoding_width);
+	sdf_pack_input_kernel<<<fgrid(n), dim3(FB), 0, n2_stream(stream)>>>(d_xyz, point_stride, dim_stride, n, 3 + encoding_width, input_width,
+	                                                                   reinterpret_cast<hf*>(d_input));
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+N2_API uint64_t n2_sdf_eikonal_workspace_bytes(uint32_t n) { return 4ull * ((n + FB - 1) / FB + 1); }
+
+N2_API int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding_width, uint32_t input_width, const n2_half* d_sdf_output,
+                               const n2_half* d_dsdf_dinput, const float* d_normal_encoding, float* d_normal, float ek_weight, float loss_scale, n2_half* d_dL_doutput,
+                               float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes) {
+	N2_REQUIRE(n > 0, "n2_sdf_eikonal_loss: empty batch");
+	N2_REQUIRE(d_sdf_output && d_dsdf_dinput && d_normal_encoding && d_normal && d_dL_doutput && d_dL_dnormal && d_second_order_input && d_loss && d_workspace,
+	           "n2_sdf_eikonal_loss: null buffer");
+	N2_REQUIRE(input_width >= 3 + encoding_width && input_width <= 64, "n2_sdf_eikonal_loss: input width %u does not hold 3 + %u rows", input_width, encoding_width);
+	N2_REQUIRE(workspace_bytes >= n2_sdf_eikonal_workspace_bytes(n), "n2_sdf_eikonal_loss: workspace of %llu bytes, %llu needed",
+	           (unsigned long long)workspace_bytes, (unsigned long long)n2_sdf_eikonal_workspace_bytes(n));
+	hipStream_t s = n2_stream(stream);
+	float* parts = reinterpret_cast<float*>(d_workspace);
+	sdf_eikonal_loss_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, 3 + encoding_width, input_width, reinterpret_cast<const hf*>(d_sdf_output),
+	                                                      reinterpret_cast<const hf*>(d_dsdf_dinput), d_normal_encoding, d_normal, ek_weight, loss_scale / (float)n,
+	                                                      reinterpret_cast<hf*>(d_dL_doutput), d_dL_dnormal, reinterpret_cast<hf*>(d_second_order_input), parts);
+	N2_LAUNCH_CHECK();
+	sdf_loss_sum_kernel<<<dim3(1), dim3(256), 0, s>>>(parts, fgrid(n).x, 1.f / (float)n, d_loss);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
 static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n,
                           n2_half* d_output, bool density) {
 	if (int rc = check_field(f, fn, n)) return rc;

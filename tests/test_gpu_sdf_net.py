@@ -61,7 +61,7 @@ def test_sdf_eikonal_step_matches_oracle(oracle, kind):
     gP, gW = torch.zeros_like(dP), torch.zeros_like(dW)
     net.set_params(dP, gP, dW, gW)
     ctx = net.forward(dev(x))
-    loss = float(net.loss_backward(ctx, ek_weight=0.1, loss_scale=128.0))
+    loss = float(net.loss_backward(ctx, ek_weight=0.1, loss_scale=128.0).item())
     ref = oracle_step(oracle, P, W, x, 0.1, 128.0)
     assert_close(host(ctx["sdf"]), ref["sdf"], what="sdf", outlier_frac=1e-3)
     assert_close(host(ctx["normal"]), ref["normal"], what="normal", outlier_frac=2e-3)
