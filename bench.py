@@ -37,7 +37,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 # scatter pair = bin (43.2 + 105.9 MiB) + reduce (110.9 + 24.0 MiB); forward = 82.3 + 115.2 MiB
 STEP_TRAFFIC_BYTES = {"grid_backward_params": int(283.9 * 2**20), "grid_forward": int(197.6 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
-        "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8}
+        "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9}
 
 
 def build_scene(n_cameras=64, resolution=512):
@@ -55,8 +55,10 @@ def profile_read(lib, name):
     return float(ms.value), int(n.value)
 
 
-def cpu_baseline(cams, rgba, bits, sdf_weights, budget_s=20.0):
-    """The oracle's full training step on the host cores, on a bounded sample of the same workload."""
+def cpu_baseline(cams, rgba, bits, sdf_weights, n_rays, n_inference, budget_s=20.0):
+    """The oracle's full training step on the host cores at the benchmark's own batch: the same scene, initialisation,
+    ray count and 2^18 target as the GPU's timed steps (one step is about 1.5 s on 16 threads, so the bounded sample is a
+    few whole steps)."""
     import numpy as np
     from oracle import oracle as orc
     from oracle.field import Field
@@ -71,18 +73,16 @@ def cpu_baseline(cams, rgba, bits, sdf_weights, budget_s=20.0):
         po = int(c["pixel_offset"])
         ocams.append(orc.Camera((orc.C.c_float * 12)(*c["xform"]), (orc.C.c_float * 2)(*c["focal"]),
                                 (orc.C.c_float * 2)(*c["principal"]), (orc.C.c_uint32 * 2)(*c["res"]), po & 0xFFFFFFFF, po >> 32))
-    T = 1 << 15
-    n_rays = 768  # about 45% of the rays hit the shell, ~115 marched samples each -> a little over T samples
     best, done, t_all = None, 0, time.time()
-    while done < 3 or (time.time() - t_all < budget_s and done < 8):
+    while done < 2 or (time.time() - t_all < budget_s and done < 8):
         t0 = time.time()
-        r = training_step(st, ocams, rgba, bits, n_rays, 16 * T, seed=done, target_batch_size=T)
+        r = training_step(st, ocams, rgba, bits, n_rays, n_inference, seed=done, target_batch_size=TARGET)
         dt = time.time() - t0
         best = dt if best is None else min(best, dt)
         done += 1
-    return {"value": T / best, "unit": "samples/s", "cores": orc.num_threads(), "kind": "port",
-            "sample": f"one full training step at a 2^15-sample batch ({r['rays']} rays, {r['samples']} marched samples, "
-                      f"same scene and initialisation), best of {done} runs, {best * 1e3:.0f} ms"}
+    return {"value": TARGET / best, "unit": "samples/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": f"{done} full training steps at the benchmark's 2^18-sample batch ({r['rays']} rays, {r['samples']} marched samples, "
+                      f"same scene and initialisation), best step {best * 1e3:.0f} ms"}
 
 
 def run_step_workload(args):
@@ -186,9 +186,66 @@ def run_step_workload(args):
         "kernels_note": "grid_backward_params is timed with HIP events inside the timed region (every fourth step's launch); the other entries come from a "
                         "second, untimed pass of the same steps with every listed kernel bracketed by events",
     }
+    # untimed extras (the driver's fields above come from the one timed region before them)
+    # (i) spread: further regions of K steps each, every one bracketed like the timed region
+    regions = [elapsed / args.steps * 1e3]
+    for _ in range(args.extra_regions):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            tr.step(n_rays=n_rays, n_inference=n_inf)
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0) / args.steps * 1e3)
+    srt = sorted(regions)
+    result["regions"] = {"ms_per_step": regions, "median": srt[len(srt) // 2], "min": srt[0], "max": srt[-1],
+                         "note": f"{len(regions)} consecutive regions of {args.steps} steps; the first one is the timed region of `value`"}
+    # (ii) the same loop on a trained field: rays stop at the surface, so a step marches more samples than it keeps
+    if args.trained_steps > 0:
+        result["trained_state"] = trained_state_leg(tr, args, lib)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cams, rgba, bits, sdf_w)
+        result["cpu_baseline"] = cpu_baseline(cams, rgba, bits, sdf_w, n_rays, n_inf)
     return result
+
+
+def trained_state_leg(tr, args, lib):
+    """Trains the benchmark's scene for args.trained_steps steps at learning rate 1e-2 (configs/nerf/dtu.json:15) with the ray
+    budget's feedback every 20 steps, then times K steps exactly like the main region."""
+    import ctypes as C
+    import torch
+    from neus2_amd.capi import check
+    check(lib.n2_trainer_set_learning_rate(tr._h, C.c_float(1e-2)), "n2_trainer_set_learning_rate")
+    for it in range(args.trained_steps):
+        tr.step()
+        if it % 20 == 19:
+            counters, ok = tr.update_budget()
+            if not ok:
+                return {"error": f"no samples at step {it}: {counters}"}
+    n_rays, n_inf = tr.budget.rays_per_batch, tr.budget.n_inference()
+    for _ in range(args.warmup):
+        tr.step(n_rays=n_rays, n_inference=n_inf)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        tr.step(n_rays=n_rays, n_inference=n_inf)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    c = tr.read_counters()
+    return {"ms_per_step": elapsed / args.steps * 1e3, "value": args.steps * min(c["compacted"], TARGET) / elapsed, "unit": "samples/s",
+            "trained_steps": args.trained_steps, "rays_per_step": n_rays, "marched_samples_per_step": c["samples"], "inference_batch": n_inf,
+            "compacted_before_rollover": c["compacted"], "loss": c["loss"],
+            "note": "same timed loop after training; `value` counts the samples the rays kept (the batch is padded to 2^18 by rollover)"}
+
+
+def timed_best(fn, budget_s=15.0, min_runs=2, max_runs=8):
+    """Best wall time of fn() over a bounded number of runs (host-side baselines)."""
+    best, done, t_all = None, 0, time.time()
+    while done < min_runs or (time.time() - t_all < budget_s and done < max_runs):
+        t0 = time.time()
+        fn()
+        dt = time.time() - t0
+        best = dt if best is None else min(best, dt)
+        done += 1
+    return best, done
 
 
 def run_grid_workload(args):
@@ -227,13 +284,28 @@ def run_grid_workload(args):
         kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
     dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
     achieved = ALGO_BYTES[dom] * TARGET / (kernels[dom]["avg_us"] * 1e-6) / 1e9
-    return {"metric": "hash-grid fwd+bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": "hash-grid encoding only, forward + backward (BASELINE configs[1])", "batch": TARGET},
-            "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": achieved / HBM_PEAK_GBS, "traffic": None},
-            "kernels": kernels}
+    result = {"metric": "hash-grid fwd+bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
+              "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+              "config": {"workload": "hash-grid encoding only, forward + backward (BASELINE configs[1])", "batch": TARGET},
+              "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": ALGO_BYTES[dom],
+                           "samples_per_launch": TARGET, "avg_launch_us": kernels[dom]["avg_us"]},
+              "kernels": kernels}
+    if not args.no_cpu_baseline:
+        from oracle import oracle as orc
+        og = orc.Grid()
+        P, xs, dys = params.float().cpu().numpy(), x.cpu().numpy(), dy.float().cpu().numpy()
+
+        def cpu_step():
+            og.forward(P, xs, want_dy_dx=True)
+            og.backward(P, xs, dys)
+
+        best, done = timed_best(cpu_step)
+        result["cpu_baseline"] = {"value": TARGET / best, "unit": "samples/s", "cores": orc.num_threads(), "kind": "port",
+                                  "sample": f"the same 2^18 points and gradients: forward with dy_dx + backward (parameters and input), "
+                                            f"best of {done} runs, {best * 1e3:.0f} ms"}
+    return result
 
 
 def run_sdf_workload(args):
@@ -276,17 +348,26 @@ def run_sdf_workload(args):
             total += ms / args.steps
     sc = kernels["grid_backward_params"]["avg_us"] * 1e-6
     achieved = ALGO_BYTES["grid_second_order"] * TARGET / sc / 1e9
-    return {"metric": "SDF net + eikonal fwd/bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": "hash grid + SDF MLP 48-64-16, forward, normals, first and second order backward of "
-                                   "mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 (BASELINE configs[2]); 2^18 uniform points",
-                       "batch": TARGET, "loss": float(loss), "kernel_ms_per_step": total},
-            "roofline": {"kernel": "grid_backward_params (merged first+second order scatter)", "bound": "hbm", "achieved": achieved,
-                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                         "algorithmic_bytes_per_sample": ALGO_BYTES["grid_second_order"], "samples_per_launch": TARGET,
-                         "avg_launch_us": kernels["grid_backward_params"]["avg_us"]},
-            "kernels": kernels}
+    result = {"metric": "SDF net + eikonal fwd/bwd samples/sec @2^18 batch (1 GPU)", "value": args.steps * TARGET / elapsed, "unit": "samples/s",
+              "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+              "config": {"workload": "hash grid + SDF MLP 48-64-16, forward, normals, first and second order backward of "
+                                     "mean|sdf| + 0.1 mean(|grad sdf| - 1)^2 (BASELINE configs[2]); 2^18 uniform points",
+                         "batch": TARGET, "loss": float(loss), "kernel_ms_per_step": total},
+              "roofline": {"kernel": "grid_backward_params (merged first+second order scatter)", "bound": "hbm", "achieved": achieved,
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                           "algorithmic_bytes_per_sample": ALGO_BYTES["grid_second_order"], "samples_per_launch": TARGET,
+                           "avg_launch_us": kernels["grid_backward_params"]["avg_us"]},
+              "kernels": kernels}
+    if not args.no_cpu_baseline:
+        from oracle import oracle as orc
+        from oracle.sdf_step import sdf_eikonal_step
+        Pn, Wn, xn = P.float().cpu().numpy(), W.float().cpu().numpy(), x.cpu().numpy()
+        best, done = timed_best(lambda: sdf_eikonal_step(Pn, Wn, xn, 0.1, 128.0))
+        result["cpu_baseline"] = {"value": TARGET / best, "unit": "samples/s", "cores": orc.num_threads(), "kind": "port",
+                                  "sample": f"the same 2^18 points, one forward + normals + first and second order backward, best of {done} "
+                                            f"runs, {best * 1e3:.0f} ms"}
+    return result
 
 
 def run_lattice_workload(args):
@@ -330,25 +411,47 @@ def run_lattice_workload(args):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.n2_profile_enable(0)
+    kernels, dom, dom_us, algo = inference_kernels(lib, args.steps)
+    achieved = algo * CH / (dom_us * 1e-6) / 1e9
+    mlp_us = dom_us if dom == "field_forward" else kernels["mlp_forward"]["avg_us"]
+    mlp_tflops = 8192 * CH / (mlp_us * 1e-6) / 1e12
+    result = {"metric": "SDF inference points/sec over a 512^3 lattice in 2^22-point chunks (1 GPU)", "value": args.steps * CH / elapsed,
+              "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+              "config": {"workload": "hash grid + SDF MLP forward over the 512^3 lattice (BASELINE configs[4]), geometric-init SDF MLP, "
+                                     "grid U(-1e-4, 1e-4) seed 1", "chunk": CH, "chunks_in_lattice": n_chunks,
+                         "sdf_mean_abs": float(out[0].float().abs().mean())},
+              "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": algo,
+                           "samples_per_launch": CH, "avg_launch_us": dom_us},
+              "mfma": {"kernel": "SDF net 48-64-16 forward" + (" (inside the fused launch)" if dom == "field_forward" else ""), "flops_per_sample": 8192,
+                       "achieved_tflops": mlp_tflops, "peak_tflops": MFMA_PEAK_TFLOPS, "frac": mlp_tflops / MFMA_PEAK_TFLOPS},
+              "kernels": kernels}
+    if not args.no_cpu_baseline:
+        from oracle import oracle as orc
+        from oracle.field import Field
+        f = Field(fp16=True)
+        sub = 128
+        gi = np.arange(sub ** 3, dtype=np.int64)
+        sx = np.stack(((gi % sub) / sub, ((gi // sub) % sub) / sub, (gi // (sub * sub)) / sub)).astype(np.float32)
+        p16 = params.float().cpu().numpy()
+        best, done = timed_best(lambda: f.sdf_values(p16, sx))
+        result["cpu_baseline"] = {"value": sub ** 3 / best, "unit": "points/s", "cores": orc.num_threads(), "kind": "port",
+                                  "sample": f"the 128^3 lattice p = (i, j, k) / 128 of the same network (1/64 of the points), best of {done} "
+                                            f"runs, {best * 1e3:.0f} ms"}
+    return result
+
+
+def inference_kernels(lib, steps):
+    """Event timings of an inference workload's launches: the fused launch (grid gather + SDF net in one kernel,
+    algorithmic bytes 12 xyz + 128 x 4 gathers + 32 output = 556 per point) or the grid forward (588) followed by the MLP."""
     kernels = {}
-    for name in ("grid_forward", "mlp_forward"):
+    for name in ("field_forward", "grid_forward", "mlp_forward"):
         ms, n = profile_read(lib, name)
-        kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
-    gf = kernels["grid_forward"]["avg_us"] * 1e-6
-    achieved = (12 + 128 * 4 + 64) * CH / gf / 1e9
-    mlp_tflops = 8192 * CH / (kernels["mlp_forward"]["avg_us"] * 1e-6) / 1e12
-    return {"metric": "SDF inference points/sec over a 512^3 lattice in 2^22-point chunks (1 GPU)", "value": args.steps * CH / elapsed,
-            "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": "hash grid + SDF MLP forward over the 512^3 lattice (BASELINE configs[4]), geometric-init SDF MLP, "
-                                   "grid U(-1e-4, 1e-4) seed 1", "chunk": CH, "chunks_in_lattice": n_chunks,
-                       "sdf_mean_abs": float(out[0].float().abs().mean())},
-            "roofline": {"kernel": "grid_forward", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": 588,
-                         "samples_per_launch": CH, "avg_launch_us": kernels["grid_forward"]["avg_us"]},
-            "mfma": {"kernel": "mlp_forward (SDF net 48-64-16)", "flops_per_sample": 8192, "achieved_tflops": mlp_tflops,
-                     "peak_tflops": MFMA_PEAK_TFLOPS, "frac": mlp_tflops / MFMA_PEAK_TFLOPS},
-            "kernels": kernels}
+        if n:
+            kernels[name] = {"ms_per_step": ms / steps, "launches_per_step": n / steps, "avg_us": ms / n * 1e3}
+    dom = "field_forward" if "field_forward" in kernels else "grid_forward"
+    return kernels, dom, kernels[dom]["avg_us"], 556 if dom == "field_forward" else 588
 
 
 def run_occupancy_workload(args):
@@ -375,21 +478,17 @@ def run_occupancy_workload(args):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.n2_profile_enable(0)
-    kernels = {}
-    for name in ("grid_forward", "mlp_forward"):
-        ms, n = profile_read(lib, name)
-        kernels[name] = {"ms_per_step": ms / args.steps, "avg_us": ms / n * 1e3}
-    gf = kernels["grid_forward"]["avg_us"] * 1e-6
-    achieved = 588 * GRID_CELLS / gf / 1e9
+    kernels, dom, dom_us, algo = inference_kernels(lib, args.steps)
+    achieved = algo * GRID_CELLS / (dom_us * 1e-6) / 1e9
     result = {"metric": "occupancy-grid cells updated per second (128^3 cells per update, 1 GPU)", "value": args.steps * GRID_CELLS / elapsed,
               "unit": "cells/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
               "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
               "config": {"workload": "update_density_grid_nerf over all 128^3 cells of one cascade: PCG32 sample generation, field density "
                                      "(hash grid + SDF MLP forward) on 2^21 points, max-splat, decayed maximum, mean, bitfield + 7 mips",
                          "cells": GRID_CELLS, "occupied_fraction": float(np.unpackbits(occ.bitfield[:GRID_CELLS // 8].cpu().numpy()).mean())},
-              "roofline": {"kernel": "grid_forward", "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": 588,
-                           "samples_per_launch": GRID_CELLS, "avg_launch_us": kernels["grid_forward"]["avg_us"]},
+              "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_sample": algo,
+                           "samples_per_launch": GRID_CELLS, "avg_launch_us": dom_us},
               "kernels": kernels}
     if not args.no_cpu_baseline:
         from oracle import oracle as orc
@@ -453,6 +552,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice", "occupancy", "mesh"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extra-regions", type=int, default=5, help="step workload: untimed repeat regions of K steps (spread of the figure)")
+    ap.add_argument("--trained-steps", type=int, default=3000,
+                    help="step workload: training steps before the trained-state leg (0 switches the leg off)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
     args = ap.parse_args()

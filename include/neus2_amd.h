@@ -387,14 +387,18 @@ int n2_field_density(n2_field_t* field, n2_stream_t stream, const float* d_xyz, 
  *                         passes take: d_dL_doutput (fp16 SoA 16 x n: row 0 = sign(sdf) loss_scale / n), d_dL_dnormal
  *                         (fp32 SoA 3 x n, times loss_scale) and rows 0..2 and the padding rows of the network's
  *                         second-order input (fp16 SoA input_width x n, nerf_network.h:546-557; rows 3.. are the encoding's
- *                         dL_ddLdoutput, written by n2_grid_backward_fused).  d_loss: one float.
+ *                         dL_ddLdoutput: written by n2_grid_backward_fused when d_dy_dx is null; with d_dy_dx, the Jacobian
+ *                         n2_grid_forward saved for the same points, this call writes them as dy_dx . d_dL_dnormal and
+ *                         n2_grid_backward_fused can be called with d_dL_ddLdy = null, which spares its pass over the
+ *                         table).  d_loss: one float.
  * ---------------------------------------------------------------------- */
 int n2_sdf_pack_input(n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n,
                       uint32_t encoding_width, uint32_t input_width, n2_half* d_input);
 uint64_t n2_sdf_eikonal_workspace_bytes(uint32_t n);
 int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding_width, uint32_t input_width, const n2_half* d_sdf_output,
                         const n2_half* d_dsdf_dinput, const float* d_normal_encoding, float* d_normal, float ek_weight, float loss_scale, n2_half* d_dL_doutput,
-                        float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes);
+                        float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes,
+                        const float* d_dy_dx);
 
 /* ------------------------------------------------------------------------
  * Adam on fp32 master weights with an fp16 working copy: tcnn's Adam as the

@@ -574,7 +574,7 @@ __global__ void __launch_bounds__(FB) sdf_pack_input_kernel(const float* __restr
 __global__ void __launch_bounds__(FB) sdf_eikonal_loss_kernel(uint32_t N, uint32_t first_pad, uint32_t in_w, const hf* __restrict__ sdf_out,
                                                               const hf* __restrict__ g, const float* __restrict__ normal_enc, float* __restrict__ normal, float ek_weight, float scale,
                                                               hf* __restrict__ dL_dy, float* __restrict__ v, hf* __restrict__ v_in,
-                                                              float* __restrict__ parts) {
+                                                              float* __restrict__ parts, const float* __restrict__ dy_dx) {
 	__shared__ float part[FB / 64];
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
 	float term = 0.f;
@@ -592,11 +592,27 @@ __global__ void __launch_bounds__(FB) sdf_eikonal_loss_kernel(uint32_t N, uint32
 		dL_dy[i] = (hf)((sdf > 0.f ? 1.f : sdf < 0.f ? -1.f : 0.f) * scale);
 		for (uint32_t r = 1; r < 16; ++r) dL_dy[(size_t)r * N + i] = (hf)0;
 		const float k = 2.f * ek_weight * (len - 1.f) / len * scale;
+		float x[3];
 #pragma unroll
 		for (int d = 0; d < 3; ++d) {
-			const float x = nrm[d] * k;  // d loss / d normal
-			v[(size_t)d * N + i] = x;
-			v_in[(size_t)d * N + i] = (hf)x;
+			x[d] = nrm[d] * k;  // d loss / d normal
+			v[(size_t)d * N + i] = x[d];
+			v_in[(size_t)d * N + i] = (hf)x[d];
+		}
+		if (dy_dx) {
+			// the encoding's dL_ddLdoutput = J v from the Jacobian the forward saved ([row][N][3]), eight rows' loads in flight
+			const uint32_t enc_w = first_pad - 3;
+			for (uint32_t r0 = 0; r0 < enc_w; r0 += 8) {
+				float j[8][3];
+#pragma unroll
+				for (uint32_t u = 0; u < 8; ++u) {
+					const float* q = dy_dx + ((size_t)min(r0 + u, enc_w - 1) * N + i) * 3;
+					j[u][0] = q[0]; j[u][1] = q[1]; j[u][2] = q[2];
+				}
+#pragma unroll
+				for (uint32_t u = 0; u < 8; ++u)
+					if (r0 + u < enc_w) v_in[(size_t)(3 + r0 + u) * N + i] = (hf)fmaf(j[u][0], x[0], fmaf(j[u][1], x[1], j[u][2] * x[2]));
+			}
 		}
 		for (uint32_t r = first_pad; r < in_w; ++r) v_in[(size_t)r * N + i] = (hf)0;
 	}
@@ -635,7 +651,8 @@ N2_API uint64_t n2_sdf_eikonal_workspace_bytes(uint32_t n) { return 4ull * ((n +
 
 N2_API int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding_width, uint32_t input_width, const n2_half* d_sdf_output,
                                const n2_half* d_dsdf_dinput, const float* d_normal_encoding, float* d_normal, float ek_weight, float loss_scale, n2_half* d_dL_doutput,
-                               float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes) {
+                               float* d_dL_dnormal, n2_half* d_second_order_input, float* d_loss, void* d_workspace, uint64_t workspace_bytes,
+                               const float* d_dy_dx) {
 	N2_REQUIRE(n > 0, "n2_sdf_eikonal_loss: empty batch");
 	N2_REQUIRE(d_sdf_output && d_dsdf_dinput && d_normal_encoding && d_normal && d_dL_doutput && d_dL_dnormal && d_second_order_input && d_loss && d_workspace,
 	           "n2_sdf_eikonal_loss: null buffer");
@@ -646,7 +663,8 @@ N2_API int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding
 	float* parts = reinterpret_cast<float*>(d_workspace);
 	sdf_eikonal_loss_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, 3 + encoding_width, input_width, reinterpret_cast<const hf*>(d_sdf_output),
 	                                                      reinterpret_cast<const hf*>(d_dsdf_dinput), d_normal_encoding, d_normal, ek_weight, loss_scale / (float)n,
-	                                                      reinterpret_cast<hf*>(d_dL_doutput), d_dL_dnormal, reinterpret_cast<hf*>(d_second_order_input), parts);
+	                                                      reinterpret_cast<hf*>(d_dL_doutput), d_dL_dnormal, reinterpret_cast<hf*>(d_second_order_input), parts,
+	                                                      d_dy_dx);
 	N2_LAUNCH_CHECK();
 	sdf_loss_sum_kernel<<<dim3(1), dim3(256), 0, s>>>(parts, fgrid(n).x, 1.f / (float)n, d_loss);
 	N2_LAUNCH_CHECK();
@@ -663,7 +681,8 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	hipStream_t s = n2_stream(stream);
 	if (f->fused && fused_ok(f)) {
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
-		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, d_output, nullptr, density);
+		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, d_output, nullptr, density,
+		                          n2_grid_lattice_order(f->grid) ? nullptr : reinterpret_cast<n2_half*>(f->sdf_in));
 	}
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->xyz);

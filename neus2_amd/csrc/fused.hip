@@ -260,13 +260,17 @@ __device__ __forceinline__ void sh4(float x, float y, float z, float* o) {
 // ----------------------------------------------------------------------------
 constexpr uint32_t FG_BLOCK = 256;
 
+// FULL: positions from the [N][7] coordinates, slopes and the coordinate rows are written; else positions with the
+// strides (ps, ds) and the feature rows only (inference on points in no particular order).
+template <bool FULL>
 __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
 	const uint32_t level = blockIdx.x / tiles, i = (blockIdx.x - level * tiles) * FG_BLOCK + threadIdx.x;
 	const uint32_t N = a.N;
 	if (i >= N) return;
-	const float* q = a.coords + (size_t)i * 7;
-	const float p[3] = {q[0], q[1], q[2]};
-	if (level == 0) {
+	const float* q = FULL ? a.coords + (size_t)i * 7 : a.pos + (size_t)i * a.ps;
+	const size_t qs = FULL ? 1 : a.ds;
+	const float p[3] = {q[0], q[qs], q[2 * qs]};
+	if (FULL && level == 0) {
 #pragma unroll
 		for (int d = 0; d < 3; ++d) {
 			a.sdf_in[(size_t)d * N + i] = (hf)p[d] - (hf)0.5f;
@@ -288,21 +292,23 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 		const char* base = reinterpret_cast<const char*>(a.table);
 #pragma unroll
 		for (int k = 0; k < 8; ++k) it.raw[k] = *reinterpret_cast<const uint32_t*>(base + boff[k]);
-		item_finish<true>(it, feat, J);
+		item_finish<FULL>(it, feat, J);
 	}
 	a.sdf_in[(size_t)(3 + 2 * level) * N + i] = (hf)feat[0];
 	a.sdf_in[(size_t)(4 + 2 * level) * N + i] = (hf)feat[1];
-	const float six[6] = {J[0][0], J[0][1], J[0][2], J[1][0], J[1][1], J[1][2]};
-	a.slopes[(size_t)level * N + i] = n2_slopes_pack(six);
+	if (FULL) {
+		const float six[6] = {J[0][0], J[0][1], J[0][2], J[1][0], J[1][1], J[1][2]};
+		a.slopes[(size_t)level * N + i] = n2_slopes_pack(six);
+	}
 }
 
 // ----------------------------------------------------------------------------
 // the network kernel: a wave takes 32 samples per pass, lane (n, g) works for sample b0 + n on the levels l(j, g).
-// GATHER: the features come from the table (inference); else from the rows the gather kernel wrote.
+// GATHER: the features come from the table (inference on points in lattice order); else from the rows the gather kernel wrote.
 // ----------------------------------------------------------------------------
 template <bool FULL, bool GATHER>
 __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const FusedArgs a) {
-	static_assert(FULL != GATHER, "the full forward reads the gather kernel's rows, inference gathers itself");
+	static_assert(!(FULL && GATHER), "the full forward reads the gather kernel's rows");
 	extern __shared__ __align__(16) unsigned char smem[];
 	hf* F = reinterpret_cast<hf*>(smem);
 	uint4* LV = reinterpret_cast<uint4*>(smem + (size_t)(FULL ? FF_COUNT : FF_SDF_COUNT) * 1024);
@@ -341,9 +347,15 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 			FF_STEP(0) FF_STEP(1) FF_STEP(2) FF_STEP(3) FF_STEP(4) FF_STEP(5) FF_STEP(6) FF_STEP(7)
 #undef FF_STEP
 		} else {
-			const float* q = a.coords + (size_t)col * 7;
+			if (FULL) {
+				const float* q = a.coords + (size_t)col * 7;
 #pragma unroll
-			for (int d = 0; d < 3; ++d) { p[d] = q[d]; dir[d] = q[4 + d]; }
+				for (int d = 0; d < 3; ++d) { p[d] = q[d]; dir[d] = q[4 + d]; }
+			} else {
+				const float* q = a.pos + (size_t)col * a.ps;
+#pragma unroll
+				for (int d = 0; d < 3; ++d) p[d] = q[(size_t)d * a.ds];
+			}
 #pragma unroll
 			for (int j = 0; j < 8; ++j) {
 				const uint32_t level = 4u * (j >> 1) + 2u * g + (j & 1);
@@ -351,7 +363,7 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 				const uint32_t lr = 2u * level < a.enc_w ? level : 0u;
 				xs[j >> 2][2 * (j & 3)] = a.sdf_in[(size_t)(3 + 2 * lr) * N + col];
 				xs[j >> 2][2 * (j & 3) + 1] = a.sdf_in[(size_t)(4 + 2 * lr) * N + col];
-				slope[j] = a.slopes[(size_t)lr * N + col];
+				if (FULL) slope[j] = a.slopes[(size_t)lr * N + col];
 			}
 		}
 		xs[2] = zero8();
@@ -543,7 +555,7 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 	a.rgb_in = reinterpret_cast<hf*>(rgb_in);
 	a.output = reinterpret_cast<hf*>(d_output);
 	const uint32_t tiles = (n + FG_BLOCK - 1) / FG_BLOCK;
-	field_gather_kernel<<<dim3(tiles * nets.tab->n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
+	field_gather_kernel<true><<<dim3(tiles * nets.tab->n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
 	N2_LAUNCH_CHECK();
 	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();
@@ -551,13 +563,24 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 }
 
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
-                       float* d_row0, bool density) {
+                       float* d_row0, bool density, n2_half* sdf_in) {
 	FusedArgs a = fused_base(nets, n);
 	a.pos = d_xyz; a.ps = ps; a.ds = ds;
 	a.sdf_out = reinterpret_cast<hf*>(d_out_soa);
 	a.row0 = d_row0;
 	a.density = density ? 1 : 0;
-	field_fused_forward_kernel<false, true><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
+	if (sdf_in == nullptr) {
+		field_fused_forward_kernel<false, true><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
+		N2_LAUNCH_CHECK();
+		return N2_OK;
+	}
+	// points in no particular order: a sample-major walk would touch all tables at once, so the features are gathered level
+	// by level into the network's input rows first
+	a.sdf_in = reinterpret_cast<hf*>(sdf_in);
+	const uint32_t tiles = (n + FG_BLOCK - 1) / FG_BLOCK;
+	field_gather_kernel<false><<<dim3(tiles * nets.tab->n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
+	N2_LAUNCH_CHECK();
+	field_fused_forward_kernel<false, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -87,9 +87,11 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 // d feature / d position without the level's scale factor, n2_slopes_pack) and the [n][16] output.
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
                            void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output);
-// NerfNetwork::sdf / density in one kernel: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
+// NerfNetwork::sdf / density: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
+// sdf_in null: one kernel that gathers sample by sample (points in lattice order, whose table lines stay cached);
+// else a level-major gather into the feature rows 3.. of sdf_in (SoA, n columns) followed by the network kernel.
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
-                       float* d_row0, bool density);
+                       float* d_row0, bool density, n2_half* sdf_in);
 
 // n2_mlp_backward_rows / n2_mlp_backward_and_second_order whose input is read through an index: sample i of the batch is
 // column d_index[i] of d_input, a matrix with n_cols columns (d_index null: column i of n columns).  Every other operand is

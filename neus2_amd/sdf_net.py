@@ -74,7 +74,8 @@ class SdfNet:
         n = ctx["x"].shape[1]
         check(capi.lib().n2_sdf_eikonal_loss(_stream(), C.c_uint32(n), C.c_uint32(self.enc_w), C.c_uint32(self.in_w), ptr(ctx["y"]), ptr(ctx["g"]),
                                              ptr(self._normal_enc), ptr(self._normal), C.c_float(ek_weight), C.c_float(loss_scale), ptr(self._dL_dy),
-                                             ptr(self._v), ptr(self._v_in), ptr(self._loss), ptr(self._ws), C.c_uint64(self._ws_bytes)),
+                                             ptr(self._v), ptr(self._v_in), ptr(self._loss), ptr(self._ws), C.c_uint64(self._ws_bytes),
+                                             ptr(ctx["dy_dx"])),
               "n2_sdf_eikonal_loss")
         ctx["weights"] = (ek_weight, loss_scale)
 
@@ -84,12 +85,12 @@ class SdfNet:
         x, inp, g, n = ctx["x"], ctx["inp"], ctx["g"], ctx["x"].shape[1]
         if ctx["weights"] != (ek_weight, loss_scale):
             self._eikonal(ctx, ek_weight, loss_scale)
-        # first order through the MLP, then both orders through the grid in one pass; the grid's dL_ddLdoutput lands in
-        # rows 3.. of the MLP's second-order input
+        # first order through the MLP, then both orders through the grid in one pass; the grid's dL_ddLdoutput (rows 3.. of
+        # the MLP's second-order input) was already formed from the saved Jacobian by n2_sdf_eikonal_loss
         check(L.n2_mlp_backward(self.mlp._h, s, ptr(inp), C.c_uint32(n), ptr(self._dL_dy), C.c_int(LAYOUT_SOA), ptr(self._d_inp), C.c_int(GRAD_OVERWRITE)),
               "n2_mlp_backward")
         check(L.n2_grid_backward_fused(self.grid._h, s, ptr(x), C.c_uint32(1), C.c_uint32(n), C.c_uint32(n), ptr(self._d_inp[3:3 + self.enc_w]),
-                                       ptr(self._v), ptr(g[3:3 + self.enc_w]), ptr(self._v_in[3:3 + self.enc_w]), C.c_int(GRAD_OVERWRITE)),
+                                       ptr(self._v), ptr(g[3:3 + self.enc_w]), None, C.c_int(GRAD_OVERWRITE)),
               "n2_grid_backward_fused")
         # second order through the MLP: its first-order output gradient was e_0
         check(L.n2_mlp_backward_backward_input(self.mlp._h, s, ptr(inp), C.c_uint32(n), ptr(self._v_in), None, None, C.c_int(GRAD_ACCUMULATE)),

@@ -12,36 +12,6 @@ pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
-def oracle_step(oracle, P, W, x, ek_weight, loss_scale):
-    og = oracle.Grid(16, 19, 16, 1.447)
-    om = oracle.Mlp(48, 64, 1, 16)
-    n = x.shape[1]
-    enc, J = og.forward(P, x, want_dy_dx=True)
-    inp = np.zeros((48, n), np.float32)
-    inp[0:3] = q16(q16(x) - 0.5)
-    inp[3:35] = q16(enc)
-    y, h = om.forward(W, inp, round_hidden=True)
-    e0 = np.zeros((16, n), np.float32)
-    e0[0] = 1
-    g, _ = om.backward(W, inp, h, e0, want_dW=False)
-    g = q16(g)
-    normal = np.einsum("rnd,rn->dn", J, g[3:35]) + g[0:3]
-    sdf = q16(y[0])
-    norm = np.maximum(np.linalg.norm(normal, axis=0), 1e-12)
-    loss = np.abs(sdf).mean() + ek_weight * ((norm - 1) ** 2).mean()
-    dL_dy = np.zeros((16, n), np.float32)
-    dL_dy[0] = q16(np.sign(sdf) * (loss_scale / n))
-    v = (normal * (2 * ek_weight * (norm - 1) / norm * (loss_scale / n))).astype(np.float32)
-    d_inp, dW = om.backward(W, inp, h, dL_dy)
-    grad, _ = og.backward(P, x, q16(d_inp)[3:35], want_dx=False)
-    grad, jv, _ = og.backward_backward_input(P, x, v, g[3:35], grad=grad, want_dinput=False)
-    v_in = np.zeros((48, n), np.float32)
-    v_in[0:3] = q16(v)
-    v_in[3:35] = q16(jv)
-    dW, _ = om.backward_backward_input(W, h, v_in, e0, dW=dW)
-    return dict(sdf=sdf, normal=normal, loss=loss, grid_grad=grad, mlp_grad=dW, offset=og.offset)
-
-
 @pytest.mark.parametrize("kind", ["uniform", "rays"])
 def test_sdf_eikonal_step_matches_oracle(oracle, kind):
     from neus2_amd.sdf_net import SdfNet
@@ -62,7 +32,8 @@ def test_sdf_eikonal_step_matches_oracle(oracle, kind):
     net.set_params(dP, gP, dW, gW)
     ctx = net.forward(dev(x))
     loss = float(net.loss_backward(ctx, ek_weight=0.1, loss_scale=128.0).item())
-    ref = oracle_step(oracle, P, W, x, 0.1, 128.0)
+    from oracle.sdf_step import sdf_eikonal_step
+    ref = sdf_eikonal_step(P, W, x, 0.1, 128.0)
     assert_close(host(ctx["sdf"]), ref["sdf"], what="sdf", outlier_frac=1e-3)
     assert_close(host(ctx["normal"]), ref["normal"], what="normal", outlier_frac=2e-3)
     assert abs(loss - ref["loss"]) <= 2e-3 * abs(ref["loss"])
