@@ -126,20 +126,36 @@ constexpr uint32_t RAYS_PER_BLOCK = 4;                // one wave per ray
 // from 2^-3 up, so a window crosses at most one boundary: the lanes behind it continue from the one real addition that
 // crosses it with the next binade's increment.  Below 2^-3 (a camera inside the volume) the additions are done one by one.
 // Must be called by all 64 lanes.
-__device__ __forceinline__ float window_t(float t_first, uint32_t lane) {
-	if (!(t_first >= 0.125f && t_first < 1e30f)) {
+// What window_t found: with `linear` set, the t of step k of the window is window_step(w, t_first, k) for any k in 0..63.
+struct WindowShape {
+	bool linear;   // false: the additions were done one by one (no closed form)
+	uint32_t kc;   // steps 0 .. kc-1 lie in the binade of t_first (64: all of them)
+	float d1, d2, t_cross;
+};
+__device__ __forceinline__ float window_step(const WindowShape& w, float t_first, uint32_t k) {
+	return k < w.kc ? __fmaf_rn((float)k, w.d1, t_first) : __fmaf_rn((float)(k - w.kc), w.d2, w.t_cross);
+}
+__device__ __forceinline__ float window_t(float t_first, uint32_t lane, WindowShape& w) {
+	w.linear = t_first >= 0.125f && t_first < 1e30f;
+	w.kc = 64u; w.d1 = STEP; w.d2 = STEP; w.t_cross = 3.4e38f;
+	if (!w.linear) {
 		float t = t_first;
 		for (uint32_t a = 0; a < lane; ++a) t += STEP;
 		return t;
 	}
 	const float lo = __uint_as_float(__float_as_uint(t_first) & 0x7F800000u), hi = lo + lo;
-	const float d1 = (lo + STEP) - lo, d2 = (hi + STEP) - hi;
-	const float x = __fmaf_rn((float)lane, d1, t_first);  // exact below hi; at or above hi only the comparison is used
-	const unsigned long long below = __ballot(x < hi);     // lanes 0 .. kc-1 (lane 0 always)
-	const uint32_t kc = (uint32_t)__popcll(below);
-	if (kc == 64u) return x;
-	const float t_cross = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)kc - 1)) + STEP;
-	return lane < kc ? x : __fmaf_rn((float)(lane - kc), d2, t_cross);
+	w.d1 = (lo + STEP) - lo;
+	w.d2 = (hi + STEP) - hi;
+	const float x = __fmaf_rn((float)lane, w.d1, t_first);  // exact below hi; at or above hi only the comparison is used
+	const unsigned long long below = __ballot(x < hi);       // lanes 0 .. kc-1 (lane 0 always)
+	w.kc = (uint32_t)__popcll(below);
+	if (w.kc == 64u) return x;
+	w.t_cross = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)w.kc - 1)) + STEP;
+	return lane < w.kc ? x : __fmaf_rn((float)(lane - w.kc), w.d2, w.t_cross);
+}
+__device__ __forceinline__ float window_t(float t_first, uint32_t lane) {
+	WindowShape w;
+	return window_t(t_first, lane, w);
 }
 
 // Returns the number of samples; mask[2 w], mask[2 w + 1]: which steps of window w emitted; t_first[w]: t of its first step.
@@ -150,7 +166,8 @@ __device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t*
 	float t_first = r.startt;  // t of the window's first step
 	float pending = -3.4e38f;  // steps with t below this are skipped (target of the last visited empty step)
 	for (uint32_t w = 0; w < WINDOWS; ++w) {
-		const float t = window_t(t_first, lane);
+		WindowShape ws;
+		const float t = window_t(t_first, lane, ws);
 		float pos[3];
 #pragma unroll
 		for (int k = 0; k < 3; ++k) pos[k] = __fmaf_rn(t, r.dir[k], r.o[k]);
@@ -163,7 +180,47 @@ __device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t*
 		bool done = false;
 		const unsigned long long reach = __ballot(t >= pending);  // steps not skipped by the pending target
 		uint32_t cur = reach ? (uint32_t)__ffsll((long long)reach) - 1u : 64u;
-		while (cur < 64u) {
+		// The walk without a loop.  Every lane works out the step the serial walk would visit after its own: the end of
+		// its run for an occupied step, the first later step whose t reaches its target for an empty one (estimated by a
+		// division, then checked against the exact t of the steps around the estimate).  Steps fall into groups that
+		// share that successor; when every group's successor is the step right behind the group, the walk, wherever it
+		// enters a group, leaves it for the first step of the next one: it visits every occupied step from `cur` on and
+		// the first step of every empty group, and the last of those sets the pending target.  A window where that does
+		// not hold (a step next to a voxel face that the two tests place differently), one that leaves the unit cube or
+		// reaches the sample limit, or one without the closed form of t takes the loop below.
+		bool walked = false;
+		if (cur < 64u && ws.linear) {
+			const unsigned long long ge = ~0ull << cur;
+			if ((~m_inside & ge) == 0ull && j + (uint32_t)__popcll(m_occ & ge) < MARCH_STEPS) {
+				uint32_t nxt;
+				bool good = true;
+				if (occ) {
+					const unsigned long long rest = ~(m_occ >> lane);  // bit 64 - lane and up are set: the run ends inside the window or at its end
+					nxt = lane + min((uint32_t)__ffsll((long long)rest) - 1u, 64u - lane);
+				} else {
+					const bool second = target >= ws.t_cross;
+					const float est = second ? __fdividef(target - ws.t_cross, ws.d2) + (float)ws.kc : __fdividef(target - t_first, ws.d1);
+					uint32_t k0 = (uint32_t)fminf(fmaxf(ceilf(est), 0.f), 64.f);
+					if (k0 > 0u && window_step(ws, t_first, k0 - 1u) >= target) --k0;
+					if (k0 < 64u && window_step(ws, t_first, k0) < target) ++k0;
+					good = (k0 == 0u || window_step(ws, t_first, k0 - 1u) < target) && (k0 == 64u || window_step(ws, t_first, k0) >= target);
+					nxt = max(k0, lane + 1u);  // the serial form always moves on by at least one step
+				}
+				const uint32_t nxt_up = (uint32_t)__shfl_down((int)nxt, 1);
+				const bool occ_up = (m_occ >> ((lane + 1u) & 63u)) & 1ull;
+				const bool chained = nxt == lane + 1u || (occ == occ_up && nxt == nxt_up);
+				const unsigned long long bad = __ballot(lane >= cur && (!good || (lane < 63u && !chained)));
+				if (bad == 0ull) {
+					walked = true;
+					emit = m_occ & ge;
+					j += (uint32_t)__popcll(emit);
+					const unsigned long long ends = __ballot(nxt == lane + 1u);
+					const unsigned long long firsts = ((ends << 1) | (1ull << cur)) & ge & ~m_occ;  // visited empty steps
+					if (firsts) pending = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(target), 63 - (int)__clzll((long long)firsts)));
+				}
+			}
+		}
+		while (!walked && cur < 64u) {
 			if (!((m_inside >> cur) & 1ull)) { done = true; break; }
 			if ((m_occ >> cur) & 1ull) {
 				// a run of occupied steps: each emits and moves on by one step

@@ -6,6 +6,10 @@
 // the scene and the seed) may run ahead on a stream the trainer owns, into the
 // other of two sample sets, while this step's field kernels occupy the GPU.
 #include "n2_common.h"
+#ifndef N2_EXP
+#define N2_EXP 0
+#endif
+
 
 #include <cstring>
 #include <new>
@@ -303,10 +307,19 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		                                    t->cfg.composite.background, t->bitfield, n_inference, set.counters, set.counters + 1, set.ray_indices,
 		                                    set.numsteps, set.rgb_target, set.coords, set.ws_sampler, t->ws_sampler_bytes);
 	};
+	// the following step's samples on the side stream, assuming the same ray count and the next seed; everything enqueued on
+	// s so far precedes the generator
+	auto prefetch = [&](uint32_t cur_set) -> int {
+		t->pf_valid = false;
+		N2_HIP(hipEventRecord(t->ev_main, s));
+		N2_HIP(hipStreamWaitEvent(t->side, t->ev_main, 0));
+		if (int rc = sample(t->sets[1u - cur_set], t->side, t->n_rays_total, seed + 1)) return rc;
+		N2_HIP(hipEventRecord(t->ev_ready, t->side));
+		t->pf_valid = true; t->pf_set = 1u - cur_set; t->pf_n_rays = n_rays; t->pf_n_inference = n_inference; t->pf_seed = seed + 1; t->pf_ray_base = t->n_rays_total;
+		return N2_OK;
+	};
 	uint32_t cur;
 	if (t->side) {
-		// everything enqueued by earlier steps precedes this marker: the set the generator overwrites next is free after it
-		N2_HIP(hipEventRecord(t->ev_main, s));
 		const bool hit = t->pf_valid && t->pf_n_rays == n_rays && t->pf_n_inference == n_inference && t->pf_seed == seed && t->pf_ray_base == t->n_rays_total;
 		if (hit) {
 			cur = t->pf_set;
@@ -317,12 +330,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 			if (int rc = sample(t->sets[cur], s, t->n_rays_total, seed)) return rc;
 		}
 		t->n_rays_total += n_rays;
-		// the following step's samples, assuming the same ray count and the next seed
-		t->pf_valid = false;
-		N2_HIP(hipStreamWaitEvent(t->side, t->ev_main, 0));
-		if (int rc = sample(t->sets[1u - cur], t->side, t->n_rays_total, seed + 1)) return rc;
-		N2_HIP(hipEventRecord(t->ev_ready, t->side));
-		t->pf_valid = true; t->pf_set = 1u - cur; t->pf_n_rays = n_rays; t->pf_n_inference = n_inference; t->pf_seed = seed + 1; t->pf_ray_base = t->n_rays_total;
+		if (N2_EXP == 0) {
+			if (int rc = prefetch(cur)) return rc;
+		}
 	} else {
 		cur = 0;
 		if (int rc = sample(t->sets[0], s, t->n_rays_total, seed)) return rc;
@@ -346,6 +356,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, t->src_index, ray_counter, n_rays,
 	                                                                     t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
+	if (N2_EXP == 1 && t->side) {
+		if (int rc = prefetch(cur)) return rc;
+	}
 	// forward + backward on the compacted batch, then the optimiser.  Every compacted sample is one of the marched
 	// samples the field has just been evaluated on: unless asked to run the field again, the activations saved for it
 	// are selected instead (the same values, a fraction of the work).
