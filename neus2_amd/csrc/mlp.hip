@@ -27,6 +27,7 @@
 #include <new>
 
 #include "mlp_device.h"
+#include "mlp_wgrad.h"
 
 struct n2_mlp {
 	uint32_t in_w, n_hidden, n_params;
@@ -586,6 +587,11 @@ static inline uint32_t stream_grid(uint32_t n, uint32_t waves_per_tile) {
 	return blocks < (uint32_t)MLP_MAX_SLABS ? blocks : (uint32_t)MLP_MAX_SLABS;
 }
 static inline size_t frag_bytes(int n_frags) { return (size_t)n_frags * 64 * 16; }
+// workgroups of the weight-gradient kernels: rounds of 128 samples in a grid-stride loop, two workgroups per CU
+static inline uint32_t wgrad_grid(uint32_t n) {
+	const uint32_t rounds = (n + WG_SAMPLES - 1) / WG_SAMPLES;
+	return rounds < (uint32_t)MLP_MAX_SLABS ? rounds : (uint32_t)MLP_MAX_SLABS;
+}
 
 #define MLP_DISPATCH(in_w, n_hidden, CALL)                                            \
 	do {                                                                              \
@@ -719,12 +725,13 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	           "n2_mlp_backward: buffers must be 16-byte aligned");
 	hipStream_t s = n2_stream(stream);
 	const bool want_dw = mode != N2_GRAD_IGNORE, want_dx = d_dL_dinput != nullptr;
+	N2_REQUIRE(!want_dw || unit_row < 0, "n2_mlp_backward: a constant output gradient goes with mode IGNORE");
 	if (n == 0) {
 		if (mode == N2_GRAD_OVERWRITE) return n2_fill_zero_u32(s, mlp->grads, mlp->n_params * sizeof(hf));
 		return N2_OK;
 	}
 	if (!want_dw && !want_dx) return N2_OK;
-	const uint32_t blocks = stream_grid(n, want_dw ? 2 : 1);
+	const uint32_t blocks = want_dw ? wgrad_grid(n) : stream_grid(n, 1);
 	if (int rc = check_pending(mlp, "n2_mlp_backward", blocks, mode)) return rc;
 	const hf* X = reinterpret_cast<const hf*>(d_input);
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
@@ -733,10 +740,17 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 #define LAUNCH(IC, NH, DX, DW)                                                                                      \
 	do {                                                                                                            \
-		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT); /* >= the fp32 parameter image laid over it */      \
+		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT);                                                      \
 		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
 		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, next_slabs(mlp), \
 			nullptr, 0, nullptr, nullptr, -1, x_index, x_cols);                                                         \
+	} while (0)
+#define LAUNCH_W(IC, NH, DX)                                                                                        \
+	do {                                                                                                            \
+		const size_t lds = mlp_wgrad_lds<IC, NH, false>();                                                          \
+		if (int rc = allow_lds(mlp_wgrad_kernel<IC, NH, DX, false>, lds)) return rc;                                \
+		mlp_wgrad_kernel<IC, NH, DX, false><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1, (int)dy_rows, dX, \
+			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols);                                                  \
 	} while (0)
 #define LAUNCH_Y(IC, NH)                                                                                            \
 	do {                                                                                                            \
@@ -748,13 +762,14 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 #define CALL(IC, NH)                                   \
 	do {                                               \
 		if (d_output) LAUNCH_Y(IC, NH);                        \
-		else if (want_dx && want_dw) LAUNCH(IC, NH, true, true);    \
+		else if (want_dx && want_dw) LAUNCH_W(IC, NH, true);        \
 		else if (want_dx) LAUNCH(IC, NH, true, false);         \
-		else LAUNCH(IC, NH, false, true);                      \
+		else LAUNCH_W(IC, NH, false);                          \
 	} while (0)
 	MLP_DISPATCH(mlp->in_w, mlp->n_hidden, CALL);
 #undef CALL
 #undef LAUNCH
+#undef LAUNCH_W
 #undef LAUNCH_Y
 	N2_LAUNCH_CHECK();
 	if (want_dw) return reduce_partials(mlp, s, blocks, mode);
@@ -825,19 +840,19 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 		if (mode == N2_GRAD_OVERWRITE) return n2_fill_zero_u32(s, mlp->grads, mlp->n_params * sizeof(hf));
 		return N2_OK;
 	}
-	const uint32_t blocks = stream_grid(n, 2);
+	const uint32_t blocks = wgrad_grid(n);
 	if (int rc = check_pending(mlp, fn, blocks, mode)) return rc;
-	const int aos = (dL_layout == N2_LAYOUT_AOS ? 1 : 0) | (MLP_OUT << 8);
+	const int aos = dL_layout == N2_LAYOUT_AOS ? 1 : 0;
 	const int unit_row2 = d_second_dL_doutput == nullptr ? 0 : -1;
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 	switch (mlp->in_w / 16) {
 #define CASE(IC)                                                                                                           \
 	case IC: {                                                                                                             \
-		const size_t lds = frag_bytes(FragMap<IC, 1>::COUNT);                                                              \
-		if (int rc = allow_lds(mlp_backward_kernel<IC, 1, true, true, false, true>, lds)) return rc;                       \
-		mlp_backward_kernel<IC, 1, true, true, false, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,        \
-			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, -1,                   \
-			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), nullptr, 0, reinterpret_cast<const hf*>(d_dL_ddLdinput),  \
+		const size_t lds = mlp_wgrad_lds<IC, 1, true>();                                                                   \
+		if (int rc = allow_lds(mlp_wgrad_kernel<IC, 1, true, true>, lds)) return rc;                                       \
+		mlp_wgrad_kernel<IC, 1, true, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,                        \
+			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,              \
+			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),              \
 			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);                                 \
 		break;                                                                                                             \
 	}
