@@ -260,88 +260,17 @@ __device__ __forceinline__ void sh4(float x, float y, float z, float* o) {
 // ----------------------------------------------------------------------------
 constexpr uint32_t FG_BLOCK = 256;
 
-#ifndef N2_EXP
-#define N2_EXP 0
-#endif
-// Piece x of the level-major list of (level, tile) items belongs to the workgroups with blockIdx.x % 8 == x, i.e. to XCD x.
-struct GatherPlan {
-	uint32_t begin[9];
-};
-
-// The eight corner values of one (sample, level) with one load per (y, z) corner pair where the two x neighbours allow it.
-//  dense level:  the x neighbours are consecutive entries: one 8-byte load (4-byte aligned).
-//  hashed level: entry = x ^ h(y, z), so the neighbours differ in the low bits that x and x + 1 differ in: for three x in
-//                four both lie in the aligned block of four entries that one 16-byte load fetches.
-// A pair that this does not cover (the dense index wraps, x + 1 carries beyond bit 1) takes a second, 4-byte load.
-// The memory pipeline looks up one cache line per lane and load, so it sees 4 to 5 lines per item instead of 8.
-template <int KIND>  // 0: dense, 1: hashed
-__device__ __forceinline__ void gather_wide(const LaneLevel& L, const uint32_t (&c)[3], const char* __restrict__ base, uint32_t (&raw)[8]) {
-	if (KIND == 0) {
-		const uint32_t r = L.res;
-		const uint32_t dx0 = min(c[0], r), dx1 = min(c[0] + 1u, r);
-		const uint32_t y0 = min(c[1], r) * r, y1 = min(c[1] + 1u, r) * r, z0 = min(c[2], r) * r * r, z1 = min(c[2] + 1u, r) * r * r;
-		const uint32_t dyz[4] = {y0 + z0, y1 + z0, y0 + z1, y1 + z1};
-		uint2 v[4];
-		uint32_t i1[4];
-		bool far[4];
-#pragma unroll
-		for (int j = 0; j < 4; ++j) {
-			uint32_t i0 = dx0 + dyz[j];
-			i0 = min(i0, i0 - L.entries);
-			i1[j] = dx1 + dyz[j];
-			i1[j] = min(i1[j], i1[j] - L.entries);
-			far[j] = i1[j] != i0 + 1u;
-			// at the last entry of the last level the upper half of this load lies behind the table: the field's parameter
-			// block continues there (the variance values), and the half is not used (far is set)
-			v[j] = *reinterpret_cast<const uint2*>(base + ((size_t)(L.offset + i0) << 2));
-		}
-#pragma unroll
-		for (int j = 0; j < 4; ++j) {
-			raw[2 * j] = v[j].x;
-			raw[2 * j + 1] = v[j].y;
-			if (far[j]) raw[2 * j + 1] = *reinterpret_cast<const uint32_t*>(base + ((size_t)(L.offset + i1[j]) << 2));
-		}
-	} else {
-		const uint32_t mask = L.entries - 1u;
-		const uint32_t y0 = c[1] * 2654435761u, y1 = y0 + 2654435761u, z0 = c[2] * 805459861u, z1 = z0 + 805459861u;
-		const uint32_t hyz[4] = {(y0 ^ z0) & mask, (y1 ^ z0) & mask, (y0 ^ z1) & mask, (y1 ^ z1) & mask};
-		const uint32_t hx0 = c[0] & mask, hx1 = (c[0] + 1u) & mask;
-		const bool far = ((hx0 ^ hx1) & ~3u) != 0u;  // the same for the four pairs of an item
-		uint4 v[4];
-		uint32_t i0[4], i1[4];
-#pragma unroll
-		for (int j = 0; j < 4; ++j) {
-			i0[j] = hx0 ^ hyz[j];
-			i1[j] = hx1 ^ hyz[j];
-			v[j] = *reinterpret_cast<const uint4*>(base + ((size_t)(L.offset + (i0[j] & ~3u)) << 2));
-		}
-		auto pick = [](const uint4& q, uint32_t k) { return (k & 2u) ? ((k & 1u) ? q.w : q.z) : ((k & 1u) ? q.y : q.x); };
-#pragma unroll
-		for (int j = 0; j < 4; ++j) {
-			raw[2 * j] = pick(v[j], i0[j]);
-			raw[2 * j + 1] = pick(v[j], i1[j]);
-		}
-		if (far) {
-#pragma unroll
-			for (int j = 0; j < 4; ++j) raw[2 * j + 1] = *reinterpret_cast<const uint32_t*>(base + ((size_t)(L.offset + i1[j]) << 2));
-		}
-	}
-}
-
 // FULL: positions from the [N][7] coordinates, slopes and the coordinate rows are written; else positions with the
 // strides (ps, ds) and the feature rows only (inference on points in no particular order).
-template <bool FULL, bool XCD, bool WIDE>
-__global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles, const GatherPlan plan) {
-	uint32_t level, tile;
-	if (XCD) {
-		const uint32_t xcd = blockIdx.x & 7u, item = plan.begin[xcd] + (blockIdx.x >> 3);
-		if (item >= plan.begin[xcd + 1]) return;
-		level = item / tiles;
-		tile = item - level * tiles;
-	} else {
-		level = blockIdx.x / tiles;
-		tile = blockIdx.x - level * tiles;
-	}
+template <bool FULL>
+__global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
+	// level-major workgroup ids: the workgroups that run at one time work on one or two levels, whose tables stay in every
+	// L2.  Measured on the training step's 2.7e5 ray-ordered samples and dropped: whole levels dealt to XCDs by a cost plan
+	// (+9 us), one 8- or 16-byte load per pair of x neighbours instead of two 4-byte loads (+12 us).  Staging the coarse
+	// levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch and the five dense
+	// levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the positions and writing
+	// 320 bytes of features and slopes per sample.
+	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
 	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
 	const uint32_t N = a.N;
 	if (i >= N) return;
@@ -366,15 +295,10 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 		for (int d = 0; d < 3; ++d) n2_locate(p[d], L.scale, it.w[d], c[d]);
 		it.scale = 1.f;  // slopes are stored without the level's scale factor
 		const char* base = reinterpret_cast<const char*>(a.table);
-		if (WIDE) {
-			if (L.hashed) gather_wide<1>(L, c, base, it.raw);
-			else gather_wide<0>(L, c, base, it.raw);
-		} else {
-			if (L.hashed) corner_offsets<1>(L, c, boff);
-			else corner_offsets<0>(L, c, boff);
+		if (L.hashed) corner_offsets<1>(L, c, boff);
+		else corner_offsets<0>(L, c, boff);
 #pragma unroll
-			for (int k = 0; k < 8; ++k) it.raw[k] = *reinterpret_cast<const uint32_t*>(base + boff[k]);
-		}
+		for (int k = 0; k < 8; ++k) it.raw[k] = *reinterpret_cast<const uint32_t*>(base + boff[k]);
 		item_finish<FULL>(it, feat, J);
 	}
 	a.sdf_in[(size_t)(3 + 2 * level) * N + i] = (hf)feat[0];
@@ -597,32 +521,10 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 	return true;
 }
 
-// Launch of the level-major gather.  dense_cost: cost of a dense level's tile relative to a hashed one's (the levels are
-// dealt to the XCDs in pieces of equal estimated cost).
 template <bool FULL>
-static void launch_gather(const FusedArgs& a, const N2LevelTable& tab, hipStream_t s, float dense_cost) {
-	constexpr bool XCD = (N2_EXP & 1) != 0, WIDE = (N2_EXP & 2) != 0;
-	const uint32_t tiles = (a.N + FG_BLOCK - 1) / FG_BLOCK, L = tab.n_levels;
-	GatherPlan plan{};
-	uint32_t blocks = tiles * L;
-	if (XCD) {
-		double total = 0.0, cost[FF_LEVELS];
-		for (uint32_t l = 0; l < L; ++l) { cost[l] = ((a.lv.hash_mask >> l) & 1u) ? 1.0 : (double)dense_cost; total += cost[l] * tiles; }
-		uint32_t level = 0, longest = 0;
-		double before = 0.0;
-		for (uint32_t x = 1; x < 8; ++x) {
-			const double target = total * x / 8;
-			while (level + 1 < L && before + cost[level] * tiles <= target) { before += cost[level] * tiles; ++level; }
-			double in_level = (target - before) / cost[level];
-			in_level = in_level < 0.0 ? 0.0 : in_level > tiles ? (double)tiles : in_level;
-			uint32_t b = level * tiles + (uint32_t)(in_level + 0.5);
-			plan.begin[x] = b < plan.begin[x - 1] ? plan.begin[x - 1] : b;
-		}
-		plan.begin[8] = L * tiles;
-		for (uint32_t x = 0; x < 8; ++x) longest = plan.begin[x + 1] - plan.begin[x] > longest ? plan.begin[x + 1] - plan.begin[x] : longest;
-		blocks = longest * 8;
-	}
-	field_gather_kernel<FULL, XCD, WIDE><<<dim3(blocks), dim3(FG_BLOCK), 0, s>>>(a, tiles, plan);
+static void launch_gather(const FusedArgs& a, const N2LevelTable& tab, hipStream_t s) {
+	const uint32_t tiles = (a.N + FG_BLOCK - 1) / FG_BLOCK;
+	field_gather_kernel<FULL><<<dim3(tiles * tab.n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
 }
 
 static uint32_t fused_grid(uint32_t n) {
@@ -665,7 +567,7 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 	a.dsdf_din = reinterpret_cast<hf*>(dsdf_din);
 	a.rgb_in = reinterpret_cast<hf*>(rgb_in);
 	a.output = reinterpret_cast<hf*>(d_output);
-	launch_gather<true>(a, *nets.tab, s, 0.6f);
+	launch_gather<true>(a, *nets.tab, s);
 	N2_LAUNCH_CHECK();
 	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();
@@ -687,7 +589,7 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 	// points in no particular order: a sample-major walk would touch all tables at once, so the features are gathered level
 	// by level into the network's input rows first
 	a.sdf_in = reinterpret_cast<hf*>(sdf_in);
-	launch_gather<false>(a, *nets.tab, s, 1.0f);
+	launch_gather<false>(a, *nets.tab, s);
 	N2_LAUNCH_CHECK();
 	field_fused_forward_kernel<false, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);
 	N2_LAUNCH_CHECK();

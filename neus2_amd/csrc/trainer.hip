@@ -6,9 +6,6 @@
 // the scene and the seed) may run ahead on a stream the trainer owns, into the
 // other of two sample sets, while this step's field kernels occupy the GPU.
 #include "n2_common.h"
-#ifndef N2_EXP
-#define N2_EXP 0
-#endif
 
 
 #include <cstring>
@@ -330,9 +327,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 			if (int rc = sample(t->sets[cur], s, t->n_rays_total, seed)) return rc;
 		}
 		t->n_rays_total += n_rays;
-		if (N2_EXP == 0) {
-			if (int rc = prefetch(cur)) return rc;
-		}
+		if (int rc = prefetch(cur)) return rc;
 	} else {
 		cur = 0;
 		if (int rc = sample(t->sets[0], s, t->n_rays_total, seed)) return rc;
@@ -356,9 +351,6 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, t->src_index, ray_counter, n_rays,
 	                                                                     t->ray_loss, t->counters);
 	N2_LAUNCH_CHECK();
-	if (N2_EXP == 1 && t->side) {
-		if (int rc = prefetch(cur)) return rc;
-	}
 	// forward + backward on the compacted batch, then the optimiser.  Every compacted sample is one of the marched
 	// samples the field has just been evaluated on: unless asked to run the field again, the activations saved for it
 	// are selected instead (the same values, a fraction of the work).
