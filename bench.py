@@ -201,22 +201,31 @@ def run_step_workload(args):
                          "note": f"{len(regions)} consecutive regions of {args.steps} steps; the first one is the timed region of `value`"}
     # (ii) the same loop on a trained field: rays stop at the surface, so a step marches more samples than it keeps
     if args.trained_steps > 0:
-        result["trained_state"] = trained_state_leg(tr, args, lib)
+        del tr
+        result["trained_state"] = trained_state_leg(args, lib, d_cams, len(cams), d_rgba, sdf_w)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cams, rgba, bits, sdf_w, n_rays, n_inf)
     return result
 
 
-def trained_state_leg(tr, args, lib):
-    """Trains the benchmark's scene for args.trained_steps steps at learning rate 1e-2 (configs/nerf/dtu.json:15) with the ray
-    budget's feedback every 20 steps, then times K steps exactly like the main region."""
+def trained_state_leg(args, lib, d_cams, n_cams, d_rgba, sdf_w):
+    """The same timed loop on a trained field.  A second trainer runs the loop the way the reference drives it
+    (src/testbed.cu:2641-2674): occupancy-grid updates on their cadence from step 0 (the rays march through the trainer's own
+    density grid instead of the analytic shell), learning rate 1e-2 (configs/nerf/dtu.json:15), the ray budget's feedback every
+    16 steps.  After args.trained_steps steps K steps are timed exactly like the main region (no occupancy update inside)."""
     import ctypes as C
+    import numpy as np
     import torch
-    from neus2_amd.capi import check
-    check(lib.n2_trainer_set_learning_rate(tr._h, C.c_float(1e-2)), "n2_trainer_set_learning_rate")
+    from neus2_amd.training import GRID_CELLS, OccupancyGrid, Trainer, default_config
+    tr = Trainer(default_config(target_batch_size=TARGET, max_rays_per_batch=1 << 16, max_samples=16 * TARGET, learning_rate=1e-2))
+    occ = OccupancyGrid(1, seed=1337, max_chunk=1 << 21)
+    tr.set_scene(d_cams, n_cams, d_rgba, occ.bitfield)
+    tr.attach_occupancy(occ)
+    tr.initialize_params(seed=1337, sdf_mlp_weights=sdf_w)
     for it in range(args.trained_steps):
+        tr.training_prep()
         tr.step()
-        if it % 20 == 19:
+        if it % 16 == 15 or it < 16:
             counters, ok = tr.update_budget()
             if not ok:
                 return {"error": f"no samples at step {it}: {counters}"}
@@ -230,10 +239,12 @@ def trained_state_leg(tr, args, lib):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     c = tr.read_counters()
+    occupied = float(np.unpackbits(occ.bitfield[:GRID_CELLS // 8].cpu().numpy()).mean())
     return {"ms_per_step": elapsed / args.steps * 1e3, "value": args.steps * min(c["compacted"], TARGET) / elapsed, "unit": "samples/s",
             "trained_steps": args.trained_steps, "rays_per_step": n_rays, "marched_samples_per_step": c["samples"], "inference_batch": n_inf,
-            "compacted_before_rollover": c["compacted"], "loss": c["loss"],
-            "note": "same timed loop after training; `value` counts the samples the rays kept (the batch is padded to 2^18 by rollover)"}
+            "compacted_before_rollover": c["compacted"], "occupied_cells": occupied, "loss": c["loss"],
+            "note": "same timed loop after training with the occupancy grid updated on its cadence; `value` counts the samples the "
+                    "rays kept (the batch is padded to 2^18 by rollover)"}
 
 
 def timed_best(fn, budget_s=15.0, min_runs=2, max_runs=8):

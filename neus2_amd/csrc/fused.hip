@@ -265,11 +265,14 @@ constexpr uint32_t FG_BLOCK = 256;
 template <bool FULL>
 __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
 	// level-major workgroup ids: the workgroups that run at one time work on one or two levels, whose tables stay in every
-	// L2.  Measured on the training step's 2.7e5 ray-ordered samples and dropped: whole levels dealt to XCDs by a cost plan
-	// (+9 us), one 8- or 16-byte load per pair of x neighbours instead of two 4-byte loads (+12 us).  Staging the coarse
-	// levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch and the five dense
-	// levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the positions and writing
-	// 320 bytes of features and slopes per sample.
+	// L2.  The launch is bound by the L2s' request rate: 13.1 M requests for the training step's 2.7e5 ray-ordered samples
+	// (four lines per sample on every level whose cells are smaller than the marching step), 63 % of them hits.  Measured on
+	// that workload and dropped: whole levels dealt to XCDs by a cost plan (the launch then fetches a third of the 278 MiB,
+	// but takes 9 to 20 us longer with every cost model tried), one 8- or 16-byte load per pair of x neighbours instead of
+	// two 4-byte loads (+12 us), a pair of lanes per sample so that the x neighbours' line is looked up once (+2 us).
+	// Staging the coarse levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch
+	// and the five dense levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the
+	// positions and writing 320 bytes of features and slopes per sample.
 	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
 	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
 	const uint32_t N = a.N;
@@ -326,6 +329,8 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 	const uint32_t N = a.N, hash_mask = a.lv.hash_mask, active = a.lv.active_levels;
 	const uint32_t n_tiles = (N + 31u) / 32u;
 	const uint32_t wave_gid = blockIdx.x * (FF_BLOCK / 64) + (threadIdx.x >> 6), n_waves = gridDim.x * (FF_BLOCK / 64);
+	// (Loading a wave's next tile while the current one is computed, into the registers the current operands have left, was
+	// measured on the full forward: no change; neither did three workgroups per CU at 168 registers, which spills.)
 	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
 		const uint32_t col_raw = tile * 32u + n;
 		const bool valid = col_raw < N;
