@@ -28,14 +28,11 @@ HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 # two passes the reference launches would be 588 + 664).
 ALGO_BYTES = {"grid_backward_params": 588, "grid_forward": 588, "grid_second_order": 664}
 STEP_ALGO_BYTES = {"grid_backward_params": 664, "grid_forward": 588}
-# MFMA work of one launch of the colour-network backward (the largest matrix kernel of a step), per sample:
-# recomputed forward 2 x (48x64 + 64x64) + data backward 2 x (16x64 + 64x64 + 64x48) + weight gradients 2 x (48x64 + 64x64 + 64x16)
-COLOUR_BACKWARD_FLOPS = 14336 + 16384 + 16384
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 # HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
 # (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
-# scatter pair = bin (43.2 + 105.9 MiB) + reduce (110.9 + 24.0 MiB); forward = 82.3 + 115.2 MiB
-STEP_TRAFFIC_BYTES = {"grid_backward_params": int(283.9 * 2**20), "grid_forward": int(197.6 * 2**20)}
+# scatter pair = bin (41.0 + 101.9 MiB) + reduce (110.9 + 24.0 MiB)
+STEP_TRAFFIC_BYTES = {"grid_backward_params": int(277.8 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9}
 
@@ -153,13 +150,14 @@ def run_step_workload(args):
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
-    # MFMA side of the metric: algorithmic flops of every MLP kernel of a step (SDF net 48-64-16: forward 8192 + input
-    # gradient 8192 per marched sample, backward 24576 + second order 14336 per batch sample; colour net 48-64-64-16:
-    # forward 16384 per marched sample, backward with the recomputed forward 47104 per batch sample) over their summed
-    # durations from the untimed per-kernel pass
-    mlp_flops = n_inf * (8192 + 8192 + 16384) + TARGET * (24576 + 14336 + 47104)
-    mlp_ms = sum(kernels[k]["ms_per_step"] for k in ("mlp_forward", "mlp_backward", "mlp_second_order") if k in kernels)
-    mfma = {"kernels": "mlp_forward + mlp_backward + mlp_second_order (all MLP launches of a step)", "algorithmic_flops_per_step": mlp_flops,
+    # MFMA side of the metric: the two weight-gradient launches of a step (colour net: recomputed forward 14336 + data
+    # gradients 16384 + weight gradients 16384 flop per batch sample; SDF net: 24576 + its second-order pass 14336), algorithmic
+    # flops over their summed durations from the untimed per-kernel pass.  The networks' forward passes run inside the fused
+    # field forward, which is timed together with the gather ("field_forward") and is bound by memory.
+    mlp_flops = TARGET * (24576 + 14336 + 47104)
+    mlp_ms = kernels["mlp_backward"]["ms_per_step"] if "mlp_backward" in kernels else 0.0
+    mfma = {"kernels": "mlp_wgrad (colour net) + mlp_wgrad (SDF net with second order): the weight-gradient launches of a step",
+            "algorithmic_flops_per_step": mlp_flops,
             "ms_per_step": mlp_ms, "achieved_tflops": mlp_flops / (mlp_ms * 1e-3) / 1e12 if mlp_ms else None, "peak_tflops": MFMA_PEAK_TFLOPS,
             "frac": mlp_flops / (mlp_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS if mlp_ms else None}
     result = {

@@ -122,3 +122,29 @@ def test_progressive_levels_schedule(oracle):
     steps = [f(s) for s in range(0, 5000, 100)]
     assert steps == sorted(steps)
     assert oracle.progressive_levels(16, 0.2, 0.02, 0, 5) == 16   # base_training_step 0: off
+
+
+def test_progressive_levels_tables_of_the_shipped_configs(oracle):
+    """The level schedule the adopted reading gives for the keys the reference ships (configs/nerf/base.json:31,36-38 and
+    configs/nerf/dtu.json:30,35-37: 14 levels, base 0.2, +0.02 per 100 resp. 200 steps), as (first step, levels in use):
+    closed form floor((0.2 + 0.02 (step // T)) 14 + 1e-3), i.e. level k + 1 joins at the first multiple of T with
+    0.02 (step // T) >= (k + 1) / 14 - 0.2 up to fp32 rounding."""
+    def table(period):
+        out, prev = [], None
+        for s in range(0, 40 * period + 1, period):
+            lv = oracle.progressive_levels(14, 0.2, 0.02, period, s)
+            assert lv == oracle.progressive_levels(14, 0.2, 0.02, period, s + period - 1)  # constant inside a period
+            if lv != prev:
+                out.append((s, lv))
+                prev = lv
+        return out
+    base = [(0, 2), (100, 3), (500, 4), (800, 5), (1200, 6), (1500, 7), (1900, 8), (2300, 9), (2600, 10), (3000, 11), (3300, 12),
+            (3700, 13), (4000, 14)]
+    assert table(100) == base
+    assert table(200) == [(2 * s, lv) for s, lv in base]
+    # the same schedule by the closed form in exact arithmetic: levels = floor(2.8 + 0.28 k) for k = step // T < 40
+    # (no k puts 2.8 + 0.28 k within the fp32 rounding and the 1e-3 guard of an integer except k = 40, which gives 14)
+    import fractions
+    for k in range(0, 41):
+        exact = min(14, int(fractions.Fraction(14, 5) + fractions.Fraction(7, 25) * k))
+        assert oracle.progressive_levels(14, 0.2, 0.02, 100, 100 * k) == exact, k
