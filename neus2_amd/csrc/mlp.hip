@@ -8,10 +8,11 @@
 // the first layer to the last (MFMA accumulators are re-packed in place into
 // the next layer's B operand), hidden activations are never written to memory
 // and the backward passes recompute them from the input.  Weights live in LDS
-// as ready-made MFMA operands (not in registers), and the batch-reduction
-// products of the weight gradients take their operands from a second set of
-// MFMAs with swapped arguments (see hidden_N) instead of a transposition
-// through memory.
+// as ready-made MFMA operands (not in registers).  The passes that produce
+// weight gradients (backward, backward + second order) are in mlp_wgrad.h:
+// their batch-reduction products read row-lane operands from an LDS staging
+// buffer.  The stand-alone second-order kernel here (mlp_bbi_kernel) still
+// takes them from a second set of MFMAs with swapped arguments (hidden_N).
 //
 // MFMA tiling (v_mfma_f32_32x32x16_f16, wave64):
 //   A (32 x 16, weights)      lane l holds A[l%32][8*(l/32) + 0..7]
@@ -104,7 +105,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_forward_kernel(const hf* __r
 }
 
 // ----------------------------------------------------------------------------
-// weight-gradient accumulators of one wave
+// weight-gradient accumulators of one wave (mlp_bbi_kernel)
 // ----------------------------------------------------------------------------
 // A wave with role r owns the gradient rows of neuron tile r (neurons 32r .. 32r+31):
 //   gW0[nt]    : dW_0  rows 32r + drow, columns 32nt + n
@@ -153,46 +154,28 @@ struct GradAcc {
 };
 
 // ----------------------------------------------------------------------------
-// backward kernel: recomputes the hidden activations, then
+// backward kernel WITHOUT weight gradients (input gradient, forward + input gradient): recomputes the hidden
+// activations, then
 //   dL_dh_last = mask * W_out^T dL_dy ; ... ; dL_dx = W_0^T dL_dh_0
-//   dW_out = dL_dy h_last^T ; dW_k = dL_dh_k h_{k-1}^T ; dW_0 = dL_dh_0 x^T
-// With WANT_DW two waves (roles 0 and 1) work on the same 64 samples; each accumulates the gradient
-// rows of one neuron tile (and computes one row tile of dL_dx), both run the cheap data chain.
-// Weight gradients are summed per workgroup in fp32 and written to one slab of `partials` per
-// workgroup; a second tiny kernel reduces the slabs.
-// ----------------------------------------------------------------------------
+// all in registers; a wave owns 64 samples as two 32-column tiles.  (The passes that also produce weight gradients are
+// mlp_wgrad_kernel, mlp_wgrad.h.)
 // WANT_Y: the forward output is written as well (the recomputed hidden activations are at hand): forward and input
 // gradient of the SDF net in one pass over its input.
-// Register cap: amdgpu_num_vgpr counts half of the unified vector registers on this part, so 120 means 240.  Two of
-// these waves then leave 32 of a SIMD's 512 registers free, enough for one small wave of another kernel: with the
-// 248 the compiler takes by itself, a CU that holds a single wave of the sample generator (which runs beside the
-// training step on its own stream) could start only one of these workgroups at a time, and the colour net's backward
-// took 67 us instead of 46.
-// SECOND (one hidden layer, with WANT_DW): the second-order pass of mlp_bbi_kernel rides along.  Its weight gradients
-//   dW_0 += (m * W_out^T g) v^T,  dW_out += g (m * W_0 v)^T
-// have the shape of the first-order ones, so they go into the same accumulators: the pass costs its own MFMAs but
-// shares the input loads, the activation mask, the fragment set-up and the slab of partial sums.
-template <int IC, int NH, bool WANT_DX, bool WANT_DW, bool WANT_Y = false, bool SECOND = false>
+// Register cap: amdgpu_num_vgpr counts half of the unified vector registers on this part, so 120 means 240.
+// ----------------------------------------------------------------------------
+template <int IC, int NH, bool WANT_Y = false>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(120))) mlp_backward_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N,
                                                                     const hf* __restrict__ dY, int dy_aos, int unit_row,
-                                                                    hf* __restrict__ dX, float* __restrict__ partials,
-                                                                    hf* __restrict__ Y = nullptr, int y_aos = 0,
-                                                                    const hf* __restrict__ V = nullptr, const hf* __restrict__ G2 = nullptr,
-                                                                    int unit_row2 = -1, const uint32_t* __restrict__ x_index = nullptr, uint32_t x_cols = 0) {
-	static_assert(!SECOND || (NH == 1 && WANT_DW), "the second-order pass needs one hidden layer and weight gradients");
+                                                                    hf* __restrict__ dX, hf* __restrict__ Y = nullptr, int y_aos = 0,
+                                                                    const uint32_t* __restrict__ x_index = nullptr, uint32_t x_cols = 0) {
 	using M = FragMap<IC, NH>;
-	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT, ROLES = WANT_DW ? 2 : 1;
-	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
+	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT;
 	extern __shared__ __align__(16) unsigned char smem[];
 	hf* F = reinterpret_cast<hf*>(smem);
-	build_frags<IC, NH>(F, W, M::COUNT);
+	build_frags<IC, NH>(F, W, M::SEL);
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, g = lane >> 5;
-	const int role = WANT_DW ? __builtin_amdgcn_readfirstlane(wave & 1) : 0;
 	const uint32_t n_tiles = (N + MLP_TILE - 1) / MLP_TILE;
-	const uint32_t slot = (blockIdx.x * (MLP_BLOCK / 64) + wave) / ROLES, n_slots = gridDim.x * (MLP_BLOCK / 64) / ROLES;
-	GradAcc<IC, NH> acc;
-	if (WANT_DW) acc.clear();
-
+	const uint32_t slot = blockIdx.x * (MLP_BLOCK / 64) + wave, n_slots = gridDim.x * (MLP_BLOCK / 64);
 	for (uint32_t tile = slot; tile < n_tiles; tile += n_slots) {
 		const uint32_t col_raw = tile * MLP_TILE + 2 * n;
 		const bool valid = col_raw < N;
@@ -204,18 +187,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 		else load_input<IC>(X, N, col, g, xp);
 		outgrad_frag(dY, N, col, g, (dy_aos & 1) != 0, unit_row, dy_aos >> 8, dyp[0], dyp[1]);
 		if (!valid) { dyp[0] = zero8(); dyp[1] = zero8(); }
-		half8 vp[2][IC], gp[2];
-		if (SECOND) {
-			load_input<IC>(V, N, col, g, vp);
-			outgrad_frag(G2, N, col, g, false, unit_row2, MLP_OUT, gp[0], gp[1]);
-			if (!valid) {
-				gp[0] = zero8(); gp[1] = zero8();
-#pragma unroll
-				for (int c = 0; c < IC; ++c) { vp[0][c] = zero8(); vp[1][c] = zero8(); }
-			}
-		}
-		constexpr int DX_TILES = WANT_DW ? 1 : IN_MT;  // with two roles each computes one row tile of dL_dx
-		half8 dx_keep[DX_TILES][2];                    // tile 0's rows until tile 1's are known (sample-pair stores)
+		half8 dx_keep[IN_MT][2];  // tile 0's rows until tile 1's are known (sample-pair stores)
 		half4 y_keep[2];
 #pragma unroll
 		for (int t = 0; t < 2; ++t) {
@@ -245,57 +217,12 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 				}
 			}
 			// ---- output layer ----
-			// dhN: gradient of the pre-activations of the current layer, neuron tile `role`, neuron-lane form
-			half8 dhN[2];
-			if (WANT_DW) {
-				half8 hN[2], dyN[2];
-				hidden_N<IC, NH>(F, lane, NH - 1, role, x, h, hN);
-				plain_pack(N2_MFMA(dy, frag(F, M::ID, lane), zero16()), dyN[0], dyN[1]);
-				acc.gWo = N2_MFMA(dyN[0], hN[0], acc.gWo);
-				acc.gWo = N2_MFMA(dyN[1], hN[1], acc.gWo);
-				mask_pack(N2_MFMA(dy, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], dhN[0], dhN[1]);
-				if (SECOND) {  // hN is the hidden layer itself here: its sign is the mask m
-					half8 v[IC], aN[2], bN[2], gN[2];
-					split_pairs<IC>(vp, t, v);
-					const half8 gg = gp[t];
-					float16v a = zero16();
-#pragma unroll
-					for (int c = 0; c < IC; ++c) a = N2_MFMA(v[c], frag(F, M::W0 + role * IC + c, lane), a);
-					mask_pack(a, hN[0], hN[1], aN[0], aN[1]);
-					mask_pack(N2_MFMA(gg, frag(F, M::WOT + role, lane), zero16()), hN[0], hN[1], bN[0], bN[1]);
-					plain_pack(N2_MFMA(gg, frag(F, M::ID, lane), zero16()), gN[0], gN[1]);
-					acc.gWo = N2_MFMA(gN[0], aN[0], acc.gWo);
-					acc.gWo = N2_MFMA(gN[1], aN[1], acc.gWo);
-#pragma unroll
-					for (int nt = 0; nt < IN_MT; ++nt) {
-						half8 vN[2];
-						input_N<IC, NH>(F, lane, nt, v, vN);
-						acc.gW0[nt] = N2_MFMA(bN[0], vN[0], acc.gW0[nt]);
-						acc.gW0[nt] = N2_MFMA(bN[1], vN[1], acc.gW0[nt]);
-					}
-				}
-			}
 #pragma unroll
 			for (int mt = 0; mt < 2; ++mt)
 				mask_pack(N2_MFMA(frag(F, M::WOT + mt, lane), dy, zero16()), h[NH - 1][2 * mt], h[NH - 1][2 * mt + 1], dh[2 * mt], dh[2 * mt + 1]);
 			// ---- hidden layers, last to first ----
 #pragma unroll
 			for (int k = NH - 1; k >= 1; --k) {
-				if (WANT_DW) {
-#pragma unroll
-					for (int nt = 0; nt < 2; ++nt) {
-						half8 hN[2];
-						hidden_N<IC, NH>(F, lane, k - 1, nt, x, h, hN);
-						acc.gWh[k - 1][nt] = N2_MFMA(dhN[0], hN[0], acc.gWh[k - 1][nt]);
-						acc.gWh[k - 1][nt] = N2_MFMA(dhN[1], hN[1], acc.gWh[k - 1][nt]);
-					}
-					half8 hN[2];
-					hidden_N<IC, NH>(F, lane, k - 1, role, x, h, hN);
-					float16v a = zero16();
-#pragma unroll
-					for (int c = 0; c < 4; ++c) a = N2_MFMA(dh[c], frag(F, M::WHT + (k - 1) * 8 + role * 4 + c, lane), a);
-					mask_pack(a, hN[0], hN[1], dhN[0], dhN[1]);
-				}
 				half8 dprev[4];
 #pragma unroll
 				for (int mt = 0; mt < 2; ++mt) {
@@ -308,42 +235,28 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) __attribute__((amdgpu_num_vgpr(1
 				for (int c = 0; c < 4; ++c) dh[c] = dprev[c];
 			}
 			// ---- first layer ----
-			if (WANT_DW) {
 #pragma unroll
-				for (int nt = 0; nt < IN_MT; ++nt) {
-					half8 xN[2];
-					input_N<IC, NH>(F, lane, nt, x, xN);
-					acc.gW0[nt] = N2_MFMA(dhN[0], xN[0], acc.gW0[nt]);
-					acc.gW0[nt] = N2_MFMA(dhN[1], xN[1], acc.gW0[nt]);
-				}
-			}
-			if (WANT_DX) {
+			for (int mt = 0; mt < IN_MT; ++mt) {
+				float16v d = zero16();
 #pragma unroll
-				for (int j = 0; j < DX_TILES; ++j) {
-					const int mt = WANT_DW ? role : j;
-					if (mt >= IN_MT) continue;
-					float16v d = zero16();
+				for (int c = 0; c < 4; ++c) d = N2_MFMA(frag(F, M::W0T + mt * 4 + c, lane), dh[c], d);
+				half8 lo, hi;
+				plain_pack(d, lo, hi);
+				if (t == 0) {
+					dx_keep[mt][0] = lo; dx_keep[mt][1] = hi;
+				} else if (valid) {
 #pragma unroll
-					for (int c = 0; c < 4; ++c) d = N2_MFMA(frag(F, M::W0T + mt * 4 + c, lane), dh[c], d);
-					half8 lo, hi;
-					plain_pack(d, lo, hi);
-					if (t == 0) {
-						dx_keep[j][0] = lo; dx_keep[j][1] = hi;
-					} else if (valid) {
-#pragma unroll
-						for (int e = 0; e < 8; ++e) {
-							// rows 32mt + drow(e, g) and 32mt + drow(8 + e, g); the 4g part is in off4
-							const int r0 = 32 * mt + 8 * (e >> 2) + (e & 3), r1 = r0 + 16;
-							if (r0 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r0 * N + off4) = half2v{dx_keep[j][0][e], lo[e]};
-							if (r1 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r1 * N + off4) = half2v{dx_keep[j][1][e], hi[e]};
-						}
+					for (int e = 0; e < 8; ++e) {
+						// rows 32mt + drow(e, g) and 32mt + drow(8 + e, g); the 4g part is in off4
+						const int r0 = 32 * mt + 8 * (e >> 2) + (e & 3), r1 = r0 + 16;
+						if (r0 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r0 * N + off4) = half2v{dx_keep[mt][0][e], lo[e]};
+						if (r1 + 4 * g < IN_W) *reinterpret_cast<half2v*>(dX + (size_t)r1 * N + off4) = half2v{dx_keep[mt][1][e], hi[e]};
 					}
 				}
 			}
 			tile_fence();
 		}
 	}
-	if (WANT_DW) acc.write_slab(reinterpret_cast<float*>(smem), partials + (size_t)blockIdx.x * N_PARAMS, N_PARAMS, wave, role, n, g);
 }
 
 // ----------------------------------------------------------------------------
@@ -738,12 +651,11 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
 	const int aos = (dL_layout == N2_LAYOUT_AOS ? 1 : 0) | ((int)dy_rows << 8);  // layout flag and the number of rows in use
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
-#define LAUNCH(IC, NH, DX, DW)                                                                                      \
+#define LAUNCH(IC, NH)                                                                                              \
 	do {                                                                                                            \
-		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT);                                                      \
-		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, DX, DW>, lds)) return rc;                                \
-		mlp_backward_kernel<IC, NH, DX, DW><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, next_slabs(mlp), \
-			nullptr, 0, nullptr, nullptr, -1, x_index, x_cols);                                                         \
+		const size_t lds = frag_bytes(FragMap<IC, NH>::SEL);                                                        \
+		if (int rc = allow_lds(mlp_backward_kernel<IC, NH>, lds)) return rc;                                        \
+		mlp_backward_kernel<IC, NH><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, nullptr, 0, x_index, x_cols); \
 	} while (0)
 #define LAUNCH_W(IC, NH, DX)                                                                                        \
 	do {                                                                                                            \
@@ -754,16 +666,16 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	} while (0)
 #define LAUNCH_Y(IC, NH)                                                                                            \
 	do {                                                                                                            \
-		const size_t lds = frag_bytes(FragMap<IC, NH>::COUNT);                                                      \
-		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, true, false, true>, lds)) return rc;                     \
-		mlp_backward_kernel<IC, NH, true, false, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, \
-			mlp->workspace, reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0);                  \
+		const size_t lds = frag_bytes(FragMap<IC, NH>::SEL);                                                        \
+		if (int rc = allow_lds(mlp_backward_kernel<IC, NH, true>, lds)) return rc;                                  \
+		mlp_backward_kernel<IC, NH, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos, unit_row, dX, \
+			reinterpret_cast<hf*>(d_output), out_layout == N2_LAYOUT_AOS ? 1 : 0);                                  \
 	} while (0)
 #define CALL(IC, NH)                                   \
 	do {                                               \
 		if (d_output) LAUNCH_Y(IC, NH);                        \
 		else if (want_dx && want_dw) LAUNCH_W(IC, NH, true);        \
-		else if (want_dx) LAUNCH(IC, NH, true, false);         \
+		else if (want_dx) LAUNCH(IC, NH);                      \
 		else LAUNCH_W(IC, NH, false);                          \
 	} while (0)
 	MLP_DISPATCH(mlp->in_w, mlp->n_hidden, CALL);
