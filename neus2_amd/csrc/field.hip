@@ -504,7 +504,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	const uint32_t n_src = f->last_n;
 	// colour net: only rows 0..2 of dL_doutput belong to it
 	if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
-	                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode)) return rc;
+	                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode, true)) return rc;
 	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
 	if (int rc = zero_padding(s, f->d_density_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.d_density_in)) return rc;
 	LevelScales scales{};
@@ -520,7 +520,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	// net (the reference's backward_backward_input with Accumulate) rides along
 	if (int rc = n2_mlp_backward_and_second_order_indexed(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n_src, index, n,
 	                                                      reinterpret_cast<const n2_half*>(f->d_rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in),
-	                                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, mode)) return rc;
+	                                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, mode, true)) return rc;
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)
 	if (int rc = n2_grid_backward_fused_indexed(f->grid, stream, f->xyz, n_src, index, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,

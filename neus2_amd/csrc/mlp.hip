@@ -629,7 +629,7 @@ static int allow_lds(K kernel, size_t bytes) {
 static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                              const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode,
                              n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA, uint32_t dy_rows = MLP_OUT,
-                             const uint32_t* x_index = nullptr, uint32_t x_cols = 0) {
+                             const uint32_t* x_index = nullptr, uint32_t x_cols = 0, bool dx_out_and_normal_only = false) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
@@ -664,6 +664,12 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 		mlp_wgrad_kernel<IC, NH, DX, false><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1, (int)dy_rows, dX, \
 			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols);                                                  \
 	} while (0)
+	// the field's colour net (48 inputs, two hidden layers): only the rows the field reads are stored
+	if (want_dx && want_dw && dx_out_and_normal_only && mlp->in_w == 48 && mlp->n_hidden == 2) {
+		LAUNCH_W(3, 2, WG_DX_OUT_AND_NORMAL);
+		N2_LAUNCH_CHECK();
+		return reduce_partials(mlp, s, blocks, mode);
+	}
 #define LAUNCH_Y(IC, NH)                                                                                            \
 	do {                                                                                                            \
 		const size_t lds = frag_bytes(FragMap<IC, NH>::SEL);                                                        \
@@ -674,9 +680,9 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 #define CALL(IC, NH)                                   \
 	do {                                               \
 		if (d_output) LAUNCH_Y(IC, NH);                        \
-		else if (want_dx && want_dw) LAUNCH_W(IC, NH, true);        \
+		else if (want_dx && want_dw) LAUNCH_W(IC, NH, WG_DX_ALL);   \
 		else if (want_dx) LAUNCH(IC, NH);                      \
-		else LAUNCH_W(IC, NH, false);                          \
+		else LAUNCH_W(IC, NH, WG_DX_NONE);                     \
 	} while (0)
 	MLP_DISPATCH(mlp->in_w, mlp->n_hidden, CALL);
 #undef CALL
@@ -709,10 +715,12 @@ N2_API int n2_mlp_backward_rows(n2_mlp_t* mlp, n2_stream_t stream, const n2_half
 }
 
 int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
-                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode) {
+                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode,
+                                 bool dx_out_and_normal_only) {
 	N2_REQUIRE(n_rows >= 1 && n_rows <= (uint32_t)MLP_OUT, "n2_mlp_backward_rows: n_rows %u outside [1, %d]", n_rows, MLP_OUT);
 	N2_REQUIRE(d_index == nullptr || n_cols >= 1, "n2_mlp_backward_rows: an indexed input needs at least one column");
-	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows, d_index, n_cols);
+	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows, d_index, n_cols,
+	                         dx_out_and_normal_only);
 }
 
 N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,
@@ -726,12 +734,13 @@ N2_API int n2_mlp_backward_and_second_order(n2_mlp_t* mlp, n2_stream_t stream, c
                                             const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode) {
 	return n2_mlp_backward_and_second_order_indexed(mlp, stream, d_input, 0, nullptr, n, d_dL_doutput, dL_layout, d_dL_dinput, d_dL_ddLdinput,
-	                                                d_second_dL_doutput, mode);
+	                                                d_second_dL_doutput, mode, false);
 }
 
 int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
                                              uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
-                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode) {
+                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode,
+                                             bool dx_encoding_only) {
 	const char* fn = "n2_mlp_backward_and_second_order";
 	N2_REQUIRE(d_index == nullptr || n_cols >= 1, "%s: an indexed input needs at least one column", fn);
 	if (int rc = check_mlp_batch(mlp, fn, d_input, n)) return rc;
@@ -757,12 +766,23 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 	const int aos = dL_layout == N2_LAYOUT_AOS ? 1 : 0;
 	const int unit_row2 = d_second_dL_doutput == nullptr ? 0 : -1;
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
+	if (dx_encoding_only && mlp->in_w == 48) {
+		// the field's SDF net: only the encoding's rows of dL/dinput are stored
+		const size_t lds = mlp_wgrad_lds<3, 1, true>();
+		if (int rc = allow_lds(mlp_wgrad_kernel<3, 1, WG_DX_ENCODING, true>, lds)) return rc;
+		mlp_wgrad_kernel<3, 1, WG_DX_ENCODING, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,
+			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,
+			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);
+		N2_LAUNCH_CHECK();
+		return reduce_partials(mlp, s, blocks, mode);
+	}
 	switch (mlp->in_w / 16) {
 #define CASE(IC)                                                                                                           \
 	case IC: {                                                                                                             \
 		const size_t lds = mlp_wgrad_lds<IC, 1, true>();                                                                   \
-		if (int rc = allow_lds(mlp_wgrad_kernel<IC, 1, true, true>, lds)) return rc;                                       \
-		mlp_wgrad_kernel<IC, 1, true, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,                        \
+		if (int rc = allow_lds(mlp_wgrad_kernel<IC, 1, WG_DX_ALL, true>, lds)) return rc;                                  \
+		mlp_wgrad_kernel<IC, 1, WG_DX_ALL, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,                   \
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,              \
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),              \
 			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);                                 \

@@ -64,7 +64,20 @@ __device__ __forceinline__ void load_tile_rows(const hf* __restrict__ X, uint32_
 		for (int e = 0; e < 8; ++e) x[c][e] = *reinterpret_cast<const hf*>(reinterpret_cast<const char*>(X + (size_t)(16 * c + e) * n_cols) + b);
 }
 
-template <int IC, int NH, bool WANT_DX, bool SECOND>
+// Which rows of dL/dinput a launch stores: all of them, or only those its caller reads (rows that differ between the two
+// halves of a wave turn into a predicate on the half, rows nobody reads cost no instruction)
+enum : int {
+	WG_DX_NONE = 0,
+	WG_DX_ALL = 1,
+	WG_DX_OUT_AND_NORMAL = 2,  // rows 0..15 and 35..37: the field's colour net (gradient of the SDF net's output and of the normal)
+	WG_DX_ENCODING = 3         // rows 3..34: the field's SDF net (gradient of the encoding; positions are not optimised)
+};
+__device__ __forceinline__ constexpr bool wg_dx_row(int mode, int row, int in_w) {
+	return row < in_w && (mode == WG_DX_ALL || (mode == WG_DX_OUT_AND_NORMAL && (row < 16 || (row >= 35 && row < 38))) ||
+	                      (mode == WG_DX_ENCODING && row >= 3 && row < 35));
+}
+
+template <int IC, int NH, int WANT_DX, bool SECOND>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N, const hf* __restrict__ dY,
                                                                  int dy_aos, int dy_rows, hf* __restrict__ dX, float* __restrict__ partials,
                                                                  const hf* __restrict__ V, const hf* __restrict__ G2, int unit_row2,
@@ -117,7 +130,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 				for (int c = 0; c < 4; ++c) a = N2_MFMA(frag(F, M::WHT + (k - 1) * 8 + t * 4 + c, lane), dh[k][c], a);
 				mask_pack(a, h[k - 1][2 * t], h[k - 1][2 * t + 1], dh[k - 1][2 * t], dh[k - 1][2 * t + 1]);
 			}
-		if (WANT_DX) {
+		if (WANT_DX != WG_DX_NONE) {
 #pragma unroll
 			for (int t = 0; t < IN_MT; ++t) {
 				float16v d = zero16();
@@ -127,7 +140,10 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 #pragma unroll
 					for (int r = 0; r < 16; ++r) {
 						const int row = 32 * t + 8 * (r >> 2) + (r & 3);  // + 4 g
-						if (row + 4 * g < IN_W) dX[(size_t)(row + 4 * g) * N + col] = (hf)d[r];
+						const bool lo = wg_dx_row(WANT_DX, row, IN_W), hi = wg_dx_row(WANT_DX, row + 4, IN_W);
+						if (lo && hi) dX[(size_t)(row + 4 * g) * N + col] = (hf)d[r];
+						else if (lo) { if (g == 0) dX[(size_t)row * N + col] = (hf)d[r]; }
+						else if (hi) { if (g == 1) dX[(size_t)(row + 4) * N + col] = (hf)d[r]; }
 					}
 				}
 			}

@@ -96,11 +96,16 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 // n2_mlp_backward_rows / n2_mlp_backward_and_second_order whose input is read through an index: sample i of the batch is
 // column d_index[i] of d_input, a matrix with n_cols columns (d_index null: column i of n columns).  Every other operand is
 // indexed by i.  The field's backward uses them to read the activations its forward saved for ALL marched samples.
+// dx_out_and_normal_only (48-input network with two hidden layers, the field's colour net): of d_dL_dinput only rows 0..15
+// and 35..37 are written (the gradients of the SDF net's output and of the normal; nothing reads the others).
+// dx_encoding_only (48-input network, the field's SDF net): only rows 3..34, the encoding's, are written.
 int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
-                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode);
+                                 const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode,
+                                 bool dx_out_and_normal_only);
 int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
                                              uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
-                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode);
+                                             const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode,
+                                             bool dx_encoding_only);
 // n2_adam_step that does nothing when *d_gate is zero on the device (d_gate null: always steps)
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
