@@ -175,14 +175,13 @@ __global__ void __launch_bounds__(FB) field_finish_output_kernel(const float* __
 //  * the variance gradient is the sum of row 7: every workgroup leaves its partial sum in var_part[blockIdx.x] and
 //    the launch that reduces the networks' weight gradients adds them up in a fixed order.
 struct LevelScales { float s[16]; };
-// SLOPES: the Jacobian comes as the fused forward stores it, 16 bytes per level and sample [level][n_src] without the level's scale factor
-// (scales.s[level] multiplies it back in); else as the grid encoding's fp32 dy_dx [enc_w][n_src][3].
-template <bool SLOPES>
+// The unfused path's form of this work (the Jacobian as the grid encoding's fp32 dy_dx [enc_w][n_src][3]); after a fused
+// forward the same work rides in the colour net's backward launch (N2FieldPrepTail), which reads the slopes instead.
 __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uint32_t enc_w, hf* __restrict__ d_rgb_in,
                                                                  const hf* __restrict__ dL_dout, float ek_batch, const float* __restrict__ dy_dx,
                                                                  float* __restrict__ v, hf* __restrict__ d_density_in,
                                                                  float* __restrict__ var_part, const uint32_t* __restrict__ src_index,
-                                                                 uint32_t n_src, LevelScales scales) {
+                                                                 uint32_t n_src) {
 	typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 	__shared__ float part[FB / 64];
 	const uint32_t i = blockIdx.x * FB + threadIdx.x;
@@ -203,28 +202,7 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 			v[(size_t)d * N + i] = x;
 			d_density_in[(size_t)d * N + i] = (hf)x;
 		}
-		if (SLOPES) {
-			const uint4* slopes = reinterpret_cast<const uint4*>(dy_dx);
-			constexpr uint32_t U = 8;  // eight levels' loads in flight per lane
-			for (uint32_t l0 = 0; 2 * l0 < enc_w; l0 += U) {
-				uint4 q[U];
-#pragma unroll
-				for (uint32_t u = 0; u < U; ++u) {
-					const uint32_t l = 2 * (l0 + u) < enc_w ? l0 + u : l0;
-					q[u] = slopes[(size_t)l * jn + js];
-				}
-#pragma unroll
-				for (uint32_t u = 0; u < U; ++u) {
-					if (2 * (l0 + u) < enc_w) {
-						float m[6];
-						const float unit = n2_slopes_unpack(q[u], m) * scales.s[l0 + u];
-						d_density_in[(size_t)(3 + 2 * (l0 + u)) * N + i] = (hf)((m[0] * vv[0] + m[1] * vv[1] + m[2] * vv[2]) * unit);
-						d_density_in[(size_t)(4 + 2 * (l0 + u)) * N + i] = (hf)((m[3] * vv[0] + m[4] * vv[1] + m[5] * vv[2]) * unit);
-					}
-				}
-			}
-		} else {
-		// eight rows' loads in flight per lane (see the normals kernel)
+		// eight rows' loads in flight per lane
 		constexpr uint32_t U = 8;
 		uint32_t r = 0;
 		for (; r + U <= enc_w; r += U) {
@@ -240,7 +218,6 @@ __global__ void __launch_bounds__(FB) field_backward_prep_kernel(uint32_t N, uin
 		for (; r < enc_w; ++r) {
 			const float* j = dy_dx + ((size_t)r * jn + js) * 3;
 			d_density_in[(size_t)(3 + r) * N + i] = (hf)(j[0] * vv[0] + j[1] * vv[1] + j[2] * vv[2]);
-		}
 		}
 	}
 #pragma unroll
@@ -369,7 +346,7 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.d_sdf_in = take(2ull * f->sdf_in_w * n);
 	c.v = take(12ull * n);
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
-	c.var_part = take(4ull * ((n + FB - 1) / FB + 1));
+	c.var_part = take(4ull * ((n + 127) / 128 + 1));  // one float per workgroup of whichever kernel forms the partial sums
 	c.sel_index = take(4ull * n);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
@@ -502,20 +479,34 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	// with a selection, sample i of the batch is column index[i] of the rows the forward saved over its n_src samples
 	const uint32_t* index = sel ? f->sel_use : nullptr;
 	const uint32_t n_src = f->last_n;
-	// colour net: only rows 0..2 of dL_doutput belong to it
-	if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
-	                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode, true)) return rc;
-	// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
 	if (int rc = zero_padding(s, f->d_density_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.d_density_in)) return rc;
 	LevelScales scales{};
 	for (uint32_t l = 0; l < 16 && 2 * l < f->enc_w; ++l) scales.s[l] = n2_grid_table(f->grid)->scale[l];
-	if (f->slopes_saved)
-		field_backward_prep_kernel<true><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-		                                                               f->d_density_in, f->var_part, index, f->last_n, scales);
-	else
-		field_backward_prep_kernel<false><<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v,
-		                                                                f->d_density_in, f->var_part, index, f->last_n, scales);
-	N2_LAUNCH_CHECK();
+	uint32_t var_parts = fgrid(n).x;
+	if (f->slopes_saved) {
+		// colour net (only rows 0..2 of dL_doutput belong to it); dL/dnormal, the second-order inputs, the direct gradient of
+		// the SDF output and the variance gradient's partial sums ride in the same launch
+		N2FieldPrepTail tail{};
+		tail.ek_batch = (float)ek_batch_size;
+		tail.slopes = f->dy_dx;
+		tail.n_src = f->last_n;
+		tail.enc_w = f->enc_w;
+		for (int l = 0; l < 16; ++l) tail.scale[l] = scales.s[l];
+		tail.v = f->v;
+		tail.d_density_in = f->d_density_in;
+		tail.var_part = f->var_part;
+		var_parts = n2_mlp_wgrad_blocks(n);
+		if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
+		                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode, true, &tail)) return rc;
+	} else {
+		// colour net: only rows 0..2 of dL_doutput belong to it
+		if (int rc = n2_mlp_backward_rows_indexed(f->rgb, stream, reinterpret_cast<const n2_half*>(f->rgb_in), n_src, index, n, d_dL_doutput, N2_LAYOUT_AOS, 3,
+		                                          reinterpret_cast<n2_half*>(f->d_rgb_in), mode, true)) return rc;
+		// dL/dnormal, the second-order inputs, the direct gradient of the SDF output and the variance gradient
+		field_backward_prep_kernel<<<fgrid(n), dim3(FB), 0, s>>>(n, f->enc_w, f->d_rgb_in, dL, (float)ek_batch_size, f->dy_dx, f->v, f->d_density_in,
+		                                                         f->var_part, index, f->last_n);
+		N2_LAUNCH_CHECK();
+	}
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient; the second-order pass through the
 	// net (the reference's backward_backward_input with Accumulate) rides along
 	if (int rc = n2_mlp_backward_and_second_order_indexed(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n_src, index, n,
@@ -527,7 +518,7 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	                                            reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n_src), mode)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
 	// pending: one launch sums them, and with them the partial sums of the variance gradient
-	return n2_mlp_reduce_deferred_sum(f->rgb, f->sdf, stream, f->var_part, fgrid(n).x, reinterpret_cast<n2_half*>(f->grads + f->off_var),
+	return n2_mlp_reduce_deferred_sum(f->rgb, f->sdf, stream, f->var_part, var_parts, reinterpret_cast<n2_half*>(f->grads + f->off_var),
 	                                  mode == N2_GRAD_ACCUMULATE ? 1 : 0);
 }
 

@@ -505,6 +505,7 @@ static inline uint32_t wgrad_grid(uint32_t n) {
 	const uint32_t rounds = (n + WG_SAMPLES - 1) / WG_SAMPLES;
 	return rounds < (uint32_t)MLP_MAX_SLABS ? rounds : (uint32_t)MLP_MAX_SLABS;
 }
+uint32_t n2_mlp_wgrad_blocks(uint32_t n) { return wgrad_grid(n); }
 
 #define MLP_DISPATCH(in_w, n_hidden, CALL)                                            \
 	do {                                                                              \
@@ -629,7 +630,8 @@ static int allow_lds(K kernel, size_t bytes) {
 static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n,
                              const n2_half* d_dL_doutput, n2_layout dL_layout, int unit_row, n2_half* d_dL_dinput, n2_grad_mode mode,
                              n2_half* d_output = nullptr, n2_layout out_layout = N2_LAYOUT_SOA, uint32_t dy_rows = MLP_OUT,
-                             const uint32_t* x_index = nullptr, uint32_t x_cols = 0, bool dx_out_and_normal_only = false) {
+                             const uint32_t* x_index = nullptr, uint32_t x_cols = 0, bool dx_out_and_normal_only = false,
+                             const N2FieldPrepTail* tail = nullptr) {
 	if (int rc = check_mlp_batch(mlp, "n2_mlp_backward", d_input, n)) return rc;
 	if (int rc = check_grad_mode(mlp, "n2_mlp_backward", mode)) return rc;
 	N2_REQUIRE(dL_layout == N2_LAYOUT_SOA || dL_layout == N2_LAYOUT_AOS, "n2_mlp_backward: bad layout %d", (int)dL_layout);
@@ -665,8 +667,18 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols);                                                  \
 	} while (0)
 	// the field's colour net (48 inputs, two hidden layers): only the rows the field reads are stored
+	N2_REQUIRE(tail == nullptr || (want_dx && want_dw && dx_out_and_normal_only && mlp->in_w == 48 && mlp->n_hidden == 2 && (aos & 1) && dy_rows <= 8),
+	           "n2_mlp_backward: the field's tail goes with the colour net's launch (48 inputs, two hidden layers, AoS output gradient)");
 	if (want_dx && want_dw && dx_out_and_normal_only && mlp->in_w == 48 && mlp->n_hidden == 2) {
-		LAUNCH_W(3, 2, WG_DX_OUT_AND_NORMAL);
+		if (tail) {
+			WgFieldPrepTail t{*tail};
+			const size_t lds = mlp_wgrad_lds<3, 2, false>();
+			if (int rc = allow_lds(mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail>, lds)) return rc;
+			mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1,
+				(int)dy_rows, dX, next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, t);
+		} else {
+			LAUNCH_W(3, 2, WG_DX_OUT_AND_NORMAL);
+		}
 		N2_LAUNCH_CHECK();
 		return reduce_partials(mlp, s, blocks, mode);
 	}
@@ -716,11 +728,11 @@ N2_API int n2_mlp_backward_rows(n2_mlp_t* mlp, n2_stream_t stream, const n2_half
 
 int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
                                  const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode,
-                                 bool dx_out_and_normal_only) {
+                                 bool dx_out_and_normal_only, const N2FieldPrepTail* tail) {
 	N2_REQUIRE(n_rows >= 1 && n_rows <= (uint32_t)MLP_OUT, "n2_mlp_backward_rows: n_rows %u outside [1, %d]", n_rows, MLP_OUT);
 	N2_REQUIRE(d_index == nullptr || n_cols >= 1, "n2_mlp_backward_rows: an indexed input needs at least one column");
 	return mlp_backward_impl(mlp, stream, d_input, n, d_dL_doutput, dL_layout, -1, d_dL_dinput, mode, nullptr, N2_LAYOUT_SOA, n_rows, d_index, n_cols,
-	                         dx_out_and_normal_only);
+	                         dx_out_and_normal_only, tail);
 }
 
 N2_API int n2_mlp_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_t dim, const n2_half* d_input, uint32_t n,

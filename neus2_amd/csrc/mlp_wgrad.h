@@ -17,6 +17,7 @@
 // matrix has two tiles only, the waves split the samples or the two products.  Each wave then holds 48 accumulator
 // registers instead of 128, and no activation is computed twice.
 #pragma once
+#include "grid_device.h"
 #include "mlp_device.h"
 
 constexpr int WG_SAMPLES = 128;              // samples per workgroup round (4 waves x 32)
@@ -77,12 +78,25 @@ __device__ __forceinline__ constexpr bool wg_dx_row(int mode, int row, int in_w)
 	                      (mode == WG_DX_ENCODING && row >= 3 && row < 35));
 }
 
-template <int IC, int NH, int WANT_DX, bool SECOND>
+// A tail: work on the same samples that rides along with a launch.  The field hangs the preparation of its SDF net's
+// backward on the colour net's kernel (N2FieldPrepTail, n2_common.h): that work streams 256 bytes of slopes per sample, and
+// inside this kernel, whose waves wait for barriers and matrix results half of their time, it costs less than as a launch
+// of its own between the two networks' kernels.
+struct WgNoTail {
+	static constexpr bool active = false;
+};
+struct WgFieldPrepTail {
+	static constexpr bool active = true;
+	N2FieldPrepTail a;
+};
+
+template <int IC, int NH, int WANT_DX, bool SECOND, class Tail = WgNoTail>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N, const hf* __restrict__ dY,
                                                                  int dy_aos, int dy_rows, hf* __restrict__ dX, float* __restrict__ partials,
                                                                  const hf* __restrict__ V, const hf* __restrict__ G2, int unit_row2,
-                                                                 const uint32_t* __restrict__ x_index, uint32_t x_cols) {
+                                                                 const uint32_t* __restrict__ x_index, uint32_t x_cols, const Tail tail = Tail()) {
 	static_assert(!SECOND || NH == 1, "the second-order pass needs one hidden layer");
+	static_assert(!Tail::active || (IC == 3 && NH == 2 && WANT_DX == WG_DX_OUT_AND_NORMAL), "the field's tail goes with the colour net");
 	using M = FragMap<IC, NH>;
 	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
@@ -98,6 +112,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 	const int G = lane >> 4;
 	const unsigned char* const tr = S + (4 * (G & 1) + (lane & 3)) * WG_QP + (8 * (G >> 1) + ((lane & 15) >> 2)) * 8;
 	float16v gW0 = zero16(), gWh = zero16(), gWo = zero16();
+	float var_acc = 0.f;  // tail: this lane's part of the variance gradient
 	const uint32_t n_rounds = (N + WG_SAMPLES - 1) / WG_SAMPLES;
 	for (uint32_t round = blockIdx.x; round < n_rounds; round += gridDim.x) {
 		const uint32_t col_raw = round * WG_SAMPLES + s_local;
@@ -105,14 +120,15 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 		const uint32_t col = valid ? col_raw : N - 1u;
 		// ---- the chain of this wave's 32 samples ----
 		half8 x[IC], dy, h[NH][4];
-		if (x_index) load_tile_rows<IC>(X, x_cols, min(x_index[col], x_cols - 1u), g, x);
-		else load_tile_rows<IC>(X, N, col, g, x);
+		const uint32_t col_src = x_index ? min(x_index[col], x_cols - 1u) : col;  // the sample's column in X
+		load_tile_rows<IC>(X, x_index ? x_cols : N, col_src, g, x);
 		if (dy_aos) {
 			dy = *reinterpret_cast<const half8*>(dY + (size_t)col * MLP_OUT + 8 * g);
 		} else {
 #pragma unroll
 			for (int e = 0; e < 8; ++e) dy[e] = dY[(size_t)(8 * g + e) * N + col];
 		}
+		const half8 dy_all = dy;  // tail: all 16 rows of the output gradient
 #pragma unroll
 		for (int e = 0; e < 8; ++e)
 			if (!valid || 8 * g + e >= dy_rows) dy[e] = (hf)0;
@@ -130,12 +146,18 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 				for (int c = 0; c < 4; ++c) a = N2_MFMA(frag(F, M::WHT + (k - 1) * 8 + t * 4 + c, lane), dh[k][c], a);
 				mask_pack(a, h[k - 1][2 * t], h[k - 1][2 * t + 1], dh[k - 1][2 * t], dh[k - 1][2 * t + 1]);
 			}
+		hf dn[2] = {(hf)0, (hf)0};  // tail: g = 0: row 35; g = 1: rows 36, 37 of dL/dinput
 		if (WANT_DX != WG_DX_NONE) {
 #pragma unroll
 			for (int t = 0; t < IN_MT; ++t) {
 				float16v d = zero16();
 #pragma unroll
 				for (int c = 0; c < 4; ++c) d = N2_MFMA(frag(F, M::W0T + t * 4 + c, lane), dh[0][c], d);
+				if constexpr (Tail::active) {
+					// row 0 also takes the direct gradient of the SDF output (row 3 of dL/doutput); rows 35..37 are dL/dnormal
+					if (t == 0 && g == 0) d[0] = (float)((hf)d[0] + dy_all[3]);
+					if (t == 1) { dn[0] = (hf)(g == 0 ? d[3] : d[0]); dn[1] = (hf)d[1]; }
+				}
 				if (valid) {
 #pragma unroll
 					for (int r = 0; r < 16; ++r) {
@@ -212,9 +234,60 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 		for (int c = 0; c < 4; ++c) stage_chained(st_ch + (4 * c) * WG_QP, dh[0][c]);
 #pragma unroll
 		for (int c = 0; c < IC; ++c) stage_natural(st_nat + (16 + 4 * c) * WG_QP, x[c]);
+		uint4 sl[Tail::active ? 8 : 1];
+		if constexpr (Tail::active) {
+			// the slopes of this lane's 8 levels (level 4 (j / 2) + 2 g + j % 2), in flight during the last products
+#pragma unroll
+			for (int j = 0; j < 8; ++j) {
+				const uint32_t level = 4u * (j >> 1) + 2u * g + (j & 1);
+				sl[j] = reinterpret_cast<const uint4*>(tail.a.slopes)[(size_t)(2u * level < tail.a.enc_w ? level : 0u) * tail.a.n_src + col_src];
+			}
+		}
 		__syncthreads();
 		if (nt < IN_MT) wgrad_tile<8>(tr, 8 * mt, 16 + 8 * nt, 0, gW0);
 		__syncthreads();
+		if constexpr (Tail::active) {
+			// dL/dnormal = row 35..37 of dL/dinput + rows 4..6 of dL/doutput / ek_batch + rows 8..10 of dL/doutput; its pieces
+			// sit in the two halves of the wave: g = 0 holds dn[0] and rows 4..6, g = 1 holds dn[0..1] (rows 36, 37) and rows 8..10
+			auto pk = [](hf a, hf b) { return (uint32_t)__builtin_bit_cast(unsigned short, a) | ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16); };
+			auto lo16 = [](uint32_t w) { return (float)__builtin_bit_cast(hf, (unsigned short)(w & 0xFFFFu)); };
+			auto hi16 = [](uint32_t w) { return (float)__builtin_bit_cast(hf, (unsigned short)(w >> 16)); };
+			const uint32_t m0 = g == 0 ? pk(dn[0], dy_all[4]) : pk(dn[0], dn[1]);
+			const uint32_t m1 = g == 0 ? pk(dy_all[5], dy_all[6]) : pk(dy_all[0], dy_all[1]);
+			const uint32_t m2 = g == 0 ? 0u : pk(dy_all[2], (hf)0);
+			const uint32_t o0 = (uint32_t)__shfl_xor((int)m0, 32), o1 = (uint32_t)__shfl_xor((int)m1, 32), o2 = (uint32_t)__shfl_xor((int)m2, 32);
+			const uint32_t a0 = g == 0 ? m0 : o0, a1 = g == 0 ? m1 : o1;             // what the lower half holds
+			const uint32_t b0 = g == 0 ? o0 : m0, b1 = g == 0 ? o1 : m1, b2 = g == 0 ? o2 : m2;  // what the upper half holds
+			float vv[3] = {lo16(a0), lo16(b0), hi16(b0)};
+			const float r4[3] = {hi16(a0), lo16(a1), hi16(a1)}, r8[3] = {lo16(b1), hi16(b1), lo16(b2)};
+#pragma unroll
+			for (int d = 0; d < 3; ++d) {
+				vv[d] += r4[d] / tail.a.ek_batch;
+				vv[d] += r8[d];
+			}
+			if (valid) {
+				if (g == 0) {
+					var_acc += (float)dy_all[7];
+#pragma unroll
+					for (int d = 0; d < 3; ++d) {
+						tail.a.v[(size_t)d * N + col] = vv[d];
+						reinterpret_cast<hf*>(tail.a.d_density_in)[(size_t)d * N + col] = (hf)vv[d];
+					}
+				}
+				// rows 3.. of the SDF net's second-order input: the encoding's dL_ddLdoutput = J v
+#pragma unroll
+				for (int j = 0; j < 8; ++j) {
+					const uint32_t level = 4u * (j >> 1) + 2u * g + (j & 1);
+					if (2u * level < tail.a.enc_w) {
+						float m[6];
+						const float unit = n2_slopes_unpack(sl[j], m) * tail.a.scale[level];
+						hf* o = reinterpret_cast<hf*>(tail.a.d_density_in) + (size_t)(3 + 2 * level) * N + col;
+						o[0] = (hf)((m[0] * vv[0] + m[1] * vv[1] + m[2] * vv[2]) * unit);
+						o[N] = (hf)((m[3] * vv[0] + m[4] * vv[1] + m[5] * vv[2]) * unit);
+					}
+				}
+			}
+		}
 		if constexpr (SECOND) {
 #pragma unroll
 			for (int c = 0; c < 4; ++c) stage_chained(st_ch + (4 * c) * WG_QP, sb[c]);
@@ -252,6 +325,15 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 	__syncthreads();
 	float* slab = partials + (size_t)blockIdx.x * N_PARAMS;
 	for (int i = threadIdx.x; i < N_PARAMS; i += MLP_BLOCK) slab[i] = Wl[i];
+	if constexpr (Tail::active) {
+		// the workgroup's part of the variance gradient (row 7 of dL/doutput), summed in a fixed order
+#pragma unroll
+		for (int o = 32; o > 0; o >>= 1) var_acc += __shfl_xor(var_acc, o);
+		__syncthreads();
+		if (lane == 0) Wl[wave] = var_acc;
+		__syncthreads();
+		if (threadIdx.x == 0) tail.a.var_part[blockIdx.x] = (Wl[0] + Wl[1]) + (Wl[2] + Wl[3]);
+	}
 }
 
 // dynamic LDS of the kernel: fragments, then the staging buffer (40 quad rows with the second-order pass, else 32)

@@ -93,6 +93,24 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
                        float* d_row0, bool density, n2_half* sdf_in);
 
+// What the field hangs on its colour net's backward launch (n2_mlp_backward_rows_indexed): for the same samples,
+//   * row 0 of d_dL_dinput also takes row 3 of d_dL_doutput (the direct gradient of the SDF output);
+//   * v[d] = row 35 + d of d_dL_dinput + row 4 + d of d_dL_doutput / ek_batch + row 8 + d of d_dL_doutput (dL/dnormal), written
+//     as fp32 rows (v, [3][n]) and as rows 0..2 of the SDF net's second-order input (d_density_in, fp16 rows of n columns);
+//   * rows 3.. of that input: the encoding's dL_ddLdoutput = J v from the slopes the fused forward saved ([levels][n_src] 16-byte
+//     blocks, read at the sample's column of the index; scale[l] = the level's scale factor);
+//   * var_part[workgroup] = the workgroup's sum of row 7 of d_dL_doutput (n2_mlp_wgrad_blocks(n) workgroups).
+struct N2FieldPrepTail {
+	float ek_batch;
+	const void* slopes;
+	uint32_t n_src, enc_w;
+	float scale[16];
+	float* v;
+	void* d_density_in;
+	float* var_part;
+};
+uint32_t n2_mlp_wgrad_blocks(uint32_t n);
+
 // n2_mlp_backward_rows / n2_mlp_backward_and_second_order whose input is read through an index: sample i of the batch is
 // column d_index[i] of d_input, a matrix with n_cols columns (d_index null: column i of n columns).  Every other operand is
 // indexed by i.  The field's backward uses them to read the activations its forward saved for ALL marched samples.
@@ -101,7 +119,7 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 // dx_encoding_only (48-input network, the field's SDF net): only rows 3..34, the encoding's, are written.
 int n2_mlp_backward_rows_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index, uint32_t n,
                                  const n2_half* d_dL_doutput, n2_layout dL_layout, uint32_t n_rows, n2_half* d_dL_dinput, n2_grad_mode mode,
-                                 bool dx_out_and_normal_only);
+                                 bool dx_out_and_normal_only, const N2FieldPrepTail* tail = nullptr);
 int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_input, uint32_t n_cols, const uint32_t* d_index,
                                              uint32_t n, const n2_half* d_dL_doutput, n2_layout dL_layout, n2_half* d_dL_dinput,
                                              const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode,
