@@ -45,10 +45,10 @@ def test_forward(oracle, in_w, n_hidden, n):
 
 
 @pytest.mark.parametrize("in_w,n_hidden", SHAPES)
-def test_backward_all_modes(oracle, in_w, n_hidden):
+@pytest.mark.parametrize("n", [8, 136, 10000])  # less than one wave's tile, a ragged second round of 128, many rounds per workgroup
+def test_backward_all_modes(oracle, in_w, n_hidden, n):
     from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_IGNORE, GRAD_OVERWRITE, LAYOUT_AOS, LAYOUT_SOA
     om, gm, W, dW, dG, rng = make(oracle, in_w, n_hidden, 2)
-    n = 10000
     x = q16(rng.standard_normal((in_w, n)))
     dy = q16(rng.standard_normal((16, n)))
     _, h = om.forward(W, x, round_hidden=True)
