@@ -136,22 +136,62 @@ __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uin
 	if (lane == 0) { scratch[ray] = RayScratch{{r0, r1, r2}, kept}; kept_of[ray] = kept; }
 }
 
+// before_of[r] = kept_of[0] + ... + kept_of[r - 1].  One workgroup per 1024 consecutive rays: it adds up the counts of all
+// rays before its own (coalesced, sixteen loads in flight per thread) and scans its own 1024 counts (lane shifts, the sixteen
+// wave totals through LDS).
+constexpr uint32_t OFFSETS_BLOCK = 1024;
+constexpr uint32_t OFFSETS_MIN_RAYS = 8192;
+__global__ void __launch_bounds__(OFFSETS_BLOCK) composite_offsets_kernel(uint32_t n_rays, const uint32_t* __restrict__ kept_of,
+                                                                          uint32_t* __restrict__ before_of) {
+	__shared__ uint32_t wave_before[OFFSETS_BLOCK / 64], wave_total[OFFSETS_BLOCK / 64];
+	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+	const uint32_t first = blockIdx.x * OFFSETS_BLOCK, ray = first + threadIdx.x;
+	const uint32_t own = ray < n_rays ? kept_of[ray] : 0u;
+	uint32_t before = 0;
+	for (uint32_t r0 = 0; r0 < first; r0 += 16 * OFFSETS_BLOCK) {
+		uint32_t v[16];
+#pragma unroll
+		for (uint32_t u = 0; u < 16; ++u) {
+			const uint32_t r = r0 + u * OFFSETS_BLOCK + threadIdx.x;
+			v[u] = r < first ? kept_of[r] : 0u;
+		}
+#pragma unroll
+		for (uint32_t u = 0; u < 16; ++u) before += v[u];
+	}
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
+	uint32_t incl = own;
+#pragma unroll
+	for (int o = 1; o < 64; o <<= 1) {
+		const uint32_t up = __shfl_up(incl, o);
+		if ((int)lane >= o) incl += up;
+	}
+	if (lane == 63u) { wave_before[wave] = before; wave_total[wave] = incl; }
+	__syncthreads();
+	uint32_t base = 0;
+#pragma unroll
+	for (uint32_t w = 0; w < OFFSETS_BLOCK / 64; ++w) base += wave_before[w] + (w < wave ? wave_total[w] : 0u);
+	if (ray < n_rays) before_of[ray] = base + incl - own;
+}
+
 __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, uint32_t n_rays, uint32_t* __restrict__ numsteps,
                                                                 const hf* __restrict__ net_out, const float* __restrict__ coords,
                                                                 const float* __restrict__ rgb_target, const RayScratch* __restrict__ scratch,
                                                                 const uint32_t* __restrict__ kept_of, uint32_t max_compacted,
                                                                 uint32_t* __restrict__ counter, float* __restrict__ coords_out,
-                                                                hf* __restrict__ dloss, float* __restrict__ loss, uint32_t* __restrict__ source_index) {
+                                                                hf* __restrict__ dloss, float* __restrict__ loss, uint32_t* __restrict__ source_index,
+                                                                const uint32_t* __restrict__ before_of) {
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 	// Where this workgroup's rays start in the compacted batch: the kept samples of all rays before them, in ray order
-	// (deterministic).  Every workgroup adds up the counts of its predecessors itself: a few KiB of L2 reads each
-	// instead of a scan kernel in between.
+	// (deterministic).  With a few thousand rays every workgroup adds up the counts of its predecessors itself: a few KiB
+	// of L2 reads each instead of a scan kernel in between.  That work grows with the square of the ray count, so beyond
+	// OFFSETS_MIN_RAYS rays composite_offsets_kernel has left the sums in before_of.
 	__shared__ uint32_t part[CB / 64];
 	const uint32_t first = blockIdx.x * (CB / 64);
 	uint32_t before = 0;
 	// eight loads in flight per lane: the last workgroups add up thousands of counts, and one dependent L2 round trip per
 	// CB of them was most of this kernel's duration
-	for (uint32_t r0 = 0; r0 < first; r0 += 8 * CB) {
+	for (uint32_t r0 = 0; r0 < (before_of ? 0u : first); r0 += 8 * CB) {
 		uint32_t v[8];
 #pragma unroll
 		for (uint32_t u = 0; u < 8; ++u) {
@@ -168,9 +208,13 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 	const uint32_t ray = first + wave;
 	if (ray >= n_rays) return;
 	uint32_t cb = 0;
+	if (before_of) {
+		cb = before_of[ray];
+	} else {
 #pragma unroll
-	for (int w = 0; w < CB / 64; ++w) cb += part[w];
-	for (int w = 0; w < wave; ++w) cb += kept_of[first + w];
+		for (int w = 0; w < CB / 64; ++w) cb += part[w];
+		for (int w = 0; w < wave; ++w) cb += kept_of[first + w];
+	}
 	const uint32_t kept = kept_of[ray];
 	const uint32_t m = min(max_compacted - min(max_compacted, cb), kept);  // the batch holds max_compacted samples
 	if (ray == n_rays - 1 && lane == 0) *counter = cb + kept;
@@ -357,13 +401,19 @@ N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_conf
 	unsigned char* w = reinterpret_cast<unsigned char*>(d_workspace);
 	RayScratch* scratch = reinterpret_cast<RayScratch*>(w);
 	uint32_t* kept_of = reinterpret_cast<uint32_t*>(w + up256(sizeof(RayScratch) * (uint64_t)n_rays));
+	uint32_t* before_of = n_rays >= OFFSETS_MIN_RAYS ? kept_of + up256(4ull * n_rays) / 4 : nullptr;
 	const dim3 grid((n_rays + CB / 64 - 1) / (CB / 64)), block(CB);
 	const hf* out = reinterpret_cast<const hf*>(d_network_output);
 	N2ProfScope prof(N2_PROF_COMPOSITE, s);
 	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch, kept_of);
 	N2_LAUNCH_CHECK();
+	if (before_of) {
+		composite_offsets_kernel<<<dim3((n_rays + OFFSETS_BLOCK - 1) / OFFSETS_BLOCK), dim3(OFFSETS_BLOCK), 0, s>>>(n_rays, kept_of, before_of);
+		N2_LAUNCH_CHECK();
+	}
 	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, kept_of, max_samples_compacted,
-	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss, d_source_index);
+	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss, d_source_index,
+	                                                 before_of);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

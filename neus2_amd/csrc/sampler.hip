@@ -255,7 +255,9 @@ __device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t*
 __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                             uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
                                                             const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts,
-                                                            uint32_t* __restrict__ mask, float* __restrict__ t_first) {
+                                                            uint32_t* __restrict__ mask, float* __restrict__ t_first,
+                                                            uint32_t* __restrict__ ray_counter) {
+	if (blockIdx.x == 0 && threadIdx.x == 0) *ray_counter = 0u;  // the scan kernel adds the kept rays up
 	const uint32_t i = blockIdx.x * RAYS_PER_BLOCK + (threadIdx.x >> 6);
 	if (i >= n_rays) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
@@ -263,43 +265,67 @@ __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_count_kernel(uint
 	if ((threadIdx.x & 63u) == 0) counts[i] = n;
 }
 
-// base[i] = exclusive sum of counts; slot[i] = rank among rays that have samples and fit the budget
+// Sum of the counts and number of non-zero counts of each block of 1024 consecutive rays.
+__global__ void __launch_bounds__(1024) sampler_block_totals_kernel(uint32_t n_rays, const uint32_t* __restrict__ counts,
+                                                                    uint32_t* __restrict__ block_sum, uint32_t* __restrict__ block_nz) {
+	__shared__ uint32_t ws[16], wn[16];
+	const uint32_t r = blockIdx.x * 1024u + threadIdx.x;
+	const uint32_t k = r < n_rays ? counts[r] : 0u;
+	uint32_t sum = k, nz = k ? 1u : 0u;
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) { sum += __shfl_xor(sum, o); nz += __shfl_xor(nz, o); }
+	if ((threadIdx.x & 63u) == 0) { ws[threadIdx.x >> 6] = sum; wn[threadIdx.x >> 6] = nz; }
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint32_t a = 0, c = 0;
+#pragma unroll
+		for (int w = 0; w < 16; ++w) { a += ws[w]; c += wn[w]; }
+		block_sum[blockIdx.x] = a;
+		block_nz[blockIdx.x] = c;
+	}
+}
+
+// base[i] = exclusive sum of counts; slot[i] = rank among rays that have samples and fit the budget.  One workgroup per block
+// of 1024 consecutive rays: it adds up the totals of the blocks before its own and scans its own counts.  The sums never
+// decrease, so once a ray with samples does not fit, no later one does: if the counts before this block fit the budget,
+// every earlier ray with samples was kept; if they do not, none of this block's rays is.  The number of kept rays is added
+// up over the workgroups with an integer atomic (*ray_counter was cleared by the count kernel).
 __global__ void __launch_bounds__(1024) sampler_scan_kernel(uint32_t n_rays, uint32_t max_samples, const uint32_t* __restrict__ counts,
+                                                            const uint32_t* __restrict__ block_sum, const uint32_t* __restrict__ block_nz,
                                                             uint32_t* __restrict__ base, uint32_t* __restrict__ slot,
                                                             uint32_t* __restrict__ ray_counter, uint32_t* __restrict__ sample_counter) {
-	__shared__ uint32_t wt_a[16], wt_b[16];
-	__shared__ uint32_t carry_a, carry_b;
+	__shared__ uint32_t before_a[16], before_nz[16], wt_a[16], wt_b[16];
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	if (threadIdx.x == 0) { carry_a = 0; carry_b = 0; }
+	const uint32_t r = blockIdx.x * 1024u + threadIdx.x;
+	const uint32_t k = r < n_rays ? counts[r] : 0u;
+	uint32_t sum = 0, nz = 0;
+	for (uint32_t q = threadIdx.x; q < blockIdx.x; q += 1024u) { sum += block_sum[q]; nz += block_nz[q]; }
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) { sum += __shfl_xor(sum, o); nz += __shfl_xor(nz, o); }
+	uint32_t v = k;
+#pragma unroll
+	for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(v, o); if (lane >= o) v += u; }
+	if (lane == 63) { before_a[wave] = sum; before_nz[wave] = nz; wt_a[wave] = v; }
 	__syncthreads();
-	for (uint32_t r0 = 0; r0 < n_rays; r0 += 1024) {
-		const uint32_t r = r0 + threadIdx.x;
-		const uint32_t k = r < n_rays ? counts[r] : 0u;
-		uint32_t v = k;
+	uint32_t all_before = 0, kept_before = 0, before = 0;
 #pragma unroll
-		for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(v, o); if (lane >= o) v += u; }
-		if (lane == 63) wt_a[wave] = v;
-		__syncthreads();
-		uint32_t before = carry_a;
-		for (int w = 0; w < wave; ++w) before += wt_a[w];
-		const uint32_t excl = before + v - k;
-		const uint32_t keep = (k > 0 && (uint64_t)excl + k <= max_samples) ? 1u : 0u;
-		uint32_t f = keep;
+	for (int w = 0; w < 16; ++w) { all_before += before_a[w]; kept_before += before_nz[w]; before += w < wave ? wt_a[w] : 0u; }
+	const uint32_t excl = all_before + before + v - k;
+	const uint32_t keep = (k > 0 && (uint64_t)excl + k <= max_samples) ? 1u : 0u;
+	uint32_t f = keep;
 #pragma unroll
-		for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(f, o); if (lane >= o) f += u; }
-		if (lane == 63) wt_b[wave] = f;
-		__syncthreads();
-		uint32_t before_b = carry_b;
-		for (int w = 0; w < wave; ++w) before_b += wt_b[w];
-		if (r < n_rays) {
-			base[r] = excl;
-			slot[r] = keep ? before_b + f - 1u : 0xFFFFFFFFu;
-		}
-		__syncthreads();
-		if (threadIdx.x == 1023) { carry_a = excl + k; carry_b = before_b + f; }
-		__syncthreads();
+	for (int o = 1; o < 64; o <<= 1) { const uint32_t u = __shfl_up(f, o); if (lane >= o) f += u; }
+	if (lane == 63) wt_b[wave] = f;
+	__syncthreads();
+	uint32_t before_b = all_before <= max_samples ? kept_before : 0u, kept_here = 0;
+#pragma unroll
+	for (int w = 0; w < 16; ++w) { before_b += w < wave ? wt_b[w] : 0u; kept_here += wt_b[w]; }
+	if (r < n_rays) {
+		base[r] = excl;
+		slot[r] = keep ? before_b + f - 1u : 0xFFFFFFFFu;
 	}
-	if (threadIdx.x == 0) { *ray_counter = carry_b; *sample_counter = carry_a; }
+	if (threadIdx.x == 0 && kept_here) atomicAdd(ray_counter, kept_here);
+	if (threadIdx.x == 1023 && blockIdx.x + 1 == gridDim.x) *sample_counter = excl + k;
 }
 
 // Coordinates of the samples the march marked, one wave per ray: lane l of window w is the step at t_first[w] plus l
@@ -346,7 +372,11 @@ __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_emit_kernel(uint3
 
 static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
 
-N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) { return 3 * up256(4ull * max_rays) + 2 * up256(4ull * 2 * WINDOWS * max_rays); }
+static inline uint32_t scan_blocks(uint32_t n_rays) { return (n_rays + 1023u) / 1024u; }
+
+N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) {
+	return 3 * up256(4ull * max_rays) + 2 * up256(4ull * 2 * WINDOWS * max_rays) + 2 * up256(4ull * scan_blocks(max_rays));
+}
 
 N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
                                         const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
@@ -372,12 +402,17 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	uint32_t* slot = reinterpret_cast<uint32_t*>(w + 2 * up256(4ull * n_rays));
 	uint32_t* mask = reinterpret_cast<uint32_t*>(w + 3 * up256(4ull * n_rays));
 	float* t_first = reinterpret_cast<float*>(w + 3 * up256(4ull * n_rays) + up256(4ull * 2 * WINDOWS * n_rays));
+	uint32_t* block_sum = reinterpret_cast<uint32_t*>(w + 3 * up256(4ull * n_rays) + 2 * up256(4ull * 2 * WINDOWS * n_rays));
+	uint32_t* block_nz = block_sum + up256(4ull * scan_blocks(n_rays)) / 4;
 	const dim3 grid((n_rays + RAYS_PER_BLOCK - 1) / RAYS_PER_BLOCK), block(64 * RAYS_PER_BLOCK);
 	N2ProfScope prof(N2_PROF_SAMPLER, s);
 	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                            background[2], d_bitfield, counts, mask, t_first);
+	                                            background[2], d_bitfield, counts, mask, t_first, d_ray_counter);
 	N2_LAUNCH_CHECK();
-	sampler_scan_kernel<<<dim3(1), dim3(1024), 0, s>>>(n_rays, max_samples, counts, base, slot, d_ray_counter, d_sample_counter);
+	sampler_block_totals_kernel<<<dim3(scan_blocks(n_rays)), dim3(1024), 0, s>>>(n_rays, counts, block_sum, block_nz);
+	N2_LAUNCH_CHECK();
+	sampler_scan_kernel<<<dim3(scan_blocks(n_rays)), dim3(1024), 0, s>>>(n_rays, max_samples, counts, block_sum, block_nz, base, slot, d_ray_counter,
+	                                                                 d_sample_counter);
 	N2_LAUNCH_CHECK();
 	sampler_emit_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
 	                                           background[2], mask, t_first, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);

@@ -151,7 +151,16 @@ __global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, c
 		__shared__ float part[4];
 		const uint32_t n = min(set_counters[0], max_rays);
 		float s = 0.f;
-		for (uint32_t i = threadIdx.x; i < n; i += 256) s += ray_loss[i];
+		for (uint32_t i0 = 0; i0 < n; i0 += 16u * 256u) {  // sixteen loads in flight per thread: tens of thousands of rays once they end at the surface
+			float v[16];
+#pragma unroll
+			for (uint32_t u = 0; u < 16; ++u) {
+				const uint32_t i = i0 + u * 256u + threadIdx.x;
+				v[u] = i < n ? ray_loss[i] : 0.f;
+			}
+#pragma unroll
+			for (uint32_t u = 0; u < 16; ++u) s += v[u];
+		}
 #pragma unroll
 		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
 		if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
