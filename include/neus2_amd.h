@@ -677,9 +677,11 @@ typedef struct n2_occupancy_buffers {
 	float* density_grid_tmp;  /* [n_cascades][128^3] maxima splatted by the last update */
 	uint8_t* bitfield;        /* [8][128^3 / 8] */
 	float* mean;              /* [1] mean of max(density, 0) over the first cascade */
-	float* positions;         /* [n_samples][3] sample positions of the last update */
-	uint32_t* indices;        /* [n_samples] their cells */
-	uint32_t n_samples, n_cascades, ema_step;
+	float* positions;         /* [n_samples][3] sample positions of the last update: first the n_uniform samples of the */
+	uint32_t* indices;        /* [n_samples] their cells            uniform group, then the others.  Within a group of n */
+	                          /* samples, slot t holds the reference's sample t (56924617^-1 mod 2^32) mod n when n is a   */
+	                          /* power of two (consecutive slots then fall into consecutive cells), else sample t          */
+	uint32_t n_samples, n_cascades, ema_step, n_uniform;
 	uint64_t rng_state, rng_inc;
 } n2_occupancy_buffers;
 

@@ -67,7 +67,7 @@ class OccupancyBuffers(C.Structure):
     """struct n2_occupancy_buffers"""
     _fields_ = [("density_grid", C.c_void_p), ("density_grid_tmp", C.c_void_p), ("bitfield", C.c_void_p), ("mean", C.c_void_p),
                 ("positions", C.c_void_p), ("indices", C.c_void_p), ("n_samples", C.c_uint32), ("n_cascades", C.c_uint32),
-                ("ema_step", C.c_uint32), ("rng_state", C.c_uint64), ("rng_inc", C.c_uint64)]
+                ("ema_step", C.c_uint32), ("n_uniform", C.c_uint32), ("rng_state", C.c_uint64), ("rng_inc", C.c_uint64)]
 
 
 class N2Error(RuntimeError):

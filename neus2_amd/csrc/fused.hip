@@ -269,7 +269,9 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 	// (four lines per sample on every level whose cells are smaller than the marching step), 63 % of them hits.  Measured on
 	// that workload and dropped: whole levels dealt to XCDs by a cost plan (the launch then fetches a third of the 278 MiB,
 	// but takes 9 to 20 us longer with every cost model tried), one 8- or 16-byte load per pair of x neighbours instead of
-	// two 4-byte loads (+12 us), a pair of lanes per sample so that the x neighbours' line is looked up once (+2 us).
+	// two 4-byte loads (+12 us), a pair of lanes per sample so that the x neighbours' line is looked up once (+2 us), loads of
+	// the hashed levels that bypass the L1 (agent- or system-scope: +27 us, the x neighbour's line is then requested twice and
+	// a request is no cheaper) or carry the non-temporal hint (no change).
 	// Staging the coarse levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch
 	// and the five dense levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the
 	// positions and writing 320 bytes of features and slopes per sample.

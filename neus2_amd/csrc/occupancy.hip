@@ -36,7 +36,7 @@ struct n2_occupancy {
 	uint8_t* bitfield;   // [8][128^3 / 8]
 	float* partial;      // [OCC_MEAN_BLOCKS]
 	float* mean;         // [1]
-	uint32_t last_n;
+	uint32_t last_n, last_n_uniform;
 };
 
 // ---------------------------------------------------------------------------
@@ -91,20 +91,38 @@ __device__ __forceinline__ uint32_t occ_morton3d_invert(uint32_t x) {
 
 // generate_grid_samples_nerf_nonuniform (:630-660), unit aabb.  Slots [n, n_pad) are filled with the cube centre
 // so that the field can run on a multiple of 8 points.
+//
+// Which sample a slot holds.  The first candidate cell of sample i is ((i + step n) P + R) mod 128^3 with P = 56924617: a
+// pseudo-random walk over the cells, so that consecutive samples would splat their maxima into unrelated memory lines
+// (one atomic request per sample).  The samples are independent of each other, so the order they are generated and
+// evaluated in is free: when n is a power of two, slot t holds sample i(t) = t P^-1 mod n (P^-1 mod 2^32, masked), whose
+// candidate cell is t + const mod n: consecutive slots splat into consecutive cells of (at most 128^3 / n) runs, and a
+// wave's 64 atomics fall into a few lines.  Other n: slot t holds sample t.
+constexpr uint32_t OCC_WALK = 56924617u;
+constexpr uint32_t occ_inverse_mod_2_32(uint32_t a) {  // a odd; Newton's iteration doubles the number of correct low bits
+	uint32_t x = a;                                     // a * a = 1 mod 8
+	for (int k = 0; k < 5; ++k) x *= 2u - a * x;
+	return x;
+}
+constexpr uint32_t OCC_WALK_INV = occ_inverse_mod_2_32(OCC_WALK);
+static_assert(OCC_WALK * OCC_WALK_INV == 1u, "inverse of the walk's multiplier");
+static inline uint32_t occ_order_mul(uint32_t n) { return (n >= 2 && (n & (n - 1)) == 0) ? OCC_WALK_INV : 0u; }
+
 __global__ void __launch_bounds__(OCC_BLOCK) occ_generate_kernel(uint32_t n, uint32_t n_pad, Pcg32 rng, uint32_t step, const float* __restrict__ grid,
-                                                                 uint32_t n_cascades, float thresh, float* __restrict__ positions,
-                                                                 uint32_t* __restrict__ indices) {
-	const uint32_t i = blockIdx.x * OCC_BLOCK + threadIdx.x;
-	if (i >= n_pad) return;
-	if (i >= n) {
-		positions[(size_t)i * 3] = 0.5f; positions[(size_t)i * 3 + 1] = 0.5f; positions[(size_t)i * 3 + 2] = 0.5f;
+                                                                 uint32_t n_cascades, float thresh, uint32_t order_mul,
+                                                                 float* __restrict__ positions, uint32_t* __restrict__ indices) {
+	const uint32_t slot = blockIdx.x * OCC_BLOCK + threadIdx.x;
+	if (slot >= n_pad) return;
+	if (slot >= n) {
+		positions[(size_t)slot * 3] = 0.5f; positions[(size_t)slot * 3 + 1] = 0.5f; positions[(size_t)slot * 3 + 2] = 0.5f;
 		return;
 	}
+	const uint32_t i = order_mul ? (slot * order_mul) & (n - 1u) : slot;
 	rng.advance((uint64_t)i * 4);
 	const uint32_t level = (uint32_t)(rng.next_float() * n_cascades) % n_cascades;
 	uint32_t idx = 0;
 	for (uint32_t j = 0; j < 10; ++j) {
-		idx = ((i + step * n) * 56924617u + j * 19349663u + 96925573u) % OCC_CELLS;
+		idx = ((i + step * n) * OCC_WALK + j * 19349663u + 96925573u) % OCC_CELLS;
 		idx += level * OCC_CELLS;
 		if (grid[idx] > thresh) break;
 	}
@@ -114,9 +132,9 @@ __global__ void __launch_bounds__(OCC_BLOCK) occ_generate_kernel(uint32_t n, uin
 	for (int d = 0; d < 3; ++d) {
 		const float c = (float)occ_morton3d_invert(pos_idx >> d);
 		const float u = rng.next_float();
-		positions[(size_t)i * 3 + d] = ((c + u) / (float)OCC_GRIDSIZE - 0.5f) * scale + 0.5f;
+		positions[(size_t)slot * 3 + d] = ((c + u) / (float)OCC_GRIDSIZE - 0.5f) * scale + 0.5f;
 	}
-	indices[i] = idx;
+	indices[slot] = idx;
 }
 
 // splat_grid_samples_nerf_max_nearest_neighbor (:662-680): positive floats order like their bit patterns
@@ -273,6 +291,7 @@ N2_API int n2_occupancy_set_workspace(n2_occupancy_t* occ, void* d_workspace, ui
 	occ->partial = reinterpret_cast<float*>(b + c.partial);
 	occ->mean = reinterpret_cast<float*>(b + c.mean);
 	occ->last_n = 0;
+	occ->last_n_uniform = 0;
 	return N2_OK;
 }
 
@@ -326,15 +345,15 @@ N2_API int n2_occupancy_update(n2_occupancy_t* occ, n2_field_t* field, n2_stream
 		// slots of the second group are written by the second launch; only the last launch pads
 		const uint32_t pad = n_nonuniform ? n_uniform : (n_uniform + 7) / 8 * 8;
 		occ_generate_kernel<<<ogrid(pad), dim3(OCC_BLOCK), 0, s>>>(n_uniform, pad, rng, occ->ema_step, occ->grid, occ->n_cascades, -0.01f,
-		                                                          occ->positions, occ->indices);
+		                                                          occ_order_mul(n_uniform), occ->positions, occ->indices);
 		N2_LAUNCH_CHECK();
 	}
 	rng.advance(1ull << 32);
 	if (n_nonuniform) {
 		const uint32_t pad = (n + 7) / 8 * 8 - n_uniform;
 		occ_generate_kernel<<<ogrid(pad), dim3(OCC_BLOCK), 0, s>>>(n_nonuniform, pad, rng, occ->ema_step, occ->grid, occ->n_cascades,
-		                                                          OCC_MIN_OPTICAL_THICKNESS, occ->positions + (size_t)n_uniform * 3,
-		                                                          occ->indices + n_uniform);
+		                                                          OCC_MIN_OPTICAL_THICKNESS, occ_order_mul(n_nonuniform),
+		                                                          occ->positions + (size_t)n_uniform * 3, occ->indices + n_uniform);
 		N2_LAUNCH_CHECK();
 	}
 	rng.advance(1ull << 32);
@@ -351,6 +370,7 @@ N2_API int n2_occupancy_update(n2_occupancy_t* occ, n2_field_t* field, n2_stream
 	N2_LAUNCH_CHECK();
 	occ->ema_step += 1;
 	occ->last_n = n;
+	occ->last_n_uniform = n_uniform;
 	return occ_bitfield_from_partials(occ, s);
 }
 
@@ -364,6 +384,7 @@ N2_API int n2_occupancy_view(n2_occupancy_t* occ, n2_occupancy_buffers* out) {
 	out->positions = occ->positions;
 	out->indices = occ->indices;
 	out->n_samples = occ->last_n;
+	out->n_uniform = occ->last_n_uniform;
 	out->n_cascades = occ->n_cascades;
 	out->ema_step = occ->ema_step;
 	out->rng_state = occ->rng_state;

@@ -187,9 +187,17 @@ class OccupancyGrid:
         return self._tensor(self.view().mean, 4, torch.float32)
 
     def last_samples(self):
+        """Positions [n, 3] and cells [n] of the last update's samples, in the reference's order (the uniform group, then
+        the others; the library keeps a group of 2^k samples in the order that walks the cells in sequence)."""
         v = self.view()
-        return (self._tensor(v.positions, 12 * v.n_samples, torch.float32).view(-1, 3),
-                self._tensor(v.indices, 4 * v.n_samples, torch.int32))
+        pos = self._tensor(v.positions, 12 * v.n_samples, torch.float32).view(-1, 3)
+        idx = self._tensor(v.indices, 4 * v.n_samples, torch.int32)
+        slot = torch.arange(v.n_samples, dtype=torch.int64, device=pos.device)
+        for first, n in ((0, v.n_uniform), (v.n_uniform, v.n_samples - v.n_uniform)):
+            if n >= 2 and n & (n - 1) == 0:  # sample i sits in slot i * 56924617 mod n of its group
+                i = torch.arange(n, dtype=torch.int64, device=pos.device)
+                slot[first:first + n] = first + (i * 56924617) % n
+        return pos[slot], idx[slot]
 
 
 class Trainer:
