@@ -32,7 +32,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 # HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
 # (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
 # scatter pair = bin (41.0 + 101.9 MiB) + reduce (110.9 + 24.0 MiB)
-STEP_TRAFFIC_BYTES = {"grid_backward_params": int(277.8 * 2**20)}
+STEP_TRAFFIC_BYTES = {"grid_backward_params": int(277.9 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9}
 
@@ -519,8 +519,8 @@ def run_occupancy_workload(args):
 
 
 def run_mesh_workload(args):
-    """The consumer of configuration 5 of BASELINE.json: marching cubes over the 512^3 SDF lattice (count, prefix sums, vertices, faces,
-    normals).  The lattice is evaluated once, untimed (that part is `--workload lattice`); a step is one full extraction."""
+    """The consumer of configuration 5 of BASELINE.json: marching cubes over the 512^3 SDF lattice (count per tile, prefix sums over
+    the tiles, vertices, faces, normals).  The lattice is evaluated once, untimed (that part is `--workload lattice`); a step is one full extraction."""
     import numpy as np
     import torch
     from neus2_amd.mesh import density_on_grid, marching_cubes
@@ -538,9 +538,9 @@ def run_mesh_workload(args):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     n_pts = RES ** 3
-    # algorithmic bytes per lattice point: density read once by each of count, vertices, faces (12) + two counters written,
-    # scanned (read + write, twice) and read back (8 + 16 + 16 + 8 = 48); output vertices / indices / normals are small
-    algo = 60
+    # algorithmic bytes per lattice point: the density is read once (4); the emitting passes touch only the tiles the surface
+    # crosses, and vertices / indices / normals are small next to the lattice
+    algo = 4
     achieved = algo * n_pts / (elapsed / args.steps) / 1e9
     return {"metric": "marching-cubes lattice points/sec over a 512^3 SDF lattice (1 GPU)", "value": args.steps * n_pts / elapsed, "unit": "points/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True,

@@ -725,10 +725,11 @@ uint64_t n2_marching_cubes_workspace_bytes(const uint32_t res[3]);
 int n2_marching_cubes_count(n2_stream_t stream, const uint32_t res[3], const float aabb_min[3], const float aabb_max[3],
                             float thresh, const float* d_density, void* d_workspace, uint64_t workspace_bytes,
                             uint32_t* n_vertices, uint32_t* n_triangles);
-/* Second pass with the workspace of the first: d_vertices fp32 [n_vertices][3], d_indices uint32 [n_triangles][3],
+/* Second pass with the workspace of the first (it holds the per-tile prefix sums; this pass adds the vertex slots of
+ * the lattice points that own a vertex): d_vertices fp32 [n_vertices][3], d_indices uint32 [n_triangles][3],
  * d_normals fp32 [n_vertices][3] or NULL (not normalised, like the reference's). */
 int n2_marching_cubes_emit(n2_stream_t stream, const uint32_t res[3], const float aabb_min[3], const float aabb_max[3],
-                           float thresh, const float* d_density, const void* d_workspace, float* d_vertices,
+                           float thresh, const float* d_density, void* d_workspace, float* d_vertices,
                            uint32_t* d_indices, float* d_normals, uint32_t n_vertices, uint32_t n_triangles);
 /* get_density_on_grid: the field's SDF (row 0 of NerfNetwork::sdf, fp16 widened to fp32) at the lattice points
  * (x, y, z)/res * (aabb_max - aabb_min) + aabb_min, evaluated `chunk` points at a time (a multiple of 8, at most the

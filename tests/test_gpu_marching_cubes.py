@@ -18,7 +18,8 @@ def test_case_table_equals_the_oracles():
     np.testing.assert_array_equal(case_table(), omc.TRIANGLE_TABLE)
 
 
-@pytest.mark.parametrize("res,kind", [((40, 48, 32), "sphere"), ((17, 9, 33), "noise"), ((2, 2, 2), "noise"), ((64, 64, 64), "two")])
+@pytest.mark.parametrize("res,kind", [((40, 48, 32), "sphere"), ((17, 9, 33), "noise"), ((2, 2, 2), "noise"), ((64, 64, 64), "two"),
+                                      ((100, 24, 10), "noise"), ((130, 9, 7), "noise"), ((96, 80, 72), "sphere")])  # rows that end inside a wave's 64 points
 def test_mesh_matches_oracle(res, kind):
     from neus2_amd.mesh import marching_cubes
     rng = np.random.default_rng(res[0])
