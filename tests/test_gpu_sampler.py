@@ -18,7 +18,8 @@ def sc(oracle):
     return cams, rgba, bits
 
 
-@pytest.mark.parametrize("n_rays,total,seed,cap", [(4096, 0, 1, 1 << 19), (1000, 7777, 5, 1 << 19), (4096, 0, 2, 20000), (1, 0, 3, 4096)])
+@pytest.mark.parametrize("n_rays,total,seed,cap", [(4096, 0, 1, 1 << 19), (1000, 7777, 5, 1 << 19), (4096, 0, 2, 20000), (1, 0, 3, 4096),
+                                                  (70000, 0, 4, 1 << 19)])  # dozens of scan blocks, the budget cut in the middle
 def test_sampler_bit_exact(oracle, sc, n_rays, total, seed, cap):
     from neus2_amd.tcnn_api import generate_training_samples, pack_cameras
     cams, rgba, bits = sc
