@@ -49,9 +49,10 @@ def _same(a, b):
 
 def test_static_scratch_matches_workspace_entry_point():
     rng = np.random.default_rng(11)
-    # first call: 3000 rays; second call, right after it on the same GPU: 700 rays (the array keeps the first call's rows)
-    for n_rays, cap, sharp in ((3000, 1 << 18, True), (700, 1 << 14, False)):
-        numsteps, out, coords, target = make_rays(rng, n_rays, lo=1, hi=150, sharp=sharp)
+    # first call: 3000 rays; then 9000 (from 8192 rays on the rays' places come from a scan kernel, whose sums sit in the
+    # scratch as well); then, right after it on the same GPU, 700 rays (the array keeps the earlier calls' rows)
+    for n_rays, cap, sharp, hi in ((3000, 1 << 18, True, 150), (9000, 1 << 18, True, 40), (700, 1 << 14, False, 150)):
+        numsteps, out, coords, target = make_rays(rng, n_rays, lo=1, hi=hi, sharp=sharp)
         ref = _call(False, numsteps, out, coords, target, cap)
         got = _call(True, numsteps, out, coords, target, cap)
         assert int(ref["counter"][0]) > 0
