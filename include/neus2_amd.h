@@ -481,12 +481,13 @@ int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* con
 
 /* n2_composite_loss_indexed without a workspace argument, for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
- * per-ray scratch (composited colour and kept-sample count of every ray, 24 bytes per ray) lives in an array inside
+ * per-ray scratch (composited colour, kept-sample count and the count's prefix sum of every ray, 24 bytes per ray) lives in an array inside
  * the library's device image, 1.5 MiB that each GPU the library runs on holds until the process ends; the call
  * allocates and frees nothing.  n_rays above N2_COMPOSITE_STATIC_MAX_RAYS is rejected with N2_ERR_INVALID_ARGUMENT.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or host threads
  * without ordering between them) race; calls ordered on one stream are safe.  Nothing in the array has to start at
- * zero: the forward kernel writes every ray's slot below n_rays before the backward kernel reads it.  Results are
+ * zero: the forward kernel writes every ray's slot below n_rays (and, from 8192 rays on, the scan kernel every prefix sum)
+ * before the backward kernel reads it.  Results are
  * bit-identical to n2_composite_loss_indexed's. */
 #define N2_COMPOSITE_STATIC_MAX_RAYS 65536u
 int n2_composite_loss_static(n2_stream_t stream, const n2_composite_config* config, uint32_t n_rays,

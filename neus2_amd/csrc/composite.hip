@@ -334,7 +334,7 @@ N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg,
 	                                 d_workspace, workspace_bytes);
 }
 
-// Scratch of n2_composite_loss_static: per-ray colour and kept counts for up to N2_COMPOSITE_STATIC_MAX_RAYS rays, held
+// Scratch of n2_composite_loss_static: per-ray colour, kept counts and their prefix sums for up to N2_COMPOSITE_STATIC_MAX_RAYS rays, held
 // by every GPU the library runs on until the process ends.  In host code the array's name stands for the symbol only;
 // the device address of each GPU's copy is looked up once per device (static_scratch) and that pointer is what the
 // kernels receive.
