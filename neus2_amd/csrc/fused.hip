@@ -61,6 +61,7 @@ struct FusedArgs {
 	uint32_t sdf_in_w, enc_w;
 	float sdf_bias;
 	uint32_t N;
+	const uint32_t* live;   // or null: only samples below min(*live, N) are evaluated (N stays the column count of the matrices)
 	const float* pos;       // coordinate d of sample i at pos[i * ps + d * ds]
 	uint32_t ps, ds;
 	const float* coords;    // full field: [N][7] NerfCoordinate (direction at 4..6)
@@ -278,7 +279,7 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
 	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
 	const uint32_t N = a.N;
-	if (i >= N) return;
+	if (i >= N || (a.live && i >= *a.live)) return;
 	const float* q = FULL ? a.coords + (size_t)i * 7 : a.pos + (size_t)i * a.ps;
 	const size_t qs = FULL ? 1 : a.ds;
 	const float p[3] = {q[0], q[qs], q[2 * qs]};
@@ -329,14 +330,15 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 	build_fused_frags(F, a, FULL ? FF_COUNT : FF_SDF_COUNT);
 	const int lane = threadIdx.x & 63, n = lane & 31, g = lane >> 5;
 	const uint32_t N = a.N, hash_mask = a.lv.hash_mask, active = a.lv.active_levels;
-	const uint32_t n_tiles = (N + 31u) / 32u;
+	const uint32_t n_live = a.live ? min(*a.live, N) : N;
+	const uint32_t n_tiles = (n_live + 31u) / 32u;
 	const uint32_t wave_gid = blockIdx.x * (FF_BLOCK / 64) + (threadIdx.x >> 6), n_waves = gridDim.x * (FF_BLOCK / 64);
 	// (Loading a wave's next tile while the current one is computed, into the registers the current operands have left, was
 	// measured on the full forward: no change; neither did three workgroups per CU at 168 registers, which spills.)
 	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
 		const uint32_t col_raw = tile * 32u + n;
-		const bool valid = col_raw < N;
-		const uint32_t col = valid ? col_raw : N - 1u;
+		const bool valid = col_raw < n_live;
+		const uint32_t col = valid ? col_raw : n_live - 1u;
 		half8 xs[3];               // SDF net input, B operands
 		float p[3], dir[3] = {0.f, 0.f, 0.f};
 		uint4 slope[8];            // FULL: the slopes of the lane's 8 levels as stored
@@ -561,12 +563,14 @@ static FusedArgs fused_base(const N2FusedNets& nets, uint32_t n) {
 	a.enc_w = tab.n_levels * 2;
 	a.sdf_bias = nets.sdf_bias;
 	a.N = n;
+	a.live = nullptr;
 	return a;
 }
 
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output) {
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live) {
 	FusedArgs a = fused_base(nets, n);
+	a.live = d_live;
 	a.coords = d_coords;
 	a.sdf_in = reinterpret_cast<hf*>(sdf_in);
 	a.xyz_rows = xyz_rows;

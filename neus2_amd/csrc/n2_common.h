@@ -85,8 +85,12 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 // NerfNetwork::forward_impl as a level-major gather kernel plus one kernel for everything behind it: writes the network
 // inputs and d sdf / d input (SoA, n columns), the slopes of the encoding (16 bytes per level and sample, [n_levels][n]:
 // d feature / d position without the level's scale factor, n2_slopes_pack) and the [n][16] output.
+// d_live (or null): a device counter; only samples below min(*d_live, n) are evaluated, n stays the matrices' column count.
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output);
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live = nullptr);
+// n2_field_forward over the samples below min(*d_live, n): the trainer's marched samples fill only part of the window it
+// evaluates (the window is the count measured some steps earlier, rounded up); what lies behind them is not computed.
+int n2_field_forward_live(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output);
 // NerfNetwork::sdf / density: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
 // sdf_in null: one kernel that gathers sample by sample (points in lattice order, whose table lines stay cached);
 // else a level-major gather into the feature rows 3.. of sdf_in (SoA, n columns) followed by the network kernel.

@@ -345,8 +345,8 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	t->last_set = cur;
 	const n2_trainer::SampleSet& set = t->sets[cur];
 	const uint32_t* ray_counter = set.counters;
-	// field over every marched sample
-	if (int rc = n2_field_forward(t->field, stream, set.coords, n_inference, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	// field over every marched sample: the window of n_inference samples, of which the generator filled set.counters[1]
+	if (int rc = n2_field_forward_live(t->field, stream, set.coords, n_inference, set.counters + 1, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
 	// compositing, loss, gradients w.r.t. the outputs, compaction
 	n2_composite_config cc = t->cfg.composite;
 	cc.n_rays_norm = n_rays;
