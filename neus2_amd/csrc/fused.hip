@@ -276,6 +276,9 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 	// Staging the coarse levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch
 	// and the five dense levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the
 	// positions and writing 320 bytes of features and slopes per sample.
+	// The trainer's sample generator runs beside this kernel on a second stream: where a wave of each is ready on a SIMD, this
+	// one issues first (the generator has the rest of the step to finish; measured 4 us on the forward, 2 us on the step).
+	__builtin_amdgcn_s_setprio(3);
 	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
 	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
 	const uint32_t N = a.N;
