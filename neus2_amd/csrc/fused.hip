@@ -266,7 +266,7 @@ constexpr uint32_t FG_BLOCK = 256;
 template <bool FULL>
 __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
 	// level-major workgroup ids: the workgroups that run at one time work on one or two levels, whose tables stay in every
-	// L2.  The launch is bound by the L2s' request rate: 13.1 M requests for the training step's 2.7e5 ray-ordered samples
+	// L2.  The launch is bound by the L2s' request rate: 10 M requests for the training step's 2.6e5 ray-ordered samples
 	// (four lines per sample on every level whose cells are smaller than the marching step), 63 % of them hits.  Measured on
 	// that workload and dropped: whole levels dealt to XCDs by a cost plan (the launch then fetches a third of the 278 MiB,
 	// but takes 9 to 20 us longer with every cost model tried), one 8- or 16-byte load per pair of x neighbours instead of
