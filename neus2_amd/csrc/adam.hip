@@ -3,6 +3,7 @@
 // accesses; parameters whose gradient is zero (most of the hash table in any
 // one step) cost only the 2-byte gradient read.
 #include "n2_common.h"
+#include "slab_reduce.h"
 
 #include <cmath>
 #include <mutex>
@@ -45,14 +46,48 @@ __device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float lo
 	return true;
 }
 
+// parameters whose gradients a slab summation produces (r.units > 0): the workgroups that run its units step them
+__device__ __forceinline__ bool adam_summed(const N2SlabReduce& r, const hf* grads, uint32_t i) {
+	if (r.units == 0) return false;
+	const hf* g = grads + i;
+	return (g >= r.ga && g < r.ga + r.params_a) || (g >= r.gb && g < r.gb + r.params_b) || (r.extra_n > 0 && g == r.extra_out);
+}
+
 __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
                                                         uint32_t slot, const uint32_t* __restrict__ gate, float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
-                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps) {
-	const uint32_t q = blockIdx.x * 256 + threadIdx.x;
-	const uint32_t i0 = q * 4;
-	if (i0 >= n) return;
+                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps, N2SlabReduce sums) {
 	if (gate != nullptr && *gate == 0u) return;  // a step without samples leaves the parameters and the optimiser state alone
 	const float* table = g_adam_bias[slot];
+	if (blockIdx.x < sums.units) {
+		// The first workgroups add up the slabs of 32 parameters each (25 MB of streaming reads that would otherwise be a launch
+		// of their own in front of this one), store the fp16 gradient and step the parameter with it.
+		__shared__ float fold[32][33];
+		n2_slab_reduce_unit(sums, blockIdx.x, fold, [&](const hf* at, hf g16) {
+			const uint32_t i = (uint32_t)(at - grads);
+			float w = master[i], a = m1[i], b = m2[i];
+			uint32_t t = steps[i];
+			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g16, w, a, b, t)) {
+				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+			}
+		});
+		return;
+	}
+	const uint32_t q = (blockIdx.x - sums.units) * 256 + threadIdx.x;
+	const uint32_t i0 = q * 4;
+	if (i0 >= n) return;
+	if (adam_summed(sums, grads, i0) || adam_summed(sums, grads, min(i0 + 3u, n - 1u))) {
+		// a quad that touches summed parameters (the networks' weights are whole quads; the single extra value may share its
+		// quad with others): one parameter at a time, leaving out the summed ones
+		for (uint32_t i = i0; i < min(i0 + 4u, n); ++i) {
+			if (adam_summed(sums, grads, i)) continue;
+			float w = master[i], a = m1[i], b = m2[i];
+			uint32_t t = steps[i];
+			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)grads[i], w, a, b, t)) {
+				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+			}
+		}
+		return;
+	}
 	if (i0 + 4 <= n) {
 		const half4 g = *reinterpret_cast<const half4*>(grads + i0);
 		const bool all_zero = g[0] == (hf)0 && g[1] == (hf)0 && g[2] == (hf)0 && g[3] == (hf)0;
@@ -91,7 +126,7 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate) {
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums) {
 	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
 	if (n_params == 0) return N2_OK;
 	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
@@ -141,8 +176,17 @@ int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_
 	int exp2 = 0;
 	const float inv_loss_scale = (std::frexp(loss_scale, &exp2) == 0.5f && exp2 > -120 && exp2 < 120) ? 1.f / loss_scale : 0.f;
 	N2ProfScope prof(N2_PROF_ADAM, s);
-	adam_step_kernel<<<dim3((quads + 255) / 256), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate,
-		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps);
+	N2SlabReduce plan = {};
+	if (sums != nullptr && sums->units > 0) {
+		plan = *sums;
+		// the summed gradients must be this call's: inside d_gradients (the kernel turns their addresses into parameter numbers)
+		const hf* g0 = reinterpret_cast<const hf*>(d_gradients);
+		auto inside = [&](const hf* p, uint32_t count) { return count == 0 || (p >= g0 && p + count <= g0 + n_params); };
+		N2_REQUIRE(inside(plan.ga, plan.params_a) && inside(plan.gb, plan.params_b) && inside(plan.extra_out, plan.extra_n > 0 ? 1u : 0u),
+		           "n2_adam_step: the summed gradients do not lie inside d_gradients");
+	}
+	adam_step_kernel<<<dim3((quads + 255) / 256 + plan.units), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate,
+		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

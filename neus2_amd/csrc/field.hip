@@ -9,6 +9,7 @@
 // writes rows 3..34 of the MLP's second-order input), which leaves three glue
 // kernels in the forward and three in the backward.
 #include "n2_common.h"
+#include "slab_reduce.h"
 #include "grid_device.h"
 
 #include <new>
@@ -466,6 +467,14 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 
 N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n,
                              const n2_half* d_dL_doutput, uint32_t ek_batch_size, n2_grad_mode mode) {
+	N2SlabReduce sums = {};
+	if (int rc = n2_field_backward_deferred(f, stream, d_coords, n, d_dL_doutput, ek_batch_size, mode, &sums)) return rc;
+	return n2_slab_reduce_launch(stream, sums);
+}
+
+int n2_field_backward_deferred(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t ek_batch_size,
+                               n2_grad_mode mode, N2SlabReduce* sums) {
+	*sums = N2SlabReduce{};
 	if (int rc = check_field(f, "n2_field_backward", n)) return rc;
 	N2_REQUIRE(n <= f->max_batch_bwd, "n2_field_backward: batch %u exceeds the workspace's backward capacity %u", n, f->max_batch_bwd);
 	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_field_backward: mode must be OVERWRITE or ACCUMULATE");
@@ -521,9 +530,10 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	if (int rc = n2_grid_backward_fused_indexed(f->grid, stream, f->xyz, n_src, index, n, reinterpret_cast<const n2_half*>(f->d_sdf_in + (size_t)3 * n), f->v,
 	                                            reinterpret_cast<const n2_half*>(f->dsdf_din + (size_t)3 * n_src), mode)) return rc;
 	// the three weight-gradient passes (colour net, SDF net first and second order) left their per-workgroup partial sums
-	// pending: one launch sums them, and with them the partial sums of the variance gradient
-	return n2_mlp_reduce_deferred_sum(f->rgb, f->sdf, stream, f->var_part, var_parts, reinterpret_cast<n2_half*>(f->grads + f->off_var),
-	                                  mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+	// pending: one plan sums them, and with them the partial sums of the variance gradient (the caller runs it: as a launch,
+	// or inside the optimiser's kernel)
+	return n2_mlp_reduce_deferred_plan(f->rgb, f->sdf, f->var_part, var_parts, reinterpret_cast<n2_half*>(f->grads + f->off_var),
+	                                   mode == N2_GRAD_ACCUMULATE ? 1 : 0, sums);
 }
 
 N2_API int n2_field_select(n2_field_t* f, n2_stream_t stream, const uint32_t* d_source_index, uint32_t n_source, uint32_t n) {

@@ -29,6 +29,7 @@
 
 #include "mlp_device.h"
 #include "mlp_wgrad.h"
+#include "slab_reduce.h"
 
 struct n2_mlp {
 	uint32_t in_w, n_hidden, n_params;
@@ -351,74 +352,10 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_bbi_kernel(const hf* __restr
 	if (partials) acc.write_slab(reinterpret_cast<float*>(smem), partials + (size_t)blockIdx.x * N_PARAMS, N_PARAMS, wave, role, n, g);
 }
 
-// grads (fp16) = [grads +] sum over slabs.  A workgroup owns 32 consecutive parameters (one 128-byte line of every
-// slab): 8 lanes cover the line with 16-byte loads, 32 lane groups share the slabs, eight loads in flight per lane,
-// LDS folds the groups.  n_params is a multiple of 16, so lines are never ragged.
-__device__ __forceinline__ void mlp_reduce_line(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params, hf* __restrict__ grads,
-                                                int accumulate, uint32_t line, float (*fold)[33]) {
-	const uint32_t q = threadIdx.x & 7, grp = threadIdx.x >> 3;
-	const uint32_t i = line * 32 + q * 4;
-	float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-	if (i < n_params) {
-		const float* p = partials + i;
-		uint32_t k = grp;
-		for (; k + 7 * 32 < n_slabs; k += 8 * 32) {
-			float4 v[8];
-#pragma unroll
-			for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(p + (size_t)(k + u * 32) * n_params);
-#pragma unroll
-			for (int u = 0; u < 8; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
-		}
-		for (; k < n_slabs; k += 32) {
-			const float4 v = *reinterpret_cast<const float4*>(p + (size_t)k * n_params);
-			acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-		}
-	}
-	fold[grp][q * 4 + 0] = acc.x;
-	fold[grp][q * 4 + 1] = acc.y;
-	fold[grp][q * 4 + 2] = acc.z;
-	fold[grp][q * 4 + 3] = acc.w;
-	__syncthreads();
-	// 8 lanes per parameter fold 4 groups each, then a shuffle tree
-	const uint32_t pl = threadIdx.x >> 3, part = threadIdx.x & 7;
-	float t = fold[part * 4][pl] + fold[part * 4 + 1][pl] + fold[part * 4 + 2][pl] + fold[part * 4 + 3][pl];
-	t += __shfl_xor(t, 1);
-	t += __shfl_xor(t, 2);
-	t += __shfl_xor(t, 4);
-	const uint32_t o = line * 32 + pl;
-	if (part == 0 && o < n_params) {
-		if (accumulate) t += (float)grads[o];
-		grads[o] = (hf)t;
-	}
-}
-
-__global__ void __launch_bounds__(256) mlp_reduce_partials_kernel(const float* __restrict__ partials, uint32_t n_slabs, uint32_t n_params,
-                                                                  hf* __restrict__ grads, int accumulate) {
+// grads (fp16) = [grads +] sum over slabs: n2_slab_reduce_unit (slab_reduce.h), one unit per workgroup.
+__global__ void __launch_bounds__(256) mlp_reduce_units_kernel(N2SlabReduce r) {
 	__shared__ float fold[32][33];
-	mlp_reduce_line(partials, n_slabs, n_params, grads, accumulate, blockIdx.x, fold);
-}
-
-// two parameter sets in one launch; one more workgroup (when extra_n > 0) adds up extra_n floats in a fixed order into a
-// single fp16 value: the field's variance gradient rides along instead of taking a launch of its own
-__global__ void __launch_bounds__(256) mlp_reduce_two_kernel(const float* __restrict__ pa, uint32_t slabs_a, uint32_t params_a, hf* __restrict__ ga, int acc_a,
-                                                             uint32_t blocks_a, const float* __restrict__ pb, uint32_t slabs_b, uint32_t params_b,
-                                                             hf* __restrict__ gb, int acc_b, uint32_t blocks_b, const float* __restrict__ extra,
-                                                             uint32_t extra_n, hf* __restrict__ extra_out, int extra_acc) {
-	__shared__ float fold[32][33];
-	if (blockIdx.x < blocks_a) mlp_reduce_line(pa, slabs_a, params_a, ga, acc_a, blockIdx.x, fold);
-	else if (blockIdx.x < blocks_a + blocks_b) mlp_reduce_line(pb, slabs_b, params_b, gb, acc_b, blockIdx.x - blocks_a, fold);
-	else {
-		float s = 0.f;
-		for (uint32_t i = threadIdx.x; i < extra_n; i += 256) s += extra[i];
-#pragma unroll
-		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-		if ((threadIdx.x & 63) == 0) fold[0][threadIdx.x >> 6] = s;
-		__syncthreads();
-		if (threadIdx.x == 0) {
-			const float t = (fold[0][0] + fold[0][1]) + (fold[0][2] + fold[0][3]);
-			extra_out[0] = extra_acc ? (hf)((float)extra_out[0] + t) : (hf)t;
-		}
-	}
+	n2_slab_reduce_unit(r, blockIdx.x, fold, [](const hf*, hf) {});
 }
 
 // ----------------------------------------------------------------------------
@@ -551,11 +488,24 @@ N2_API int n2_mlp_forward(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d_in
 // where the next gradient-producing kernel writes its slabs
 static float* next_slabs(n2_mlp_t* mlp) { return mlp->workspace + (size_t)mlp->pending_slabs * mlp->n_params; }
 
-static int reduce_now(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
-	mlp_reduce_partials_kernel<<<dim3((mlp->n_params + 31) / 32), dim3(256), 0, s>>>(mlp->workspace, n_slabs, mlp->n_params,
-		mlp->grads, mode == N2_GRAD_ACCUMULATE ? 1 : 0);
+static void slab_set(N2SlabReduce& r, bool second, const n2_mlp_t* mlp, uint32_t n_slabs, n2_grad_mode mode) {
+	const uint32_t units = (mlp->n_params + 31) / 32;
+	if (!second) { r.pa = mlp->workspace; r.slabs_a = n_slabs; r.params_a = mlp->n_params; r.ga = mlp->grads; r.acc_a = mode == N2_GRAD_ACCUMULATE ? 1 : 0; r.units_a = units; }
+	else { r.pb = mlp->workspace; r.slabs_b = n_slabs; r.params_b = mlp->n_params; r.gb = mlp->grads; r.acc_b = mode == N2_GRAD_ACCUMULATE ? 1 : 0; r.units_b = units; }
+	r.units = r.units_a + r.units_b + (r.extra_n > 0 ? 1u : 0u);
+}
+
+int n2_slab_reduce_launch(n2_stream_t stream, const N2SlabReduce& r) {
+	if (r.units == 0) return N2_OK;
+	mlp_reduce_units_kernel<<<dim3(r.units), dim3(256), 0, n2_stream(stream)>>>(r);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
+}
+
+static int reduce_now(n2_mlp_t* mlp, hipStream_t s, uint32_t n_slabs, n2_grad_mode mode) {
+	N2SlabReduce r = {};
+	slab_set(r, false, mlp, n_slabs, mode);
+	return n2_slab_reduce_launch(reinterpret_cast<n2_stream_t>(s), r);
 }
 
 // a kernel has just written n_slabs slabs at next_slabs(mlp)
@@ -583,32 +533,27 @@ N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 
 N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) { return n2_mlp_reduce_deferred_sum(a, b, stream, nullptr, 0, nullptr, 0); }
 
+int n2_mlp_reduce_deferred_plan(n2_mlp_t* a, n2_mlp_t* b, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate, N2SlabReduce* out) {
+	N2_REQUIRE(out != nullptr, "n2_mlp_reduce_deferred: plan is null");
+	N2SlabReduce r = {};
+	if (n_parts > 0) { r.extra = d_parts; r.extra_n = n_parts; r.extra_out = reinterpret_cast<hf*>(d_sum); r.extra_acc = accumulate; r.units = 1; }
+	bool second = false;
+	n2_mlp_t* nets[2] = {a, b};
+	for (n2_mlp_t* m : nets) {
+		if (m == nullptr || m->pending_slabs == 0) continue;
+		slab_set(r, second, m, m->pending_slabs, m->pending_mode);
+		m->pending_slabs = 0;
+		second = true;
+	}
+	*out = r;
+	return N2_OK;
+}
+
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate) {
 	N2_REQUIRE(a != nullptr, "n2_mlp_reduce_deferred: mlp is null");
-	hipStream_t s = n2_stream(stream);
-	if (b != nullptr && b->pending_slabs == 0) b = nullptr;
-	if (a->pending_slabs == 0) { a = b; b = nullptr; }
-	if (a == nullptr || a->pending_slabs == 0 || (b == nullptr && n_parts > 0)) {
-		// nothing or one network pending: the sum, if any, goes alone
-		if (n_parts > 0) {
-			mlp_reduce_two_kernel<<<dim3(1), dim3(256), 0, s>>>(nullptr, 0, 0, nullptr, 0, 0, nullptr, 0, 0, nullptr, 0, 0, d_parts, n_parts, reinterpret_cast<hf*>(d_sum), accumulate);
-			N2_LAUNCH_CHECK();
-		}
-		if (a == nullptr || a->pending_slabs == 0) return N2_OK;
-	}
-	if (b == nullptr) {
-		const int rc = reduce_now(a, s, a->pending_slabs, a->pending_mode);
-		a->pending_slabs = 0;
-		return rc;
-	}
-	const uint32_t blocks_a = (a->n_params + 31) / 32, blocks_b = (b->n_params + 31) / 32;
-	mlp_reduce_two_kernel<<<dim3(blocks_a + blocks_b + (n_parts > 0 ? 1u : 0u)), dim3(256), 0, s>>>(a->workspace, a->pending_slabs, a->n_params, a->grads,
-		a->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0, blocks_a, b->workspace, b->pending_slabs, b->n_params, b->grads,
-		b->pending_mode == N2_GRAD_ACCUMULATE ? 1 : 0, blocks_b, d_parts, n_parts, reinterpret_cast<hf*>(d_sum), accumulate);
-	N2_LAUNCH_CHECK();
-	a->pending_slabs = 0;
-	b->pending_slabs = 0;
-	return N2_OK;
+	N2SlabReduce r;
+	if (int rc = n2_mlp_reduce_deferred_plan(a, b, d_parts, n_parts, d_sum, accumulate, &r)) return rc;
+	return n2_slab_reduce_launch(stream, r);
 }
 
 static int check_grad_mode(const n2_mlp_t* mlp, const char* fn, n2_grad_mode mode) {

@@ -34,6 +34,8 @@ void n2_set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 constexpr uint32_t N2_MAX_LEVELS = 32;
 
+struct N2SlabReduce;  // slab_reduce.h
+
 // How a level turns integer grid coordinates into an entry index.
 enum : uint32_t {
 	N2_LEVEL_DENSE = 0,  // x + y*res + z*res^2, one conditional subtract stands in for the modulo
@@ -129,11 +131,21 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
                                              const n2_half* d_dL_ddLdinput, const n2_half* d_second_dL_doutput, n2_grad_mode mode,
                                              bool dx_encoding_only);
 // n2_adam_step that does nothing when *d_gate is zero on the device (d_gate null: always steps)
+// sums (or null): a slab summation whose gradients lie inside d_gradients; the kernel's first workgroups run it, store the
+// fp16 gradients and step those parameters themselves (the other workgroups leave them alone)
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate);
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums = nullptr);
 // n2_mlp_reduce_deferred that also adds up n_parts floats, in a fixed order, into one fp16 value ([+=] when accumulate)
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
+// The same work as a plan instead of a launch: what is pending is handed to *out (and no longer pending), for
+// n2_slab_reduce_launch or for a kernel that carries the summation (n2_adam_step_gated).
+int n2_mlp_reduce_deferred_plan(n2_mlp_t* a, n2_mlp_t* b, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate, N2SlabReduce* out);
+int n2_slab_reduce_launch(n2_stream_t stream, const N2SlabReduce& plan);
+// n2_field_backward that leaves the summation of the networks' weight-gradient slabs and of the variance gradient's partial
+// sums to the caller: *sums is the plan (their fp16 gradients are not written until it has run)
+int n2_field_backward_deferred(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t n_rays_ek,
+                               n2_grad_mode mode, N2SlabReduce* sums);
 // n2_field_select without the copy of the index: d_source_index must stay valid and unchanged until the backward has run
 int n2_field_select_borrow(n2_field_t* field, const uint32_t* d_source_index, uint32_t n_source, uint32_t n);
 // n2_grid_backward_fused whose positions (SoA 3 x n_cols) and d_dL_dy_second rows (n_cols columns) are read through d_index.

@@ -1,0 +1,81 @@
+// Summation of the per-workgroup partial sums (slabs) that the weight-gradient kernels of the MLPs leave behind, as a device
+// function for any kernel with 256-thread workgroups: mlp.hip launches it as a kernel of its own, and the trainer's Adam
+// step runs it in its first workgroups (25 MB of streaming reads inside a kernel that streams 350 MB anyway), so that a
+// training step has no reduction launch.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+struct N2SlabReduce {
+	// two parameter sets: grads (fp16) = [grads +] sum over the slabs, a unit per 32 consecutive parameters
+	const float* pa; uint32_t slabs_a, params_a; _Float16* ga; int acc_a; uint32_t units_a;
+	const float* pb; uint32_t slabs_b, params_b; _Float16* gb; int acc_b; uint32_t units_b;
+	// one more unit (when extra_n > 0) adds up extra_n floats in a fixed order into a single fp16 value
+	const float* extra; uint32_t extra_n; _Float16* extra_out; int extra_acc;
+	uint32_t units;  // units_a + units_b + (extra_n > 0)
+};
+
+// Unit `unit` of the plan, run by the 256 threads of a workgroup.  A unit owns 32 consecutive parameters (one 128-byte line
+// of every slab): 8 lanes cover the line with 16-byte loads, 32 lane groups share the slabs, eight loads in flight per
+// lane, LDS folds the groups.  n_params is a multiple of 16, so lines are never ragged.  The fp16 gradient is stored, and
+// done(address of the stored gradient, its value) is called by the thread that stored it.  Contains one __syncthreads().
+template <class Done>
+__device__ __forceinline__ void n2_slab_reduce_unit(const N2SlabReduce& r, uint32_t unit, float (*fold)[33], Done done) {
+	const uint32_t tid = threadIdx.x;
+	if (unit >= r.units_a + r.units_b) {  // the extra sum
+		float s = 0.f;
+		for (uint32_t i = tid; i < r.extra_n; i += 256) s += r.extra[i];
+#pragma unroll
+		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+		if ((tid & 63u) == 0) fold[0][tid >> 6] = s;
+		__syncthreads();
+		if (tid == 0) {
+			const float t = (fold[0][0] + fold[0][1]) + (fold[0][2] + fold[0][3]);
+			const _Float16 h = r.extra_acc ? (_Float16)((float)r.extra_out[0] + t) : (_Float16)t;
+			r.extra_out[0] = h;
+			done(r.extra_out, h);
+		}
+		return;
+	}
+	const bool first = unit < r.units_a;
+	const float* partials = first ? r.pa : r.pb;
+	const uint32_t n_slabs = first ? r.slabs_a : r.slabs_b, n_params = first ? r.params_a : r.params_b, line = first ? unit : unit - r.units_a;
+	_Float16* grads = first ? r.ga : r.gb;
+	const int accumulate = first ? r.acc_a : r.acc_b;
+	const uint32_t q = tid & 7u, grp = tid >> 3;
+	const uint32_t i = line * 32 + q * 4;
+	float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+	if (i < n_params) {
+		const float* p = partials + i;
+		uint32_t k = grp;
+		for (; k + 7 * 32 < n_slabs; k += 8 * 32) {
+			float4 v[8];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(p + (size_t)(k + u * 32) * n_params);
+#pragma unroll
+			for (int u = 0; u < 8; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
+		}
+		for (; k < n_slabs; k += 32) {
+			const float4 v = *reinterpret_cast<const float4*>(p + (size_t)k * n_params);
+			acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+		}
+	}
+	fold[grp][q * 4 + 0] = acc.x;
+	fold[grp][q * 4 + 1] = acc.y;
+	fold[grp][q * 4 + 2] = acc.z;
+	fold[grp][q * 4 + 3] = acc.w;
+	__syncthreads();
+	// 8 lanes per parameter fold 4 groups each, then a shuffle tree
+	const uint32_t pl = tid >> 3, part = tid & 7u;
+	float t = fold[part * 4][pl] + fold[part * 4 + 1][pl] + fold[part * 4 + 2][pl] + fold[part * 4 + 3][pl];
+	t += __shfl_xor(t, 1);
+	t += __shfl_xor(t, 2);
+	t += __shfl_xor(t, 4);
+	const uint32_t o = line * 32 + pl;
+	if (part == 0 && o < n_params) {
+		if (accumulate) t += (float)grads[o];
+		const _Float16 h = (_Float16)t;
+		grads[o] = h;
+		done(grads + o, h);
+	}
+}

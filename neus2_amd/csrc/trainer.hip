@@ -6,6 +6,7 @@
 // the scene and the seed) may run ahead on a stream the trainer owns, into the
 // other of two sample sets, while this step's field kernels occupy the GPU.
 #include "n2_common.h"
+#include "slab_reduce.h"
 
 
 #include <cstring>
@@ -368,10 +369,12 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	} else {
 		if (int rc = n2_field_select_borrow(t->field, t->src_index, n_inference, T)) return rc;
 	}
-	if (int rc = n2_field_backward(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE)) return rc;
+	// the summation of the networks' weight-gradient slabs rides in the optimiser's kernel instead of taking a launch
+	N2SlabReduce sums;
+	if (int rc = n2_field_backward_deferred(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE, &sums)) return rc;
 	// a step whose rays kept no sample (counter 2 is zero) must not apply the previous step's gradients again
 	if (int rc = n2_adam_step_gated(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter)) return rc;
+	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums)) return rc;
 	t->optimizer_steps += 1;
 	t->training_step += 1;
 	if (t->ema) {
