@@ -436,6 +436,22 @@ def run_lattice_workload(args):
               "mfma": {"kernel": "SDF net 48-64-16 forward" + (" (inside the fused launch)" if dom == "field_forward" else ""), "flops_per_sample": 8192,
                        "achieved_tflops": mlp_tflops, "peak_tflops": MFMA_PEAK_TFLOPS, "frac": mlp_tflops / MFMA_PEAK_TFLOPS},
               "kernels": kernels}
+    # the consumer's form of the same job (Testbed::get_density_on_grid): lattice points formed inside the kernel, only the SDF
+    # row kept, as fp32; the whole 512^3 lattice
+    from neus2_amd.mesh import density_on_grid
+    from neus2_amd.training import Trainer, default_config
+    tr = Trainer(default_config(target_batch_size=TARGET, max_rays_per_batch=1 << 12, max_samples=CH))
+    tr.initialize_params(seed=1, sdf_mlp_weights=np.load(os.path.join(ROOT, "tests", "golden", "sdf_mlp_weights_48.npy")))
+    d = density_on_grid(tr._field, (RES, RES, RES), chunk=CH)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        d = density_on_grid(tr._field, (RES, RES, RES), chunk=CH)
+    torch.cuda.synchronize()
+    dog = (time.perf_counter() - t0) / 3
+    result["density_on_grid"] = {"ms_per_lattice": dog * 1e3, "ms_per_chunk": dog * 1e3 / n_chunks, "points_per_s": RES ** 3 / dog,
+                                 "note": "n2_density_on_grid over all 32 chunks: no position array, fp32 SDF row only"}
+    del d, tr
     if not args.no_cpu_baseline:
         from oracle import oracle as orc
         from oracle.field import Field

@@ -703,6 +703,44 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	return N2_OK;
 }
 
+__global__ void __launch_bounds__(FB) field_widen_row_kernel(uint32_t n, const hf* __restrict__ in, float* __restrict__ out) {
+	const uint32_t i = blockIdx.x * FB + threadIdx.x;
+	if (i < n) out[i] = (float)in[i];
+}
+
+// Row 0 of n2_field_sdf as fp32 (the fp16 value widened; what get_density_on_grid keeps, src/testbed_nerf.cu:4082-4133):
+// the fused kernel writes it directly and the other 15 rows not at all; d_scratch16 ([16][n] fp16) serves the unfused path.
+int n2_field_sdf_row0(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, uint32_t n_keep, float* d_row0,
+                      n2_half* d_scratch16) {
+	if (int rc = check_field(f, "n2_field_sdf", n)) return rc;
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_xyz != nullptr && d_row0 != nullptr, "n2_field_sdf: null buffer");
+	N2_REQUIRE(ps >= 1 && ds >= 1, "n2_field_sdf: strides must be >= 1");
+	hipStream_t s = n2_stream(stream);
+	if (f->fused && fused_ok(f)) {
+		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, nullptr, d_row0, false,
+		                          n2_grid_lattice_order(f->grid) ? nullptr : reinterpret_cast<n2_half*>(f->sdf_in), n_keep);
+	}
+	if (int rc = field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, ps, ds, n, d_scratch16, false)) return rc;
+	const uint32_t keep = n_keep < n ? n_keep : n;
+	field_widen_row_kernel<<<fgrid(keep), dim3(FB), 0, s>>>(keep, reinterpret_cast<const hf*>(d_scratch16), d_row0);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
+}
+
+bool n2_field_sdf_row0_lattice(n2_field_t* f, n2_stream_t stream, const N2Lattice& lattice, uint32_t n, uint32_t n_keep, float* d_row0, int* rc) {
+	*rc = check_field(f, "n2_field_sdf", n);
+	if (*rc != N2_OK) return true;
+	if (!(f->fused && fused_ok(f) && n2_grid_lattice_order(f->grid))) return false;
+	if (n == 0) return true;
+	if (d_row0 == nullptr) { n2_set_error("n2_field_sdf: null buffer"); *rc = N2_ERR_INVALID_ARGUMENT; return true; }
+	hipStream_t s = n2_stream(stream);
+	N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+	*rc = n2_fused_field_sdf(fused_nets(f), s, nullptr, 0, 0, n, nullptr, d_row0, false, nullptr, n_keep, &lattice);
+	return true;
+}
+
 N2_API int n2_field_sdf(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n,
                         n2_half* d_output) {
 	return field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, point_stride, dim_stride, n, d_output, false);

@@ -62,8 +62,9 @@ struct FusedArgs {
 	float sdf_bias;
 	uint32_t N;
 	const uint32_t* live;   // or null: only samples below min(*live, N) are evaluated (N stays the column count of the matrices)
-	const float* pos;       // coordinate d of sample i at pos[i * ps + d * ds]
+	const float* pos;       // coordinate d of sample i at pos[i * ps + d * ds]; null: sample i is point lat.first + i of a lattice
 	uint32_t ps, ds;
+	N2Lattice lat;
 	const float* coords;    // full field: [N][7] NerfCoordinate (direction at 4..6)
 	// full field: what the backward pass reads, and the output
 	hf* sdf_in;             // [sdf_in_w][N]  rows 0..2 centred coordinates, 3.. features
@@ -74,7 +75,8 @@ struct FusedArgs {
 	hf* output;             // [N][16]
 	// SDF only
 	hf* sdf_out;            // [16][N] or null
-	float* row0;            // [N] fp32 copy of row 0, or null
+	float* row0;            // [row0_n] fp32 copy of row 0 of the first row0_n samples, or null
+	uint32_t row0_n;
 	int density;            // row 0 becomes the logistic density
 };
 
@@ -346,9 +348,19 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 		float p[3], dir[3] = {0.f, 0.f, 0.f};
 		uint4 slope[8];            // FULL: the slopes of the lane's 8 levels as stored
 		if (GATHER) {
-			const float* q = a.pos + (size_t)col * a.ps;
+			if (a.pos) {
+				const float* q = a.pos + (size_t)col * a.ps;
 #pragma unroll
-			for (int d = 0; d < 3; ++d) p[d] = q[(size_t)d * a.ds];
+				for (int d = 0; d < 3; ++d) p[d] = q[(size_t)d * a.ds];
+			} else {
+				// lattice point (x, y, z), x fastest: (c / res) * extent + corner, each step rounded on its own (the positions are
+				// part of a bit-exact contract); points behind the lattice's end sit at the centre
+				const uint32_t idx = a.lat.first + col;
+				const uint32_t c[3] = {idx % a.lat.res[0], (idx / a.lat.res[0]) % a.lat.res[1], idx / (a.lat.res[0] * a.lat.res[1])};
+#pragma unroll
+				for (int d = 0; d < 3; ++d)
+					p[d] = idx < a.lat.total ? __fadd_rn(__fmul_rn(__fmul_rn((float)c[d], a.lat.inv_res[d]), a.lat.extent[d]), a.lat.corner[d]) : 0.5f;
+			}
 			// the lane's 8 levels, the next level's loads in flight while one is finished
 			Item cur, nxt;
 			float unused[2][3];
@@ -414,7 +426,7 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 					s = is * sig * ((hf)1.0f - sig);
 				}
 				y[0] = s;
-				if (a.row0 && valid) a.row0[col] = (float)s;
+				if (a.row0 && col_raw < a.row0_n) a.row0[col] = (float)s;
 			}
 			if (a.sdf_out && valid) {
 #pragma unroll
@@ -589,11 +601,16 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 }
 
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
-                       float* d_row0, bool density, n2_half* sdf_in) {
+                       float* d_row0, bool density, n2_half* sdf_in, uint32_t row0_n, const N2Lattice* lattice) {
 	FusedArgs a = fused_base(nets, n);
 	a.pos = d_xyz; a.ps = ps; a.ds = ds;
+	if (lattice) {
+		if (d_xyz != nullptr || sdf_in != nullptr) { n2_set_error("n2_fused_field_sdf: lattice points are generated in the one-launch form only"); return N2_ERR_INVALID_ARGUMENT; }
+		a.lat = *lattice;
+	}
 	a.sdf_out = reinterpret_cast<hf*>(d_out_soa);
 	a.row0 = d_row0;
+	a.row0_n = row0_n < n ? row0_n : n;
 	a.density = density ? 1 : 0;
 	if (sdf_in == nullptr) {
 		field_fused_forward_kernel<false, true><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_SDF_COUNT), s>>>(a);

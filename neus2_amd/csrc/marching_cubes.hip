@@ -564,11 +564,6 @@ __global__ void __launch_bounds__(MC_BLOCK) mc_lattice_positions_kernel(McGrid g
 #pragma unroll
 	for (int d = 0; d < 3; ++d) p[d] = ((float)c[d] * (1.f / (float)r[d])) * g.scale[d] + g.offset[d];
 }
-__global__ void __launch_bounds__(MC_BLOCK) mc_widen_kernel(uint32_t n, const hf* __restrict__ in, float* __restrict__ out) {
-	const uint32_t i = blockIdx.x * MC_BLOCK + threadIdx.x;
-	if (i < n) out[i] = (float)in[i];
-}
-
 N2_API uint64_t n2_density_on_grid_scratch_bytes(uint32_t chunk) { return m256(12ull * chunk) + m256(32ull * chunk); }
 
 N2_API int n2_density_on_grid(n2_field_t* field, n2_stream_t stream, const uint32_t res[3], const float aabb_min[3], const float aabb_max[3],
@@ -591,9 +586,14 @@ N2_API int n2_density_on_grid(n2_field_t* field, n2_stream_t stream, const uint3
 	int rc = N2_OK;
 	for (uint64_t first = 0; first < n && rc == N2_OK; first += chunk) {
 		const uint32_t m = (uint32_t)((n - first < chunk) ? n - first : chunk), m8 = (m + 7) / 8 * 8;
+		// the fused kernel forms the lattice points itself; other fields get them written out
+		N2Lattice lat;
+		for (int d = 0; d < 3; ++d) { lat.res[d] = res[d]; lat.inv_res[d] = 1.f / (float)res[d]; lat.extent[d] = g.scale[d]; lat.corner[d] = g.offset[d]; }
+		lat.first = (uint32_t)first; lat.total = (uint32_t)n;
+		if (n < (1ull << 32) && n2_field_sdf_row0_lattice(field, stream, lat, m8, m, d_density + first, &rc)) continue;
 		mc_lattice_positions_kernel<<<mgrid(m8), dim3(MC_BLOCK), 0, s>>>(g, first, m, m8, positions);
-		rc = n2_field_sdf(field, stream, positions, 3, 1, m8, reinterpret_cast<n2_half*>(mlp_out));
-		if (rc == N2_OK) mc_widen_kernel<<<mgrid(m), dim3(MC_BLOCK), 0, s>>>(m, mlp_out, d_density + first);
+		// the padded tail of the last chunk (m8 - m points at most 7) is evaluated but not kept
+		rc = n2_field_sdf_row0(field, stream, positions, 3, 1, m8, m, d_density + first, reinterpret_cast<n2_half*>(mlp_out));
 	}
 	n2_grid_set_point_order(n2_field_encoding(field), 0);
 	if (rc != N2_OK) return rc;

@@ -96,8 +96,13 @@ int n2_field_forward_live(n2_field_t* field, n2_stream_t stream, const float* d_
 // NerfNetwork::sdf / density: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
 // sdf_in null: one kernel that gathers sample by sample (points in lattice order, whose table lines stay cached);
 // else a level-major gather into the feature rows 3.. of sdf_in (SoA, n columns) followed by the network kernel.
+// lattice (with d_xyz and sdf_in null): sample i is lattice point first + i, x fastest, at (c / res) * extent + corner.
+struct N2Lattice {
+	uint32_t res[3], first, total;  // total = res[0] res[1] res[2]
+	float inv_res[3], extent[3], corner[3];
+};
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
-                       float* d_row0, bool density, n2_half* sdf_in);
+                       float* d_row0, bool density, n2_half* sdf_in, uint32_t row0_n = 0xFFFFFFFFu, const N2Lattice* lattice = nullptr);
 
 // What the field hangs on its colour net's backward launch (n2_mlp_backward_rows_indexed): for the same samples,
 //   * row 0 of d_dL_dinput also takes row 3 of d_dL_doutput (the direct gradient of the SDF output);
@@ -152,6 +157,13 @@ int n2_field_select_borrow(n2_field_t* field, const uint32_t* d_source_index, ui
 int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz_rows, uint32_t n_cols, const uint32_t* d_index,
                                    uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,
                                    n2_grad_mode mode);
+
+// row 0 of n2_field_sdf for the first n_keep <= n samples as fp32 (d_scratch16: [16][n] fp16, used when the fused kernels do not serve the field)
+int n2_field_sdf_row0(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n, uint32_t n_keep,
+                      float* d_row0, n2_half* d_scratch16);
+// the same on n points of a lattice, generated inside the kernel; false when the field's fused kernels do not serve it (the
+// caller then writes the positions out and uses n2_field_sdf_row0)
+bool n2_field_sdf_row0_lattice(n2_field_t* field, n2_stream_t stream, const N2Lattice& lattice, uint32_t n, uint32_t n_keep, float* d_row0, int* rc);
 
 static inline hipStream_t n2_stream(n2_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
