@@ -708,10 +708,11 @@ __global__ void __launch_bounds__(FB) field_widen_row_kernel(uint32_t n, const h
 	if (i < n) out[i] = (float)in[i];
 }
 
-// Row 0 of n2_field_sdf as fp32 (the fp16 value widened; what get_density_on_grid keeps, src/testbed_nerf.cu:4082-4133):
+// Row 0 of n2_field_sdf (or n2_field_density) as fp32 (the fp16 value widened; what get_density_on_grid keeps,
+// src/testbed_nerf.cu:4082-4133, and what the occupancy update splats):
 // the fused kernel writes it directly and the other 15 rows not at all; d_scratch16 ([16][n] fp16) serves the unfused path.
 int n2_field_sdf_row0(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, uint32_t n_keep, float* d_row0,
-                      n2_half* d_scratch16) {
+                      n2_half* d_scratch16, bool density) {
 	if (int rc = check_field(f, "n2_field_sdf", n)) return rc;
 	if (n == 0) return N2_OK;
 	N2_REQUIRE(d_xyz != nullptr && d_row0 != nullptr, "n2_field_sdf: null buffer");
@@ -719,10 +720,10 @@ int n2_field_sdf_row0(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uin
 	hipStream_t s = n2_stream(stream);
 	if (f->fused && fused_ok(f)) {
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
-		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, nullptr, d_row0, false,
+		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, nullptr, d_row0, density,
 		                          n2_grid_lattice_order(f->grid) ? nullptr : reinterpret_cast<n2_half*>(f->sdf_in), n_keep);
 	}
-	if (int rc = field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, ps, ds, n, d_scratch16, false)) return rc;
+	if (int rc = field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, ps, ds, n, d_scratch16, density)) return rc;
 	const uint32_t keep = n_keep < n ? n_keep : n;
 	field_widen_row_kernel<<<fgrid(keep), dim3(FB), 0, s>>>(keep, reinterpret_cast<const hf*>(d_scratch16), d_row0);
 	N2_LAUNCH_CHECK();

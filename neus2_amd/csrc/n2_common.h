@@ -158,9 +158,9 @@ int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const fl
                                    uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,
                                    n2_grad_mode mode);
 
-// row 0 of n2_field_sdf for the first n_keep <= n samples as fp32 (d_scratch16: [16][n] fp16, used when the fused kernels do not serve the field)
+// row 0 of n2_field_sdf (density: of n2_field_density) for the first n_keep <= n samples as fp32 (d_scratch16: [16][n] fp16, used when the fused kernels do not serve the field)
 int n2_field_sdf_row0(n2_field_t* field, n2_stream_t stream, const float* d_xyz, uint32_t point_stride, uint32_t dim_stride, uint32_t n, uint32_t n_keep,
-                      float* d_row0, n2_half* d_scratch16);
+                      float* d_row0, n2_half* d_scratch16, bool density = false);
 // the same on n points of a lattice, generated inside the kernel; false when the field's fused kernels do not serve it (the
 // caller then writes the positions out and uses n2_field_sdf_row0)
 bool n2_field_sdf_row0_lattice(n2_field_t* field, n2_stream_t stream, const N2Lattice& lattice, uint32_t n, uint32_t n_keep, float* d_row0, int* rc);

@@ -32,7 +32,7 @@ struct n2_occupancy {
 	float* tmp;          // same
 	float* positions;    // [max_samples + 8][3]
 	uint32_t* indices;   // [max_samples + 8]
-	hf* mlp_out;         // [16][chunk]
+	hf* mlp_out;         // [16][chunk] fp16 (the field's full output, unfused path only), then [chunk] fp32: the density row
 	uint8_t* bitfield;   // [8][128^3 / 8]
 	float* partial;      // [OCC_MEAN_BLOCKS]
 	float* mean;         // [1]
@@ -138,11 +138,11 @@ __global__ void __launch_bounds__(OCC_BLOCK) occ_generate_kernel(uint32_t n, uin
 }
 
 // splat_grid_samples_nerf_max_nearest_neighbor (:662-680): positive floats order like their bit patterns
-__global__ void __launch_bounds__(OCC_BLOCK) occ_splat_kernel(uint32_t n, const uint32_t* __restrict__ indices, const hf* __restrict__ density,
+__global__ void __launch_bounds__(OCC_BLOCK) occ_splat_kernel(uint32_t n, const uint32_t* __restrict__ indices, const float* __restrict__ density,
                                                               float* __restrict__ tmp) {
 	const uint32_t i = blockIdx.x * OCC_BLOCK + threadIdx.x;
 	if (i >= n) return;
-	atomicMax(reinterpret_cast<uint32_t*>(tmp) + indices[i], __float_as_uint((float)density[i]));
+	atomicMax(reinterpret_cast<uint32_t*>(tmp) + indices[i], __float_as_uint(density[i]));
 }
 
 // ema_grid_samples_nerf (:698-727), fused with the partial sums of max(v, 0) over the first cascade (:3383).
@@ -233,7 +233,7 @@ static OccCarve occ_carve(uint32_t n_cascades, uint32_t max_samples, uint32_t ch
 	c.tmp = take(4ull * n_cascades * OCC_CELLS);
 	c.positions = take(12ull * ((uint64_t)max_samples + 8));
 	c.indices = take(4ull * ((uint64_t)max_samples + 8));
-	c.mlp_out = take(32ull * chunk);
+	c.mlp_out = take(32ull * chunk + 4ull * chunk);
 	c.bitfield = take((uint64_t)OCC_LEVELS * OCC_LEVEL_BYTES);
 	c.partial = take(4ull * OCC_MEAN_BLOCKS);
 	c.mean = take(4);
@@ -361,8 +361,10 @@ N2_API int n2_occupancy_update(n2_occupancy_t* occ, n2_field_t* field, n2_stream
 	// densities, a chunk at a time (row 0 of the field's 16 x chunk output)
 	for (uint32_t a = 0; a < n; a += occ->chunk) {
 		const uint32_t m = (n - a < occ->chunk) ? n - a : occ->chunk, m8 = (m + 7) / 8 * 8;
-		if (int rc = n2_field_density(field, stream, occ->positions + (size_t)a * 3, 3, 1, m8, reinterpret_cast<n2_half*>(occ->mlp_out))) return rc;
-		occ_splat_kernel<<<ogrid(m), dim3(OCC_BLOCK), 0, s>>>(m, occ->indices + a, occ->mlp_out, occ->tmp);
+		// only the density row is kept, as fp32 (the fp16 output widened); the row sits behind the fp16 scratch the unfused path needs
+		float* row0 = reinterpret_cast<float*>(occ->mlp_out + (size_t)16 * occ->chunk);
+		if (int rc = n2_field_sdf_row0(field, stream, occ->positions + (size_t)a * 3, 3, 1, m8, m8, row0, reinterpret_cast<n2_half*>(occ->mlp_out), true)) return rc;
+		occ_splat_kernel<<<ogrid(m), dim3(OCC_BLOCK), 0, s>>>(m, occ->indices + a, row0, occ->tmp);
 		N2_LAUNCH_CHECK();
 	}
 	occ_ema_kernel<true><<<dim3((n_elements + OCC_BLOCK * 32 - 1) / (OCC_BLOCK * 32)), dim3(OCC_BLOCK), 0, s>>>(n_elements, decay, occ->grid, occ->tmp,
