@@ -32,7 +32,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
 # HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
 # (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
 # scatter pair = bin (41.0 + 101.9 MiB) + reduce (110.9 + 24.0 MiB)
-STEP_TRAFFIC_BYTES = {"grid_backward_params": int(273.0 * 2**20)}
+STEP_TRAFFIC_BYTES = {"grid_backward_params": int(272.8 * 2**20)}
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
         "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9}
 
