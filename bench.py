@@ -107,10 +107,10 @@ def run_step_workload(args):
     for _ in range(args.warmup):
         tr.step(n_rays=n_rays, n_inference=n_inf)
     torch.cuda.synchronize()
-    # timed region: K steps; only the roofline kernel (the parameter scatter) carries events, and only in every fourth
-    # step, because every event pair costs stream time (about 13 us) that is charged to the step
+    # timed region: K steps; only the roofline kernel (the parameter scatter) carries events, and only in five of the
+    # steps, because every event pair costs stream time (about 13 us) that is charged to the step
     dom = "grid_backward_params"
-    period = 4 if args.steps >= 8 else 1
+    period = max(1, args.steps // 5)  # five timed launches per region
     lib.n2_profile_reset()
     lib.n2_profile_select(C.c_uint32(1 << PROF[dom]))
     lib.n2_profile_set_period(C.c_uint32(period))
@@ -181,7 +181,7 @@ def run_step_workload(args):
                      "avg_launch_us": kernels[dom]["avg_us"], "timed_launches": dom_n},
         "mfma": mfma,
         "kernels": kernels,
-        "kernels_note": "grid_backward_params is timed with HIP events inside the timed region (every fourth step's launch); the other entries come from a "
+        "kernels_note": "grid_backward_params is timed with HIP events inside the timed region (five launches spread over the region); the other entries come from a "
                         "second, untimed pass of the same steps with every listed kernel bracketed by events",
     }
     # untimed extras (the driver's fields above come from the one timed region before them)
@@ -573,8 +573,8 @@ def run_mesh_workload(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)   # 85 ms of timed region for the default workload
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["step", "grid", "sdf", "lattice", "occupancy", "mesh"], default="step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra-regions", type=int, default=5, help="step workload: untimed repeat regions of K steps (spread of the figure)")
