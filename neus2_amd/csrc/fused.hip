@@ -471,8 +471,15 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 		sh4(dir[0] * 2.f - 1.f, dir[1] * 2.f - 1.f, dir[2] * 2.f - 1.f, sh);
 		half8 xc[3];
 		xc[0] = y;
+		{
+			// both halves are formed and one is picked value by value: picking between sh[e] and sh[8 + e] inside the
+			// conversion turns into an index that depends on the lane, and the array then lives in scratch memory
+			half8 lo8, hi8;
 #pragma unroll
-		for (int e = 0; e < 8; ++e) xc[1][e] = (hf)(g ? sh[8 + e] : sh[e]);
+			for (int e = 0; e < 8; ++e) { lo8[e] = (hf)sh[e]; hi8[e] = (hf)sh[8 + e]; }
+			const uint4 lo = __builtin_bit_cast(uint4, lo8), hi = __builtin_bit_cast(uint4, hi8);
+			xc[1] = __builtin_bit_cast(half8, make_uint4(g ? hi.x : lo.x, g ? hi.y : lo.y, g ? hi.z : lo.z, g ? hi.w : lo.w));
+		}
 		xc[2] = zero8();
 		if (g == 0) {
 #pragma unroll
