@@ -34,10 +34,10 @@ struct n2_field {
 	// carved from the workspace
 	hf* sdf_in;        // [sdf_in_w][N]
 	float* xyz;        // [3][N]  positions of the last forward, row per coordinate (the grid kernels read each row 16 times)
-	hf* rgb_in;        // [48][N]
+	hf* rgb_in;        // [48][N]; after a fused forward [N][N2_RGB_IN_PITCH] (sample-major: the networks' kernels hold 8 consecutive rows per lane)
 	float* dy_dx;      // [enc_w][N][3] fp32, or (slopes_saved) 16-byte slope blocks [levels][N] without the levels' scale factors
 	hf* dsdf_din;      // [sdf_in_w][N]  d sdf / d (SDF net input)
-	hf* d_rgb_in;      // [48][N]
+	hf* d_rgb_in;      // [48][N]; behind a fused forward [N][16], rows 0..15 only
 	hf* d_sdf_in;      // [sdf_in_w][N]
 	float* v;          // [3][N]  dL / d normal
 	hf* d_density_in;  // [sdf_in_w][N]  second-order input of the SDF net
@@ -443,9 +443,9 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 	f->last_n = n;
 	f->sel_n = 0;
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
-	if (int rc = zero_padding(s, f->rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.rgb_in)) return rc;
 	f->slopes_saved = f->fused && fused_ok(f);
 	if (f->slopes_saved) {
+		f->pad_n.rgb_in = 0;  // the fused kernel writes sample-major, over what the row layout keeps zero
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
 		return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx,
 		                              reinterpret_cast<n2_half*>(f->dsdf_din), reinterpret_cast<n2_half*>(f->rgb_in), d_output, d_live);
@@ -454,6 +454,7 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), f->dy_dx)) return rc;
 	// SDF net forward (into rows 0..15 of the colour net's input) and d sdf / d input in one pass over the input
+	if (int rc = zero_padding(s, f->rgb_in, RGB_IN_ROWS, f->rgb_in_w, n, f->pad_n.rgb_in)) return rc;
 	if (int rc = n2_mlp_forward_and_input_gradient(f->sdf, stream, 0, reinterpret_cast<const n2_half*>(f->sdf_in), n,
 	                                               reinterpret_cast<n2_half*>(f->rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->dsdf_din))) return rc;
 	field_normals_rgb_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, n, f->enc_w, f->dsdf_din, f->dy_dx, f->rgb_in);
@@ -523,7 +524,8 @@ int n2_field_backward_deferred(n2_field_t* f, n2_stream_t stream, const float* d
 	// SDF net: its output gradient is rows 0..15 of the colour net's input gradient; the second-order pass through the
 	// net (the reference's backward_backward_input with Accumulate) rides along
 	if (int rc = n2_mlp_backward_and_second_order_indexed(f->sdf, stream, reinterpret_cast<const n2_half*>(f->sdf_in), n_src, index, n,
-	                                                      reinterpret_cast<const n2_half*>(f->d_rgb_in), N2_LAYOUT_SOA, reinterpret_cast<n2_half*>(f->d_sdf_in),
+	                                                      reinterpret_cast<const n2_half*>(f->d_rgb_in), f->slopes_saved ? N2_LAYOUT_AOS : N2_LAYOUT_SOA,
+	                                                      reinterpret_cast<n2_half*>(f->d_sdf_in),
 	                                                      reinterpret_cast<const n2_half*>(f->d_density_in), nullptr, mode, true)) return rc;
 	// grid: first-order and second-order gradients in one scatter pass (the reference's backward with
 	// Overwrite followed by backward_backward_input with Accumulate)

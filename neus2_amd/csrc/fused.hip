@@ -71,7 +71,7 @@ struct FusedArgs {
 	float* xyz_rows;        // [3][N]
 	uint4* slopes;          // [n_levels][N]: d feature / d position of each level (2 x 3 values, see n2_slopes_pack), without the level's scale
 	hf* dsdf_din;           // [sdf_in_w][N]
-	hf* rgb_in;             // [48][N]
+	hf* rgb_in;             // [N][N2_RGB_IN_PITCH]: sample-major
 	hf* output;             // [N][16]
 	// SDF only
 	hf* sdf_out;            // [16][N] or null
@@ -330,6 +330,8 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 	extern __shared__ __align__(16) unsigned char smem[];
 	hf* F = reinterpret_cast<hf*>(smem);
 	uint4* LV = reinterpret_cast<uint4*>(smem + (size_t)(FULL ? FF_COUNT : FF_SDF_COUNT) * 1024);
+	// FULL: each wave's staging area for the colour net's input (32 samples)
+	unsigned char* const stage = smem + (size_t)(FULL ? FF_COUNT : FF_SDF_COUNT) * 1024 + FF_LEVELS * sizeof(uint4) + (threadIdx.x >> 6) * (32 * 2 * N2_RGB_IN_PITCH);
 	if (threadIdx.x < FF_LEVELS)
 		LV[threadIdx.x] = make_uint4(__float_as_uint(a.lv.scale[threadIdx.x]), a.lv.res[threadIdx.x], a.lv.entries[threadIdx.x], a.lv.offset[threadIdx.x]);
 	build_fused_frags(F, a, FULL ? FF_COUNT : FF_SDF_COUNT);
@@ -485,21 +487,30 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 #pragma unroll
 			for (int d = 0; d < 3; ++d) { xc[2][d] = (hf)p[d]; xc[2][3 + d] = hn[d]; }
 		}
+		{
+			// The colour net's input goes out sample-major for the backward pass (N2_RGB_IN_PITCH = 40 values per sample: rows
+			// 38, 39 zero, rows 40..47 of the padded input left out): the wave's 32 samples are 2560 consecutive bytes.  A
+			// lane's registers are runs of 4 and 8 rows of its sample; stored from there, every 16 bytes would be a write
+			// request of their own.  Through LDS (80 bytes per sample: the 16-byte writes of 16 lanes fall on different
+			// banks) the wave writes whole lines.
+			unsigned char* sp = stage + n * (2 * N2_RGB_IN_PITCH);
+			*reinterpret_cast<half4v*>(sp + 8 * g) = half4v{y[0], y[1], y[2], y[3]};
+			*reinterpret_cast<half4v*>(sp + 16 + 8 * g) = half4v{y[4], y[5], y[6], y[7]};
+			*reinterpret_cast<half8*>(sp + 32 + 16 * g) = xc[1];
+			if (g == 0) *reinterpret_cast<half8*>(sp + 64) = xc[2];
+			__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+			__builtin_amdgcn_wave_barrier();
+			__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+			const uint32_t chunks = 5u * min(32u, n_live - tile * 32u);  // 16-byte chunks of the tile's samples
+			unsigned char* out = reinterpret_cast<unsigned char*>(a.rgb_in) + (size_t)tile * (32u * 2u * N2_RGB_IN_PITCH);
+#pragma unroll
+			for (int i = 0; i < 3; ++i) {
+				const uint32_t k = (uint32_t)lane + 64u * i;
+				if (k < chunks) *reinterpret_cast<uint4*>(out + (size_t)k * 16u) = *reinterpret_cast<const uint4*>(stage + k * 16u);
+			}
+		}
 		if (valid) {
-			// what the backward pass reads of the two networks
-#pragma unroll
-			for (int e = 0; e < 4; ++e) {
-				a.rgb_in[(size_t)e * N + off4] = y[e];
-				a.rgb_in[(size_t)(8 + e) * N + off4] = y[4 + e];
-			}
-#pragma unroll
-			for (int e = 0; e < 8; ++e) a.rgb_in[(size_t)(16 + 8 * g + e) * N + col] = xc[1][e];
-			if (g == 0) {
-#pragma unroll
-				for (int d = 0; d < 6; ++d) a.rgb_in[(size_t)(32 + d) * N + col] = xc[2][d];
-#pragma unroll
-				for (int d = 0; d < 3; ++d) a.dsdf_din[(size_t)d * N + col] = gx[d];
-			}
+			// (rows 0..2 of d sdf / d input, gx, have no reader behind this kernel)
 #pragma unroll
 			for (int r = 0; r < 16; ++r) {
 				const uint32_t level = 4u * (r >> 2) + 2u * g + ((r >> 1) & 1);
@@ -562,7 +573,9 @@ static uint32_t fused_grid(uint32_t n) {
 	const uint32_t tiles = (n + 31u) / 32u, blocks = (tiles + 3u) / 4u;
 	return blocks < 512u ? blocks : 512u;
 }
-static size_t fused_lds(int n_frags) { return (size_t)n_frags * 1024 + FF_LEVELS * sizeof(uint4); }
+static size_t fused_lds(int n_frags, bool staged = false) {
+	return (size_t)n_frags * 1024 + FF_LEVELS * sizeof(uint4) + (staged ? (size_t)(FF_BLOCK / 64) * 32 * 2 * N2_RGB_IN_PITCH : 0);
+}
 
 static FusedArgs fused_base(const N2FusedNets& nets, uint32_t n) {
 	FusedArgs a{};
@@ -602,7 +615,7 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 	a.output = reinterpret_cast<hf*>(d_output);
 	launch_gather<true>(a, *nets.tab, s);
 	N2_LAUNCH_CHECK();
-	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT), s>>>(a);
+	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT, true), s>>>(a);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

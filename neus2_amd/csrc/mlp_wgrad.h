@@ -85,6 +85,9 @@ __device__ __forceinline__ constexpr bool wg_dx_row(int mode, int row, int in_w)
 struct WgNoTail {
 	static constexpr bool active = false;
 };
+// With the tail, the launch also takes the field's layouts: X holds a column's first N2_RGB_IN_PITCH values side by side
+// (column c at X + N2_RGB_IN_PITCH c), and rows 0..15 of dL/dinput are written the same way (16 values per column, dX + 16 c); nothing else of
+// dL/dinput is stored.
 struct WgFieldPrepTail {
 	static constexpr bool active = true;
 	N2FieldPrepTail a;
@@ -121,7 +124,15 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 		// ---- the chain of this wave's 32 samples ----
 		half8 x[IC], dy, h[NH][4];
 		const uint32_t col_src = x_index ? min(x_index[col], x_cols - 1u) : col;  // the sample's column in X
-		load_tile_rows<IC>(X, x_index ? x_cols : N, col_src, g, x);
+		if constexpr (Tail::active) {
+			// the field keeps the colour net's input sample-major (N2_RGB_IN_PITCH values per column, the rows behind them
+			// are the padding's zeros): an operand is one 16-byte load
+#pragma unroll
+			for (int c = 0; c < IC; ++c)
+				x[c] = 16 * c + 8 * g < (int)N2_RGB_IN_PITCH ? *reinterpret_cast<const half8*>(X + (size_t)col_src * N2_RGB_IN_PITCH + 16 * c + 8 * g) : zero8();
+		} else {
+			load_tile_rows<IC>(X, x_index ? x_cols : N, col_src, g, x);
+		}
 		if (dy_aos) {
 			dy = *reinterpret_cast<const half8*>(dY + (size_t)col * MLP_OUT + 8 * g);
 		} else {
@@ -157,8 +168,16 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 					// row 0 also takes the direct gradient of the SDF output (row 3 of dL/doutput); rows 35..37 are dL/dnormal
 					if (t == 0 && g == 0) d[0] = (float)((hf)d[0] + dy_all[3]);
 					if (t == 1) { dn[0] = (hf)(g == 0 ? d[3] : d[0]); dn[1] = (hf)d[1]; }
+					// rows 0..15 go out sample-major (16 values per column, the SDF net's output gradient): the lane holds
+					// rows 4 g .. 4 g + 3 and 8 + 4 g .. 8 + 4 g + 3; rows 35..37 stay in registers (dn)
+					if (t == 0 && valid) {
+						const half4v lo = {(hf)d[0], (hf)d[1], (hf)d[2], (hf)d[3]}, hi = {(hf)d[4], (hf)d[5], (hf)d[6], (hf)d[7]};
+						hf* o = dX + (size_t)col * MLP_OUT + 4 * g;
+						*reinterpret_cast<half4v*>(o) = lo;
+						*reinterpret_cast<half4v*>(o + 8) = hi;
+					}
 				}
-				if (valid) {
+				if (!Tail::active && valid) {
 #pragma unroll
 					for (int r = 0; r < 16; ++r) {
 						const int row = 32 * t + 8 * (r >> 2) + (r & 3);  // + 4 g

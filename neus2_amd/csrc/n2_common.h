@@ -111,6 +111,9 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 //   * rows 3.. of that input: the encoding's dL_ddLdoutput = J v from the slopes the fused forward saved ([levels][n_src] 16-byte
 //     blocks, read at the sample's column of the index; scale[l] = the level's scale factor);
 //   * var_part[workgroup] = the workgroup's sum of row 7 of d_dL_doutput (n2_mlp_wgrad_blocks(n) workgroups).
+// With it the launch takes d_input sample-major ([n_cols][N2_RGB_IN_PITCH], the rows behind are zero) and writes only rows 0..15 of d_dL_dinput, sample-major too
+// ([n][16]: the AoS output gradient of the SDF net's backward).
+constexpr uint32_t N2_RGB_IN_PITCH = 40;  // values per sample of the colour net's saved input (38 in use)
 struct N2FieldPrepTail {
 	float ek_batch;
 	const void* slopes;
