@@ -236,10 +236,11 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	if (rc == N2_OK) rc = n2_fill_zero_u32(nullptr, b + c.coords[0], c.ws_sampler[0] - c.coords[0]);
 	if (rc == N2_OK && hipStreamSynchronize(nullptr) != hipSuccess) { n2_set_error("n2_trainer_create: workspace initialisation failed"); rc = N2_ERR_HIP; }
 	if (rc == N2_OK && cfg->prefetch_samples) {
-		// default priority on purpose: the stream only has to run beside the caller's, not ahead of it
+		// default priority on purpose: the stream only has to run beside the caller's, not ahead of it.  The two events order
+		// kernels of this GPU only (the host never waits on them), so they skip the system-scope fence: 2.5 us per step
 		if (hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking) != hipSuccess ||
-		    hipEventCreateWithFlags(&t->ev_main, hipEventDisableTiming) != hipSuccess ||
-		    hipEventCreateWithFlags(&t->ev_ready, hipEventDisableTiming) != hipSuccess) {
+		    hipEventCreateWithFlags(&t->ev_main, hipEventDisableTiming | hipEventDisableSystemFence) != hipSuccess ||
+		    hipEventCreateWithFlags(&t->ev_ready, hipEventDisableTiming | hipEventDisableSystemFence) != hipSuccess) {
 			n2_set_error("n2_trainer_create: cannot create the sample-generation stream");
 			rc = N2_ERR_HIP;
 		}
