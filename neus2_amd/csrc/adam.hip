@@ -55,14 +55,40 @@ __device__ __forceinline__ bool adam_summed(const N2SlabReduce& r, const hf* gra
 
 __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
                                                         uint32_t slot, const uint32_t* __restrict__ gate, float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
-                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps, N2SlabReduce sums) {
+                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps, N2SlabReduce sums,
+                                                        N2StepEpilogue epi) {
+	const uint32_t epi_blocks = epi.values != nullptr ? 1u : 0u;
+	if (epi_blocks && blockIdx.x == 0) {
+		// the caller's bookkeeping (the trainer: the loss of the step's rays and its counters), whether the step is gated or not
+		__shared__ float part[4];
+		const uint32_t n_val = min(*epi.n_ptr, epi.n_max);
+		float s = 0.f;
+		for (uint32_t i0 = 0; i0 < n_val; i0 += 16u * 256u) {  // sixteen loads in flight per thread
+			float v[16];
+#pragma unroll
+			for (uint32_t u = 0; u < 16; ++u) {
+				const uint32_t i = i0 + u * 256u + threadIdx.x;
+				v[u] = i < n_val ? epi.values[i] : 0.f;
+			}
+#pragma unroll
+			for (uint32_t u = 0; u < 16; ++u) s += v[u];
+		}
+#pragma unroll
+		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+		if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+		__syncthreads();
+		if (threadIdx.x == 0) *epi.sum_out = (part[0] + part[1]) + (part[2] + part[3]);
+		if (threadIdx.x < epi.copy_n) epi.copy_dst[threadIdx.x] = epi.copy_src[threadIdx.x];
+		return;
+	}
 	if (gate != nullptr && *gate == 0u) return;  // a step without samples leaves the parameters and the optimiser state alone
 	const float* table = g_adam_bias[slot];
-	if (blockIdx.x < sums.units) {
+	const uint32_t block = blockIdx.x - epi_blocks;
+	if (block < sums.units) {
 		// The first workgroups add up the slabs of 32 parameters each (25 MB of streaming reads that would otherwise be a launch
 		// of their own in front of this one), store the fp16 gradient and step the parameter with it.
 		__shared__ float fold[32][33];
-		n2_slab_reduce_unit(sums, blockIdx.x, fold, [&](const hf* at, hf g16) {
+		n2_slab_reduce_unit(sums, block, fold, [&](const hf* at, hf g16) {
 			const uint32_t i = (uint32_t)(at - grads);
 			float w = master[i], a = m1[i], b = m2[i];
 			uint32_t t = steps[i];
@@ -72,7 +98,7 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		});
 		return;
 	}
-	const uint32_t q = (blockIdx.x - sums.units) * 256 + threadIdx.x;
+	const uint32_t q = (block - sums.units) * 256 + threadIdx.x;
 	const uint32_t i0 = q * 4;
 	if (i0 >= n) return;
 	if (adam_summed(sums, grads, i0) || adam_summed(sums, grads, min(i0 + 3u, n - 1u))) {
@@ -126,7 +152,7 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums) {
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums, const N2StepEpilogue* epilogue) {
 	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
 	if (n_params == 0) return N2_OK;
 	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
@@ -185,8 +211,14 @@ int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_
 		N2_REQUIRE(inside(plan.ga, plan.params_a) && inside(plan.gb, plan.params_b) && inside(plan.extra_out, plan.extra_n > 0 ? 1u : 0u),
 		           "n2_adam_step: the summed gradients do not lie inside d_gradients");
 	}
-	adam_step_kernel<<<dim3((quads + 255) / 256 + plan.units), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate,
-		d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan);
+	N2StepEpilogue epi = {};
+	if (epilogue != nullptr && epilogue->values != nullptr) {
+		epi = *epilogue;
+		N2_REQUIRE(epi.n_ptr != nullptr && epi.sum_out != nullptr && epi.copy_n <= 256 && (epi.copy_n == 0 || (epi.copy_src && epi.copy_dst)),
+		           "n2_adam_step: incomplete step epilogue");
+	}
+	adam_step_kernel<<<dim3((quads + 255) / 256 + plan.units + (epi.values ? 1u : 0u)), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale,
+		inv_loss_scale, saturated, slot, d_gate, d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan, epi);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -96,44 +96,55 @@ constexpr int CB = 256;  // 4 rays per workgroup
 __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uint32_t n_rays, const uint32_t* __restrict__ ray_counter,
                                                                const uint32_t* __restrict__ numsteps, const hf* __restrict__ net_out,
                                                                const float* __restrict__ coords, RayScratch* __restrict__ scratch,
-                                                               uint32_t* __restrict__ kept_of) {
+                                                               uint32_t* __restrict__ kept_of, uint32_t* __restrict__ kept_of_block) {
 	const int lane = threadIdx.x & 63;
 	const uint32_t ray = blockIdx.x * (CB / 64) + (threadIdx.x >> 6);
-	if (ray >= n_rays) return;
 	const uint32_t live = ray_counter ? min(*ray_counter, n_rays) : n_rays;
-	if (ray >= live) {
-		if (lane == 0) { scratch[ray] = RayScratch{{0.f, 0.f, 0.f}, 0u}; kept_of[ray] = 0u; }
-		return;
-	}
-	const uint32_t n = numsteps[2 * ray], base = numsteps[2 * ray + 1];
-	float dir[3] = {0.f, 0.f, 0.f};
-	if (n > 0) ray_dir(net_out, base, dir);
-	float T = 1.f, r0 = 0.f, r1 = 0.f, r2 = 0.f;
 	uint32_t kept = 0;
-	for (uint32_t c0 = 0; c0 < n; c0 += 64) {
-		const uint32_t s = c0 + lane;
-		const bool valid = s < n;
-		float alpha = 0.f, rgb[3] = {0.f, 0.f, 0.f};
-		if (valid) {
-			float o[16];
-			load_out(net_out, (size_t)base + s, o);
-			const Sample sm = eval_sample(o, net_out[((size_t)base + s) * 16 + 7], coords[((size_t)base + s) * 7 + 3], dir, c);
-			alpha = sm.alpha; rgb[0] = sm.rgb[0]; rgb[1] = sm.rgb[1]; rgb[2] = sm.rgb[2];
+	if (ray < n_rays && ray >= live) {
+		if (lane == 0) { scratch[ray] = RayScratch{{0.f, 0.f, 0.f}, 0u}; kept_of[ray] = 0u; }
+	} else if (ray < n_rays) {
+		const uint32_t n = numsteps[2 * ray], base = numsteps[2 * ray + 1];
+		float dir[3] = {0.f, 0.f, 0.f};
+		if (n > 0) ray_dir(net_out, base, dir);
+		float T = 1.f, r0 = 0.f, r1 = 0.f, r2 = 0.f;
+		for (uint32_t c0 = 0; c0 < n; c0 += 64) {
+			const uint32_t s = c0 + lane;
+			const bool valid = s < n;
+			float alpha = 0.f, rgb[3] = {0.f, 0.f, 0.f};
+			if (valid) {
+				float o[16];
+				load_out(net_out, (size_t)base + s, o);
+				const Sample sm = eval_sample(o, net_out[((size_t)base + s) * 16 + 7], coords[((size_t)base + s) * 7 + 3], dir, c);
+				alpha = sm.alpha; rgb[0] = sm.rgb[0]; rgb[1] = sm.rgb[1]; rgb[2] = sm.rgb[2];
+			}
+			const float Tb = T * wave_excl_prod(1.f - alpha, lane);
+			// samples are consumed while the transmittance before them is >= 1e-4
+			const unsigned long long stop = __ballot(!valid || Tb < T_EPS);
+			const int n_proc = stop ? (int)__ffsll((long long)stop) - 1 : 64;
+			const float w = lane < n_proc ? alpha * Tb : 0.f;
+			r0 += wave_sum(w * rgb[0]);
+			r1 += wave_sum(w * rgb[1]);
+			r2 += wave_sum(w * rgb[2]);
+			kept += n_proc;
+			if (n_proc > 0) T = __shfl(Tb * (1.f - alpha), n_proc - 1);
+			if (n_proc < 64) break;
 		}
-		const float Tb = T * wave_excl_prod(1.f - alpha, lane);
-		// samples are consumed while the transmittance before them is >= 1e-4
-		const unsigned long long stop = __ballot(!valid || Tb < T_EPS);
-		const int n_proc = stop ? (int)__ffsll((long long)stop) - 1 : 64;
-		const float w = lane < n_proc ? alpha * Tb : 0.f;
-		r0 += wave_sum(w * rgb[0]);
-		r1 += wave_sum(w * rgb[1]);
-		r2 += wave_sum(w * rgb[2]);
-		kept += n_proc;
-		if (n_proc > 0) T = __shfl(Tb * (1.f - alpha), n_proc - 1);
-		if (n_proc < 64) break;
+		if (kept == n) { r0 += T * c.bg[0]; r1 += T * c.bg[1]; r2 += T * c.bg[2]; }
+		if (lane == 0) { scratch[ray] = RayScratch{{r0, r1, r2}, kept}; kept_of[ray] = kept; }
 	}
-	if (kept == n) { r0 += T * c.bg[0]; r1 += T * c.bg[1]; r2 += T * c.bg[2]; }
-	if (lane == 0) { scratch[ray] = RayScratch{{r0, r1, r2}, kept}; kept_of[ray] = kept; }
+	// the workgroup's count: the backward kernel adds up a quarter as many values to place its rays in the batch
+	if (kept_of_block) {
+		__shared__ uint32_t wave_kept[CB / 64];
+		if (lane == 0) wave_kept[threadIdx.x >> 6] = kept;
+		__syncthreads();
+		if (threadIdx.x == 0) {
+			uint32_t sum = 0;
+#pragma unroll
+			for (int w = 0; w < CB / 64; ++w) sum += wave_kept[w];
+			kept_of_block[blockIdx.x] = sum;
+		}
+	}
 }
 
 // before_of[r] = kept_of[0] + ... + kept_of[r - 1].  One workgroup per 1024 consecutive rays: it adds up the counts of all
@@ -180,41 +191,54 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
                                                                 const uint32_t* __restrict__ kept_of, uint32_t max_compacted,
                                                                 uint32_t* __restrict__ counter, float* __restrict__ coords_out,
                                                                 hf* __restrict__ dloss, float* __restrict__ loss, uint32_t* __restrict__ source_index,
-                                                                const uint32_t* __restrict__ before_of) {
+                                                                const uint32_t* __restrict__ before_of, uint32_t pad,
+                                                                const uint32_t* __restrict__ kept_of_block) {
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 	// Where this workgroup's rays start in the compacted batch: the kept samples of all rays before them, in ray order
 	// (deterministic).  With a few thousand rays every workgroup adds up the counts of its predecessors itself: a few KiB
 	// of L2 reads each instead of a scan kernel in between.  That work grows with the square of the ray count, so beyond
 	// OFFSETS_MIN_RAYS rays composite_offsets_kernel has left the sums in before_of.
-	__shared__ uint32_t part[CB / 64];
+	//
+	// pad: the batch is also filled up to max_compacted samples here.  With n_in = min(all kept samples, max_compacted), slot
+	// j >= n_in holds a copy of slot j % n_in whose output gradient is scaled by n_in / max_compacted (fill_rollover on the
+	// coordinates, fill_rollover_and_rescale on the gradients, src/testbed_nerf.cu:3908-3916): the ray that writes slot p also
+	// writes slots p + n_in, p + 2 n_in, ...  That needs the count of ALL rays, which the same loop adds up.
+	__shared__ uint32_t part[CB / 64], part_all[CB / 64];
 	const uint32_t first = blockIdx.x * (CB / 64);
-	uint32_t before = 0;
+	uint32_t before = 0, all = 0;
 	// eight loads in flight per lane: the last workgroups add up thousands of counts, and one dependent L2 round trip per
 	// CB of them was most of this kernel's duration
-	for (uint32_t r0 = 0; r0 < (before_of ? 0u : first); r0 += 8 * CB) {
+	// (kept_of_block: the forward kernel's counts per workgroup of CB / 64 rays, the same workgroups as here)
+	const uint32_t n_counts = before_of ? 0u : (pad ? gridDim.x : blockIdx.x);
+	for (uint32_t r0 = 0; r0 < n_counts; r0 += 8 * CB) {
 		uint32_t v[8];
 #pragma unroll
 		for (uint32_t u = 0; u < 8; ++u) {
 			const uint32_t r = r0 + u * CB + threadIdx.x;
-			v[u] = r < first ? kept_of[r] : 0u;
+			v[u] = r < n_counts ? kept_of_block[r] : 0u;
 		}
 #pragma unroll
-		for (uint32_t u = 0; u < 8; ++u) before += v[u];
+		for (uint32_t u = 0; u < 8; ++u) {
+			all += v[u];
+			before += r0 + u * CB + threadIdx.x < blockIdx.x ? v[u] : 0u;
+		}
 	}
 #pragma unroll
-	for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
-	if (lane == 0) part[wave] = before;
+	for (int o = 32; o > 0; o >>= 1) { before += __shfl_xor(before, o); all += __shfl_xor(all, o); }
+	if (lane == 0) { part[wave] = before; part_all[wave] = all; }
 	__syncthreads();
 	const uint32_t ray = first + wave;
 	if (ray >= n_rays) return;
-	uint32_t cb = 0;
+	uint32_t cb = 0, total = 0;
 	if (before_of) {
 		cb = before_of[ray];
+		if (pad) total = before_of[n_rays - 1] + kept_of[n_rays - 1];
 	} else {
 #pragma unroll
-		for (int w = 0; w < CB / 64; ++w) cb += part[w];
+		for (int w = 0; w < CB / 64; ++w) { cb += part[w]; total += part_all[w]; }
 		for (int w = 0; w < wave; ++w) cb += kept_of[first + w];
 	}
+	const uint32_t n_in = min(total, max_compacted);  // pad: the samples the batch holds before it is filled up
 	const uint32_t kept = kept_of[ray];
 	const uint32_t m = min(max_compacted - min(max_compacted, cb), kept);  // the batch holds max_compacted samples
 	if (ray == n_rays - 1 && lane == 0) *counter = cb + kept;
@@ -299,6 +323,23 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 #pragma unroll
 			for (int k = 0; k < 7; ++k) co[k] = ci[k];
 			if (source_index) source_index[cb + s] = base + s;  // which marched sample this compacted sample is
+			if (pad && n_in > 0 && n_in < max_compacted) {
+				for (uint32_t j = cb + s + n_in; j < max_compacted; j += n_in) {
+					half8 lo_f, hi_f;
+#pragma unroll
+					for (int k = 0; k < 8; ++k) {
+						lo_f[k] = (hf)((float)lo[k] * (float)n_in / (float)max_compacted);
+						hi_f[k] = (hf)((float)hi[k] * (float)n_in / (float)max_compacted);
+					}
+					hf* gf = dloss + (size_t)j * 16;
+					*reinterpret_cast<half8*>(gf) = lo_f;
+					*reinterpret_cast<half8*>(gf + 8) = hi_f;
+					float* cf = coords_out + (size_t)j * 7;
+#pragma unroll
+					for (int k = 0; k < 7; ++k) cf[k] = ci[k];
+					if (source_index) source_index[j] = base + s;
+				}
+			}
 		}
 		T = __shfl(Ta, 63);
 		p0 = __shfl(q0, 63); p1 = __shfl(q1, 63); p2 = __shfl(q2, 63);
@@ -381,6 +422,15 @@ N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_conf
                                      const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
                                      uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
                                      float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes) {
+	return n2_composite_loss_filled(stream, cfg, n_rays, d_ray_counter, d_numsteps, d_network_output, d_coords, d_rgb_target, max_samples_compacted,
+	                                d_compacted_counter, d_coords_compacted, d_dloss_doutput, d_loss, d_source_index, d_workspace, workspace_bytes, false);
+}
+
+int n2_composite_loss_filled(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
+                             const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
+                             const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                             uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
+                             float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes, bool fill) {
 	N2_REQUIRE(cfg != nullptr, "n2_composite_loss: config is null");
 	N2_REQUIRE(d_compacted_counter != nullptr, "n2_composite_loss: d_compacted_counter is null");
 	hipStream_t s = n2_stream(stream);
@@ -405,7 +455,9 @@ N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_conf
 	const dim3 grid((n_rays + CB / 64 - 1) / (CB / 64)), block(CB);
 	const hf* out = reinterpret_cast<const hf*>(d_network_output);
 	N2ProfScope prof(N2_PROF_COMPOSITE, s);
-	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch, kept_of);
+	// below OFFSETS_MIN_RAYS rays the second count array holds the forward kernel's counts per workgroup instead of prefix sums
+	uint32_t* kept_of_block = before_of ? nullptr : kept_of + up256(4ull * n_rays) / 4;
+	composite_forward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_ray_counter, d_numsteps, out, d_coords, scratch, kept_of, kept_of_block);
 	N2_LAUNCH_CHECK();
 	if (before_of) {
 		composite_offsets_kernel<<<dim3((n_rays + OFFSETS_BLOCK - 1) / OFFSETS_BLOCK), dim3(OFFSETS_BLOCK), 0, s>>>(n_rays, kept_of, before_of);
@@ -413,7 +465,7 @@ N2_API int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_conf
 	}
 	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, kept_of, max_samples_compacted,
 	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss, d_source_index,
-	                                                 before_of);
+	                                                 before_of, fill ? 1u : 0u, kept_of_block);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

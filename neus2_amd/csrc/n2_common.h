@@ -34,7 +34,8 @@ void n2_set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 constexpr uint32_t N2_MAX_LEVELS = 32;
 
-struct N2SlabReduce;  // slab_reduce.h
+struct N2SlabReduce;
+struct N2StepEpilogue;  // slab_reduce.h
 
 // How a level turns integer grid coordinates into an entry index.
 enum : uint32_t {
@@ -104,6 +105,15 @@ struct N2Lattice {
 int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n, n2_half* d_out_soa,
                        float* d_row0, bool density, n2_half* sdf_in, uint32_t row0_n = 0xFFFFFFFFu, const N2Lattice* lattice = nullptr);
 
+// n2_composite_loss_indexed that also fills the compacted batch up to max_samples_compacted samples (fill = true): slot j
+// behind the n_in = min(*d_compacted_counter, max_samples_compacted) kept samples holds a copy of slot j % n_in (coordinates,
+// source index, output gradient scaled by n_in / max_samples_compacted), what n2_fill_rollover_f32 and
+// n2_fill_rollover_and_rescale_f16 would write in launches of their own.
+int n2_composite_loss_filled(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays, const uint32_t* d_ray_counter, uint32_t* d_numsteps,
+                             const n2_half* d_network_output, const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
+                             uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput, float* d_loss, uint32_t* d_source_index,
+                             void* d_workspace, uint64_t workspace_bytes, bool fill);
+
 // What the field hangs on its colour net's backward launch (n2_mlp_backward_rows_indexed): for the same samples,
 //   * row 0 of d_dL_dinput also takes row 3 of d_dL_doutput (the direct gradient of the SDF output);
 //   * v[d] = row 35 + d of d_dL_dinput + row 4 + d of d_dL_doutput / ek_batch + row 8 + d of d_dL_doutput (dL/dnormal), written
@@ -141,9 +151,11 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 // n2_adam_step that does nothing when *d_gate is zero on the device (d_gate null: always steps)
 // sums (or null): a slab summation whose gradients lie inside d_gradients; the kernel's first workgroups run it, store the
 // fp16 gradients and step those parameters themselves (the other workgroups leave them alone)
+// epilogue (or null): one more workgroup of the launch does the caller's bookkeeping (slab_reduce.h), gated or not
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums = nullptr);
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums = nullptr,
+                       const N2StepEpilogue* epilogue = nullptr);
 // n2_mlp_reduce_deferred that also adds up n_parts floats, in a fixed order, into one fp16 value ([+=] when accumulate)
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
 // The same work as a plan instead of a launch: what is pending is handed to *out (and no longer pending), for

@@ -15,6 +15,13 @@ struct N2SlabReduce {
 	uint32_t units;  // units_a + units_b + (extra_n > 0)
 };
 
+// Bookkeeping of a training step that rides in the optimiser's launch as one workgroup (values null: none):
+// *sum_out = values[0] + ... + values[min(*n_ptr, n_max) - 1], added up in a fixed order, and copy_n words copied.
+struct N2StepEpilogue {
+	const float* values; const uint32_t* n_ptr; uint32_t n_max; float* sum_out;
+	const uint32_t* copy_src; uint32_t* copy_dst; uint32_t copy_n;
+};
+
 // Unit `unit` of the plan, run by the 256 threads of a workgroup.  A unit owns 32 consecutive parameters (one 128-byte line
 // of every slab): 8 lanes cover the line with 16-byte loads, 32 lane groups share the slabs, eight loads in flight per
 // lane, LDS folds the groups.  n_params is a multiple of 16, so lines are never ragged.  The fp16 gradient is stored, and

@@ -132,48 +132,6 @@ __global__ void __launch_bounds__(256) trainer_cast_params_kernel(uint32_t n, co
 	if (i < n) params[i] = (hf)master[i];
 }
 
-// After compositing, in one launch: pad the compacted batch to exactly T samples (fill_rollover_and_rescale on the fp16
-// output gradients, fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916) and, in the last workgroup, sum the
-// per-ray losses of the live rays and publish the sample set's counters.
-__global__ void __launch_bounds__(256) trainer_finish_batch_kernel(uint32_t T, const uint32_t* __restrict__ n_in_ptr, hf* __restrict__ dloss,
-                                                                   float* __restrict__ coords, uint32_t* __restrict__ src_index,
-                                                                   const uint32_t* __restrict__ set_counters, uint32_t max_rays,
-                                                                   const float* __restrict__ ray_loss, uint32_t* __restrict__ counters) {
-	const uint32_t n_in = *n_in_ptr;
-	if (blockIdx.x + 1 < gridDim.x) {
-		// the padding is usually a small tail of the batch: the workgroups stride over it instead of covering all of T
-		if (n_in == 0 || n_in >= T) return;
-		const size_t stride = (size_t)(gridDim.x - 1) * 256, first = (size_t)blockIdx.x * 256 + threadIdx.x;
-		const size_t lim16 = (size_t)n_in * 16, lim7 = (size_t)n_in * 7;
-		for (size_t i = lim16 + first; i < (size_t)T * 16; i += stride) dloss[i] = (hf)((float)dloss[i % lim16] * (float)n_in / (float)T);
-		for (size_t i = lim7 + first; i < (size_t)T * 7; i += stride) coords[i] = coords[i % lim7];
-		for (size_t i = n_in + first; i < T; i += stride) src_index[i] = src_index[i % n_in];
-	} else {
-		__shared__ float part[4];
-		const uint32_t n = min(set_counters[0], max_rays);
-		float s = 0.f;
-		for (uint32_t i0 = 0; i0 < n; i0 += 16u * 256u) {  // sixteen loads in flight per thread: tens of thousands of rays once they end at the surface
-			float v[16];
-#pragma unroll
-			for (uint32_t u = 0; u < 16; ++u) {
-				const uint32_t i = i0 + u * 256u + threadIdx.x;
-				v[u] = i < n ? ray_loss[i] : 0.f;
-			}
-#pragma unroll
-			for (uint32_t u = 0; u < 16; ++u) s += v[u];
-		}
-#pragma unroll
-		for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
-		if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
-		__syncthreads();
-		if (threadIdx.x == 0) {
-			counters[0] = set_counters[0];
-			counters[1] = set_counters[1];
-			reinterpret_cast<float*>(counters)[4] = (part[0] + part[1]) + (part[2] + part[3]);
-		}
-	}
-}
-
 N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, uint64_t workspace_bytes, n2_trainer_t** out) {
 	N2_REQUIRE(out != nullptr, "n2_trainer_create: out is null");
 	*out = nullptr;
@@ -353,15 +311,11 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	n2_composite_config cc = t->cfg.composite;
 	cc.n_rays_norm = n_rays;
 	cc.loss_scale = t->cfg.loss_scale;
-	if (int rc = n2_composite_loss_indexed(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
-	                                       set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss),
-	                                       t->ray_loss, t->src_index, t->ws_composite, t->ws_composite_bytes)) return rc;
-	// pad the compacted batch to exactly T samples; loss sum and counters
-	uint32_t pad_blocks = (uint32_t)(((size_t)T * 16 + 255) / 256);
-	if (pad_blocks > 512) pad_blocks = 512;
-	trainer_finish_batch_kernel<<<dim3(pad_blocks + 1), dim3(256), 0, s>>>(T, compacted_counter, t->dloss, t->coords_compacted, t->src_index, ray_counter, n_rays,
-	                                                                     t->ray_loss, t->counters);
-	N2_LAUNCH_CHECK();
+	// (the compacted batch comes back filled up to exactly T samples: fill_rollover_and_rescale on the output gradients,
+	// fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916)
+	if (int rc = n2_composite_loss_filled(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
+	                                      set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss),
+	                                      t->ray_loss, t->src_index, t->ws_composite, t->ws_composite_bytes, true)) return rc;
 	// forward + backward on the compacted batch, then the optimiser.  Every compacted sample is one of the marched
 	// samples the field has just been evaluated on: unless asked to run the field again, the activations saved for it
 	// are selected instead (the same values, a fraction of the work).
@@ -373,9 +327,13 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	// the summation of the networks' weight-gradient slabs rides in the optimiser's kernel instead of taking a launch
 	N2SlabReduce sums;
 	if (int rc = n2_field_backward_deferred(t->field, stream, t->coords_compacted, T, reinterpret_cast<const n2_half*>(t->dloss), T, N2_GRAD_OVERWRITE, &sums)) return rc;
-	// a step whose rays kept no sample (counter 2 is zero) must not apply the previous step's gradients again
+	// a step whose rays kept no sample (counter 2 is zero) must not apply the previous step's gradients again.  The step's
+	// bookkeeping rides along: the sum of the live rays' losses (counter 4, as a float) and the sample set's counters
+	N2StepEpilogue epi{};
+	epi.values = t->ray_loss; epi.n_ptr = ray_counter; epi.n_max = n_rays; epi.sum_out = reinterpret_cast<float*>(t->counters) + 4;
+	epi.copy_src = set.counters; epi.copy_dst = t->counters; epi.copy_n = 2;
 	if (int rc = n2_adam_step_gated(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums)) return rc;
+	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums, &epi)) return rc;
 	t->optimizer_steps += 1;
 	t->training_step += 1;
 	if (t->ema) {

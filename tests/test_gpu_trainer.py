@@ -60,6 +60,28 @@ def test_one_step_matches_oracle_pipeline(oracle, setup):
     np.testing.assert_array_equal(host(tr.params), q16(host(tr.master)))
 
 
+def test_a_small_batch_rolls_over_several_times(oracle, setup):
+    """Few rays: the kept samples fill less than half of the batch, so every kept sample is copied (and its output
+    gradient rescaled) more than once; every stage of the step against the oracle, as above."""
+    from oracle.field import Field
+    from oracle.step import verify_step
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    _, cams, rgba, bits, T = setup
+    tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=2048, max_samples=16 * T, background=(1.0, 1.0, 1.0)))
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), dev(bits))
+    tr.initialize_params(seed=7, sdf_mlp_weights=None)
+    params16 = host(tr.params)
+    n_rays, seed, n_inf = 40, 3, 16 * T
+    tr.step(n_rays=n_rays, n_inference=n_inf, seed=seed)
+    c = tr.read_counters()
+    assert 0 < c["compacted"] < T // 2, c
+    gpu = {k: host(v) for k, v in tr.last_step(c["rays"], c["samples"], n_inf).items()}
+    res = verify_step(Field(fp16=True), params16, oc_cams(oracle, cams), rgba, bits, n_rays, 0, seed, n_inf, T, c, gpu,
+                      host(tr.grads), background=(1.0, 1.0, 1.0))
+    assert res["compacted"] == c["compacted"]
+
+
 def test_training_reduces_the_loss(setup):
     """End-to-end: a sign error anywhere in the first- or second-order backward would stop this from converging."""
     tr, cams, rgba, bits, T = setup
