@@ -3,6 +3,7 @@
 // accesses; parameters whose gradient is zero (most of the hash table in any
 // one step) cost only the 2-byte gradient read.
 #include "n2_common.h"
+#include <hip/hip_ext.h>
 #include "slab_reduce.h"
 
 #include <cmath>
@@ -152,7 +153,7 @@ N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32
 
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums, const N2StepEpilogue* epilogue) {
+                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums, const N2StepEpilogue* epilogue, hipEvent_t done_event) {
 	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
 	if (n_params == 0) return N2_OK;
 	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
@@ -217,8 +218,17 @@ int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_
 		N2_REQUIRE(epi.n_ptr != nullptr && epi.sum_out != nullptr && epi.copy_n <= 256 && (epi.copy_n == 0 || (epi.copy_src && epi.copy_dst)),
 		           "n2_adam_step: incomplete step epilogue");
 	}
-	adam_step_kernel<<<dim3((quads + 255) / 256 + plan.units + (epi.values ? 1u : 0u)), dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale,
-		inv_loss_scale, saturated, slot, d_gate, d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan, epi);
+	const dim3 grid((quads + 255) / 256 + plan.units + (epi.values ? 1u : 0u));
+	if (done_event != nullptr) {
+		// the event is tied to this launch's own completion: no packet of its own behind the kernel, where an event record costs
+		// the stream about 5 us before its next kernel starts
+		hipExtLaunchKernelGGL(adam_step_kernel, grid, dim3(256), 0, s, nullptr, done_event, 0, *config, n_params, n_matrix_params, loss_scale, inv_loss_scale,
+		                      saturated, slot, d_gate, d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps,
+		                      plan, epi);
+	} else {
+		adam_step_kernel<<<grid, dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate, d_master,
+			reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan, epi);
+	}
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

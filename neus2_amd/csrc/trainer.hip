@@ -57,6 +57,7 @@ struct n2_trainer {
 	uint32_t n_rays_total;
 	// sample generation running ahead of the step that uses it
 	hipStream_t side;
+	bool ev_main_from_adam;   // ev_main stands for the completion of the last step's Adam launch
 	hipEvent_t ev_main, ev_ready;
 	bool pf_valid;
 	uint32_t pf_set, pf_n_rays, pf_n_inference, pf_seed, pf_ray_base;
@@ -273,11 +274,15 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		                                    t->cfg.composite.background, t->bitfield, n_inference, set.counters, set.counters + 1, set.ray_indices,
 		                                    set.numsteps, set.rgb_target, set.coords, set.ws_sampler, t->ws_sampler_bytes);
 	};
-	// the following step's samples on the side stream, assuming the same ray count and the next seed; everything enqueued on
-	// s so far precedes the generator
+	// the following step's samples on the side stream, assuming the same ray count and the next seed
+	bool main_event_is_last_step = false;
 	auto prefetch = [&](uint32_t cur_set) -> int {
 		t->pf_valid = false;
-		N2_HIP(hipEventRecord(t->ev_main, s));
+		// The generator overwrites the other sample set, which the previous step's kernels read: it waits for that step's
+		// last launch, whose completion is ev_main (no packet on s).  When anything else may have been enqueued on s since
+		// (the first step, a step that missed its prefetch: the caller has changed the scene, the bitfield or the
+		// arguments), the event is recorded here, behind everything on s.
+		if (!main_event_is_last_step) N2_HIP(hipEventRecord(t->ev_main, s));
 		N2_HIP(hipStreamWaitEvent(t->side, t->ev_main, 0));
 		if (int rc = sample(t->sets[1u - cur_set], t->side, t->n_rays_total, seed + 1)) return rc;
 		N2_HIP(hipEventRecord(t->ev_ready, t->side));
@@ -289,6 +294,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		const bool hit = t->pf_valid && t->pf_n_rays == n_rays && t->pf_n_inference == n_inference && t->pf_seed == seed && t->pf_ray_base == t->n_rays_total;
 		if (hit) {
 			cur = t->pf_set;
+			main_event_is_last_step = t->ev_main_from_adam;
 			N2_HIP(hipStreamWaitEvent(s, t->ev_ready, 0));
 		} else {
 			// a generation that ran ahead with other arguments is abandoned (it stays ordered on the side stream)
@@ -333,7 +339,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	epi.values = t->ray_loss; epi.n_ptr = ray_counter; epi.n_max = n_rays; epi.sum_out = reinterpret_cast<float*>(t->counters) + 4;
 	epi.copy_src = set.counters; epi.copy_dst = t->counters; epi.copy_n = 2;
 	if (int rc = n2_adam_step_gated(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums, &epi)) return rc;
+	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums, &epi,
+	                                t->side ? t->ev_main : nullptr)) return rc;
+	t->ev_main_from_adam = t->side != nullptr;
 	t->optimizer_steps += 1;
 	t->training_step += 1;
 	if (t->ema) {
