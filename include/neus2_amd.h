@@ -602,15 +602,20 @@ int n2_trainer_set_learning_rate(n2_trainer_t* trainer, float learning_rate);
 
 /* Optimizer state inside the workspace (what Trainer::serialize(include_optimizer_state) stores, src/testbed.cu:3134-3137):
  * Adam moments and per-parameter step counters, the fp32 moving average of the Ema wrapper (NULL without it) and the
- * parameters to use for inference (the Ema copy when it exists, else the working copy). */
+ * parameters to use for inference (the Ema copy when it exists, else the working copy).
+ * The step counters are param_steps_bits wide: uint32_t, or uint16_t that stop at 65535 when the Adam betas are such that
+ * 1 - beta^t is exactly 1 in fp32 from step 4096 on (the defaults are): the bias correction no longer depends on the
+ * count then, and the narrow counters save 4 bytes of traffic per parameter and step.  n2_snapshot_save and
+ * n2_snapshot_read take either width and keep the file's 32-bit form. */
 typedef struct n2_trainer_optimizer_buffers {
 	float* first_moments;
 	float* second_moments;
-	uint32_t* param_steps;
+	void* param_steps;
 	float* ema_weights;
 	n2_half* inference_params;
 	uint32_t optimizer_steps;
 	float learning_rate;
+	uint32_t param_steps_bits;
 } n2_trainer_optimizer_buffers;
 int n2_trainer_optimizer_state(n2_trainer_t* trainer, n2_trainer_optimizer_buffers* out);
 int n2_trainer_set_optimizer_steps(n2_trainer_t* trainer, uint32_t steps);
@@ -757,7 +762,7 @@ typedef struct n2_snapshot_desc {
 	uint32_t include_optimizer_state;
 	const float* d_first_moments;    /* Adam state, n_params each (only with include_optimizer_state) */
 	const float* d_second_moments;
-	const uint32_t* d_param_steps;
+	const void* d_param_steps;       /* uint32_t, or uint16_t when param_steps_bits (below) is 16 */
 	const float* d_ema_weights;      /* fp32 moving average of the Ema wrapper, or NULL */
 	uint32_t optimizer_steps;
 	float learning_rate;
@@ -769,6 +774,7 @@ typedef struct n2_snapshot_desc {
 	uint32_t rays_per_batch, measured_batch_size, measured_batch_size_before_compaction;
 	uint32_t training_step;
 	float loss;
+	uint32_t param_steps_bits;       /* width of d_param_steps: 16, or 32 (0 reads as 32); the file always holds 32-bit counters */
 } n2_snapshot_desc;
 
 /* Testbed::save_snapshot(path, include_optimizer_state).  Synchronises with the stream. */
@@ -796,10 +802,11 @@ typedef struct n2_snapshot_targets {
 	uint64_t density_grid_cells;
 	float* d_first_moments;
 	float* d_second_moments;
-	uint32_t* d_param_steps;
+	void* d_param_steps;             /* uint32_t, or uint16_t when param_steps_bits is 16 (counts above 65535 stop there) */
 	float* d_ema_weights;
 	void* d_scratch;                 /* device staging: max(params_binary bytes, 2 bytes per density cell) */
 	uint64_t scratch_bytes;
+	uint32_t param_steps_bits;       /* 16, or 32 (0 reads as 32) */
 } n2_snapshot_targets;
 
 /* Testbed::load_snapshot: reads and checks the file ("does not contain a snapshot", parameter count, grid size). */

@@ -53,7 +53,7 @@ class TrainerOptimizerBuffers(C.Structure):
     """struct n2_trainer_optimizer_buffers"""
     _fields_ = [("first_moments", C.c_void_p), ("second_moments", C.c_void_p), ("param_steps", C.c_void_p),
                 ("ema_weights", C.c_void_p), ("inference_params", C.c_void_p), ("optimizer_steps", C.c_uint32),
-                ("learning_rate", C.c_float)]
+                ("learning_rate", C.c_float), ("param_steps_bits", C.c_uint32)]
 
 
 class TrainerStepView(C.Structure):

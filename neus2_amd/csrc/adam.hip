@@ -7,6 +7,7 @@
 #include "slab_reduce.h"
 
 #include <cmath>
+#include <type_traits>
 #include <mutex>
 
 typedef _Float16 hf;
@@ -47,6 +48,24 @@ __device__ __forceinline__ bool adam_one(uint32_t i, uint32_t n_matrix, float lo
 	return true;
 }
 
+// Step counters are 32 bits wide, or 16 bits saturating at 65535 (the trainer's, when both beta powers have underflowed
+// long before: past the table the correction is exactly 1 then, so the count no longer matters; 4 bytes less traffic per
+// touched parameter).
+__device__ __forceinline__ uint32_t step_load(const uint32_t* p) { return *p; }
+__device__ __forceinline__ uint32_t step_load(const uint16_t* p) { return *p; }
+__device__ __forceinline__ void step_store(uint32_t* p, uint32_t t) { *p = t; }
+__device__ __forceinline__ void step_store(uint16_t* p, uint32_t t) { *p = (uint16_t)min(t, 65535u); }
+__device__ __forceinline__ uint4 step_load4(const uint32_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint4 step_load4(const uint16_t* p) {
+	const ushort4 v = *reinterpret_cast<const ushort4*>(p);
+	return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void step_store4(uint32_t* p, uint4 t) { *reinterpret_cast<uint4*>(p) = t; }
+__device__ __forceinline__ void step_store4(uint16_t* p, uint4 t) {
+	*reinterpret_cast<ushort4*>(p) = make_ushort4((unsigned short)min(t.x, 65535u), (unsigned short)min(t.y, 65535u), (unsigned short)min(t.z, 65535u),
+	                                              (unsigned short)min(t.w, 65535u));
+}
+
 // parameters whose gradients a slab summation produces (r.units > 0): the workgroups that run its units step them
 __device__ __forceinline__ bool adam_summed(const N2SlabReduce& r, const hf* grads, uint32_t i) {
 	if (r.units == 0) return false;
@@ -54,9 +73,10 @@ __device__ __forceinline__ bool adam_summed(const N2SlabReduce& r, const hf* gra
 	return (g >= r.ga && g < r.ga + r.params_a) || (g >= r.gb && g < r.gb + r.params_b) || (r.extra_n > 0 && g == r.extra_out);
 }
 
+template <typename StepT>
 __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32_t n, uint32_t n_matrix, float loss_scale, float inv_loss_scale, int saturated,
                                                         uint32_t slot, const uint32_t* __restrict__ gate, float* __restrict__ master, hf* __restrict__ params, const hf* __restrict__ grads,
-                                                        float* __restrict__ m1, float* __restrict__ m2, uint32_t* __restrict__ steps, N2SlabReduce sums,
+                                                        float* __restrict__ m1, float* __restrict__ m2, StepT* __restrict__ steps, N2SlabReduce sums,
                                                         N2StepEpilogue epi) {
 	const uint32_t epi_blocks = epi.values != nullptr ? 1u : 0u;
 	if (epi_blocks && blockIdx.x == 0) {
@@ -92,9 +112,9 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		n2_slab_reduce_unit(sums, block, fold, [&](const hf* at, hf g16) {
 			const uint32_t i = (uint32_t)(at - grads);
 			float w = master[i], a = m1[i], b = m2[i];
-			uint32_t t = steps[i];
+			uint32_t t = step_load(steps + i);
 			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g16, w, a, b, t)) {
-				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+				master[i] = w; m1[i] = a; m2[i] = b; step_store(steps + i, t); params[i] = (hf)w;
 			}
 		});
 		return;
@@ -108,9 +128,9 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		for (uint32_t i = i0; i < min(i0 + 4u, n); ++i) {
 			if (adam_summed(sums, grads, i)) continue;
 			float w = master[i], a = m1[i], b = m2[i];
-			uint32_t t = steps[i];
+			uint32_t t = step_load(steps + i);
 			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)grads[i], w, a, b, t)) {
-				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+				master[i] = w; m1[i] = a; m2[i] = b; step_store(steps + i, t); params[i] = (hf)w;
 			}
 		}
 		return;
@@ -122,7 +142,7 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		float4 w = *reinterpret_cast<float4*>(master + i0);
 		float4 a = *reinterpret_cast<float4*>(m1 + i0);
 		float4 b = *reinterpret_cast<float4*>(m2 + i0);
-		uint4 t = *reinterpret_cast<uint4*>(steps + i0);
+		uint4 t = step_load4(steps + i0);
 		bool any = false;
 		any |= adam_one(i0 + 0, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[0], w.x, a.x, b.x, t.x);
 		any |= adam_one(i0 + 1, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)g[1], w.y, a.y, b.y, t.y);
@@ -132,28 +152,34 @@ __global__ void __launch_bounds__(256) adam_step_kernel(n2_adam_config c, uint32
 		*reinterpret_cast<float4*>(master + i0) = w;
 		*reinterpret_cast<float4*>(m1 + i0) = a;
 		*reinterpret_cast<float4*>(m2 + i0) = b;
-		*reinterpret_cast<uint4*>(steps + i0) = t;
+		step_store4(steps + i0, t);
 		*reinterpret_cast<half4*>(params + i0) = half4{(hf)w.x, (hf)w.y, (hf)w.z, (hf)w.w};
 	} else {
 		for (uint32_t i = i0; i < n; ++i) {
 			float w = master[i], a = m1[i], b = m2[i];
-			uint32_t t = steps[i];
+			uint32_t t = step_load(steps + i);
 			if (adam_one(i, n_matrix, loss_scale, inv_loss_scale, saturated, c, table, (float)grads[i], w, a, b, t)) {
-				master[i] = w; m1[i] = a; m2[i] = b; steps[i] = t; params[i] = (hf)w;
+				master[i] = w; m1[i] = a; m2[i] = b; step_store(steps + i, t); params[i] = (hf)w;
 			}
 		}
 	}
 }
 
+bool n2_adam_counters_may_saturate(float beta1, float beta2) {
+	const double small = std::ldexp(1.0, -26);
+	return std::pow((double)beta1, (double)ADAM_TABLE) < small && std::pow((double)beta2, (double)ADAM_TABLE) < small;
+}
+
 N2_API int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                         float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
                         float* d_m2, uint32_t* d_steps) {
-	return n2_adam_step_gated(stream, config, n_params, n_matrix_params, loss_scale, d_master, d_params, d_gradients, d_m1, d_m2, d_steps, nullptr);
+	return n2_adam_step_gated(stream, config, n_params, n_matrix_params, loss_scale, d_master, d_params, d_gradients, d_m1, d_m2, d_steps, 32, nullptr);
 }
 
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums, const N2StepEpilogue* epilogue, hipEvent_t done_event) {
+                       float* d_m2, void* d_steps, uint32_t steps_bits, const uint32_t* d_gate, const N2SlabReduce* sums, const N2StepEpilogue* epilogue,
+                       hipEvent_t done_event) {
 	N2_REQUIRE(config != nullptr, "n2_adam_step: config is null");
 	if (n_params == 0) return N2_OK;
 	N2_REQUIRE(d_master && d_params && d_gradients && d_m1 && d_m2 && d_steps, "n2_adam_step: null buffer");
@@ -198,8 +224,7 @@ int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_
 		slots[dev][slot].used = ++clock;
 	}
 	// 1 - beta^t == 1 in fp32 for every t past the table?
-	const double small = std::ldexp(1.0, -26);
-	const int saturated = (std::pow((double)config->beta1, (double)ADAM_TABLE) < small && std::pow((double)config->beta2, (double)ADAM_TABLE) < small) ? 1 : 0;
+	const int saturated = n2_adam_counters_may_saturate(config->beta1, config->beta2) ? 1 : 0;
 	int exp2 = 0;
 	const float inv_loss_scale = (std::frexp(loss_scale, &exp2) == 0.5f && exp2 > -120 && exp2 < 120) ? 1.f / loss_scale : 0.f;
 	N2ProfScope prof(N2_PROF_ADAM, s);
@@ -219,16 +244,23 @@ int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_
 		           "n2_adam_step: incomplete step epilogue");
 	}
 	const dim3 grid((quads + 255) / 256 + plan.units + (epi.values ? 1u : 0u));
-	if (done_event != nullptr) {
-		// the event is tied to this launch's own completion: no packet of its own behind the kernel, where an event record costs
-		// the stream about 5 us before its next kernel starts
-		hipExtLaunchKernelGGL(adam_step_kernel, grid, dim3(256), 0, s, nullptr, done_event, 0, *config, n_params, n_matrix_params, loss_scale, inv_loss_scale,
-		                      saturated, slot, d_gate, d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps,
-		                      plan, epi);
-	} else {
-		adam_step_kernel<<<grid, dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate, d_master,
-			reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, d_steps, plan, epi);
-	}
+	N2_REQUIRE(steps_bits == 32 || steps_bits == 16, "n2_adam_step: step counters of %u bits", steps_bits);
+	N2_REQUIRE(steps_bits == 32 || saturated, "n2_adam_step: 16-bit step counters need betas whose powers underflow within %u steps", ADAM_TABLE);
+	auto launch = [&](auto* steps) {
+		using StepT = std::remove_pointer_t<decltype(steps)>;
+		if (done_event != nullptr) {
+			// the event is tied to this launch's own completion: no packet of its own behind the kernel, where an event record
+			// costs the stream about 5 us before its next kernel starts
+			hipExtLaunchKernelGGL(adam_step_kernel<StepT>, grid, dim3(256), 0, s, nullptr, done_event, 0, *config, n_params, n_matrix_params, loss_scale,
+			                      inv_loss_scale, saturated, slot, d_gate, d_master, reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients),
+			                      d_m1, d_m2, steps, plan, epi);
+		} else {
+			adam_step_kernel<StepT><<<grid, dim3(256), 0, s>>>(*config, n_params, n_matrix_params, loss_scale, inv_loss_scale, saturated, slot, d_gate, d_master,
+				reinterpret_cast<hf*>(d_params), reinterpret_cast<const hf*>(d_gradients), d_m1, d_m2, steps, plan, epi);
+		}
+	};
+	if (steps_bits == 16) launch(static_cast<uint16_t*>(d_steps));
+	else launch(static_cast<uint32_t*>(d_steps));
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

@@ -151,12 +151,16 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 // n2_adam_step that does nothing when *d_gate is zero on the device (d_gate null: always steps)
 // sums (or null): a slab summation whose gradients lie inside d_gradients; the kernel's first workgroups run it, store the
 // fp16 gradients and step those parameters themselves (the other workgroups leave them alone)
+// d_steps: uint32_t (steps_bits 32) or uint16_t counters (16)
 // epilogue (or null): one more workgroup of the launch does the caller's bookkeeping (slab_reduce.h), gated or not
 // done_event (or null): recorded by the completion of the launch itself (hipExtLaunchKernel's stop event)
 int n2_adam_step_gated(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                        float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
-                       float* d_m2, uint32_t* d_steps, const uint32_t* d_gate, const N2SlabReduce* sums = nullptr,
+                       float* d_m2, void* d_steps, uint32_t steps_bits, const uint32_t* d_gate, const N2SlabReduce* sums = nullptr,
                        const N2StepEpilogue* epilogue = nullptr, hipEvent_t done_event = nullptr);
+// true when 1 - beta^t is exactly 1 in fp32 for both betas from the end of the kernel's bias-correction table on: the step
+// counters may then be 16 bits wide (steps_bits 16, saturating at 65535) instead of 32
+bool n2_adam_counters_may_saturate(float beta1, float beta2);
 // n2_mlp_reduce_deferred that also adds up n_parts floats, in a fixed order, into one fp16 value ([+=] when accumulate)
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
 // The same work as a plan instead of a launch: what is pending is handed to *out (and no longer pending), for

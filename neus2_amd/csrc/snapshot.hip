@@ -240,7 +240,19 @@ N2_API int n2_snapshot_save(const char* path, const n2_snapshot_desc* d, n2_stre
 		w.str("second_moments_binary");
 		if (int rc = append_device_bin(w, d->d_second_moments, 4ull * d->n_params)) return rc;
 		w.str("param_steps_binary");
-		if (int rc = append_device_bin(w, d->d_param_steps, 4ull * d->n_params)) return rc;
+		N2_REQUIRE(d->param_steps_bits == 0 || d->param_steps_bits == 16 || d->param_steps_bits == 32, "n2_snapshot_save: step counters of %u bits", d->param_steps_bits);
+		if (d->param_steps_bits == 16) {
+			// the file holds 32-bit counters
+			std::vector<uint16_t> narrow(d->n_params);
+			N2_HIP(hipMemcpy(narrow.data(), d->d_param_steps, 2ull * d->n_params, hipMemcpyDeviceToHost));
+			w.bin_header(4ull * d->n_params);
+			const size_t at = w.buf.size();
+			w.buf.resize(at + 4ull * d->n_params);
+			for (uint32_t i = 0; i < d->n_params; ++i) {
+				const uint32_t v = narrow[i];
+				std::memcpy(w.buf.data() + at + 4ull * i, &v, 4);
+			}
+		} else if (int rc = append_device_bin(w, d->d_param_steps, 4ull * d->n_params)) return rc;
 	}
 	w.str("density_grid_size"); w.uint(128);
 	w.str("density_grid_binary");
@@ -388,6 +400,7 @@ N2_API int n2_snapshot_read(n2_snapshot_t* sn, n2_stream_t stream, const n2_snap
 	N2_REQUIRE(sn != nullptr && t != nullptr, "n2_snapshot_read: null argument");
 	hipStream_t s = n2_stream(stream);
 	const uint64_t n = sn->info.n_params;
+	std::vector<uint16_t> narrow_steps;  // lives until the stream has been waited for
 	if (t->d_master || t->d_params) {
 		N2_REQUIRE(t->n_params == n, "n2_snapshot_read: the snapshot holds %llu parameters, the model has %u", (unsigned long long)n, t->n_params);
 		N2_REQUIRE(t->d_scratch != nullptr && t->scratch_bytes >= sn->params.bytes, "n2_snapshot_read: the parameters need %llu bytes of device scratch",
@@ -422,7 +435,18 @@ N2_API int n2_snapshot_read(n2_snapshot_t* sn, n2_stream_t stream, const n2_snap
 		N2_REQUIRE(t->n_params == n, "n2_snapshot_read: the snapshot holds %llu parameters, the model has %u", (unsigned long long)n, t->n_params);
 		if (t->d_first_moments) N2_HIP(hipMemcpyAsync(t->d_first_moments, sn->m1.data, 4 * n, hipMemcpyHostToDevice, s));
 		if (t->d_second_moments) N2_HIP(hipMemcpyAsync(t->d_second_moments, sn->m2.data, 4 * n, hipMemcpyHostToDevice, s));
-		if (t->d_param_steps) N2_HIP(hipMemcpyAsync(t->d_param_steps, sn->steps.data, 4 * n, hipMemcpyHostToDevice, s));
+		N2_REQUIRE(t->param_steps_bits == 0 || t->param_steps_bits == 16 || t->param_steps_bits == 32, "n2_snapshot_read: step counters of %u bits", t->param_steps_bits);
+		if (t->d_param_steps && t->param_steps_bits == 16) {
+			narrow_steps.resize(n);
+			for (uint64_t i = 0; i < n; ++i) {
+				uint32_t v;
+				std::memcpy(&v, sn->steps.data + 4 * i, 4);
+				narrow_steps[i] = (uint16_t)(v < 65535u ? v : 65535u);
+			}
+			N2_HIP(hipMemcpyAsync(t->d_param_steps, narrow_steps.data(), 2 * n, hipMemcpyHostToDevice, s));
+		} else if (t->d_param_steps) {
+			N2_HIP(hipMemcpyAsync(t->d_param_steps, sn->steps.data, 4 * n, hipMemcpyHostToDevice, s));
+		}
 	}
 	if (t->d_ema_weights) {
 		N2_REQUIRE(sn->info.has_ema_weights, "n2_snapshot_read: the snapshot holds no Ema weights");

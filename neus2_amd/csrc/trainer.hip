@@ -25,7 +25,8 @@ struct n2_trainer {
 	hf* grads;
 	float* m1;
 	float* m2;
-	uint32_t* steps;
+	void* steps;              // per-parameter step counters, steps_bits wide
+	uint32_t steps_bits;
 	float* ema_tmp;   // fp32 moving average of the fp16 weights (null without the Ema wrapper)
 	hf* ema;          // its fp16 copy: the inference parameters
 	uint32_t optimizer_steps;  // nested optimizer steps taken so far
@@ -83,7 +84,7 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	c.grads = take(2 * np);
 	c.m1 = take(4 * np);
 	c.m2 = take(4 * np);
-	c.steps = take(4 * np);
+	c.steps = take((n2_adam_counters_may_saturate(cfg->adam.beta1, cfg->adam.beta2) ? 2 : 4) * np);
 	const bool ema = cfg->ema_decay > 0.f;
 	c.ema_tmp = take(ema ? 4 * np : 0);
 	c.ema = take(ema ? 2 * np : 0);
@@ -162,7 +163,8 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->grads = reinterpret_cast<hf*>(b + c.grads);
 	t->m1 = reinterpret_cast<float*>(b + c.m1);
 	t->m2 = reinterpret_cast<float*>(b + c.m2);
-	t->steps = reinterpret_cast<uint32_t*>(b + c.steps);
+	t->steps = b + c.steps;
+	t->steps_bits = n2_adam_counters_may_saturate(cfg->adam.beta1, cfg->adam.beta2) ? 16u : 32u;
 	t->ema_tmp = cfg->ema_decay > 0.f ? reinterpret_cast<float*>(b + c.ema_tmp) : nullptr;
 	t->ema = cfg->ema_decay > 0.f ? reinterpret_cast<hf*>(b + c.ema) : nullptr;
 	t->optimizer_steps = 0;
@@ -339,7 +341,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	epi.values = t->ray_loss; epi.n_ptr = ray_counter; epi.n_max = n_rays; epi.sum_out = reinterpret_cast<float*>(t->counters) + 4;
 	epi.copy_src = set.counters; epi.copy_dst = t->counters; epi.copy_n = 2;
 	if (int rc = n2_adam_step_gated(stream, &t->cfg.adam, t->n_params, t->n_matrix_params, t->cfg.loss_scale, t->master, reinterpret_cast<n2_half*>(t->params),
-	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, compacted_counter, &sums, &epi,
+	                                reinterpret_cast<const n2_half*>(t->grads), t->m1, t->m2, t->steps, t->steps_bits, compacted_counter, &sums, &epi,
 	                                t->side ? t->ev_main : nullptr)) return rc;
 	t->ev_main_from_adam = t->side != nullptr;
 	t->optimizer_steps += 1;
@@ -364,6 +366,7 @@ N2_API int n2_trainer_optimizer_state(n2_trainer_t* t, n2_trainer_optimizer_buff
 	out->first_moments = t->m1;
 	out->second_moments = t->m2;
 	out->param_steps = t->steps;
+	out->param_steps_bits = t->steps_bits;
 	out->ema_weights = t->ema_tmp;
 	out->inference_params = reinterpret_cast<n2_half*>(t->ema ? t->ema : t->params);
 	out->optimizer_steps = t->optimizer_steps;

@@ -18,7 +18,7 @@ class SnapshotDesc(C.Structure):
                 ("learning_rate", C.c_float), ("d_density_grid", C.c_void_p), ("density_grid_cells", C.c_uint64),
                 ("d_scratch", C.c_void_p), ("scratch_bytes", C.c_uint64), ("aabb_scale", C.c_uint32), ("rays_per_batch", C.c_uint32),
                 ("measured_batch_size", C.c_uint32), ("measured_batch_size_before_compaction", C.c_uint32),
-                ("training_step", C.c_uint32), ("loss", C.c_float)]
+                ("training_step", C.c_uint32), ("loss", C.c_float), ("param_steps_bits", C.c_uint32)]
 
 
 class SnapshotInfo(C.Structure):
@@ -34,7 +34,8 @@ class SnapshotTargets(C.Structure):
     """struct n2_snapshot_targets"""
     _fields_ = [("n_params", C.c_uint32), ("d_master", C.c_void_p), ("d_params", C.c_void_p), ("d_density_grid", C.c_void_p),
                 ("density_grid_cells", C.c_uint64), ("d_first_moments", C.c_void_p), ("d_second_moments", C.c_void_p),
-                ("d_param_steps", C.c_void_p), ("d_ema_weights", C.c_void_p), ("d_scratch", C.c_void_p), ("scratch_bytes", C.c_uint64)]
+                ("d_param_steps", C.c_void_p), ("d_ema_weights", C.c_void_p), ("d_scratch", C.c_void_p), ("scratch_bytes", C.c_uint64),
+                ("param_steps_bits", C.c_uint32)]
 
 
 def pack_config(obj):
@@ -143,6 +144,7 @@ def save_snapshot(path, trainer, occupancy=None, config=None, include_optimizer_
     d.include_optimizer_state = 1 if include_optimizer_state else 0
     if include_optimizer_state:
         d.d_first_moments, d.d_second_moments, d.d_param_steps = st.first_moments, st.second_moments, st.param_steps
+        d.param_steps_bits = st.param_steps_bits
         d.d_ema_weights = st.ema_weights
     d.optimizer_steps, d.learning_rate = st.optimizer_steps, st.learning_rate
     scratch = None
@@ -185,6 +187,7 @@ def load_snapshot(path, trainer, occupancy=None, load_optimizer_state=True):
         with_opt = bool(load_optimizer_state and info.has_optimizer_state)
         if with_opt:
             t.d_first_moments, t.d_second_moments, t.d_param_steps = st.first_moments, st.second_moments, st.param_steps
+            t.param_steps_bits = st.param_steps_bits
             if info.has_ema_weights and st.ema_weights:
                 t.d_ema_weights = st.ema_weights
         scratch = torch.empty(need, dtype=torch.uint8, device=trainer.master.device)

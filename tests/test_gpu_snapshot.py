@@ -58,8 +58,10 @@ def test_file_contents_and_exact_resume(tmp_path):
     st = tr.optimizer_state()
     assert adam["current_step"] == 3 and abs(adam["base_learning_rate"] - 1e-3) < 1e-9
     np.testing.assert_array_equal(np.frombuffer(adam["first_moments_binary"], np.float32), tr._view(st.first_moments, tr.n_params, torch.float32).cpu().numpy())
+    # the trainer keeps 16-bit counters for the default betas; the file holds the reference's 32-bit form
+    assert st.param_steps_bits == 16
     np.testing.assert_array_equal(np.frombuffer(adam["param_steps_binary"], np.uint32),
-                                  tr._view(st.param_steps, tr.n_params, torch.int32).cpu().numpy().view(np.uint32))
+                                  tr._view(st.param_steps, tr.n_params, torch.int16).cpu().numpy().view(np.uint16).astype(np.uint32))
     np.testing.assert_array_equal(np.frombuffer(snap["optimizer"]["ema_weights_binary"], np.float32), tr.ema_weights.cpu().numpy())
     info = snapshot_info(path)
     assert info.n_params == tr.n_params and info.training_step == 3 and info.has_optimizer_state and info.has_ema_weights
@@ -117,6 +119,42 @@ def test_loads_files_of_another_writer_and_checks_shapes(tmp_path):
     p.write_bytes(msgpack.packb(doc, use_bin_type=True))
     with pytest.raises(capi.N2Error, match="cascades"):
         load_snapshot(p, tr, tr.occupancy)
+
+
+def test_step_counters_of_a_long_run_load_into_the_narrow_counters(tmp_path):
+    """The trainer keeps 16-bit per-parameter step counters for the default betas (past 4096 steps the bias correction is
+    exactly 1, so the count no longer matters); a file of another writer holds 32-bit counts, some beyond 65535: they load
+    as min(count, 65535), a step goes on from there, and the file written afterwards holds the 32-bit form again."""
+    from neus2_amd.snapshot import load_snapshot, save_snapshot
+    tr = make_trainer(ema=0.0)
+    n = tr.n_params
+    rng = np.random.default_rng(3)
+    steps = rng.integers(0, 200000, n).astype(np.uint32)
+    steps[:4] = (0, 65534, 65535, 70000)
+    doc = reference_style_file(with_optimizer=True)
+    adam = doc["snapshot"]["optimizer"]["nested"]["nested"]
+    adam.update(first_moments_binary=np.zeros(n, np.float32).tobytes(), second_moments_binary=np.ones(n, np.float32).tobytes(),
+                param_steps_binary=steps.tobytes())
+    del doc["snapshot"]["optimizer"]["ema_weights_binary"]
+    doc["snapshot"].update(n_params=n, params_type="__half", params_binary=host(tr.params).astype(np.float16).tobytes(),
+                           density_grid_binary=np.full(CELLS, 1.0, np.float16).tobytes())
+    p = tmp_path / "long_run.msgpack"
+    p.write_bytes(msgpack.packb(doc, use_bin_type=True))
+    info = load_snapshot(p, tr, tr.occupancy)
+    assert info.has_optimizer_state
+    st = tr.optimizer_state()
+    assert st.param_steps_bits == 16
+    got = tr._view(st.param_steps, n, torch.int16).cpu().numpy().view(np.uint16)
+    np.testing.assert_array_equal(got, np.minimum(steps, 65535).astype(np.uint16))
+    tr.step(n_rays=256, n_inference=1 << 17)
+    after = tr._view(st.param_steps, n, torch.int16).cpu().numpy().view(np.uint16).astype(np.uint32)
+    assert ((after == np.minimum(steps, 65535)) | (after == np.minimum(steps + 1, 65535))).all()
+    assert (after != np.minimum(steps, 65535)).any()
+    assert np.isfinite(host(tr.master)).all()
+    out = tmp_path / "after.msgpack"
+    save_snapshot(out, tr, tr.occupancy, config=CONFIG, include_optimizer_state=True)
+    saved = msgpack.unpackb(out.read_bytes(), raw=False, strict_map_key=False)["snapshot"]["optimizer"]["nested"]  # no Ema level
+    np.testing.assert_array_equal(np.frombuffer(saved["param_steps_binary"], np.uint32), after)
 
 
 def test_params_only_resume_restores_level_mask_and_restarts_ema(tmp_path):

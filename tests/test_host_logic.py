@@ -57,7 +57,7 @@ def test_trainer_config_struct_matches_header():
     assert ctypes.sizeof(capi.FieldConfig) == 32 and ctypes.sizeof(capi.AdamConfig) == 20
     assert ctypes.sizeof(capi.CompositeConfig) == 28 and ctypes.sizeof(capi.Camera) == 80
     assert ctypes.sizeof(capi.TrainerConfig) == 32 + 20 + 28 + 28
-    assert ctypes.sizeof(capi.OccupancyBuffers) == 6 * 8 + 3 * 4 + 4 + 2 * 8 and ctypes.sizeof(capi.TrainerOptimizerBuffers) == 5 * 8 + 8
+    assert ctypes.sizeof(capi.OccupancyBuffers) == 6 * 8 + 3 * 4 + 4 + 2 * 8 and ctypes.sizeof(capi.TrainerOptimizerBuffers) == 5 * 8 + 16
     L = capi.lib()
     cfg = capi.TrainerConfig()
     assert L.n2_trainer_workspace_bytes(ctypes.byref(cfg)) == 0  # all-zero config is rejected on the host
