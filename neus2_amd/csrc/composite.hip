@@ -315,6 +315,14 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 			hi[0] = (hf)(dnorm * dir[0]); hi[1] = (hf)(dnorm * dir[1]); hi[2] = (hf)(dnorm * dir[2]);
 #pragma unroll
 			for (int k = 3; k < 8; ++k) hi[k] = (hf)0;
+			// The rows are pinned in registers here: the copies that fill the batch up are formed from these fp16 values, and a
+			// second evaluation of the expressions above (which the compiler is free to contract differently) rounds to
+			// another fp16 value in a few cases per million.
+			{
+				uint4 lb = __builtin_bit_cast(uint4, lo), hb = __builtin_bit_cast(uint4, hi);
+				asm volatile("" : "+v"(lb.x), "+v"(lb.y), "+v"(lb.z), "+v"(lb.w), "+v"(hb.x), "+v"(hb.y), "+v"(hb.z), "+v"(hb.w));
+				lo = __builtin_bit_cast(half8, lb); hi = __builtin_bit_cast(half8, hb);
+			}
 			hf* g = dloss + ((size_t)cb + s) * 16;
 			*reinterpret_cast<half8*>(g) = lo;
 			*reinterpret_cast<half8*>(g + 8) = hi;

@@ -50,3 +50,30 @@ def test_two_steps_at_the_benchmark_shape(oracle, loss_scale):
         results.append(res)
         assert res["samples"] <= n_inf and 0.8 * T < res["compacted"] <= n_inf, res
     assert results[0]["samples"] != results[1]["samples"]   # two different sets of rays
+
+
+def test_many_rays_whose_batch_is_filled_up(oracle):
+    """From 8192 rays on, the compositor places the rays in the batch with the prefix sums of a scan kernel instead of sums
+    inside its backward kernel; here such a step keeps fewer samples than the batch holds, so the batch is also filled up by
+    roll-over with those offsets.  Every stage against the oracle, as above."""
+    import bench
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    from oracle.field import Field
+    from oracle.step import verify_step
+    T = 1 << 19
+    cams, rgba, bits = bench.build_scene()
+    cfg = default_config(target_batch_size=T, max_rays_per_batch=1 << 14, max_samples=T, prefetch_samples=True)
+    cfg.loss_scale = 8192.0
+    tr = Trainer(cfg)
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), dev(bits))
+    tr.initialize_params(seed=1338, sdf_mlp_weights=None)
+    n_rays, seed, n_inf = 8500, 7, T
+    params16 = host(tr.params).copy()
+    tr.step(n_rays=n_rays, n_inference=n_inf, seed=seed)
+    c = tr.read_counters()
+    assert n_rays >= 8192 and c["rays"] > 0 and 0 < c["compacted"] < T, c  # the scan kernel goes by the rays asked for
+    gpu = {k: host(v) for k, v in tr.last_step(c["rays"], c["samples"], n_inf).items()}
+    res = verify_step(Field(fp16=True), params16, oc_cams(oracle, cams), rgba, bits, n_rays, 0, seed, n_inf, T, c, gpu, host(tr.grads),
+                      background=(1.0, 1.0, 1.0), loss_scale=8192.0, rtol=RTOL)
+    assert res["compacted"] == c["compacted"]
