@@ -460,7 +460,7 @@ constexpr uint32_t PAIR_MAX_CELL = BKT_ENTRIES - 2u;  // pair records (grid_bin_
 static_assert(BKT_SHIFT <= 12, "a pair record's 16-bit key holds the entry within the bucket and four bits of carry length");
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
 constexpr uint32_t BIN_RECORDS = BIN_POINTS * 8;
-constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: two workgroups (2 x 64 KiB staging) keep 4 waves on every SIMD
+constexpr uint32_t BIN_BLOCK = 512;       // 8 waves: three workgroups (3 x 49 KiB of LDS) keep 6 waves on every SIMD, at 80 registers (with 96 or 128: pair +10 us)
 constexpr uint32_t BIN_PER_THREAD = BIN_POINTS / BIN_BLOCK;  // 2
 
 struct N2BucketPlan {
