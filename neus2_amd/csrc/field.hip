@@ -307,6 +307,10 @@ N2_API int n2_field_set_fused(n2_field_t* field, int enable) {
 	field->fused = enable != 0;
 	return N2_OK;
 }
+N2_API int n2_field_set_colour_gradient_exponent(n2_field_t* field, int exponent) {
+	N2_REQUIRE(field != nullptr, "n2_field_set_colour_gradient_exponent: field is null");
+	return n2_mlp_set_output_gradient_exponent(field->rgb, exponent);
+}
 N2_API uint32_t n2_field_n_params(const n2_field_t* f) { return f ? f->n_params : 0; }
 
 N2_API int n2_field_param_offsets(const n2_field_t* f, uint32_t offsets[5]) {
@@ -678,6 +682,16 @@ N2_API int n2_sdf_eikonal_loss(n2_stream_t stream, uint32_t n, uint32_t encoding
 	return N2_OK;
 }
 
+// The inference paths for points in no particular order gather the features into the rows of the SDF net's input, at the
+// pitch of THEIR batch: whatever the training forward left there is gone, and with another batch size the rows land on what
+// the training layout keeps as zero padding (rows 3 + enc_w .. sdf_in_w, which the weight-gradient kernels read against
+// non-zero weight columns).  So the padding counts as not cleared, and a backward pass has to follow a new forward.
+static void inference_takes_sdf_in(n2_field_t* f) {
+	f->pad_n.sdf_in = 0;
+	f->last_n = 0;
+	f->sel_n = 0;
+}
+
 static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, const float* d_xyz, uint32_t ps, uint32_t ds, uint32_t n,
                           n2_half* d_output, bool density) {
 	if (int rc = check_field(f, fn, n)) return rc;
@@ -688,10 +702,14 @@ static int field_sdf_impl(n2_field_t* f, const char* fn, n2_stream_t stream, con
 	hipStream_t s = n2_stream(stream);
 	if (f->fused && fused_ok(f)) {
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+		const bool scratch = !n2_grid_lattice_order(f->grid);
+		if (scratch) inference_takes_sdf_in(f);
 		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, d_output, nullptr, density,
-		                          n2_grid_lattice_order(f->grid) ? nullptr : reinterpret_cast<n2_half*>(f->sdf_in));
+		                          scratch ? reinterpret_cast<n2_half*>(f->sdf_in) : nullptr);
 	}
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
+	f->last_n = 0;  // the rows below are overwritten: a backward pass needs a new n2_field_forward
+	f->sel_n = 0;
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_xyz, ps, ds, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();
 	if (int rc = n2_grid_forward(f->grid, stream, f->xyz, 1, n, n, reinterpret_cast<n2_half*>(f->sdf_in + (size_t)3 * n), nullptr)) return rc;
@@ -722,8 +740,10 @@ int n2_field_sdf_row0(n2_field_t* f, n2_stream_t stream, const float* d_xyz, uin
 	hipStream_t s = n2_stream(stream);
 	if (f->fused && fused_ok(f)) {
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+		const bool scratch = !n2_grid_lattice_order(f->grid);
+		if (scratch) inference_takes_sdf_in(f);
 		return n2_fused_field_sdf(fused_nets(f), s, d_xyz, ps, ds, n, nullptr, d_row0, density,
-		                          n2_grid_lattice_order(f->grid) ? nullptr : reinterpret_cast<n2_half*>(f->sdf_in), n_keep);
+		                          scratch ? reinterpret_cast<n2_half*>(f->sdf_in) : nullptr, n_keep);
 	}
 	if (int rc = field_sdf_impl(f, "n2_field_sdf", stream, d_xyz, ps, ds, n, d_scratch16, density)) return rc;
 	const uint32_t keep = n_keep < n ? n_keep : n;

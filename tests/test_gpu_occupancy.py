@@ -148,3 +148,34 @@ def test_training_with_live_occupancy_grid(trainer):
     assert results[0][0] == results[1][0]
     np.testing.assert_array_equal(results[0][1], results[1][1])
     np.testing.assert_array_equal(results[0][2], results[1][2])
+
+
+def test_a_step_after_an_update_with_larger_chunks_matches_the_oracle(oracle):
+    """The occupancy update evaluates the field in chunks that are larger than the training step's inference batch; its
+    gather uses the SDF net's input rows as scratch at the chunk's pitch, which falls on the rows the training layout
+    keeps as zero padding.  A step behind such an update (same inference batch as the step before it) is checked stage by
+    stage: the weight-gradient kernels read the padding rows against non-zero weight columns."""
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import OccupancyGrid, Trainer, default_config
+    from oracle.field import Field
+    from oracle.step import verify_step
+    from test_oracle_sampler import oc_cams
+    cams = scene.cameras_on_sphere(8, 96)
+    rgba = scene.render_sphere_images(cams)
+    bits = scene.sphere_bitfield()
+    T, n_inf, chunk = 4096, 1 << 15, 1 << 18
+    tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=2048, max_samples=chunk, background=(1.0, 1.0, 1.0)))
+    tr.set_scene(pack_cameras(cams), len(cams), dev(rgba), dev(bits))
+    tr.initialize_params(seed=9, sdf_mlp_weights=None)   # Xavier: the padding columns of W_0 are not zero
+    occ = OccupancyGrid(1, seed=21, max_chunk=chunk)
+    n_rays = 300
+    tr.step(n_rays=n_rays, n_inference=n_inf, seed=1)
+    assert n_inf < chunk < 16 * n_inf
+    occ.update(tr._field, 2 * chunk, 0)
+    params16 = host(tr.params).copy()
+    tr.step(n_rays=n_rays, n_inference=n_inf, seed=2)
+    c = tr.read_counters()
+    gpu = {k: host(v) for k, v in tr.last_step(c["rays"], c["samples"], n_inf).items()}
+    res = verify_step(Field(fp16=True), params16, oc_cams(oracle, cams), rgba, bits, n_rays, n_rays, 2, n_inf, T, c, gpu, host(tr.grads),
+                      background=(1.0, 1.0, 1.0))
+    assert res["compacted"] > T // 2, res
