@@ -252,6 +252,20 @@ int n2_mlp_forward_and_input_gradient(n2_mlp_t* mlp, n2_stream_t stream, uint32_
  * follow) and n2_mlp_reduce_deferred folds everything pending for up to two networks in one launch.  Off by default;
  * no counterpart in the reference, which uses GEMMs for the weight gradients. */
 int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable);
+
+/* Numerical head-room of n2_mlp_backward / n2_mlp_backward_rows with weight gradients.  The fully fused network rounds the
+ * gradients of its hidden layers to fp16 for the matrix cores (as tcnn's FullyFusedMLP does); with the reference's loss scale
+ * (LOSS_SCALE = 128, testbed.h:237, divided by the ray count, src/testbed_nerf.cu:1756) the colour rows of dL/doutput lie in
+ * fp16's SUBNORMAL range and that rounding costs 1-2 % per value.  With exponent k the kernel multiplies dL/doutput by 2^k as
+ * it loads it (exact), runs the chain on the larger values and multiplies dL/dinput and the weight gradients by 2^-k in
+ * fp32 before it stores them: the same results as k = 0 wherever k = 0 loses nothing, and no subnormal intermediate.
+ * k in [-14, 14], default 0; the caller must keep |dL/doutput| * 2^k well inside fp16's range.  Ignored by the passes with
+ * a second-order part.  No counterpart in the reference. */
+int n2_mlp_set_output_gradient_exponent(n2_mlp_t* mlp, int exponent);
+/* The exponent the trainer uses for the colour net: the largest k with loss_scale / n_rays * 2^k <= 16 (clamped to
+ * [0, 14]).  The colour rows of the compositor's dL/doutput are bounded by 0.05 * loss_scale / n_rays (weight <= 1, Huber
+ * slope / 5 <= 0.2, sigmoid' <= 0.25; src/testbed_nerf.cu:1700-1760), i.e. by 0.8 after the scaling. */
+int n2_colour_gradient_exponent(float loss_scale, uint32_t n_rays);
 int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b /* may be NULL */, n2_stream_t stream);
 
 /* Network::backward_backward_input(stream, ctx, input, dL_ddLdinput, dL_doutput,
@@ -321,6 +335,9 @@ int n2_field_param_offsets(const n2_field_t* field, uint32_t offsets[5]);
  * colour net, no per-point level mask.  Off, or for other configurations: the same results from separate grid, network
  * and element-wise kernels (values agree within fp32 summation order). */
 int n2_field_set_fused(n2_field_t* field, int enable);
+/* n2_mlp_set_output_gradient_exponent for the field's colour net (rows 0..2 of n2_field_backward's dL/doutput); the
+ * trainer sets n2_colour_gradient_exponent(loss_scale, n_rays) before every step.  Default 0. */
+int n2_field_set_colour_gradient_exponent(n2_field_t* field, int exponent);
 
 /* NerfNetwork::set_params, nerf_network.h:728-772 (fp16 params and gradients, n_params each). */
 int n2_field_set_params(n2_field_t* field, const n2_half* d_params, n2_half* d_gradients);

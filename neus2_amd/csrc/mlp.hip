@@ -41,6 +41,7 @@ struct n2_mlp {
 	bool deferred;
 	uint32_t pending_slabs;       // slabs written since the last reduction
 	n2_grad_mode pending_mode;    // mode of the first of the pending calls (later ones must accumulate)
+	int dy_exponent;              // n2_mlp_set_output_gradient_exponent
 };
 
 // ----------------------------------------------------------------------------
@@ -531,6 +532,21 @@ N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 	return N2_OK;
 }
 
+N2_API int n2_mlp_set_output_gradient_exponent(n2_mlp_t* mlp, int exponent) {
+	N2_REQUIRE(mlp != nullptr, "n2_mlp_set_output_gradient_exponent: mlp is null");
+	N2_REQUIRE(exponent >= -14 && exponent <= 14, "n2_mlp_set_output_gradient_exponent: exponent %d outside [-14, 14]", exponent);
+	mlp->dy_exponent = exponent;
+	return N2_OK;
+}
+
+N2_API int n2_colour_gradient_exponent(float loss_scale, uint32_t n_rays) {
+	if (!(loss_scale > 0.f) || n_rays == 0) return 0;
+	int k = 0;
+	// largest k with loss_scale / n_rays * 2^k <= 16
+	while (k < 14 && ldexpf(loss_scale / (float)n_rays, k + 1) <= 16.f) ++k;
+	return k;
+}
+
 N2_API int n2_mlp_reduce_deferred(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream) { return n2_mlp_reduce_deferred_sum(a, b, stream, nullptr, 0, nullptr, 0); }
 
 int n2_mlp_reduce_deferred_plan(n2_mlp_t* a, n2_mlp_t* b, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate, N2SlabReduce* out) {
@@ -597,6 +613,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 	const hf* dY = reinterpret_cast<const hf*>(d_dL_doutput);
 	hf* dX = reinterpret_cast<hf*>(d_dL_dinput);
 	const int aos = (dL_layout == N2_LAYOUT_AOS ? 1 : 0) | ((int)dy_rows << 8);  // layout flag and the number of rows in use
+	const float dy_gain = ldexpf(1.f, mlp->dy_exponent), dy_gain_inv = ldexpf(1.f, -mlp->dy_exponent);
 	N2ProfScope prof(N2_PROF_MLP_BACKWARD, s);
 #define LAUNCH(IC, NH)                                                                                              \
 	do {                                                                                                            \
@@ -609,7 +626,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 		const size_t lds = mlp_wgrad_lds<IC, NH, false>();                                                          \
 		if (int rc = allow_lds(mlp_wgrad_kernel<IC, NH, DX, false>, lds)) return rc;                                \
 		mlp_wgrad_kernel<IC, NH, DX, false><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1, (int)dy_rows, dX, \
-			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols);                                                  \
+			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv);                            \
 	} while (0)
 	// the field's colour net (48 inputs, two hidden layers): only the rows the field reads are stored
 	N2_REQUIRE(tail == nullptr || (want_dx && want_dw && dx_out_and_normal_only && mlp->in_w == 48 && mlp->n_hidden == 2 && (aos & 1) && dy_rows <= 8),
@@ -620,7 +637,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 			const size_t lds = mlp_wgrad_lds<3, 2, false>();
 			if (int rc = allow_lds(mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail>, lds)) return rc;
 			mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1,
-				(int)dy_rows, dX, next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, t);
+				(int)dy_rows, dX, next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv, t);
 		} else {
 			LAUNCH_W(3, 2, WG_DX_OUT_AND_NORMAL);
 		}
@@ -730,7 +747,7 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 		mlp_wgrad_kernel<3, 1, WG_DX_ENCODING, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),
-			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f);
 		N2_LAUNCH_CHECK();
 		return reduce_partials(mlp, s, blocks, mode);
 	}
@@ -742,7 +759,7 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 		mlp_wgrad_kernel<IC, 1, WG_DX_ALL, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,                   \
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,              \
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),              \
-			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols);                                 \
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f);                       \
 		break;                                                                                                             \
 	}
 		CASE(1) CASE(2) CASE(3) CASE(4)

@@ -97,9 +97,16 @@ template <int IC, int NH, int WANT_DX, bool SECOND, class Tail = WgNoTail>
 __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __restrict__ W, const hf* __restrict__ X, uint32_t N, const hf* __restrict__ dY,
                                                                  int dy_aos, int dy_rows, hf* __restrict__ dX, float* __restrict__ partials,
                                                                  const hf* __restrict__ V, const hf* __restrict__ G2, int unit_row2,
-                                                                 const uint32_t* __restrict__ x_index, uint32_t x_cols, const Tail tail = Tail()) {
+                                                                 const uint32_t* __restrict__ x_index, uint32_t x_cols, float dy_gain, float dy_gain_inv,
+                                                                 const Tail tail = Tail()) {
 	static_assert(!SECOND || NH == 1, "the second-order pass needs one hidden layer");
 	static_assert(!Tail::active || (IC == 3 && NH == 2 && WANT_DX == WG_DX_OUT_AND_NORMAL), "the field's tail goes with the colour net");
+	// dy_gain = 2^k, dy_gain_inv = 2^-k (first-order launches only).  The output gradient is multiplied by 2^k when it is
+	// loaded and everything the launch hands on (dL/dinput, the weight-gradient slab) by 2^-k in fp32, so the chain between
+	// them, whose matrices are rounded to fp16 for the matrix cores, works on values 2^k larger: an output gradient in the
+	// subnormal range of fp16 (a loss scale of 128 over thousands of rays puts the colour rows there: steps of 6e-8 on values
+	// near 2e-6) then loses nothing, the products with a power of two being exact.  2^0 leaves every value as it is.
+	const float gain_inv = SECOND ? 1.f : dy_gain_inv;
 	using M = FragMap<IC, NH>;
 	constexpr int IN_W = 16 * IC, IN_MT = M::IN_MT;
 	constexpr int N_PARAMS = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH + MLP_OUT * MLP_WIDTH;
@@ -143,6 +150,11 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 #pragma unroll
 		for (int e = 0; e < 8; ++e)
 			if (!valid || 8 * g + e >= dy_rows) dy[e] = (hf)0;
+		if constexpr (!SECOND) {
+			const hf gain = (hf)dy_gain;
+#pragma unroll
+			for (int e = 0; e < 8; ++e) dy[e] = dy[e] * gain;
+		}
 		hidden_S<IC, NH>(F, lane, x, h);
 		half8 dh[NH][4];
 #pragma unroll
@@ -164,6 +176,8 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 				float16v d = zero16();
 #pragma unroll
 				for (int c = 0; c < 4; ++c) d = N2_MFMA(frag(F, M::W0T + t * 4 + c, lane), dh[0][c], d);
+#pragma unroll
+				for (int r = 0; r < 16; ++r) d[r] *= gain_inv;
 				if constexpr (Tail::active) {
 					// row 0 also takes the direct gradient of the SDF output (row 3 of dL/doutput); rows 35..37 are dL/dnormal
 					if (t == 0 && g == 0) d[0] = (float)((hf)d[0] + dy_all[3]);
@@ -323,23 +337,23 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 	if (nt < IN_MT) {
 #pragma unroll
 		for (int r = 0; r < 16; ++r)
-			if (32 * nt + n < IN_W) Wl[(32 * mt + drow(r, g)) * IN_W + 32 * nt + n] = gW0[r];
+			if (32 * nt + n < IN_W) Wl[(32 * mt + drow(r, g)) * IN_W + 32 * nt + n] = gW0[r] * gain_inv;
 	}
 	if (NH > 1) {
 #pragma unroll
-		for (int r = 0; r < 16; ++r) Wl[MLP_WIDTH * IN_W + (32 * mt + drow(r, g)) * MLP_WIDTH + 32 * nt + n] = gWh[r];
+		for (int r = 0; r < 16; ++r) Wl[MLP_WIDTH * IN_W + (32 * mt + drow(r, g)) * MLP_WIDTH + 32 * nt + n] = gWh[r] * gain_inv;
 	}
 	constexpr int OFF_O = MLP_WIDTH * IN_W + (NH - 1) * MLP_WIDTH * MLP_WIDTH;
 	if (mt == 0) {
 #pragma unroll
 		for (int r = 0; r < 16; ++r)
-			if (drow(r, g) < MLP_OUT) Wl[OFF_O + drow(r, g) * MLP_WIDTH + 32 * nt + n] = gWo[r];
+			if (drow(r, g) < MLP_OUT) Wl[OFF_O + drow(r, g) * MLP_WIDTH + 32 * nt + n] = gWo[r] * gain_inv;
 	}
 	__syncthreads();
 	if (mt == 1) {
 #pragma unroll
 		for (int r = 0; r < 16; ++r)
-			if (drow(r, g) < MLP_OUT) Wl[OFF_O + drow(r, g) * MLP_WIDTH + 32 * nt + n] += gWo[r];
+			if (drow(r, g) < MLP_OUT) Wl[OFF_O + drow(r, g) * MLP_WIDTH + 32 * nt + n] += gWo[r] * gain_inv;
 	}
 	__syncthreads();
 	float* slab = partials + (size_t)blockIdx.x * N_PARAMS;

@@ -270,6 +270,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	// progressive level mask: the encoding is told the number of training steps taken so far before every step
 	// (Testbed::train, src/testbed.cu:2641-2647)
 	if (int rc = n2_grid_set_training_step(n2_field_encoding(t->field), t->training_step)) return rc;
+	// the colour rows of dL/doutput are at most 0.05 * loss_scale / n_rays: the colour net's backward lifts them out of
+	// fp16's subnormal range by an exact power of two
+	if (int rc = n2_field_set_colour_gradient_exponent(t->field, n2_colour_gradient_exponent(t->cfg.loss_scale, n_rays))) return rc;
 	auto sample = [&](n2_trainer::SampleSet& set, hipStream_t on, uint32_t ray_base, uint32_t sd) {
 		// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
 		return n2_generate_training_samples(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,

@@ -237,6 +237,11 @@ class FullyFusedMLP:
             self._ws = torch.empty(nbytes, dtype=torch.uint8, device=params.device)
             check(capi.lib().n2_mlp_set_workspace(self._h, ptr(self._ws), C.c_uint64(nbytes)), "n2_mlp_set_workspace")
 
+    def set_output_gradient_exponent(self, exponent):
+        """backward() with weight gradients multiplies dL/doutput by 2**exponent while it works and divides what it
+        returns by it (n2_mlp_set_output_gradient_exponent): for output gradients in fp16's subnormal range."""
+        check(capi.lib().n2_mlp_set_output_gradient_exponent(self._h, C.c_int(exponent)), "n2_mlp_set_output_gradient_exponent")
+
     def _out(self, n, layout, device):
         shape = (n, 16) if layout == LAYOUT_AOS else (16, n)
         return torch.empty(shape, dtype=torch.float16, device=device)

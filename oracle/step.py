@@ -67,7 +67,7 @@ def _band(got, ref, rtol, what, scale=None, outlier_frac=0.0, atol=0.0):
 
 
 def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_total, seed, n_inference, target_batch_size, counters,
-                gpu, grads, background=(1.0, 1.0, 1.0), ek_loss_weight=0.01, loss_scale=128.0, rtol=2e-3, rgb_grad_rtol=None):
+                gpu, grads, background=(1.0, 1.0, 1.0), ek_loss_weight=0.01, loss_scale=128.0, rtol=2e-3):
     """Checks one GPU training step stage by stage, every stage against the oracle run on the GPU's own input to that
     stage, so that a wiring error (a wrong batch size in the eikonal term, a mis-scaled roll-over, loss_scale / n_rays)
     shows at the stage where it happens and nothing is blurred by the one-sample differences that the 1e-4
@@ -76,7 +76,6 @@ def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_
       gpu       numpy arrays of the step's device buffers (Trainer.last_step): coords, numsteps, rgb_target,
                 ray_indices, network_output, coords_compacted, dloss_doutput, source_index
       grads     the fp16 gradient vector the step left (as float32)
-      rgb_grad_rtol  bound on the colour net's weight gradients when it differs from 2 * rtol (see the full-shape test)
     Returns a dict of the figures it checked."""
     f, T = field, target_batch_size
     # 1. sample generation: bit-exact
@@ -133,7 +132,7 @@ def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_
     for name, a, b in (("sdf mlp", f.off_sdf, f.off_rgb), ("rgb mlp", f.off_rgb, f.off_grid), ("grid", f.off_grid, f.off_var)):
         r = _rel_l2(grads[a:b], ref[a:b])
         res[name] = r
-        bound = rgb_grad_rtol if (name == "rgb mlp" and rgb_grad_rtol is not None) else 2 * rtol
+        bound = 2 * rtol
         assert r <= bound, f"{name} gradient: rel_l2 {r:.3g} > {bound}"
     dv = abs(float(grads[f.off_var]) - float(ref[f.off_var]))
     res["variance"] = dv

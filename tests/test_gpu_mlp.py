@@ -1,4 +1,5 @@
 """GPU parity of the fully fused MLP kernels against the CPU oracle, through the C ABI."""
+import ctypes as C
 import os
 
 import numpy as np
@@ -72,6 +73,56 @@ def test_backward_all_modes(oracle, in_w, n_hidden, n):
     none = gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=False, mode=GRAD_ACCUMULATE)
     assert none is None
     assert_grad_close(host(dG), 2 * ref_dW, what="accumulated weight gradients")
+
+
+@pytest.mark.parametrize("in_w,n_hidden", [(48, 2), (48, 1), (32, 2)])
+def test_output_gradients_in_the_subnormal_range(oracle, in_w, n_hidden):
+    """Output gradients of 2e-6 (what a loss scale of 128 over 5000 rays gives the colour rows): the hidden layers' gradients
+    are fp16 matrices inside the kernel and would be rounded in steps of 6e-8.  With the exponent set, the kernel works on
+    2^k times the values and the results are held to the same bounds as gradients of order one; exponent 0 reproduces the
+    plain call bit for bit on gradients that lose nothing."""
+    from neus2_amd import capi
+    from neus2_amd.tcnn_api import GRAD_OVERWRITE, LAYOUT_SOA
+    om, gm, W, dW, dG, rng = make(oracle, in_w, n_hidden, 12)
+    n = 20000
+    x = q16(rng.standard_normal((in_w, n)))
+    dy = np.zeros((16, n), np.float32)
+    dy[:3] = q16(rng.standard_normal((3, n)) * 2e-6)     # subnormal fp16 values, as the compositor stores them
+    assert 0 < np.abs(dy[:3]).max() < 6.1e-5
+    _, h = om.forward(W, x, round_hidden=True)
+    ref_dx, ref_dW = om.backward(W, x, h, dy)
+    dx_, ddy = dev(x, torch.float16), dev(dy, torch.float16)
+    k = capi.lib().n2_colour_gradient_exponent(C.c_float(128.0), C.c_uint32(5000))
+    assert k == 9                                        # 128 / 5000 * 2^9 = 13.1 <= 16 < 26.2
+    gm.set_output_gradient_exponent(k)
+    gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE)
+    assert_grad_close(host(dG), ref_dW, what="weight gradients of subnormal output gradients")
+    # without it the same call misses the bound (which is what the exponent is for)
+    gm.set_output_gradient_exponent(0)
+    gm.backward(dx_, ddy, LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE)
+    assert rel_l2(host(dG), ref_dW) > RTOL
+    # gradients of order one: the exponent changes nothing but the last bit of sums whose rounding it moves
+    dy1 = q16(rng.standard_normal((16, n)))
+    ref_dx1, ref_dW1 = om.backward(W, x, h, dy1)
+    for kk in (0, 3):
+        gm.set_output_gradient_exponent(kk)
+        dx = gm.backward(dx_, dev(dy1, torch.float16), LAYOUT_SOA, want_input_grad=True, mode=GRAD_OVERWRITE)
+        assert_close(host(dx), ref_dx1, what=f"dL_dinput, exponent {kk}", outlier_frac=FLIP)
+        assert_grad_close(host(dG), ref_dW1, what=f"weight gradients, exponent {kk}")
+    gm.set_output_gradient_exponent(0)
+    with pytest.raises(capi.N2Error):
+        gm.set_output_gradient_exponent(15)
+
+
+def test_colour_gradient_exponent_rule():
+    """Largest k with loss_scale / n_rays * 2^k <= 16, clamped to [0, 14]."""
+    from neus2_amd import capi
+    f = lambda ls, n: capi.lib().n2_colour_gradient_exponent(C.c_float(ls), C.c_uint32(n))
+    assert f(128.0, 5000) == 9 and f(128.0, 50000) == 12 and f(8192.0, 5000) == 3 and f(128.0, 8) == 0 and f(128.0, 1) == 0
+    assert f(1.0, 1 << 20) == 14 and f(0.0, 10) == 0 and f(128.0, 0) == 0
+    for ls, n in ((128.0, 4992), (100.0, 777), (3.0, 65536)):
+        k = f(ls, n)
+        assert ls / n * 2.0 ** k <= 16.0 and (k == 14 or ls / n * 2.0 ** (k + 1) > 16.0)
 
 
 @pytest.mark.parametrize("in_w", [48, 32, 16, 64])
