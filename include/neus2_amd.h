@@ -113,9 +113,11 @@ uint32_t n2_grid_active_levels(const n2_grid_t* grid);
 int n2_grid_set_params(n2_grid_t* grid, const n2_half* d_params, n2_half* d_gradients);
 
 /* Optional scratch for the parameter-gradient scatter (the reference takes temporaries from tcnn's arena).
- * With it, batches of >= 4096 points scatter through an LDS counting sort (no global atomics, fp32
- * accumulation); without it, or for tables with more than 2^19 entries per level, packed fp16 global
- * atomics are used.  Results agree within the stated tolerance either way.
+ * With it, batches of up to max_points points scatter through an LDS counting sort (no global atomics, exact integer
+ * accumulation, partial sums of split buckets added in a fixed order): the gradients do not depend on the order in which the
+ * GPU runs the work, two calls on the same inputs give the same bits.  Without it, or for tables with more than 2^19
+ * entries per level, packed fp16 global atomics are used (as in the reference; sums then depend on arrival order in the
+ * last bit).  Results agree within the stated tolerance either way.
  * n2_grid_workspace_bytes returns 0 when the table shape does not support the sorted path. */
 uint64_t n2_grid_workspace_bytes(const n2_grid_t* grid, uint32_t max_points);
 int n2_grid_set_workspace(n2_grid_t* grid, void* d_workspace, uint64_t n_bytes, uint32_t max_points);
@@ -585,7 +587,8 @@ typedef struct n2_trainer_config {
 	uint32_t prefetch_samples;      /* non-zero: each step also starts the NEXT step's sample generation (same n_rays and
 	                                   n_inference, seed + 1) on a stream the trainer owns, so that it overlaps this step's
 	                                   field kernels; a following step called with other arguments regenerates in line.
-	                                   Results are identical either way.  The trainer must then be driven from one stream
+	                                   Results are bit-identical either way (every sum of a step is formed in a fixed
+	                                   order).  The trainer must then be driven from one stream
 	                                   (or from streams the caller orders against each other). */
 	float ema_decay;                /* 0: plain Adam.  In (0, 1): the Ema wrapper of configs/nerf/base.json:5-7 (0.95) keeps a
 	                                   bias-corrected moving average of the fp16 weights as the inference parameters */

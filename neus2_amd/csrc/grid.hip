@@ -13,6 +13,7 @@
 // walks every level and the table crosses the fabric 8 times per launch.)
 #include "n2_common.h"
 #include "grid_device.h"
+#include "slab_reduce.h"
 
 #include <cmath>
 #include <new>
@@ -34,9 +35,6 @@ struct n2_grid {
 	uint64_t ws_bytes;
 	uint32_t ws_max_points;
 	bool lattice_order;  // points of the next forwards come in lattice order (n2_grid_set_point_order)
-	// part of the gradient buffer the next bucketed scatter clears in its bin kernel (OVERWRITE, levels that add with atomics)
-	uint4* zero_begin;
-	uint32_t zero_count;  // in 16-byte units
 };
 
 struct N2Point {
@@ -467,6 +465,10 @@ struct N2BucketPlan {
 	uint32_t wg_begin[N2_MAX_LEVELS + 1];  // first reduce workgroup of each level
 	uint32_t n_buckets[N2_MAX_LEVELS];
 	uint32_t groups[N2_MAX_LEVELS];        // tile groups per bucket
+	// levels whose buckets are split over several workgroups (groups > 1): where the level's partial images start (images:
+	// bucket-major, then group) and the number of split buckets in the levels below
+	uint32_t part_begin[N2_MAX_LEVELS];
+	uint32_t split_begin[N2_MAX_LEVELS + 1];
 };
 
 template <uint32_t MODE, bool FIRST, bool SECOND, bool WANT_OUT, bool CLAMP_X>
@@ -692,10 +694,8 @@ __global__ void __launch_bounds__(BIN_BLOCK, 6) grid_bin_kernel(N2LevelTable tab
                                                               const float* __restrict__ v, const __half* __restrict__ g2,
                                                               const __half2* __restrict__ params, __half* __restrict__ dL_ddLdy,
                                                               uint32_t* __restrict__ rec_vals, uint16_t* __restrict__ rec_keys,
-                                                              uint16_t* __restrict__ offsets, uint4* __restrict__ zero_begin, uint32_t zero_count,
+                                                              uint16_t* __restrict__ offsets,
                                                               const uint32_t* __restrict__ index, uint32_t n_cols) {
-	// part of the gradient buffer that the reduce kernel will add to with atomics: cleared here, one 16-byte store per thread
-	for (uint32_t z = blockIdx.x * BIN_BLOCK + threadIdx.x; z < zero_count; z += gridDim.x * BIN_BLOCK) zero_begin[z] = make_uint4(0u, 0u, 0u, 0u);
 	__shared__ uint32_t hist[BKT_MAX];
 	__shared__ uint32_t prefix[BKT_MAX + 1];
 	__shared__ __align__(16) uint32_t stage_val[BIN_RECORDS];  // sorted records: packed half2 value (a pair of them on pair levels) ...
@@ -908,7 +908,8 @@ __device__ __forceinline__ void grid_reduce_runs(const uint32_t tiles, const uin
 __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable tab, N2BucketPlan plan, uint32_t tiles,
                                                                    const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
                                                                    const uint16_t* __restrict__ offsets,
-                                                                   __half2* __restrict__ grads, int accumulate) {
+                                                                   __half2* __restrict__ grads, int accumulate,
+                                                                   float2* __restrict__ partials) {
 	// one plane per feature: lanes of a wave's atomic then spread over all bank pairs (entry-major pairs of features would
 	// leave every other pair unused)
 	__shared__ unsigned long long acc[2 * BKT_ENTRIES];
@@ -934,20 +935,37 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 	__syncthreads();
 	const uint32_t entries = tab.entries[level];
 	__half2* Gd = grads + tab.offset[level];
+	if (G > 1) {
+		// Several workgroups hold parts of this bucket's sums (coarse levels of large batches).  Each leaves its image as
+		// fp32 and grid_combine_kernel adds the G images up in the order of the groups: every entry is the same sum of the
+		// same terms in the same order however the workgroups were scheduled (the images themselves are exact integer sums).
+		float2* mine = partials + ((size_t)plan.part_begin[level] + (size_t)bucket * G + group) * BKT_ENTRIES;
+		for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) mine[e] = make_float2(from_fixed(acc[e]), from_fixed(acc[BKT_ENTRIES + e]));
+		return;
+	}
 	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) {
 		const uint32_t idx = bucket * BKT_ENTRIES + e;
 		if (idx >= entries) break;
 		const float ax = from_fixed(acc[e]), ay = from_fixed(acc[BKT_ENTRIES + e]);
-		if (G > 1) {
-			// several tile groups fold into the same entries (coarse levels only)
-			if (ax != 0.f || ay != 0.f) unsafeAtomicAdd(&Gd[idx], __floats2half2_rn(ax, ay));
-		} else if (accumulate) {
+		if (accumulate) {
 			const float2 old = __half22float2(Gd[idx]);
 			Gd[idx] = __floats2half2_rn(old.x + ax, old.y + ay);
 		} else {
 			Gd[idx] = __floats2half2_rn(ax, ay);
 		}
 	}
+}
+
+// Split buckets: the sum of a bucket's G partial images in a fixed order (n2_image_combine_unit, slab_reduce.h: with the
+// images added one after the other by one thread the launch was a chain of memory round trips, 9 us for 5 MB).  Run as units
+// of the optimiser's kernel instead of a launch of its own it shortens the training step by 0.9 us (measured): not built.
+// (Doing this in the reduce kernel, by the workgroup of a bucket that finishes last, needs two device-scope fences per
+// workgroup, which write back and invalidate the L2s: the scatter took 150 us longer.  Packed fp16 atomics into the
+// gradient buffer cost nothing extra but add in arrival order.)
+static_assert(BKT_ENTRIES % N2_CMB_ENTRIES == 0, "whole units per bucket");
+__global__ void __launch_bounds__(256) grid_combine_kernel(N2ImageCombine plan) {
+	__shared__ float2 part[N2_CMB_SLICES][N2_CMB_ENTRIES];
+	n2_image_combine_unit(plan, blockIdx.x, part, [](const _Float16*, _Float16) {});
 }
 
 // ----------------------------------------------------------------------------
@@ -1025,8 +1043,6 @@ N2_API int n2_grid_create(uint32_t n_levels, uint32_t n_features_per_level, uint
 	g->ws = nullptr;
 	g->ws_bytes = 0;
 	g->ws_max_points = 0;
-	g->zero_begin = nullptr;
-	g->zero_count = 0;
 	g->lattice_order = false;
 	*out = g;
 	return N2_OK;
@@ -1218,31 +1234,14 @@ N2_API int n2_grid_corner_indices(n2_grid_t* grid, n2_stream_t stream, const flo
 static bool uses_bucketed(const n2_grid_t* grid, uint32_t n_points);
 static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_points, uint32_t tiles);
 
-// OVERWRITE: the gradient buffer starts from zero.  The bucketed scatter writes every entry of a level whose buckets
-// have one workgroup each, so only levels whose buckets are split over several workgroups (they add with atomics) need
-// clearing beforehand.
+// OVERWRITE: the gradient buffer starts from zero.  The bucketed scatter writes every entry itself (with plain stores),
+// so only the scatter with atomics needs the buffer cleared beforehand.
 static int prepare_grads(n2_grid_t* grid, const char* fn, hipStream_t stream, n2_grad_mode mode, uint32_t n_points) {
 	N2_REQUIRE(mode == N2_GRAD_IGNORE || mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "%s: bad gradient mode %d", fn, (int)mode);
-	grid->zero_begin = nullptr;
-	grid->zero_count = 0;
 	if (mode == N2_GRAD_IGNORE) return N2_OK;
 	N2_REQUIRE(grid->grads != nullptr, "%s: gradient mode %d needs a gradient buffer (n2_grid_set_params)", fn, (int)mode);
 	if (mode != N2_GRAD_OVERWRITE) return N2_OK;
 	if (!uses_bucketed(grid, n_points)) return n2_fill_zero_u32(stream, grid->grads, (size_t)grid->n_params * sizeof(__half));
-	const uint32_t tiles = (n_points + 1023u) / 1024u;
-	uint32_t first = 0xFFFFFFFFu, last = 0;
-	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
-		if (bucket_groups(grid, l, n_points, tiles) > 1) {
-			if (first == 0xFFFFFFFFu) first = l;
-			last = l;
-		}
-	}
-	if (first == 0xFFFFFFFFu) return N2_OK;
-	// the span of those levels (they are the coarse, small ones) is cleared by the bin kernel, which runs to completion
-	// before the reduce kernel adds to it; 16-byte aligned because every level holds a multiple of 8 entries
-	const size_t begin = (size_t)grid->tab.offset[first] * sizeof(__half2), end = (size_t)grid->tab.offset[last + 1] * sizeof(__half2);
-	grid->zero_begin = reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(grid->grads) + begin);
-	grid->zero_count = (uint32_t)((end - begin) / 16);
 	return N2_OK;
 }
 
@@ -1254,24 +1253,51 @@ static bool bucket_supported(const n2_grid_t* grid) {
 		if (grid->tab.entries[l] > BKT_ENTRIES * BKT_MAX) return false;
 	return true;
 }
-static uint64_t bucket_ws_bytes(const n2_grid_t* grid, uint32_t max_points) {
+// workspace: the records' values, their keys, the tiles' bucket offsets, then one fp32 image per (bucket, group) of the
+// split buckets
+struct BucketCarve {
+	uint64_t vals, keys, offsets, partials, total;
+};
+static uint32_t split_images(const n2_grid_t* grid, uint32_t n_points);
+static BucketCarve bucket_carve(const n2_grid_t* grid, uint32_t max_points) {
 	const uint64_t tiles = n_bin_tiles(max_points), L = grid->tab.n_levels;
-	const uint64_t rec = L * tiles * BIN_RECORDS * (sizeof(uint32_t) + sizeof(uint16_t));
-	const uint64_t off = (L * tiles * (BKT_MAX + 1) * sizeof(uint16_t) + 255) / 256 * 256;
-	return rec + off;
+	const uint64_t n_rec = L * tiles * BIN_RECORDS;
+	auto up = [](uint64_t x) { return (x + 255) / 256 * 256; };
+	BucketCarve c{};
+	c.vals = 0;
+	c.keys = c.vals + n_rec * sizeof(uint32_t);
+	c.offsets = c.keys + n_rec * sizeof(uint16_t);
+	c.partials = up(c.offsets + L * tiles * (BKT_MAX + 1) * sizeof(uint16_t));
+	c.total = up(c.partials + (uint64_t)split_images(grid, max_points) * BKT_ENTRIES * sizeof(float2));
+	return c;
 }
+static uint64_t bucket_ws_bytes(const n2_grid_t* grid, uint32_t max_points) { return bucket_carve(grid, max_points).total; }
 
+// With a workspace every batch size takes the bucketed scatter, whose result does not depend on the order in which
+// workgroups run; the scatter with atomics (no workspace, or more points than it was sized for) sums in arrival order.
 static bool uses_bucketed(const n2_grid_t* grid, uint32_t n_points) {
-	return grid->grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 4 * BIN_POINTS;
+	return grid->grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 1;
 }
 // workgroups per bucket of a level: aim at <= ~64k records per reduce workgroup (a level holds 8 records per point)
 static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_points, uint32_t tiles) {
 	const uint32_t nb = (grid->tab.entries[level] + BKT_ENTRIES - 1) / BKT_ENTRIES;
 	const uint64_t per_bucket = (uint64_t)n_points * 8 / nb;
 	uint32_t groups = (uint32_t)((per_bucket + 65535) / 65536);
+	if (groups > N2_CMB_MAX_GROUPS) groups = N2_CMB_MAX_GROUPS;
 	if (groups > tiles) groups = tiles;
 	if (groups < 1) groups = 1;
 	return groups;
+}
+
+// fp32 images of all split buckets of a batch (never more for a smaller batch: the groups per bucket grow with the batch)
+static uint32_t split_images(const n2_grid_t* grid, uint32_t n_points) {
+	const uint32_t tiles = n_bin_tiles(n_points);
+	uint32_t n = 0;
+	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
+		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES, groups = bucket_groups(grid, l, n_points, tiles);
+		if (groups > 1) n += nb * groups;
+	}
+	return n;
 }
 
 N2_API uint64_t n2_grid_workspace_bytes(const n2_grid_t* grid, uint32_t max_points) {
@@ -1301,18 +1327,32 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	const uint32_t tiles = n_bin_tiles(n_points), L = grid->tab.n_levels;
 	const bool first = dL_dy != nullptr, second = v != nullptr, out = dL_ddLdy != nullptr;
 	const dim3 bd(BIN_BLOCK);
-	// workspace: packed half2 values of all records, then their 16-bit keys, then the tiles' bucket offsets
-	const uint64_t n_rec = (uint64_t)L * tiles * BIN_RECORDS;
-	uint32_t* rec_vals = reinterpret_cast<uint32_t*>(grid->ws);
-	uint16_t* rec_keys = reinterpret_cast<uint16_t*>(grid->ws + n_rec * sizeof(uint32_t));
-	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + n_rec * (sizeof(uint32_t) + sizeof(uint16_t)));
+	// The records of this batch are packed as for a workspace of exactly this size (values, keys, offsets one behind the
+	// other); the images of split buckets stand where the workspace's own size put them.
+	const BucketCarve now = bucket_carve(grid, n_points), full = bucket_carve(grid, grid->ws_max_points);
+	uint32_t* rec_vals = reinterpret_cast<uint32_t*>(grid->ws + now.vals);
+	uint16_t* rec_keys = reinterpret_cast<uint16_t*>(grid->ws + now.keys);
+	uint16_t* offsets = reinterpret_cast<uint16_t*>(grid->ws + now.offsets);
+	float2* partials = reinterpret_cast<float2*>(grid->ws + full.partials);
 	const dim3 gd(tiles * L);
-	uint4* zero_begin = grid->zero_begin;
-	const uint32_t zero_count = grid->zero_count;
-	grid->zero_begin = nullptr;
-	grid->zero_count = 0;
+	N2BucketPlan plan;
+	uint32_t wg = 0, images = 0, split = 0;
+	for (uint32_t l = 0; l < L; ++l) {
+		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES;
+		const uint32_t groups = bucket_groups(grid, l, n_points, tiles);
+		plan.wg_begin[l] = wg;
+		plan.n_buckets[l] = nb;
+		plan.groups[l] = groups;
+		plan.part_begin[l] = images;
+		plan.split_begin[l] = split;
+		wg += nb * groups;
+		if (groups > 1) { images += nb * groups; split += nb; }
+	}
+	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
+	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; plan.part_begin[l] = images; }
+	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.split_begin[l] = split;
 #define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
-                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, zero_begin, zero_count, index, n_cols)
+                                                                   grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, index, n_cols)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
 	else if (second && out) LAUNCH(false, true, true);
@@ -1320,20 +1360,28 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	else LAUNCH(true, false, false);
 #undef LAUNCH
 	N2_LAUNCH_CHECK();
-	N2BucketPlan plan;
-	uint32_t wg = 0;
-	for (uint32_t l = 0; l < L; ++l) {
-		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES;
-		const uint32_t groups = bucket_groups(grid, l, n_points, tiles);
-		plan.wg_begin[l] = wg;
-		plan.n_buckets[l] = nb;
-		plan.groups[l] = groups;
-		wg += nb * groups;
-	}
-	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
-	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; }
-	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, rec_vals, rec_keys, offsets, grid->grads, accumulate ? 1 : 0);
+	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, rec_vals, rec_keys, offsets, grid->grads, accumulate ? 1 : 0, partials);
 	N2_LAUNCH_CHECK();
+	if (split > 0) {
+		// the split levels are the coarsest ones (a level has at least as many buckets as the one below it)
+		N2ImageCombine cmb{};
+		cmb.images = partials;
+		cmb.grads = reinterpret_cast<_Float16*>(grid->grads);
+		cmb.bucket_entries = BKT_ENTRIES;
+		cmb.accumulate = accumulate ? 1 : 0;
+		uint32_t k = 0;
+		while (k < L && k < N2_CMB_LEVELS && plan.groups[k] > 1) {
+			cmb.split_begin[k] = plan.split_begin[k]; cmb.groups[k] = plan.groups[k]; cmb.part_begin[k] = plan.part_begin[k];
+			cmb.entries[k] = grid->tab.entries[k]; cmb.offset[k] = grid->tab.offset[k];
+			++k;
+		}
+		cmb.n_levels = k;
+		for (uint32_t l = k; l <= N2_CMB_LEVELS; ++l) cmb.split_begin[l] = split;
+		N2_REQUIRE(k > 0 && plan.split_begin[k] == split, "grid scatter: split buckets outside the coarsest %u levels", N2_CMB_LEVELS);
+		cmb.units = split * (BKT_ENTRIES / N2_CMB_ENTRIES);
+		grid_combine_kernel<<<dim3(cmb.units), dim3(256), 0, s>>>(cmb);
+		N2_LAUNCH_CHECK();
+	}
 	return N2_OK;
 }
 
@@ -1399,7 +1447,7 @@ N2_API int n2_grid_backward_fused(n2_grid_t* grid, n2_stream_t stream, const flo
 int n2_grid_backward_fused_indexed(n2_grid_t* grid, n2_stream_t stream, const float* d_xyz_rows, uint32_t n_cols, const uint32_t* d_index,
                                    uint32_t n_points, const n2_half* d_dL_dy, const float* d_dL_ddLdx, const n2_half* d_dL_dy_second,
                                    n2_grad_mode mode) {
-	if (d_index == nullptr) return n2_grid_backward_fused(grid, stream, d_xyz_rows, 1, n_points, n_points, d_dL_dy, d_dL_ddLdx, d_dL_dy_second, nullptr, mode);
+	if (d_index == nullptr) n_cols = n_points;  // the rows hold the batch itself
 	if (int rc = check_batch(grid, "n2_grid_backward_fused", d_xyz_rows, 1, n_cols, n_points)) return rc;
 	N2_REQUIRE((d_dL_dy && d_dL_ddLdx && d_dL_dy_second) || n_points == 0, "n2_grid_backward_fused: d_dL_dy, d_dL_ddLdx and d_dL_dy_second are required");
 	N2_REQUIRE(mode == N2_GRAD_OVERWRITE || mode == N2_GRAD_ACCUMULATE, "n2_grid_backward_fused: mode must be OVERWRITE or ACCUMULATE");

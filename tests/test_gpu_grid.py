@@ -256,7 +256,7 @@ def test_backward_fused_equals_first_plus_second_order(setup, n):
 
 @pytest.mark.parametrize("kind", ["uniform", "clustered", "rays"])
 def test_sorted_scatter_path(oracle, kind):
-    """With a scatter workspace, batches of >= 4096 points go through the run-length kernel (coarsest levels) and the
+    """With a scatter workspace, batches go through the run-length kernel (coarsest levels) and the
     LDS counting sort (the others): fp32 / exact accumulation, tighter agreement with the fp32 oracle than the
     atomic path, on uniform points, on points packed into a few cells (the contention case) and on points in ray
     order (consecutive samples share cells on the coarse levels, so runs are merged before they are written)."""

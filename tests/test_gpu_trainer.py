@@ -147,12 +147,39 @@ def test_samples_generated_ahead_give_the_same_steps():
         runs.append((log, host(tr.master).copy()))
         del tr
     (log_a, m_a), (log_b, m_b) = runs
-    for a, b in zip(log_a, log_b):
-        assert (a["rays"], a["samples"]) == (b["rays"], b["samples"]) and a["rays"] > 0
-        assert abs(a["compacted"] - b["compacted"]) <= max(2, 0.005 * a["compacted"])
-        assert abs(a["loss"] - b["loss"]) <= 0.01 * abs(a["loss"]) + 1e-6
-    assert cos_sim(m_a - m_a.mean(), m_b - m_b.mean()) > 0.999
-    assert np.abs(m_a - m_b).max() < 2e-2
+    # bit for bit: every sum of a step is formed in an order that does not depend on how the GPU schedules the work
+    assert log_a == log_b and all(a["rays"] > 0 for a in log_a)
+    np.testing.assert_array_equal(m_a, m_b)
+
+
+def test_a_step_is_bit_reproducible_at_the_benchmark_batch():
+    """Two trainers run the same steps at the 2^18 batch (the encoding's coarsest levels then split their buckets over
+    several workgroups, whose partial sums meet in a fixed order): gradients, counters, loss and parameters agree bit for
+    bit after every step, with the sample generation running ahead in one of them."""
+    import bench
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import Trainer, default_config
+    T = 1 << 18
+    cams, rgba, bits = bench.build_scene()
+    d_cams, d_rgba, d_bits = pack_cameras(cams), dev(rgba), dev(bits)
+    n_inf = 280000 // 128 * 128
+    runs = []
+    for ahead in (True, False):
+        tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=1 << 16, max_samples=16 * T, prefetch_samples=ahead))
+        tr.set_scene(d_cams, len(cams), d_rgba, d_bits)
+        tr.initialize_params(seed=1337, sdf_mlp_weights=None)
+        seen = []
+        for step in range(3):
+            tr.step(n_rays=5000, n_inference=n_inf, seed=40 + step)
+            seen.append((tr.read_counters(), tr.grads.clone()))
+        runs.append((seen, tr.master.clone()))
+        del tr
+    (seen_a, m_a), (seen_b, m_b) = runs
+    for (ca, ga), (cb, gb) in zip(seen_a, seen_b):
+        assert ca == cb and ca["compacted"] > T // 2
+        assert torch.equal(ga, gb)
+        assert ga.float().abs().sum() > 0
+    assert torch.equal(m_a, m_b)
 
 
 def test_progressive_level_mask_follows_the_step_count(oracle):
