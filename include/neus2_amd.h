@@ -658,6 +658,21 @@ int n2_trainer_set_training_step(n2_trainer_t* trainer, uint32_t step);
  * src/testbed.cu:2658-2674).  No counterpart in the reference, which generates its samples inside the step. */
 int n2_trainer_invalidate_prefetch(n2_trainer_t* trainer);
 
+/* Forward pass in depth chunks.  The compositor consumes a ray's samples only while the transmittance in front of them is
+ * >= 1e-4 (src/testbed_nerf.cu:1562-1566); on a trained field most rays reach that point long before their last marched
+ * sample, and nothing behind it enters the loss, the compaction or a gradient.  With n_rounds >= 2 the step evaluates the
+ * field in rounds: every round takes the next chunk_size samples of the rays that are still in front of their cut (the
+ * last round: all that is left of them).  Parameters, gradients and counters are bit-identical to the plain step's, which
+ * evaluates every marched sample as the reference does (src/testbed_nerf.cu:3771-3777); each round costs three short
+ * launches, so the setting pays when a step marches well over one and a half times the samples it keeps.
+ * n_rounds 0 or 1: off (the default).  n_rounds <= 8.  Needs the fused field kernels. */
+int n2_trainer_set_depth_chunks(n2_trainer_t* trainer, uint32_t chunk_size, uint32_t n_rounds);
+/* How many samples each round evaluated in a recent step (n2_trainer_step_view.evaluated_counts, read by the caller when it
+ * reads the step's counters): the following steps size their launches by these figures instead of by the most a round can
+ * hold.  Estimates only decide how the work is dealt to workgroups, never what is computed.  n2_trainer_set_depth_chunks
+ * forgets them. */
+int n2_trainer_set_depth_chunk_estimates(n2_trainer_t* trainer, const uint32_t* samples_per_round, uint32_t n_rounds);
+
 /*  n_rays       rays to draw this step (<= max_rays_per_batch)
  *  n_inference  how many marched samples the first forward covers (a multiple of 8, <= max_samples); the
  *               reference uses the sample count measured in earlier steps, rounded up to 128
@@ -675,7 +690,11 @@ typedef struct n2_trainer_step_view {
 	const n2_half* network_output;    /* [n_inference][16] field output over the marched samples */
 	const float* coords_compacted;    /* [target_batch_size][7] after the roll-over */
 	const n2_half* dloss_doutput;     /* [target_batch_size][16] after the roll-over */
-	const uint32_t* source_index;     /* [target_batch_size] marched sample behind every compacted sample */
+	const uint32_t* source_index;     /* [target_batch_size] marched sample behind every compacted sample; after a step in depth
+	                                     chunks: its place in evaluated_samples */
+	const uint32_t* evaluated_samples;/* NULL, or (a step in depth chunks) the marched samples the field was evaluated on, in the
+	                                     order in which it stored them */
+	const uint32_t* evaluated_counts; /* NULL, or [8]: how many of them each round evaluated (their sum is the list's length) */
 } n2_trainer_step_view;
 int n2_trainer_last_step_view(n2_trainer_t* trainer, n2_trainer_step_view* out);
 

@@ -60,7 +60,7 @@ class TrainerStepView(C.Structure):
     """struct n2_trainer_step_view"""
     _fields_ = [("coords", C.c_void_p), ("numsteps", C.c_void_p), ("rgb_target", C.c_void_p), ("ray_indices", C.c_void_p),
                 ("network_output", C.c_void_p), ("coords_compacted", C.c_void_p), ("dloss_doutput", C.c_void_p),
-                ("source_index", C.c_void_p)]
+                ("source_index", C.c_void_p), ("evaluated_samples", C.c_void_p), ("evaluated_counts", C.c_void_p)]
 
 
 class OccupancyBuffers(C.Structure):

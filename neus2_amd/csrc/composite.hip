@@ -122,10 +122,13 @@ __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uin
 			// samples are consumed while the transmittance before them is >= 1e-4
 			const unsigned long long stop = __ballot(!valid || Tb < T_EPS);
 			const int n_proc = stop ? (int)__ffsll((long long)stop) - 1 : 64;
-			const float w = lane < n_proc ? alpha * Tb : 0.f;
-			r0 += wave_sum(w * rgb[0]);
-			r1 += wave_sum(w * rgb[1]);
-			r2 += wave_sum(w * rgb[2]);
+			// (samples behind the cut contribute exact zeros whatever their outputs hold: with a forward pass in depth chunks
+			// those outputs were never written)
+			const bool in = lane < n_proc;
+			const float w = in ? alpha * Tb : 0.f;
+			r0 += wave_sum(in ? w * rgb[0] : 0.f);
+			r1 += wave_sum(in ? w * rgb[1] : 0.f);
+			r2 += wave_sum(in ? w * rgb[2] : 0.f);
 			kept += n_proc;
 			if (n_proc > 0) T = __shfl(Tb * (1.f - alpha), n_proc - 1);
 			if (n_proc < 64) break;
@@ -192,7 +195,9 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
                                                                 uint32_t* __restrict__ counter, float* __restrict__ coords_out,
                                                                 hf* __restrict__ dloss, float* __restrict__ loss, uint32_t* __restrict__ source_index,
                                                                 const uint32_t* __restrict__ before_of, uint32_t pad,
-                                                                const uint32_t* __restrict__ kept_of_block) {
+                                                                const uint32_t* __restrict__ kept_of_block, const uint32_t* __restrict__ column_of) {
+	// column_of (or null): where the field stored what it saved for marched sample i (a forward pass in depth chunks stores
+	// the samples it evaluates side by side); source_index then names that column
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 	// Where this workgroup's rays start in the compacted batch: the kept samples of all rays before them, in ray order
 	// (deterministic).  With a few thousand rays every workgroup adds up the counts of its predecessors itself: a few KiB
@@ -330,7 +335,8 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 			float* co = coords_out + ((size_t)cb + s) * 7;
 #pragma unroll
 			for (int k = 0; k < 7; ++k) co[k] = ci[k];
-			if (source_index) source_index[cb + s] = base + s;  // which marched sample this compacted sample is
+			const uint32_t src_col = column_of ? column_of[base + s] : base + s;
+			if (source_index) source_index[cb + s] = src_col;  // which marched sample this compacted sample is
 			if (pad && n_in > 0 && n_in < max_compacted) {
 				for (uint32_t j = cb + s + n_in; j < max_compacted; j += n_in) {
 					half8 lo_f, hi_f;
@@ -345,12 +351,117 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 					float* cf = coords_out + (size_t)j * 7;
 #pragma unroll
 					for (int k = 0; k < 7; ++k) cf[k] = ci[k];
-					if (source_index) source_index[j] = base + s;
+					if (source_index) source_index[j] = src_col;
 				}
 			}
 		}
 		T = __shfl(Ta, 63);
 		p0 = __shfl(q0, 63); p1 = __shfl(q1, 63); p2 = __shfl(q2, 63);
+	}
+}
+
+// ----------------------------------------------------------------------------
+// Forward pass in depth chunks.  The compositor consumes a ray's samples only while the transmittance before them is
+// >= 1e-4 (src/testbed_nerf.cu:1562-1566); on a trained field most rays reach that point after a fraction of their
+// marched samples, and everything behind it never enters loss, compaction or gradients.  The trainer can therefore
+// evaluate the field in rounds: every round takes the next `chunk` samples of the rays that are still live, and between
+// rounds this kernel (one thread per ray) multiplies the transmittance on over the samples just evaluated, with the
+// compositor's own alpha, and retires the rays that are certainly past the cut (T < 0.5e-4: the compositor's product is
+// formed in another order, which moves T by a few units in the last place, never by a factor of two; a ray that stays
+// live a round too long costs work, never correctness).  For the live rays it appends the next samples to the list of
+// samples to evaluate; the samples of all rounds stand side by side in that list, and column_of[marched sample] is its
+// place in it (where the field stores what the backward reads).  counts[r] = samples of round r.
+// ----------------------------------------------------------------------------
+struct ChunkRay {
+	uint32_t prev, done;  // samples [prev, done) of the ray were listed last
+	float T;              // transmittance behind sample prev
+	uint32_t live;
+};
+constexpr float CHUNK_T_EPS = 0.5f * T_EPS;
+// sixteen lanes per ray, 64 rays per workgroup: every workgroup takes its places in the list with one atomic on the round's
+// counter, and those atomics, all on one address, run one after the other (16 rays per workgroup: 2500 of them, 20 us)
+constexpr uint32_t CHUNK_BLOCK = 1024, CHUNK_LANES = 16, CHUNK_RAYS = CHUNK_BLOCK / CHUNK_LANES;
+
+// One ray per sixteen lanes (a row of the data-parallel lane operations): the lanes take the ray's samples sixteen at a
+// time.  coords_listed receives the coordinate rows of the listed samples in list order, so that the field's kernels read
+// their input without going through the list.
+__global__ void __launch_bounds__(CHUNK_BLOCK) composite_chunk_kernel(CompParams c, uint32_t n_rays, const uint32_t* __restrict__ ray_counter,
+                                                                      const uint32_t* __restrict__ numsteps, const hf* __restrict__ net_out,
+                                                                      const float* __restrict__ coords, uint32_t round, uint32_t chunk,
+                                                                      ChunkRay* __restrict__ state, uint32_t* __restrict__ counts,
+                                                                      uint32_t* __restrict__ counts_other, uint32_t* __restrict__ list,
+                                                                      uint32_t* __restrict__ column_of, float* __restrict__ coords_listed) {
+	__shared__ uint32_t takes[CHUNK_RAYS], places[CHUNK_RAYS];
+	const uint32_t l = threadIdx.x % CHUNK_LANES, slot = threadIdx.x / CHUNK_LANES;
+	const uint32_t ray = blockIdx.x * CHUNK_RAYS + slot;
+	const uint32_t live_rays = ray_counter ? min(*ray_counter, n_rays) : n_rays;
+	// the counters that the following step uses start from zero
+	if (round == 0 && blockIdx.x == 0 && threadIdx.x < N2_CHUNK_MAX_ROUNDS) counts_other[threadIdx.x] = 0u;
+	uint32_t begin = 0;  // samples listed by the rounds before this one
+	for (uint32_t q = 0; q < round; ++q) begin += counts[q];
+	ChunkRay st = {0u, 0u, 1.f, 0u};
+	uint32_t n = 0, base = 0;
+	if (ray < live_rays) {
+		n = numsteps[2 * ray];
+		base = numsteps[2 * ray + 1];
+		if (round == 0) {
+			st.live = n > 0 ? 1u : 0u;
+		} else {
+			st = state[ray];
+			if (st.live) {
+				float dir[3];
+				ray_dir(net_out, base, dir);
+				float T = st.T;
+				for (uint32_t s0 = st.prev; s0 < st.done; s0 += CHUNK_LANES) {
+					const uint32_t s = s0 + l;
+					float keep = 1.f;
+					if (s < st.done) {
+						float o[16];
+						load_out(net_out, (size_t)base + s, o);
+						const Sample sm = eval_sample(o, net_out[((size_t)base + s) * 16 + 7], coords[((size_t)base + s) * 7 + 3], dir, c);
+						keep = 1.f - sm.alpha;
+					}
+#pragma unroll
+					for (int o = 1; o < (int)CHUNK_LANES; o <<= 1) keep *= __shfl_xor(keep, o);  // stays inside the sixteen lanes
+					T *= keep;
+				}
+				st.T = T;
+				if (!(T >= CHUNK_T_EPS) || st.done >= n) st.live = 0u;  // (a transmittance that is not a number retires the ray too)
+			}
+		}
+	}
+	const uint32_t take = st.live ? min(n - st.done, chunk) : 0u;
+	// places in the list: the workgroup's sixteen rays in order, one atomic per workgroup for its block of places
+	if (l == 0) takes[slot] = take;
+	__syncthreads();
+	if (threadIdx.x < 64) {  // one wave scans the 64 counts
+		static_assert(CHUNK_RAYS == 64, "one count per lane");
+		const uint32_t own = takes[threadIdx.x];
+		uint32_t incl = own;
+#pragma unroll
+		for (int o = 1; o < 64; o <<= 1) {
+			const uint32_t up = __shfl_up(incl, o);
+			if ((int)threadIdx.x >= o) incl += up;
+		}
+		const uint32_t total = __shfl(incl, 63);
+		uint32_t at = 0;
+		if (threadIdx.x == 0 && total) at = atomicAdd(&counts[round], total);
+		places[threadIdx.x] = __shfl(at, 0) + incl - own;
+	}
+	__syncthreads();
+	const uint32_t at = begin + places[slot], first = base + st.done;
+	for (uint32_t k = l; k < take; k += CHUNK_LANES) {
+		list[at + k] = first + k;
+		column_of[first + k] = at + k;
+	}
+	// the coordinate rows of the listed samples: consecutive in the input (one ray's samples) and in the output
+	const float* from = coords + (size_t)first * 7;
+	float* to = coords_listed + (size_t)at * 7;
+	for (uint32_t k = l; k < take * 7u; k += CHUNK_LANES) to[k] = from[k];
+	if (ray < live_rays && l == 0) {
+		st.prev = st.done;
+		st.done += take;
+		state[ray] = st;
 	}
 }
 
@@ -371,6 +482,28 @@ static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
 
 N2_API uint64_t n2_composite_workspace_bytes(uint32_t max_rays) {
 	return up256(sizeof(RayScratch) * (uint64_t)max_rays) + 2 * up256(4ull * max_rays);
+}
+
+uint64_t n2_composite_chunk_state_bytes(uint32_t max_rays) { return up256(sizeof(ChunkRay) * (uint64_t)max_rays); }
+
+int n2_composite_chunk_next(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays, const uint32_t* d_ray_counter, const uint32_t* d_numsteps,
+                            const n2_half* d_network_output, const float* d_coords, uint32_t round, uint32_t chunk, void* d_state, uint32_t* d_counts,
+                            uint32_t* d_counts_other, uint32_t* d_list, uint32_t* d_column_of, float* d_coords_listed) {
+	N2_REQUIRE(cfg && d_numsteps && d_network_output && d_coords && d_state && d_counts && d_counts_other && d_list && d_column_of && d_coords_listed,
+	           "n2_composite_chunk_next: null argument");
+	N2_REQUIRE(round < N2_CHUNK_MAX_ROUNDS && chunk >= 1, "n2_composite_chunk_next: round %u of at most %u, chunk %u", round, N2_CHUNK_MAX_ROUNDS, chunk);
+	if (n_rays == 0) return N2_OK;
+	CompParams c;
+	c.loss_scale = cfg->loss_scale; c.ek_loss_weight = cfg->ek_loss_weight; c.anneal = cfg->cos_anneal_ratio;
+	c.bg[0] = cfg->background[0]; c.bg[1] = cfg->background[1]; c.bg[2] = cfg->background[2];
+	c.inv_n_rays = 1.f;
+	c.min_step = 1.73205080757f / 1024.f;
+	c.max_step = c.min_step * 128.f;
+	composite_chunk_kernel<<<dim3((n_rays + CHUNK_RAYS - 1) / CHUNK_RAYS), dim3(CHUNK_BLOCK), 0, n2_stream(stream)>>>(
+		c, n_rays, d_ray_counter, d_numsteps, reinterpret_cast<const hf*>(d_network_output), d_coords, round, chunk, reinterpret_cast<ChunkRay*>(d_state),
+		d_counts, d_counts_other, d_list, d_column_of, d_coords_listed);
+	N2_LAUNCH_CHECK();
+	return N2_OK;
 }
 
 N2_API int n2_composite_loss(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays,
@@ -438,7 +571,7 @@ int n2_composite_loss_filled(n2_stream_t stream, const n2_composite_config* cfg,
                              const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
                              const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
                              uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput,
-                             float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes, bool fill) {
+                             float* d_loss, uint32_t* d_source_index, void* d_workspace, uint64_t workspace_bytes, bool fill, const uint32_t* d_column_of) {
 	N2_REQUIRE(cfg != nullptr, "n2_composite_loss: config is null");
 	N2_REQUIRE(d_compacted_counter != nullptr, "n2_composite_loss: d_compacted_counter is null");
 	hipStream_t s = n2_stream(stream);
@@ -473,7 +606,7 @@ int n2_composite_loss_filled(n2_stream_t stream, const n2_composite_config* cfg,
 	}
 	composite_backward_kernel<<<grid, block, 0, s>>>(c, n_rays, d_numsteps, out, d_coords, d_rgb_target, scratch, kept_of, max_samples_compacted,
 	                                                 d_compacted_counter, d_coords_compacted, reinterpret_cast<hf*>(d_dloss_doutput), d_loss, d_source_index,
-	                                                 before_of, fill ? 1u : 0u, kept_of_block);
+	                                                 before_of, fill ? 1u : 0u, kept_of_block, d_column_of);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

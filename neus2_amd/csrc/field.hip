@@ -50,6 +50,7 @@ struct n2_field {
 	void* ws_sdf;
 	void* ws_rgb;
 	void* ws_grid;
+	hf* frag_image;  // the fused forward's weight fragments
 	bool fused;  // forward passes go through the fused kernels where the configuration allows (n2_field_set_fused)
 	bool slopes_saved;  // the last forward left the encoding's Jacobian as fp16 slopes (fused forward), not as fp32 dy_dx
 };
@@ -332,7 +333,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 }
 
 struct FieldCarve {
-	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_index, ws_sdf, ws_rgb, ws_grid, total;
+	uint64_t sdf_in, xyz, rgb_in, dy_dx, dsdf_din, d_rgb_in, d_sdf_in, v, d_density_in, var_part, sel_index, frag_image, ws_sdf, ws_rgb, ws_grid, total;
 };
 
 // nf: largest forward batch, nbw: largest batch that is also run backward
@@ -353,6 +354,7 @@ static FieldCarve carve(const n2_field_t* f, uint32_t nf, uint32_t nbw) {
 	c.d_density_in = take(2ull * f->sdf_in_w * n);
 	c.var_part = take(4ull * ((n + 127) / 128 + 1));  // one float per workgroup of whichever kernel forms the partial sums
 	c.sel_index = take(4ull * n);
+	c.frag_image = take(N2_FUSED_FRAG_BYTES);
 	c.ws_sdf = take(n2_mlp_workspace_bytes(f->sdf));
 	c.ws_rgb = take(n2_mlp_workspace_bytes(f->rgb));
 	c.ws_grid = take(n2_grid_workspace_bytes(f->grid, (uint32_t)nbw));
@@ -386,6 +388,7 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->d_density_in = reinterpret_cast<hf*>(b + c.d_density_in);
 	f->var_part = reinterpret_cast<float*>(b + c.var_part);
 	f->sel_index = reinterpret_cast<uint32_t*>(b + c.sel_index);
+	f->frag_image = reinterpret_cast<hf*>(b + c.frag_image);
 	f->last_n = 0;
 	f->sel_n = 0;
 	f->pad_n = {0, 0, 0};
@@ -418,6 +421,7 @@ static N2FusedNets fused_nets(const n2_field_t* f) {
 	nets.variance = reinterpret_cast<const n2_half*>(f->params + f->off_var);
 	nets.sdf_in_w = f->sdf_in_w;
 	nets.sdf_bias = f->sdf_bias;
+	nets.frag_image = reinterpret_cast<n2_half*>(f->frag_image);
 	return nets;
 }
 // the level mask can change between calls (n2_grid_set_max_level_gpu), so the check is made per call
@@ -468,6 +472,24 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 	                                                         reinterpret_cast<hf*>(d_output));
 	N2_LAUNCH_CHECK();
 	return N2_OK;
+}
+
+int n2_field_forward_listed(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_list, const uint32_t* d_counts,
+                            uint32_t round, uint32_t est_samples, n2_half* d_output) {
+	if (int rc = check_field(f, "n2_field_forward", n)) return rc;
+	if (n == 0) return N2_OK;
+	N2_REQUIRE(d_coords != nullptr && d_output != nullptr && d_list != nullptr && d_counts != nullptr, "n2_field_forward: null buffer");
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_output) % 16 == 0, "n2_field_forward: d_output must be 16-byte aligned");
+	N2_REQUIRE(f->fused && fused_ok(f), "n2_field_forward: a listed pass needs the fused kernels (n2_field_set_fused, no per-point level mask)");
+	hipStream_t s = n2_stream(stream);
+	f->last_n = n;
+	f->sel_n = 0;
+	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
+	f->slopes_saved = true;
+	f->pad_n.rgb_in = 0;
+	N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
+	return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx, reinterpret_cast<n2_half*>(f->dsdf_din),
+	                              reinterpret_cast<n2_half*>(f->rgb_in), d_output, nullptr, d_list, d_counts, round, est_samples);
 }
 
 N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n,

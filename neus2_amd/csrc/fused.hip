@@ -62,6 +62,15 @@ struct FusedArgs {
 	float sdf_bias;
 	uint32_t N;
 	const uint32_t* live;   // or null: only samples below min(*live, N) are evaluated (N stays the column count of the matrices)
+	// A listed pass (full field only; list null: off) evaluates the samples begin .. begin + counts[round] of the
+	// coordinates, begin = counts[0] + ... + counts[round - 1]: sample c writes row list[c] of the output, and everything
+	// the backward reads is stored at column c.
+	const uint32_t* list;
+	const uint32_t* counts;
+	uint32_t round, n_levels;
+	// full field: the weight fragments of the network kernel as one image in global memory (FF_COUNT KiB; null: every
+	// workgroup builds them from the weights).  The gather launch in front of the network kernel writes it.
+	hf* frags;
 	const float* pos;       // coordinate d of sample i at pos[i * ps + d * ds]; null: sample i is point lat.first + i of a lattice
 	uint32_t ps, ds;
 	N2Lattice lat;
@@ -89,15 +98,16 @@ __device__ __forceinline__ int sdf_col(int row, uint32_t enc_w) {
 }
 __device__ __forceinline__ int chained_k(int c, int g, int e) { return 16 * c + 4 * g + (e & 3) + ((e >> 2) << 3); }
 
-__device__ __forceinline__ void build_fused_frags(hf* F, const FusedArgs& a, int count) {
+// lane l's 16 bytes of fragment f
+__device__ __forceinline__ half8 fused_frag_value(const FusedArgs& a, int f, int l) {
 	const hf* W0s = a.sdf_w;
 	const int ld_s = (int)a.sdf_in_w;
 	const hf* W1s = W0s + MLP_WIDTH * ld_s;
 	const hf* W0c = a.rgb_w;
 	const hf* Whc = W0c + MLP_WIDTH * 48;
 	const hf* Woc = Whc + MLP_WIDTH * MLP_WIDTH;
-	for (int idx = threadIdx.x; idx < count * 64; idx += FF_BLOCK) {
-		const int f = idx >> 6, l = idx & 63, n = l & 31, g = l >> 5;
+	{
+		const int n = l & 31, g = l >> 5;
 		half8 v = zero8();
 		if (f < S_WO) {
 			const int mt = f / 3, c = f % 3, row = 32 * mt + n;
@@ -124,9 +134,25 @@ __device__ __forceinline__ void build_fused_frags(hf* F, const FusedArgs& a, int
 		} else {
 			if (n < MLP_OUT) v = wfrag_chained(Woc, MLP_WIDTH, n, f - C_WO, g);
 		}
-		*reinterpret_cast<half8*>(F + (size_t)idx * 8) = v;
+		return v;
 	}
+}
+
+__device__ __forceinline__ void build_fused_frags(hf* F, const FusedArgs& a, int count) {
+	for (int idx = threadIdx.x; idx < count * 64; idx += FF_BLOCK) *reinterpret_cast<half8*>(F + (size_t)idx * 8) = fused_frag_value(a, idx >> 6, idx & 63);
 	__syncthreads();
+}
+// the same fragments copied from the image a gather launch left in global memory: 16 consecutive bytes per lane instead
+// of two-byte picks all over the weight matrices (5 to 7 us of a network launch went into those)
+__device__ __forceinline__ void load_fused_frags(hf* F, const hf* __restrict__ image, int count) {
+	for (int idx = threadIdx.x; idx < count * 64; idx += FF_BLOCK) *reinterpret_cast<half8*>(F + (size_t)idx * 8) = *reinterpret_cast<const half8*>(image + (size_t)idx * 8);
+	__syncthreads();
+}
+// Workgroups FRAG_BLOCKS .. of a gather launch (behind those that gather) write the image.
+constexpr uint32_t FRAG_BLOCKS = (FF_COUNT * 64 + 255) / 256;
+__device__ __forceinline__ void write_frag_image(const FusedArgs& a, uint32_t block) {
+	const uint32_t idx = block * 256u + threadIdx.x;
+	if (idx < (uint32_t)FF_COUNT * 64u) *reinterpret_cast<half8*>(a.frags + (size_t)idx * 8) = fused_frag_value(a, (int)(idx >> 6), (int)(idx & 63u));
 }
 
 // ----------------------------------------------------------------------------
@@ -265,27 +291,11 @@ constexpr uint32_t FG_BLOCK = 256;
 
 // FULL: positions from the [N][7] coordinates, slopes and the coordinate rows are written; else positions with the
 // strides (ps, ds) and the feature rows only (inference on points in no particular order).
+// one (sample, level) item: the sample's coordinates are row `src` of the input, what it writes goes to column i
 template <bool FULL>
-__global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
-	// level-major workgroup ids: the workgroups that run at one time work on one or two levels, whose tables stay in every
-	// L2.  The launch is bound by the L2s' request rate: 10 M requests for the training step's 2.6e5 ray-ordered samples
-	// (four lines per sample on every level whose cells are smaller than the marching step), 63 % of them hits.  Measured on
-	// that workload and dropped: whole levels dealt to XCDs by a cost plan (the launch then fetches a third of the 278 MiB,
-	// but takes 9 to 20 us longer with every cost model tried), one 8- or 16-byte load per pair of x neighbours instead of
-	// two 4-byte loads (+12 us), a pair of lanes per sample so that the x neighbours' line is looked up once (+2 us), loads of
-	// the hashed levels that bypass the L1 (agent- or system-scope: +27 us, the x neighbour's line is then requested twice and
-	// a request is no cheaper) or carry the non-temporal hint (no change).
-	// Staging the coarse levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch
-	// and the five dense levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the
-	// positions and writing 320 bytes of features and slopes per sample.
-	// The trainer's sample generator runs beside this kernel on a second stream: where a wave of each is ready on a SIMD, this
-	// one issues first (the generator has the rest of the step to finish; measured 4 us on the forward, 2 us on the step).
-	__builtin_amdgcn_s_setprio(3);
-	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
-	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
+__device__ __forceinline__ void gather_item(const FusedArgs& a, uint32_t level, uint32_t i, uint32_t src) {
 	const uint32_t N = a.N;
-	if (i >= N || (a.live && i >= *a.live)) return;
-	const float* q = FULL ? a.coords + (size_t)i * 7 : a.pos + (size_t)i * a.ps;
+	const float* q = FULL ? a.coords + (size_t)src * 7 : a.pos + (size_t)src * a.ps;
 	const size_t qs = FULL ? 1 : a.ds;
 	const float p[3] = {q[0], q[qs], q[2 * qs]};
 	if (FULL && level == 0) {
@@ -320,6 +330,60 @@ __global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs 
 	}
 }
 
+// first column and number of samples of a listed pass
+__device__ __forceinline__ void listed_range(const FusedArgs& a, uint32_t& begin, uint32_t& count) {
+	begin = 0;
+	for (uint32_t q = 0; q < a.round; ++q) begin += a.counts[q];
+	count = min(a.counts[a.round], a.N - min(begin, a.N));
+}
+
+// The listed pass: the number of samples is known on the device only.  The launch has est_tiles workgroups per level, level-
+// major like the other kernel's; workgroup t of a level takes the tiles t, t + est_tiles, ...: any estimate gives the right
+// result, a good one gives every workgroup one tile.  (A fixed number of workgroups that walk all items by a stride is
+// 1.6 times slower beside the trainer's sample generator: its waves keep some of them from starting until others have
+// finished their whole share.)
+__global__ void __launch_bounds__(FG_BLOCK) field_gather_list_kernel(const FusedArgs a, uint32_t est_tiles) {
+	__builtin_amdgcn_s_setprio(3);
+	const uint32_t level = blockIdx.x / est_tiles;
+	if (level >= a.n_levels) {  // the network kernel's weight fragments (round 0 only)
+		write_frag_image(a, blockIdx.x - a.n_levels * est_tiles);
+		return;
+	}
+	uint32_t begin, count;
+	listed_range(a, begin, count);
+	const uint32_t tiles = (count + FG_BLOCK - 1) / FG_BLOCK;
+	for (uint32_t tile = blockIdx.x - level * est_tiles; tile < tiles; tile += est_tiles) {
+		const uint32_t j = tile * FG_BLOCK + threadIdx.x;
+		if (j < count) gather_item<true>(a, level, begin + j, begin + j);
+	}
+}
+
+template <bool FULL>
+__global__ void __launch_bounds__(FG_BLOCK) field_gather_kernel(const FusedArgs a, uint32_t tiles) {
+	// level-major workgroup ids: the workgroups that run at one time work on one or two levels, whose tables stay in every
+	// L2.  The launch is bound by the L2s' request rate: 10 M requests for the training step's 2.6e5 ray-ordered samples
+	// (four lines per sample on every level whose cells are smaller than the marching step), 63 % of them hits.  Measured on
+	// that workload and dropped: whole levels dealt to XCDs by a cost plan (the launch then fetches a third of the 278 MiB,
+	// but takes 9 to 20 us longer with every cost model tried), one 8- or 16-byte load per pair of x neighbours instead of
+	// two 4-byte loads (+12 us), a pair of lanes per sample so that the x neighbours' line is looked up once (+2 us), loads of
+	// the hashed levels that bypass the L1 (agent- or system-scope: +27 us, the x neighbour's line is then requested twice and
+	// a request is no cheaper) or carry the non-temporal hint (no change).
+	// Staging the coarse levels in LDS has nothing to win: with all caches cold, levels 0..2 together add 2 us to the launch
+	// and the five dense levels 4 us, against 5 to 6 us for each of the fine hashed levels and 19 us for reading the
+	// positions and writing 320 bytes of features and slopes per sample.
+	// The trainer's sample generator runs beside this kernel on a second stream: where a wave of each is ready on a SIMD, this
+	// one issues first (the generator has the rest of the step to finish; measured 4 us on the forward, 2 us on the step).
+	__builtin_amdgcn_s_setprio(3);
+	const uint32_t level = blockIdx.x / tiles, tile = blockIdx.x - level * tiles;
+	if (FULL && level >= a.n_levels) {  // the workgroups behind the last level: the network kernel's weight fragments
+		write_frag_image(a, blockIdx.x - a.n_levels * tiles);
+		return;
+	}
+	const uint32_t i = tile * FG_BLOCK + threadIdx.x;
+	if (i >= a.N || (a.live && i >= *a.live)) return;
+	gather_item<FULL>(a, level, i, i);
+}
+
 // ----------------------------------------------------------------------------
 // the network kernel: a wave takes 32 samples per pass, lane (n, g) works for sample b0 + n on the levels l(j, g).
 // GATHER: the features come from the table (inference on points in lattice order); else from the rows the gather kernel wrote.
@@ -334,10 +398,12 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 	unsigned char* const stage = smem + (size_t)(FULL ? FF_COUNT : FF_SDF_COUNT) * 1024 + FF_LEVELS * sizeof(uint4) + (threadIdx.x >> 6) * (32 * 2 * N2_RGB_IN_PITCH);
 	if (threadIdx.x < FF_LEVELS)
 		LV[threadIdx.x] = make_uint4(__float_as_uint(a.lv.scale[threadIdx.x]), a.lv.res[threadIdx.x], a.lv.entries[threadIdx.x], a.lv.offset[threadIdx.x]);
-	build_fused_frags(F, a, FULL ? FF_COUNT : FF_SDF_COUNT);
+	if (FULL && a.frags) load_fused_frags(F, a.frags, FF_COUNT);
+	else build_fused_frags(F, a, FULL ? FF_COUNT : FF_SDF_COUNT);
 	const int lane = threadIdx.x & 63, n = lane & 31, g = lane >> 5;
 	const uint32_t N = a.N, hash_mask = a.lv.hash_mask, active = a.lv.active_levels;
-	const uint32_t n_live = a.live ? min(*a.live, N) : N;
+	uint32_t n_live = a.live ? min(*a.live, N) : N, col0 = 0;
+	if (FULL && a.list) listed_range(a, col0, n_live);  // a listed pass: columns col0 .. col0 + n_live
 	const uint32_t n_tiles = (n_live + 31u) / 32u;
 	const uint32_t wave_gid = blockIdx.x * (FF_BLOCK / 64) + (threadIdx.x >> 6), n_waves = gridDim.x * (FF_BLOCK / 64);
 	// (Loading a wave's next tile while the current one is computed, into the registers the current operands have left, was
@@ -345,7 +411,8 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 	for (uint32_t tile = wave_gid; tile < n_tiles; tile += n_waves) {
 		const uint32_t col_raw = tile * 32u + n;
 		const bool valid = col_raw < n_live;
-		const uint32_t col = valid ? col_raw : n_live - 1u;
+		const uint32_t col = col0 + (valid ? col_raw : n_live - 1u);
+		const uint32_t dst = (FULL && a.list) ? a.list[col] : col;  // the sample's row in the output
 		half8 xs[3];               // SDF net input, B operands
 		float p[3], dir[3] = {0.f, 0.f, 0.f};
 		uint4 slope[8];            // FULL: the slopes of the lane's 8 levels as stored
@@ -502,7 +569,7 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 			__builtin_amdgcn_wave_barrier();
 			__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 			const uint32_t chunks = 5u * min(32u, n_live - tile * 32u);  // 16-byte chunks of the tile's samples
-			unsigned char* out = reinterpret_cast<unsigned char*>(a.rgb_in) + (size_t)tile * (32u * 2u * N2_RGB_IN_PITCH);
+			unsigned char* out = reinterpret_cast<unsigned char*>(a.rgb_in) + ((size_t)col0 + (size_t)tile * 32u) * (2u * N2_RGB_IN_PITCH);
 #pragma unroll
 			for (int i = 0; i < 3; ++i) {
 				const uint32_t k = (uint32_t)lane + 64u * i;
@@ -544,7 +611,7 @@ __global__ void __launch_bounds__(FF_BLOCK, 2) field_fused_forward_kernel(const 
 			lo[0] = hn[0]; lo[1] = hn[1]; lo[2] = hn[2]; lo[3] = a.variance[0];
 		}
 		if (valid) {
-			hf* o = a.output + (size_t)col * MLP_OUT;
+			hf* o = a.output + (size_t)dst * MLP_OUT;
 			*reinterpret_cast<half4*>(o + 4 * g) = lo;
 			*reinterpret_cast<half4*>(o + 8 + 4 * g) = hi;
 		}
@@ -566,7 +633,7 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 template <bool FULL>
 static void launch_gather(const FusedArgs& a, const N2LevelTable& tab, hipStream_t s) {
 	const uint32_t tiles = (a.N + FG_BLOCK - 1) / FG_BLOCK;
-	field_gather_kernel<FULL><<<dim3(tiles * tab.n_levels), dim3(FG_BLOCK), 0, s>>>(a, tiles);
+	field_gather_kernel<FULL><<<dim3(tiles * tab.n_levels + (FULL && a.frags ? FRAG_BLOCKS : 0u)), dim3(FG_BLOCK), 0, s>>>(a, tiles);
 }
 
 static uint32_t fused_grid(uint32_t n) {
@@ -596,16 +663,26 @@ static FusedArgs fused_base(const N2FusedNets& nets, uint32_t n) {
 	a.variance = reinterpret_cast<const hf*>(nets.variance);
 	a.sdf_in_w = nets.sdf_in_w;
 	a.enc_w = tab.n_levels * 2;
+	a.n_levels = tab.n_levels;
 	a.sdf_bias = nets.sdf_bias;
 	a.N = n;
 	a.live = nullptr;
+	a.list = nullptr;
+	a.counts = nullptr;
+	a.round = 0;
+	a.frags = nullptr;
 	return a;
 }
 
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live) {
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live, const uint32_t* d_list,
+                           const uint32_t* d_counts, uint32_t round, uint32_t est_samples) {
 	FusedArgs a = fused_base(nets, n);
 	a.live = d_live;
+	a.list = d_list;
+	a.counts = d_counts;
+	a.round = round;
+	a.frags = reinterpret_cast<hf*>(nets.frag_image);
 	a.coords = d_coords;
 	a.sdf_in = reinterpret_cast<hf*>(sdf_in);
 	a.xyz_rows = xyz_rows;
@@ -613,6 +690,18 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 	a.dsdf_din = reinterpret_cast<hf*>(dsdf_din);
 	a.rgb_in = reinterpret_cast<hf*>(rgb_in);
 	a.output = reinterpret_cast<hf*>(d_output);
+	if (d_list) {
+		// est_samples: the caller's estimate of this round's sample count (it only sizes the launches)
+		const uint32_t est = est_samples < 1u ? 1u : (est_samples > n ? n : est_samples);
+		const uint32_t est_tiles = (est + FG_BLOCK - 1) / FG_BLOCK;
+		field_gather_list_kernel<<<dim3(est_tiles * a.n_levels + (a.frags && round == 0 ? FRAG_BLOCKS : 0u)), dim3(FG_BLOCK), 0, s>>>(a, est_tiles);
+		N2_LAUNCH_CHECK();
+		// one 32-sample tile per wave where the estimate holds (the weight fragments come as a copy, so small workgroups are cheap)
+		const uint32_t blocks = (est + 127u) / 128u;
+		field_fused_forward_kernel<true, false><<<dim3(blocks < 2048u ? blocks : 2048u), dim3(FF_BLOCK), fused_lds(FF_COUNT, true), s>>>(a);
+		N2_LAUNCH_CHECK();
+		return N2_OK;
+	}
 	launch_gather<true>(a, *nets.tab, s);
 	N2_LAUNCH_CHECK();
 	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT, true), s>>>(a);

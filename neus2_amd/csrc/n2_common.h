@@ -75,7 +75,9 @@ struct N2FusedNets {
 	const n2_half* variance;
 	uint32_t sdf_in_w;
 	float sdf_bias;
+	n2_half* frag_image;  // N2_FUSED_FRAG_BYTES of scratch for the full forward's weight fragments (written by its gather launch), or null
 };
+constexpr uint64_t N2_FUSED_FRAG_BYTES = 40 * 1024;
 const N2LevelTable* n2_grid_table(const n2_grid_t* grid);
 const __half2* n2_grid_params(const n2_grid_t* grid);
 bool n2_grid_lattice_order(const n2_grid_t* grid);
@@ -90,7 +92,14 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 // d feature / d position without the level's scale factor, n2_slopes_pack) and the [n][16] output.
 // d_live (or null): a device counter; only samples below min(*d_live, n) are evaluated, n stays the matrices' column count.
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
-                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live = nullptr);
+                           void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live = nullptr,
+                           const uint32_t* d_list = nullptr, const uint32_t* d_counts = nullptr, uint32_t round = 0, uint32_t est_samples = 0);
+// One round of a forward pass in depth chunks (n2_composite_chunk_next): the samples begin .. begin + d_counts[round] of
+// d_coords_listed, begin = d_counts[0] + ... + d_counts[round - 1].  The output of sample c goes to row d_list[c] of d_output;
+// what the backward reads is stored at column c (n2_field_select then takes list positions).  est_samples: the caller's
+// estimate of d_counts[round], which sizes the launches (any value gives the same results).
+int n2_field_forward_listed(n2_field_t* field, n2_stream_t stream, const float* d_coords_listed, uint32_t n, const uint32_t* d_list, const uint32_t* d_counts,
+                            uint32_t round, uint32_t est_samples, n2_half* d_output);
 // n2_field_forward over the samples below min(*d_live, n): the trainer's marched samples fill only part of the window it
 // evaluates (the window is the count measured some steps earlier, rounded up); what lies behind them is not computed.
 int n2_field_forward_live(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output);
@@ -112,7 +121,17 @@ int n2_fused_field_sdf(const N2FusedNets& nets, hipStream_t s, const float* d_xy
 int n2_composite_loss_filled(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays, const uint32_t* d_ray_counter, uint32_t* d_numsteps,
                              const n2_half* d_network_output, const float* d_coords, const float* d_rgb_target, uint32_t max_samples_compacted,
                              uint32_t* d_compacted_counter, float* d_coords_compacted, n2_half* d_dloss_doutput, float* d_loss, uint32_t* d_source_index,
-                             void* d_workspace, uint64_t workspace_bytes, bool fill);
+                             void* d_workspace, uint64_t workspace_bytes, bool fill, const uint32_t* d_column_of = nullptr);
+// Forward pass in depth chunks (composite.hip): round `round` retires the rays whose transmittance behind the samples
+// listed last is below the compositor's cut and lists the next `chunk` samples of the others.  d_counts[r]: samples of
+// round r (d_counts_other: the counters of the following step, cleared by round 0); d_list: marched sample of every listed
+// sample, rounds side by side; d_column_of: the inverse map; d_coords_listed: the coordinate rows of the listed samples in
+// list order.  d_column_of goes to n2_composite_loss_filled, whose source_index then names list positions.
+constexpr uint32_t N2_CHUNK_MAX_ROUNDS = 8;
+uint64_t n2_composite_chunk_state_bytes(uint32_t max_rays);
+int n2_composite_chunk_next(n2_stream_t stream, const n2_composite_config* cfg, uint32_t n_rays, const uint32_t* d_ray_counter, const uint32_t* d_numsteps,
+                            const n2_half* d_network_output, const float* d_coords, uint32_t round, uint32_t chunk, void* d_state, uint32_t* d_counts,
+                            uint32_t* d_counts_other, uint32_t* d_list, uint32_t* d_column_of, float* d_coords_listed);
 
 // What the field hangs on its colour net's backward launch (n2_mlp_backward_rows_indexed): for the same samples,
 //   * row 0 of d_dL_dinput also takes row 3 of d_dL_doutput (the direct gradient of the SDF output);

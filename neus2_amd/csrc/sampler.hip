@@ -56,7 +56,35 @@ __device__ __forceinline__ float to_next_voxel(const float* pos, const float* di
 struct RaySetup {
 	bool alive;
 	float o[3], dir[3], idir[3], startt, target[3];
+	float tmax;  // where the ray leaves the unit cube (below startt: it misses the cube)
 };
+
+// A coarse, dilated copy of the bitfield's first level, rebuilt by every sample generation: bit x + 32 y + 1024 z is set
+// when any of the 4^3 cells of coarse cell (x, y, z) or of its 26 neighbours is occupied.  The march uses it to leave out,
+// for certain, what cannot hold a sample: rays that pass no occupied cell at all, and the part of a ray behind the last
+// occupied cell it can reach.  (In morton order the 64 cells of an aligned 4^3 block are 64 consecutive bits.)
+constexpr uint32_t COARSE = 32, COARSE_WORDS = COARSE * COARSE * COARSE / 32;
+__global__ void __launch_bounds__(256) sampler_coarse_kernel(const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ coarse) {
+	const uint32_t cell = blockIdx.x * 256u + threadIdx.x;  // x + 32 y + 1024 z
+	const int x = (int)(cell % COARSE), y = (int)((cell / COARSE) % COARSE), z = (int)(cell / (COARSE * COARSE));
+	const unsigned long long* blocks = reinterpret_cast<const unsigned long long*>(bitfield);
+	bool any = false;
+#pragma unroll
+	for (int dz = -1; dz <= 1; ++dz)
+#pragma unroll
+		for (int dy = -1; dy <= 1; ++dy)
+#pragma unroll
+			for (int dx = -1; dx <= 1; ++dx) {
+				const int nx = x + dx, ny = y + dy, nz = z + dz;
+				// (every load is issued whatever the others return: a neighbour outside the cube reads the cell itself)
+				const bool out = nx < 0 || ny < 0 || nz < 0 || nx >= (int)COARSE || ny >= (int)COARSE || nz >= (int)COARSE;
+				const uint32_t ux = out ? (uint32_t)x : (uint32_t)nx, uy = out ? (uint32_t)y : (uint32_t)ny, uz = out ? (uint32_t)z : (uint32_t)nz;
+				const uint32_t m = expand_bits(ux) | (expand_bits(uy) << 1) | (expand_bits(uz) << 2);
+				any |= blocks[m] != 0ull;
+			}
+	const unsigned long long bits = __ballot(any);
+	if ((threadIdx.x & 63u) == 0) { coarse[cell / 32u] = (uint32_t)bits; coarse[cell / 32u + 1u] = (uint32_t)(bits >> 32); }
+}
 
 __device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
                                               const n2_camera* __restrict__ cams, uint32_t n_images, const float* __restrict__ rgba,
@@ -100,6 +128,7 @@ __device__ __forceinline__ RaySetup setup_ray(uint32_t i, uint32_t n_rays, uint3
 		if (b < tmax) tmax = b;
 	}
 	if (!hit) tmin = 3.402823466e38f;
+	r.tmax = hit ? tmax : -1.0f;
 	tmin = fmaxf(tmin, 0.0f);
 	r.startt = __fmaf_rn(STEP, rand01(seed, i, 3), tmin);
 	r.alive = true;
@@ -159,13 +188,32 @@ __device__ __forceinline__ float window_t(float t_first, uint32_t lane) {
 }
 
 // Returns the number of samples; mask[2 w], mask[2 w + 1]: which steps of window w emitted; t_first[w]: t of its first step.
-__device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ mask,
-                                               float* __restrict__ t_first_out) {
+__device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t* __restrict__ bitfield, const uint32_t* __restrict__ coarse,
+                                               uint32_t* __restrict__ mask, float* __restrict__ t_first_out) {
 	const uint32_t lane = threadIdx.x & 63u;
 	uint32_t j = 0;
 	float t_first = r.startt;  // t of the window's first step
 	float pending = -3.4e38f;  // steps with t below this are skipped (target of the last visited empty step)
+	// Where the march may stop.  The stretch of the ray inside the cube is cut into 64 pieces, one per lane; a piece is at
+	// most sqrt(3) / 64 long, less than a coarse cell (1 / 32), so every point of it lies in the coarse cell of its
+	// midpoint or in a neighbour of that cell: when the dilated bit of the midpoint's cell is clear, no step of the piece is
+	// occupied.  No bit set: the ray has no sample.  Else no step behind the last piece with a set bit is occupied: the
+	// serial march would only walk on to the cube's far side without emitting anything, so it ends there with the same
+	// samples.  (A ray outside these assumptions marches all the way.)
+	float t_stop = 3.4e38f;
+	if (coarse != nullptr && r.tmax > r.startt && r.startt >= 0.f && r.tmax - r.startt < 2.0f) {
+		const float piece = (r.tmax - r.startt) * (1.0f / 64.0f);
+		const float tm = r.startt + ((float)lane + 0.5f) * piece;
+		uint32_t c[3];
+#pragma unroll
+		for (int k = 0; k < 3; ++k) c[k] = (uint32_t)min(max((int)((tm * r.dir[k] + r.o[k]) * (float)COARSE), 0), (int)COARSE - 1);
+		const uint32_t cell = c[0] + COARSE * c[1] + COARSE * COARSE * c[2];
+		const unsigned long long maybe = __ballot((coarse[cell >> 5] >> (cell & 31u)) & 1u);
+		if (maybe == 0ull) return 0u;
+		t_stop = r.startt + ((float)(64 - (int)__clzll((long long)maybe)) + 0.5f) * piece;
+	}
 	for (uint32_t w = 0; w < WINDOWS; ++w) {
+		if (t_first > t_stop) break;  // nothing behind this point can emit
 		WindowShape ws;
 		const float t = window_t(t_first, lane, ws);
 		float pos[3];
@@ -254,14 +302,14 @@ __device__ __forceinline__ uint32_t march_wave(const RaySetup& r, const uint8_t*
 
 __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_count_kernel(uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* __restrict__ cams,
                                                             uint32_t n_images, const float* __restrict__ rgba, float bg0, float bg1, float bg2,
-                                                            const uint8_t* __restrict__ bitfield, uint32_t* __restrict__ counts,
-                                                            uint32_t* __restrict__ mask, float* __restrict__ t_first,
+                                                            const uint8_t* __restrict__ bitfield, const uint32_t* __restrict__ coarse,
+                                                            uint32_t* __restrict__ counts, uint32_t* __restrict__ mask, float* __restrict__ t_first,
                                                             uint32_t* __restrict__ ray_counter) {
 	if (blockIdx.x == 0 && threadIdx.x == 0) *ray_counter = 0u;  // the scan kernel adds the kept rays up
 	const uint32_t i = blockIdx.x * RAYS_PER_BLOCK + (threadIdx.x >> 6);
 	if (i >= n_rays) return;
 	const RaySetup r = setup_ray(i, n_rays, n_rays_total, seed, cams, n_images, rgba, bg0, bg1, bg2);
-	const uint32_t n = r.alive ? march_wave(r, bitfield, mask + (size_t)i * 2 * WINDOWS, t_first + (size_t)i * WINDOWS) : 0u;
+	const uint32_t n = r.alive ? march_wave(r, bitfield, coarse, mask + (size_t)i * 2 * WINDOWS, t_first + (size_t)i * WINDOWS) : 0u;
 	if ((threadIdx.x & 63u) == 0) counts[i] = n;
 }
 
@@ -375,7 +423,7 @@ static inline uint64_t up256(uint64_t x) { return (x + 255) / 256 * 256; }
 static inline uint32_t scan_blocks(uint32_t n_rays) { return (n_rays + 1023u) / 1024u; }
 
 N2_API uint64_t n2_sampler_workspace_bytes(uint32_t max_rays) {
-	return 3 * up256(4ull * max_rays) + 2 * up256(4ull * 2 * WINDOWS * max_rays) + 2 * up256(4ull * scan_blocks(max_rays));
+	return 3 * up256(4ull * max_rays) + 2 * up256(4ull * 2 * WINDOWS * max_rays) + 2 * up256(4ull * scan_blocks(max_rays)) + up256(4ull * COARSE_WORDS);
 }
 
 N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
@@ -404,10 +452,14 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	float* t_first = reinterpret_cast<float*>(w + 3 * up256(4ull * n_rays) + up256(4ull * 2 * WINDOWS * n_rays));
 	uint32_t* block_sum = reinterpret_cast<uint32_t*>(w + 3 * up256(4ull * n_rays) + 2 * up256(4ull * 2 * WINDOWS * n_rays));
 	uint32_t* block_nz = block_sum + up256(4ull * scan_blocks(n_rays)) / 4;
+	uint32_t* coarse = block_nz + up256(4ull * scan_blocks(n_rays)) / 4;
 	const dim3 grid((n_rays + RAYS_PER_BLOCK - 1) / RAYS_PER_BLOCK), block(64 * RAYS_PER_BLOCK);
 	N2ProfScope prof(N2_PROF_SAMPLER, s);
+	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_bitfield) % 8 == 0, "n2_generate_training_samples: d_bitfield must be 8-byte aligned");
+	sampler_coarse_kernel<<<dim3(COARSE * COARSE * COARSE / 256), dim3(256), 0, s>>>(d_bitfield, coarse);
+	N2_LAUNCH_CHECK();
 	sampler_count_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                            background[2], d_bitfield, counts, mask, t_first, d_ray_counter);
+	                                            background[2], d_bitfield, coarse, counts, mask, t_first, d_ray_counter);
 	N2_LAUNCH_CHECK();
 	sampler_block_totals_kernel<<<dim3(scan_blocks(n_rays)), dim3(1024), 0, s>>>(n_rays, counts, block_sum, block_nz);
 	N2_LAUNCH_CHECK();

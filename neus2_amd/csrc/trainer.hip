@@ -49,6 +49,16 @@ struct n2_trainer {
 	uint32_t* counters;       // [0] live rays, [1] marched samples, [2] compacted samples (+ [4] as float: loss)
 	void* ws_composite;
 	uint64_t ws_sampler_bytes, ws_composite_bytes;
+	// forward pass in depth chunks (n2_trainer_set_depth_chunks)
+	uint32_t chunk_size, chunk_rounds;
+	uint32_t chunk_estimate[N2_CHUNK_MAX_ROUNDS];  // samples per round as last measured by the caller (0: not known)
+	uint32_t chunk_parity;    // which of the two counter sets the next chunked step uses
+	bool last_chunked;        // the last step ran in depth chunks
+	uint32_t* chunk_list;     // [max_samples] marched samples in the order of their evaluation
+	uint32_t* chunk_column;   // [max_samples] inverse map
+	float* chunk_coords;      // [max_samples][7] coordinate rows in list order
+	uint32_t* chunk_counts;   // [2][N2_CHUNK_MAX_ROUNDS]
+	void* chunk_state;
 	void* ws_field;
 	// scene
 	const n2_camera* cameras;
@@ -67,7 +77,7 @@ struct n2_trainer {
 
 struct TrainerCarve {
 	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], mlp_out, dloss, coords_compacted, src_index, numsteps[2], ray_indices[2], rgb_target[2],
-		set_counters[2], ray_loss, counters, ws_sampler[2], ws_composite, ws_field, total;
+		set_counters[2], ray_loss, counters, chunk_counts, chunk_list, chunk_column, chunk_state, chunk_coords, ws_sampler[2], ws_composite, ws_field, total;
 };
 
 static inline uint64_t a256(uint64_t x) { return (x + 255) / 256 * 256; }
@@ -101,6 +111,11 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	}
 	c.ray_loss = take(4 * R);
 	c.counters = take(64);
+	c.chunk_counts = take(2 * N2_CHUNK_MAX_ROUNDS * sizeof(uint32_t));
+	c.chunk_list = take(4 * S);
+	c.chunk_column = take(4 * S);
+	c.chunk_state = take(n2_composite_chunk_state_bytes((uint32_t)R));
+	c.chunk_coords = take(28 * S);
 	for (int i = 0; i < 2; ++i) c.ws_sampler[i] = take(n2_sampler_workspace_bytes((uint32_t)R));
 	c.ws_composite = take(n2_composite_workspace_bytes((uint32_t)R));
 	c.ws_field = take(n2_field_workspace_bytes(f, (uint32_t)(S > T ? S : T), (uint32_t)T));
@@ -184,6 +199,11 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->src_index = reinterpret_cast<uint32_t*>(b + c.src_index);
 	t->ray_loss = reinterpret_cast<float*>(b + c.ray_loss);
 	t->counters = reinterpret_cast<uint32_t*>(b + c.counters);
+	t->chunk_counts = reinterpret_cast<uint32_t*>(b + c.chunk_counts);
+	t->chunk_list = reinterpret_cast<uint32_t*>(b + c.chunk_list);
+	t->chunk_column = reinterpret_cast<uint32_t*>(b + c.chunk_column);
+	t->chunk_state = b + c.chunk_state;
+	t->chunk_coords = reinterpret_cast<float*>(b + c.chunk_coords);
 	t->ws_sampler_bytes = c.ws_sampler[1] - c.ws_sampler[0];
 	t->ws_composite = b + c.ws_composite;
 	t->ws_composite_bytes = c.ws_field - c.ws_composite;
@@ -316,17 +336,39 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	t->last_set = cur;
 	const n2_trainer::SampleSet& set = t->sets[cur];
 	const uint32_t* ray_counter = set.counters;
-	// field over every marched sample: the window of n_inference samples, of which the generator filled set.counters[1]
-	if (int rc = n2_field_forward_live(t->field, stream, set.coords, n_inference, set.counters + 1, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
-	// compositing, loss, gradients w.r.t. the outputs, compaction
 	n2_composite_config cc = t->cfg.composite;
 	cc.n_rays_norm = n_rays;
 	cc.loss_scale = t->cfg.loss_scale;
+	const bool chunked = t->chunk_rounds >= 2 && !t->cfg.recompute_training_forward;
+	if (chunked) {
+		// the field over the marched samples in depth chunks: only what lies in front of the rays' cuts (and at most a chunk
+		// behind them) is evaluated
+		uint32_t* counts = t->chunk_counts + N2_CHUNK_MAX_ROUNDS * t->chunk_parity;
+		uint32_t* counts_other = t->chunk_counts + N2_CHUNK_MAX_ROUNDS * (1u - t->chunk_parity);
+		t->chunk_parity ^= 1u;
+		for (uint32_t round = 0; round < t->chunk_rounds; ++round) {
+			const uint32_t chunk = round + 1 == t->chunk_rounds ? 0xFFFFFFFFu : t->chunk_size;
+			if (int rc = n2_composite_chunk_next(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords, round, chunk,
+			                                     t->chunk_state, counts, counts_other, t->chunk_list, t->chunk_column, t->chunk_coords)) return rc;
+			// the launches are sized by what the caller measured on earlier steps (with a margin), else by the most a round can hold
+			const uint64_t most = round + 1 == t->chunk_rounds ? n_inference : (uint64_t)n_rays * t->chunk_size;
+			uint64_t est = t->chunk_estimate[round] ? (uint64_t)t->chunk_estimate[round] * 9 / 8 + 1024 : most;
+			if (est > most) est = most;
+			if (est > n_inference) est = n_inference;
+			if (int rc = n2_field_forward_listed(t->field, stream, t->chunk_coords, n_inference, t->chunk_list, counts, round, (uint32_t)est,
+			                                     reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+		}
+	} else {
+		// field over every marched sample: the window of n_inference samples, of which the generator filled set.counters[1]
+		if (int rc = n2_field_forward_live(t->field, stream, set.coords, n_inference, set.counters + 1, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+	}
+	t->last_chunked = chunked;
+	// compositing, loss, gradients w.r.t. the outputs, compaction
 	// (the compacted batch comes back filled up to exactly T samples: fill_rollover_and_rescale on the output gradients,
 	// fill_rollover on the coordinates, src/testbed_nerf.cu:3908-3916)
 	if (int rc = n2_composite_loss_filled(stream, &cc, n_rays, ray_counter, set.numsteps, reinterpret_cast<const n2_half*>(t->mlp_out), set.coords,
 	                                      set.rgb_target, T, compacted_counter, t->coords_compacted, reinterpret_cast<n2_half*>(t->dloss),
-	                                      t->ray_loss, t->src_index, t->ws_composite, t->ws_composite_bytes, true)) return rc;
+	                                      t->ray_loss, t->src_index, t->ws_composite, t->ws_composite_bytes, true, chunked ? t->chunk_column : nullptr)) return rc;
 	// forward + backward on the compacted batch, then the optimiser.  Every compacted sample is one of the marched
 	// samples the field has just been evaluated on: unless asked to run the field again, the activations saved for it
 	// are selected instead (the same values, a fraction of the work).
@@ -354,6 +396,23 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		return n2_ema_step(stream, t->n_params, t->cfg.ema_decay, t->ema_steps, reinterpret_cast<const n2_half*>(t->params), t->ema_tmp,
 		                   reinterpret_cast<n2_half*>(t->ema));
 	}
+	return N2_OK;
+}
+
+N2_API int n2_trainer_set_depth_chunks(n2_trainer_t* t, uint32_t chunk_size, uint32_t n_rounds) {
+	N2_REQUIRE(t != nullptr, "n2_trainer_set_depth_chunks: trainer is null");
+	N2_REQUIRE(n_rounds <= N2_CHUNK_MAX_ROUNDS, "n2_trainer_set_depth_chunks: %u rounds, at most %u", n_rounds, N2_CHUNK_MAX_ROUNDS);
+	N2_REQUIRE(n_rounds < 2 || chunk_size >= 1, "n2_trainer_set_depth_chunks: chunk_size must be positive");
+	t->chunk_size = chunk_size;
+	t->chunk_rounds = n_rounds < 2 ? 0u : n_rounds;
+	for (uint32_t r = 0; r < N2_CHUNK_MAX_ROUNDS; ++r) t->chunk_estimate[r] = 0;
+	return N2_OK;
+}
+
+N2_API int n2_trainer_set_depth_chunk_estimates(n2_trainer_t* t, const uint32_t* samples_per_round, uint32_t n_rounds) {
+	N2_REQUIRE(t != nullptr && (samples_per_round != nullptr || n_rounds == 0), "n2_trainer_set_depth_chunk_estimates: null argument");
+	N2_REQUIRE(n_rounds <= N2_CHUNK_MAX_ROUNDS, "n2_trainer_set_depth_chunk_estimates: %u rounds, at most %u", n_rounds, N2_CHUNK_MAX_ROUNDS);
+	for (uint32_t r = 0; r < N2_CHUNK_MAX_ROUNDS; ++r) t->chunk_estimate[r] = r < n_rounds ? samples_per_round[r] : 0u;
 	return N2_OK;
 }
 
@@ -414,6 +473,8 @@ N2_API int n2_trainer_last_step_view(n2_trainer_t* t, n2_trainer_step_view* out)
 	out->coords_compacted = t->coords_compacted;
 	out->dloss_doutput = reinterpret_cast<const n2_half*>(t->dloss);
 	out->source_index = t->src_index;
+	out->evaluated_samples = t->last_chunked ? t->chunk_list : nullptr;
+	out->evaluated_counts = t->last_chunked ? t->chunk_counts + N2_CHUNK_MAX_ROUNDS * (1u - t->chunk_parity) : nullptr;
 	return N2_OK;
 }
 

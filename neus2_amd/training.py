@@ -227,6 +227,9 @@ class Trainer:
         self.budget = RayBudget(self.cfg.target_batch_size, self.cfg.max_rays_per_batch, self.cfg.max_samples)
         self.step_index = 0
         self.lr_schedule = None  # an ExponentialDecay, when the optimizer configuration nests one
+        # update_budget switches the forward pass in depth chunks on and off by the measured ratio of marched to kept samples
+        self.auto_depth_chunks = True
+        self.depth_chunks = (0, 0)
 
     def __del__(self):
         try:
@@ -244,6 +247,12 @@ class Trainer:
         set_max_level live there; every step tells it the number of steps taken so far."""
         from .tcnn_api import GridEncoding
         return GridEncoding._borrowed(capi.lib().n2_field_encoding(self._field), self)
+
+    def set_depth_chunks(self, chunk_size, n_rounds):
+        """n2_trainer_set_depth_chunks: the field over the marched samples in rounds of ``chunk_size`` samples per ray, rays
+        past the compositor's cut dropping out between rounds (n_rounds < 2: off).  Results are bit-identical either way."""
+        check(capi.lib().n2_trainer_set_depth_chunks(self._h, C.c_uint32(chunk_size), C.c_uint32(n_rounds)), "n2_trainer_set_depth_chunks")
+        self.depth_chunks = (chunk_size, n_rounds) if n_rounds >= 2 else (0, 0)
 
     def set_parameters(self, master_np):
         self.master.copy_(torch.from_numpy(np.ascontiguousarray(master_np, np.float32)).to(self.master.device))
@@ -326,14 +335,22 @@ class Trainer:
         v = capi.TrainerStepView()
         check(capi.lib().n2_trainer_last_step_view(self._h, C.byref(v)), "n2_trainer_last_step_view")
         T = self.cfg.target_batch_size
-        return dict(coords=self._view(v.coords, n_samples * 7, torch.float32).view(-1, 7),
+        source_index = self._view(v.source_index, T, torch.int32)
+        extra = {}
+        if v.evaluated_samples:
+            # a step in depth chunks: the index names places in the list of evaluated samples
+            counts = self._view(v.evaluated_counts, 8, torch.int32)
+            evaluated = self._view(v.evaluated_samples, self.cfg.max_samples, torch.int32)[:int(counts.sum().item())]
+            source_index = evaluated[source_index.long()]
+            extra = dict(evaluated_samples=evaluated, evaluated_counts=counts)
+        return dict(**extra, coords=self._view(v.coords, n_samples * 7, torch.float32).view(-1, 7),
                     numsteps=self._view(v.numsteps, n_rays * 2, torch.int32).view(-1, 2),
                     rgb_target=self._view(v.rgb_target, n_rays * 3, torch.float32).view(-1, 3),
                     ray_indices=self._view(v.ray_indices, n_rays, torch.int32),
                     network_output=self._view(v.network_output, n_inference * 16, torch.float16).view(-1, 16),
                     coords_compacted=self._view(v.coords_compacted, T * 7, torch.float32).view(-1, 7),
                     dloss_doutput=self._view(v.dloss_doutput, T * 16, torch.float16).view(-1, 16),
-                    source_index=self._view(v.source_index, T, torch.int32))
+                    source_index=source_index)
 
     def read_counters(self):
         r, s, c, l = C.c_uint32(), C.c_uint32(), C.c_uint32(), C.c_float()
@@ -341,9 +358,30 @@ class Trainer:
               "n2_trainer_read_counters")
         return dict(rays=int(r.value), samples=int(s.value), compacted=int(c.value), loss=float(l.value))
 
+    # the forward pass in depth chunks pays (three rounds of sixteen samples) when a step marches this many times the
+    # samples it keeps, and is switched off again below the lower figure
+    DEPTH_CHUNKS_ON, DEPTH_CHUNKS_OFF = 1.6, 1.3
+    DEPTH_CHUNKS = (16, 3)
+
+    def _update_chunk_estimates(self):
+        """After a step in depth chunks: its rounds' sample counts size the launches of the following steps."""
+        v = capi.TrainerStepView()
+        check(capi.lib().n2_trainer_last_step_view(self._h, C.byref(v)), "n2_trainer_last_step_view")
+        if v.evaluated_counts and self.depth_chunks[1] >= 2:
+            counts = self._view(v.evaluated_counts, 8, torch.int32).cpu().numpy().astype(np.uint32)
+            check(capi.lib().n2_trainer_set_depth_chunk_estimates(self._h, counts.ctypes.data_as(C.c_void_p), C.c_uint32(self.depth_chunks[1])),
+                  "n2_trainer_set_depth_chunk_estimates")
+
     def update_budget(self):
         c = self.read_counters()
         ok = self.budget.update(c["rays"], c["samples"], c["compacted"])
+        if ok and self.auto_depth_chunks and not self.cfg.recompute_training_forward:
+            ratio = c["samples"] / max(1, min(c["compacted"], self.cfg.target_batch_size))
+            if ratio >= self.DEPTH_CHUNKS_ON and self.depth_chunks[1] < 2:
+                self.set_depth_chunks(*self.DEPTH_CHUNKS)
+            elif ratio <= self.DEPTH_CHUNKS_OFF and self.depth_chunks[1] >= 2:
+                self.set_depth_chunks(0, 0)
+            self._update_chunk_estimates()
         return c, ok
 
     def sdf(self, xyz):

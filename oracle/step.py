@@ -67,7 +67,7 @@ def _band(got, ref, rtol, what, scale=None, outlier_frac=0.0, atol=0.0):
 
 
 def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_total, seed, n_inference, target_batch_size, counters,
-                gpu, grads, background=(1.0, 1.0, 1.0), ek_loss_weight=0.01, loss_scale=128.0, rtol=2e-3):
+                gpu, grads, background=(1.0, 1.0, 1.0), ek_loss_weight=0.01, loss_scale=128.0, rtol=2e-3, evaluated=None):
     """Checks one GPU training step stage by stage, every stage against the oracle run on the GPU's own input to that
     stage, so that a wiring error (a wrong batch size in the eikonal term, a mis-scaled roll-over, loss_scale / n_rays)
     shows at the stage where it happens and nothing is blurred by the one-sample differences that the 1e-4
@@ -76,6 +76,8 @@ def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_
       gpu       numpy arrays of the step's device buffers (Trainer.last_step): coords, numsteps, rgb_target,
                 ray_indices, network_output, coords_compacted, dloss_doutput, source_index
       grads     the fp16 gradient vector the step left (as float32)
+      evaluated marched samples the GPU evaluated the field on when it ran the forward pass in depth chunks (the others lie
+                behind their rays' cuts and hold no output); None: all of them
     Returns a dict of the figures it checked."""
     f, T = field, target_batch_size
     # 1. sample generation: bit-exact
@@ -89,6 +91,13 @@ def verify_step(field: Field, params16, cameras, rgba, bitfield, n_rays, n_rays_
     # 2. field forward over every marched sample
     out_ref, _ = f.forward(params16, s["coords"][:S])
     out_gpu = gpu["network_output"][:S].astype(np.float32)
+    if evaluated is not None:
+        # what was not evaluated must lie behind the cut: the oracle's compositor is given its own values there, and stops
+        # at another sample than the GPU's if the GPU evaluated too little
+        skipped = np.ones(S, bool)
+        skipped[np.asarray(evaluated, np.int64)] = False
+        assert len(np.unique(evaluated)) == len(evaluated) and not skipped.all()
+        out_gpu[skipped] = orc.round_fp16(out_ref.T[skipped])
     for name, rows in (("rgb", slice(0, 3)), ("sdf", slice(3, 4)), ("normal", slice(4, 7)), ("variance", slice(7, 8)), ("dir", slice(8, 11))):
         _band(out_gpu[:, rows].T, out_ref[rows], rtol, f"field output {name}", outlier_frac=2e-4)
     # 3. compositing, loss, gradients and compaction, on the GPU's own network output

@@ -259,3 +259,69 @@ def test_step_without_samples_changes_nothing(setup):
     assert c["samples"] == 0 and c["compacted"] == 0
     assert torch.equal(tr.master, master) and torch.equal(tr.params, params)
     assert torch.equal(tr._view(st.first_moments, tr.n_params, torch.float32), m1)
+
+
+def test_depth_chunks_give_the_same_steps(oracle):
+    """On a trained field most rays pass the compositor's transmittance cut long before their last marched sample.  The
+    step can evaluate the field in rounds of a few samples per ray, dropping the rays that are past the cut between
+    rounds: parameters, gradients and counters are bit-identical to the plain step's (which evaluates every marched sample),
+    a fraction of the samples is evaluated, and a chunked step passes the stage-by-stage check against the oracle."""
+    from oracle.field import Field
+    from oracle.step import verify_step
+    from neus2_amd.tcnn_api import pack_cameras
+    from neus2_amd.training import OccupancyGrid, Trainer, default_config
+    cams = scene.cameras_on_sphere(32, 128)
+    rgba = scene.render_sphere_images(cams)
+    d_cams, d_rgba = pack_cameras(cams), dev(rgba)
+    T = 1 << 14
+    W = np.load(os.path.join(GOLD, "sdf_mlp_weights_48.npy"))
+
+    def make(bitfield=None):
+        tr = Trainer(default_config(target_batch_size=T, max_rays_per_batch=1 << 13, max_samples=1 << 19, background=(1.0, 1.0, 1.0)))
+        tr.auto_depth_chunks = False
+        tr.set_scene(d_cams, len(cams), d_rgba, bitfield if bitfield is not None else dev(scene.sphere_bitfield()))
+        return tr
+    # a trained state: the loop the reference drives (occupancy updates on their cadence, ray budget feedback)
+    a = make()
+    a.attach_occupancy(OccupancyGrid(1, seed=1337, max_chunk=1 << 19))
+    a.initialize_params(seed=1337, sdf_mlp_weights=W)
+    for it in range(500):
+        a.training_prep()
+        a.step()
+        if it % 16 == 15 or it < 16:
+            c, ok = a.update_budget()
+            assert ok, c
+    master = host(a.master).copy()
+    bits = a.occupancy.bitfield.clone()
+    n_rays, n_inf = a.budget.rays_per_batch, a.budget.n_inference()
+    assert c["samples"] > 1.3 * c["compacted"], c   # rays do end early in this state (after a hundred to two hundred samples)
+    runs = []
+    for chunks in ((0, 0), (96, 3), (16, 8), (1, 2)):
+        tr = make(bits)
+        tr.set_parameters(master)
+        tr.set_depth_chunks(*chunks)
+        seen = []
+        for step in range(4):
+            params16 = host(tr.params).copy()
+            tr.step(n_rays=n_rays, n_inference=n_inf, seed=100 + step)
+            cs = tr.read_counters()
+            view = tr.last_step(cs["rays"], cs["samples"], n_inf)
+            seen.append((cs, tr.grads.clone()))
+            if chunks[1]:
+                done = int(view["evaluated_counts"].sum().item())
+                assert min(cs["compacted"], T) <= done <= cs["samples"]
+                if chunks == (96, 3):
+                    assert done < 0.95 * cs["samples"], (done, cs)
+                if step == 1 and chunks == (96, 3):
+                    gpu = {k: host(v) for k, v in view.items()}
+                    res = verify_step(Field(fp16=True), params16, oc_cams(oracle, cams), rgba, host(bits), n_rays, n_rays, 101, n_inf, T, cs, gpu,
+                                      host(tr.grads), background=(1.0, 1.0, 1.0), evaluated=gpu["evaluated_samples"])
+                    assert res["compacted"] == cs["compacted"]
+        runs.append((seen, tr.master.clone()))
+        del tr
+    (ref_seen, ref_master) = runs[0]
+    for seen, m in runs[1:]:
+        for (ca, ga), (cb, gb) in zip(ref_seen, seen):
+            assert ca == cb and ca["compacted"] > 0
+            assert torch.equal(ga, gb)
+        assert torch.equal(ref_master, m)
