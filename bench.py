@@ -29,12 +29,72 @@ HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 ALGO_BYTES = {"grid_backward_params": 588, "grid_forward": 588, "grid_second_order": 664}
 STEP_ALGO_BYTES = {"grid_backward_params": 664, "grid_forward": 588}
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16
-# HBM bytes per launch of the step workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file
-# (profiles/training_step_2p18_hbm_traffic.txt; counters scaled by what a plain copy of known size reads):
-# scatter pair = bin (41.0 + 101.9 MiB) + reduce (110.9 + 24.0 MiB)
-STEP_TRAFFIC_BYTES = {"grid_backward_params": int(272.8 * 2**20)}
+# HBM bytes per launch of the step workload's kernels: read from profiles/training_step_2p18_hbm_traffic.json, which
+# `bench.py --summarize-traffic` writes from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this file (commands in the JSON
+# and in the .txt beside it; counters scaled by what a plain copy of known size reads in the same process)
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "training_step_2p18_hbm_traffic.json")
+SCATTER_KERNELS = ("grid_bin_kernel", "grid_reduce_kernel", "grid_combine_kernel")
 PROF = {"grid_forward": 0, "grid_backward_params": 1, "grid_second_order": 2, "mlp_forward": 3, "mlp_backward": 4,
-        "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9}
+        "mlp_second_order": 5, "composite": 6, "sampler": 7, "adam": 8, "field_forward": 9, "field_gather": 10}
+
+
+def short_kernel_name(name):
+    """Base name of a kernel as rocprofv3 prints it (mangled or not); the two weight-gradient instantiations a step
+    launches are told apart by their hidden-layer count."""
+    import re
+    m = re.search(r"([a-z][a-z0-9_]*_kernel)", name)
+    base = m.group(1) if m else name.split("(")[0][:48]
+    if base == "mlp_wgrad_kernel":
+        base += "<colour net>" if "Li3ELi2E" in name or "<3, 2," in name else "<SDF net>"
+    return base
+
+
+def step_traffic():
+    """Per-kernel HBM bytes of a step from the committed profile; the scatter's figure is what `roofline.traffic` reports."""
+    if not os.path.exists(TRAFFIC_JSON):
+        raise SystemExit(f"{TRAFFIC_JSON} is missing: run the two rocprofv3 --pmc commands it records and `bench.py --summarize-traffic`")
+    with open(TRAFFIC_JSON) as f:
+        t = json.load(f)
+    k = t["kernels"]
+    missing = [n for n in SCATTER_KERNELS[:2] if n not in k]
+    if missing:
+        raise SystemExit(f"{TRAFFIC_JSON} holds no entry for {missing}")
+    return t, sum(k[n]["fetch_bytes"] + k[n]["write_bytes"] for n in SCATTER_KERNELS if n in k)
+
+
+def summarize_traffic(fetch_csv, write_csv, copy_mib):
+    """rocprofv3 counter CSVs of `bench.py --calibrate-copy MIB` (one run with --pmc FETCH_SIZE, one with WRITE_SIZE) ->
+    the JSON this file reads: median launch of the second half of each kernel's launches (steady state), in bytes, scaled so
+    that the calibration copy reads its known size."""
+    import csv
+    import statistics
+
+    def load(path, counter):
+        per, copies = {}, []
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] != counter:
+                continue
+            v = float(r["Counter_Value"])
+            if "copyBuffer" in r["Kernel_Name"]:
+                copies.append(v)
+            per.setdefault(short_kernel_name(r["Kernel_Name"]), []).append(v)
+        if not copies:
+            raise SystemExit(f"{path}: no copy kernel found (run bench.py with --calibrate-copy)")
+        factor = copy_mib * 1024.0 / max(copies)   # the counters are in KiB
+        return {k: statistics.median(v[len(v) // 2:]) * 1024.0 * factor for k, v in per.items()}, factor
+    fetch, ff = load(fetch_csv, "FETCH_SIZE")
+    write, wf = load(write_csv, "WRITE_SIZE")
+    cmd = ("rocprofv3 --pmc {c} --kernel-trace --output-format csv -d gpurun_out/pp/{d} -o f -- python3 bench.py --no-cpu-baseline "
+           "--trained-steps 0 --extra-regions 0 --calibrate-copy %d --steps 20 --warmup 5" % copy_mib)
+    kernels = {k: {"fetch_bytes": int(fetch.get(k, 0.0)), "write_bytes": int(write.get(k, 0.0))}
+               for k in sorted(set(fetch) | set(write)) if "_kernel" in k and not k.startswith("at::")}
+    return {"workload": "default benchmark: full training step, 2^18 batch", "command_fetch": cmd.format(c="FETCH_SIZE", d="fetch"),
+            "command_write": cmd.format(c="WRITE_SIZE", d="write"),
+            "then": "python3 bench.py --calibrate-copy %d --summarize-traffic gpurun_out/pp/fetch/f_counter_collection.csv "
+                    "gpurun_out/pp/write/f_counter_collection.csv > profiles/training_step_2p18_hbm_traffic.json" % copy_mib,
+            "calibration": {"copy_mib": copy_mib, "fetch_factor": ff, "write_factor": wf,
+                            "note": "factor = known bytes of the calibration copy / what the counter read for it"},
+            "unit": "bytes per launch (median of the steady-state launches)", "kernels": kernels}
 
 
 def build_scene(n_cameras=64, resolution=512):
@@ -107,6 +167,11 @@ def run_step_workload(args):
     for _ in range(args.warmup):
         tr.step(n_rays=n_rays, n_inference=n_inf)
     torch.cuda.synchronize()
+    # one region of the same length is run and discarded first: the first region after the warm-up steps is consistently about
+    # one per cent slower than those that follow it (clocks and caches settle), and `value` is to be a steady-state figure
+    for _ in range(args.steps):
+        tr.step(n_rays=n_rays, n_inference=n_inf)
+    torch.cuda.synchronize()
     # timed region: K steps; only the roofline kernel (the parameter scatter) carries events, and only in five of the
     # steps, because every event pair costs stream time (about 13 us) that is charged to the step
     dom = "grid_backward_params"
@@ -143,6 +208,21 @@ def run_step_workload(args):
     # also runs over the marched samples, so use the average batch per launch
     per_launch = TARGET if dom != "grid_forward" else (TARGET + n_inf) / 2
     achieved = STEP_ALGO_BYTES[dom] * per_launch / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    traffic_profile, scatter_traffic = step_traffic()
+    # the other two large memory-bound launches of a step, from the untimed per-kernel pass: the gather over the marched
+    # samples (588 B per sample) and Adam (32 B per parameter with the trainer's 16-bit step counters, dense bound)
+    n_params = tr.n_params
+
+    def hbm_entry(key, kernel, bytes_per_unit, units, what):
+        if key not in kernels:
+            return None
+        gbs = bytes_per_unit * units / (kernels[key]["avg_us"] * 1e-6) / 1e9
+        k = traffic_profile["kernels"].get(kernel)
+        return {"kernel": kernel, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                "algorithmic_bytes": what, "units_per_launch": units, "avg_launch_us": kernels[key]["avg_us"],
+                "traffic": (k["fetch_bytes"] + k["write_bytes"]) if k else None}
+    rooflines = {"field_gather": hbm_entry("field_gather", "field_gather_kernel", 588, counters["samples"], "588 B per marched sample (12 xyz + 128 x 4 gathers + 64 features)"),
+                 "adam": hbm_entry("adam", "adam_step_kernel", 32, n_params, "32 B per parameter (dense bound, 16-bit step counters)")}
     if args.calibrate_copy:
         # a plain copy of known size in the same process: the scale of the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(args.calibrate_copy << 20, dtype=torch.uint8, device="cuda").zero_()
@@ -175,11 +255,13 @@ def run_step_workload(args):
                    "target_batch": TARGET, "rays_per_step": n_rays, "marched_samples_per_step": counters["samples"],
                    "inference_batch": n_inf, "compacted_before_rollover": counters["compacted"], "loss": counters["loss"]},
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": STEP_TRAFFIC_BYTES.get(dom),
-                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated; recorded from profiles/)",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": scatter_traffic,
+                     "traffic_unit": "bytes per launch of bin + reduce + combine (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated; "
+                                     "read from profiles/training_step_2p18_hbm_traffic.json)",
                      "algorithmic_bytes_per_sample": STEP_ALGO_BYTES[dom], "samples_per_launch": per_launch,
                      "avg_launch_us": kernels[dom]["avg_us"], "timed_launches": dom_n},
         "mfma": mfma,
+        "rooflines": rooflines,
         "kernels": kernels,
         "kernels_note": "grid_backward_params is timed with HIP events inside the timed region (five launches spread over the region); the other entries come from a "
                         "second, untimed pass of the same steps with every listed kernel bracketed by events",
@@ -198,9 +280,14 @@ def run_step_workload(args):
     result["regions"] = {"ms_per_step": regions, "median": srt[len(srt) // 2], "min": srt[0], "max": srt[-1],
                          "note": f"{len(regions)} consecutive regions of {args.steps} steps; the first one is the timed region of `value`"}
     # (ii) the same loop on a trained field: rays stop at the surface, so a step marches more samples than it keeps
+    result["settle_steps"] = args.steps  # the discarded region in front of the timed one (after the `warmup` steps)
     if args.trained_steps > 0:
         del tr
         result["trained_state"] = trained_state_leg(args, lib, d_cams, len(cams), d_rgba, sdf_w)
+        # both regimes side by side: `value` is the initial state (every marched sample is kept), the trained field marches
+        # about three samples for every one it keeps
+        result["config"]["trained_state_ms_per_step"] = result["trained_state"].get("ms_per_step")
+        result["config"]["trained_state_samples_per_s"] = result["trained_state"].get("value")
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cams, rgba, bits, sdf_w, n_rays, n_inf)
     return result
@@ -582,7 +669,15 @@ def main():
                     help="step workload: training steps before the trained-state leg (0 switches the leg off)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="after the timed region, copy MIB mebibytes device-to-device once (counter calibration under a profiler)")
+    ap.add_argument("--summarize-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: turn the counter CSVs of two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE, both with "
+                         "--calibrate-copy MIB) into the JSON that `roofline.traffic` is read from, on stdout")
     args = ap.parse_args()
+    if args.summarize_traffic:
+        if args.calibrate_copy <= 0:
+            raise SystemExit("--summarize-traffic needs --calibrate-copy MIB (the size of the calibration copy of the profiled runs)")
+        print(json.dumps(summarize_traffic(args.summarize_traffic[0], args.summarize_traffic[1], args.calibrate_copy), indent=1))
+        return
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs the hot path on ONE GPU (the reference has no multi-GPU path and the "
                          "benchmark metric is quoted on 1 GPU); run with --gpus 1")

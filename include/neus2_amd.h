@@ -446,7 +446,9 @@ int n2_ema_step(n2_stream_t stream, uint32_t n_params, float decay, uint32_t ste
 
 /* All buffers hold n_params elements and are caller-owned device memory:
  *  d_master fp32 weights, d_params fp16 copy (written), d_gradients fp16 (read),
- *  d_m1 / d_m2 fp32 moments, d_steps uint32 per-parameter step counters. */
+ *  d_m1 / d_m2 fp32 moments, d_steps uint32 per-parameter step counters.
+ * The first call on a device with a new pair of betas fills a table of bias corrections and waits for it (a stream
+ * synchronisation, a device synchronisation when all four table slots are taken): make that call outside graph capture. */
 int n2_adam_step(n2_stream_t stream, const n2_adam_config* config, uint32_t n_params, uint32_t n_matrix_params,
                  float loss_scale, float* d_master, n2_half* d_params, const n2_half* d_gradients, float* d_m1,
                  float* d_m2, uint32_t* d_steps);
@@ -507,7 +509,9 @@ int n2_composite_loss_indexed(n2_stream_t stream, const n2_composite_config* con
  * without ordering between them) race; calls ordered on one stream are safe.  Nothing in the array has to start at
  * zero: the forward kernel writes every ray's slot below n_rays (and, from 8192 rays on, the scan kernel every prefix sum)
  * before the backward kernel reads it.  Results are
- * bit-identical to n2_composite_loss_indexed's. */
+ * bit-identical to n2_composite_loss_indexed's.
+ * The first call on a device takes a lock and looks the array's address up (hipGetSymbolAddress, which may load the
+ * library's code object): make one call per device outside graph capture before capturing any. */
 #define N2_COMPOSITE_STATIC_MAX_RAYS 65536u
 int n2_composite_loss_static(n2_stream_t stream, const n2_composite_config* config, uint32_t n_rays,
                              const uint32_t* d_ray_counter, uint32_t* d_numsteps, const n2_half* d_network_output,
@@ -677,11 +681,16 @@ int n2_trainer_set_depth_chunk_estimates(n2_trainer_t* trainer, const uint32_t* 
  *  n_inference  how many marched samples the first forward covers (a multiple of 8, <= max_samples); the
  *               reference uses the sample count measured in earlier steps, rounded up to 128
  *               (src/testbed_nerf.cu:3751-3756)
- *  seed         seed of this step's random draws */
+ *  seed         seed of this step's random draws
+ * A step whose rays kept no sample leaves parameters and optimiser state alone (the reference stops training there,
+ * src/testbed_nerf.cu:3536-3542), but the host-side counts (optimizer_steps, the training step, the Ema's step count)
+ * advance with every call: they count calls, the device decides about the update. */
 int n2_trainer_step(n2_trainer_t* trainer, n2_stream_t stream, uint32_t n_rays, uint32_t n_inference, uint32_t seed);
 
 /* Device buffers of the last step, for inspection and tests (the reference keeps the same data in its arena allocation,
- * src/testbed_nerf.cu:3723-3749): valid until the next step overwrites them. */
+ * src/testbed_nerf.cu:3723-3749): valid until the next step overwrites them.  After this call the next n2_trainer_step
+ * orders its sample generation (which overwrites the sample set) behind everything enqueued on the step's stream so far, so
+ * work that reads the view may simply be enqueued on that stream before the next step. */
 typedef struct n2_trainer_step_view {
 	const float* coords;              /* [marched samples][7] of the step's sample set */
 	const uint32_t* numsteps;         /* [rays][2] after compositing: (kept samples, first compacted sample) per live ray */
@@ -870,7 +879,8 @@ typedef enum n2_prof_id {
 	N2_PROF_SAMPLER = 7,
 	N2_PROF_ADAM = 8,
 	N2_PROF_FIELD_FORWARD = 9, /* the fused forward kernels of the field (grid + networks in one launch) */
-	N2_PROF_COUNT = 10
+	N2_PROF_FIELD_GATHER = 10, /* the level-major gather launch inside N2_PROF_FIELD_FORWARD */
+	N2_PROF_COUNT = 11
 } n2_prof_id;
 
 int n2_profile_enable(int enable);

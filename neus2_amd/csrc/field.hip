@@ -499,8 +499,23 @@ N2_API int n2_field_backward(n2_field_t* f, n2_stream_t stream, const float* d_c
 	return n2_slab_reduce_launch(stream, sums);
 }
 
+static int field_backward_passes(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t ek_batch_size,
+                                 n2_grad_mode mode, N2SlabReduce* sums);
+
 int n2_field_backward_deferred(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t ek_batch_size,
                                n2_grad_mode mode, N2SlabReduce* sums) {
+	const int rc = field_backward_passes(f, stream, d_coords, n, d_dL_doutput, ek_batch_size, mode, sums);
+	if (rc != N2_OK && f != nullptr) {
+		// a pass that ran before the failure left partial sums pending in its network: nobody will reduce them
+		n2_mlp_drop_pending(f->rgb);
+		n2_mlp_drop_pending(f->sdf);
+		*sums = N2SlabReduce{};
+	}
+	return rc;
+}
+
+static int field_backward_passes(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t ek_batch_size,
+                                 n2_grad_mode mode, N2SlabReduce* sums) {
 	*sums = N2SlabReduce{};
 	if (int rc = check_field(f, "n2_field_backward", n)) return rc;
 	N2_REQUIRE(n <= f->max_batch_bwd, "n2_field_backward: batch %u exceeds the workspace's backward capacity %u", n, f->max_batch_bwd);

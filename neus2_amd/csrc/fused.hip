@@ -702,7 +702,10 @@ int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* 
 		N2_LAUNCH_CHECK();
 		return N2_OK;
 	}
-	launch_gather<true>(a, *nets.tab, s);
+	{
+		N2ProfScope prof(N2_PROF_FIELD_GATHER, s);
+		launch_gather<true>(a, *nets.tab, s);
+	}
 	N2_LAUNCH_CHECK();
 	field_fused_forward_kernel<true, false><<<dim3(fused_grid(n)), dim3(FF_BLOCK), fused_lds(FF_COUNT, true), s>>>(a);
 	N2_LAUNCH_CHECK();

@@ -525,6 +525,10 @@ static int check_pending(n2_mlp_t* mlp, const char* fn, uint32_t n_slabs, n2_gra
 	return N2_OK;
 }
 
+void n2_mlp_drop_pending(n2_mlp_t* mlp) {
+	if (mlp) mlp->pending_slabs = 0;
+}
+
 N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 	N2_REQUIRE(mlp != nullptr, "n2_mlp_set_deferred_reduction: mlp is null");
 	N2_REQUIRE(mlp->pending_slabs == 0, "n2_mlp_set_deferred_reduction: gradient passes are pending");

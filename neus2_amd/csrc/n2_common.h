@@ -184,6 +184,9 @@ bool n2_adam_counters_may_saturate(float beta1, float beta2);
 int n2_mlp_reduce_deferred_sum(n2_mlp_t* a, n2_mlp_t* b, n2_stream_t stream, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate);
 // The same work as a plan instead of a launch: what is pending is handed to *out (and no longer pending), for
 // n2_slab_reduce_launch or for a kernel that carries the summation (n2_adam_step_gated).
+// forgets the gradient passes that are pending (their partial sums are dropped): for the error path of a caller that will
+// not run the reduction
+void n2_mlp_drop_pending(n2_mlp_t* mlp);
 int n2_mlp_reduce_deferred_plan(n2_mlp_t* a, n2_mlp_t* b, const float* d_parts, uint32_t n_parts, n2_half* d_sum, int accumulate, N2SlabReduce* out);
 int n2_slab_reduce_launch(n2_stream_t stream, const N2SlabReduce& plan);
 // n2_field_backward that leaves the summation of the networks' weight-gradient slabs and of the variance gradient's partial

@@ -71,6 +71,8 @@ struct n2_trainer {
 	bool ev_main_from_adam;   // ev_main stands for the completion of the last step's Adam launch
 	hipEvent_t ev_main, ev_ready;
 	bool pf_valid;
+	bool view_taken;          // n2_trainer_last_step_view since the last step: the caller may have enqueued readers of the sample set
+	hipStream_t last_stream;  // stream of the last step
 	uint32_t pf_set, pf_n_rays, pf_n_inference, pf_seed, pf_ray_base;
 	uint32_t last_set;
 };
@@ -319,7 +321,9 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		const bool hit = t->pf_valid && t->pf_n_rays == n_rays && t->pf_n_inference == n_inference && t->pf_seed == seed && t->pf_ray_base == t->n_rays_total;
 		if (hit) {
 			cur = t->pf_set;
-			main_event_is_last_step = t->ev_main_from_adam;
+			// ev_main stands for the last step's Adam launch: enough unless the caller may have put readers of that step's
+			// buffers on the stream since (it asked for the view), or this step runs on another stream
+			main_event_is_last_step = t->ev_main_from_adam && !t->view_taken && s == t->last_stream;
 			N2_HIP(hipStreamWaitEvent(s, t->ev_ready, 0));
 		} else {
 			// a generation that ran ahead with other arguments is abandoned (it stays ordered on the side stream)
@@ -334,6 +338,8 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		t->n_rays_total += n_rays;
 	}
 	t->last_set = cur;
+	t->view_taken = false;
+	t->last_stream = s;
 	const n2_trainer::SampleSet& set = t->sets[cur];
 	const uint32_t* ray_counter = set.counters;
 	n2_composite_config cc = t->cfg.composite;
@@ -465,6 +471,7 @@ N2_API int n2_trainer_set_optimizer_steps(n2_trainer_t* t, uint32_t steps) {
 N2_API int n2_trainer_last_step_view(n2_trainer_t* t, n2_trainer_step_view* out) {
 	N2_REQUIRE(t != nullptr && out != nullptr, "n2_trainer_last_step_view: null argument");
 	const n2_trainer::SampleSet& set = t->sets[t->last_set];
+	t->view_taken = true;
 	out->coords = set.coords;
 	out->numsteps = set.numsteps;
 	out->rgb_target = set.rgb_target;

@@ -149,3 +149,39 @@ def test_lattice_512_chunks_and_subsample(oracle):
         e = density_on_grid(net._h, (R, R, 64), (0, 0, 0), (1, 1, 64 / R), chunk=chunk)
         assert torch.equal(e, sub), chunk
         del e
+
+
+def test_sdf_eikonal_step_2p18_against_oracle(oracle):
+    """BASELINE configuration 3 at its full size, through the entry points that configuration's benchmark times
+    (n2_sdf_pack_input, n2_grid_forward with the Jacobian, n2_mlp_forward_and_input_gradient, n2_sdf_eikonal_loss,
+    n2_mlp_backward, n2_grid_backward_fused, n2_mlp_backward_backward_input): 2^18 points uniform in the unit cube, the
+    SDF, the normals, the loss, the MLP's weight gradients and the encoding's gradients level by level against the oracle's
+    composition, at the tolerances of the small test (nerf_network.h:184-238, 402-429, 534-571)."""
+    from neus2_amd.sdf_net import SdfNet
+    from oracle.sdf_step import sdf_eikonal_step
+    rng = np.random.default_rng(70)
+    n = 1 << 18
+    net = SdfNet(max_batch=n)
+    P = q16(rng.uniform(-0.01, 0.01, net.grid.n_params()))
+    W = q16(np.load(os.path.join(GOLD, "sdf_mlp_weights_48.npy")) + rng.normal(0, 0.05, 4096))
+    x = rng.random((3, n), dtype=np.float32)
+    dP, dW = dev(P, torch.float16), dev(W, torch.float16)
+    gP, gW = torch.zeros_like(dP), torch.zeros_like(dW)
+    net.set_params(dP, gP, dW, gW)
+    ctx = net.forward(dev(x))
+    loss = float(net.loss_backward(ctx, ek_weight=0.1, loss_scale=128.0).item())
+    ref = sdf_eikonal_step(P, W, x, 0.1, 128.0)
+    assert_close(host(ctx["sdf"]), ref["sdf"], what="sdf", outlier_frac=1e-3)
+    assert_close(host(ctx["normal"]), ref["normal"], what="normal", outlier_frac=2e-3)
+    assert abs(loss - ref["loss"]) <= 2e-3 * abs(ref["loss"])
+    assert_grad_close(host(gW), ref["mlp_grad"], what="MLP gradient", rtol=5e-3)
+    got = host(gP)
+    for l in range(16):
+        a, b = int(ref["offset"][l]) * 2, int(ref["offset"][l + 1]) * 2
+        assert rel_l2(got[a:b], ref["grid_grad"][a:b]) < 5e-3, (l, rel_l2(got[a:b], ref["grid_grad"][a:b]))
+    # a second run of the same step leaves the same bits (sorted scatter, fixed-order sums)
+    g1 = gP.clone()
+    w1 = gW.clone()
+    ctx = net.forward(dev(x))
+    net.loss_backward(ctx, ek_weight=0.1, loss_scale=128.0)
+    assert torch.equal(g1, gP) and torch.equal(w1, gW)
