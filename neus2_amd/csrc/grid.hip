@@ -454,6 +454,7 @@ __global__ void __launch_bounds__(GRID_BLOCK) grid_bbi_kernel(N2LevelTable tab, 
 constexpr uint32_t BKT_SHIFT = N2_BKT_SHIFT;           // 4096 entries per bucket: a 64 KiB accumulator image, two reduce workgroups per CU
 constexpr uint32_t BKT_ENTRIES = 1u << BKT_SHIFT;
 constexpr uint32_t BKT_MAX = (1u << 19) >> BKT_SHIFT;  // buckets per level (entries <= 2^19)
+constexpr uint32_t BKT_MIN_SHIFT = 5;                  // smallest bucket of a level that chooses its own size (N2LevelTable::bucket_shift)
 constexpr uint32_t PAIR_MAX_CELL = BKT_ENTRIES - 2u;  // pair records (grid_bin_kernel): x + 1 <= BKT_ENTRIES - 1
 static_assert(BKT_SHIFT <= 12, "a pair record's 16-bit key holds the entry within the bucket and four bits of carry length");
 constexpr uint32_t BIN_POINTS = 1024;    // points per bin workgroup
@@ -574,6 +575,7 @@ __device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uin
                                               const uint32_t* __restrict__ index, uint32_t n_cols) {
 	constexpr uint32_t R = PAIR ? 4 : 8;  // sorted records per point
 	const uint32_t lane = threadIdx.x & 63u;
+	const uint32_t shift = PAIR ? BKT_SHIFT : (uint32_t)tab.bucket_shift[level], in_bucket = (1u << shift) - 1u;
 	// records of this thread: entry | rank << 19 after the counting step (REC_SKIP: merged into a later lane)
 	uint32_t re[BIN_PER_THREAD * R], rv[BIN_PER_THREAD * 8], tcode[BIN_PER_THREAD];
 #pragma unroll
@@ -630,7 +632,7 @@ __device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uin
 			if (!PAIR || (k & 1u) == 0) {
 				uint32_t rec = REC_SKIP;
 				if (emit) {
-					const uint32_t rank = atomicAdd(&hist[e[k] >> BKT_SHIFT], 1u);
+					const uint32_t rank = atomicAdd(&hist[e[k] >> shift], 1u);
 					rec = e[k] | (rank << 19);
 				}
 				re[R * j + (PAIR ? k >> 1 : k)] = rec;
@@ -663,13 +665,13 @@ __device__ __forceinline__ void grid_bin_tile(const N2LevelTable& tab, const uin
 		for (uint32_t k = 0; k < R; ++k) {
 			if (re[R * j + k] != REC_SKIP) {
 				const uint32_t e = re[R * j + k] & 0x7FFFFu, rank = re[R * j + k] >> 19;
-				const uint32_t pos = prefix[e >> BKT_SHIFT] + rank;
+				const uint32_t pos = prefix[e >> shift] + rank;
 				if (PAIR) {
 					reinterpret_cast<uint2*>(stage_val)[pos] = make_uint2(rv[8 * j + 2 * k], rv[8 * j + 2 * k + 1]);
 					stage_key[pos] = (uint16_t)((e & (BKT_ENTRIES - 1u)) | tcode[j]);
 				} else {
 					stage_val[pos] = rv[8 * j + k];
-					stage_key[pos] = (uint16_t)(e & (BKT_ENTRIES - 1u));
+					stage_key[pos] = (uint16_t)(e & in_bucket);
 				}
 			}
 		}
@@ -748,7 +750,7 @@ template <bool PAIR>
 __device__ __forceinline__ void grid_reduce_runs(const uint32_t tiles, const uint32_t level, const uint32_t bucket, const uint32_t group,
                                                  const uint32_t G, const uint32_t* __restrict__ rec_vals, const uint16_t* __restrict__ rec_keys,
                                                  const uint16_t* __restrict__ offsets, unsigned long long* acc, uint32_t* item_src,
-                                                 uint8_t* item_n, uint32_t* wave_tot) {
+                                                 uint8_t* item_n, uint32_t* wave_tot, const uint32_t bucket_entries) {
 	constexpr uint32_t SHIFT = PAIR ? PITEM_SHIFT : ITEM_SHIFT, RECS = 1u << SHIFT;
 	constexpr uint32_t TILE_RECS = PAIR ? BIN_RECORDS / 2 : BIN_RECORDS;  // records in a tile's slot of the value array
 	const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -768,7 +770,7 @@ __device__ __forceinline__ void grid_reduce_runs(const uint32_t tiles, const uin
 			len = end - begin;
 		}
 		if (c0 == 0) {
-			for (uint32_t e = threadIdx.x; e < 2 * BKT_ENTRIES; e += RED_BLOCK) acc[e] = 0ull;
+			for (uint32_t e = threadIdx.x; e < bucket_entries; e += RED_BLOCK) { acc[e] = 0ull; acc[BKT_ENTRIES + e] = 0ull; }
 		}
 		const uint32_t cnt = (len + RECS - 1u) >> SHIFT;
 		uint32_t incl = cnt;
@@ -927,11 +929,13 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 	// ids are dealt round-robin over the XCDs: XCD x takes the x-th eighth of the level's buckets, in order, so that both
 	// fetches of such a line go through the same L2 at about the same time.
 	const uint32_t nb = plan.n_buckets[level];
+	// entries per bucket: the level's own size (split buckets always have BKT_ENTRIES)
+	const uint32_t bucket_entries = ((tab.pair_levels >> level) & 1u) ? BKT_ENTRIES : 1u << tab.bucket_shift[level];
 	if (G == 1 && nb % N_XCD == 0) bucket = (blockIdx.x % N_XCD) * (nb / N_XCD) + local / N_XCD;
 	if ((tab.pair_levels >> level) & 1u)
-		grid_reduce_runs<true>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot);
+		grid_reduce_runs<true>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot, BKT_ENTRIES);
 	else
-		grid_reduce_runs<false>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot);
+		grid_reduce_runs<false>(tiles, level, bucket, group, G, rec_vals, rec_keys, offsets, acc, item_src, item_n, wave_tot, bucket_entries);
 	__syncthreads();
 	const uint32_t entries = tab.entries[level];
 	__half2* Gd = grads + tab.offset[level];
@@ -943,8 +947,8 @@ __global__ void __launch_bounds__(RED_BLOCK, 8) grid_reduce_kernel(N2LevelTable 
 		for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) mine[e] = make_float2(from_fixed(acc[e]), from_fixed(acc[BKT_ENTRIES + e]));
 		return;
 	}
-	for (uint32_t e = threadIdx.x; e < BKT_ENTRIES; e += RED_BLOCK) {
-		const uint32_t idx = bucket * BKT_ENTRIES + e;
+	for (uint32_t e = threadIdx.x; e < bucket_entries; e += RED_BLOCK) {
+		const uint32_t idx = bucket * bucket_entries + e;
 		if (idx >= entries) break;
 		const float ax = from_fixed(acc[e]), ay = from_fixed(acc[BKT_ENTRIES + e]);
 		if (accumulate) {
@@ -1279,8 +1283,27 @@ static bool uses_bucketed(const n2_grid_t* grid, uint32_t n_points) {
 	return grid->grads != nullptr && grid->ws != nullptr && n_points <= grid->ws_max_points && n_points >= 1;
 }
 // workgroups per bucket of a level: aim at <= ~64k records per reduce workgroup (a level holds 8 records per point)
+// Entries per bucket of a level (log2).  Levels that sort pair records keep 4096-entry buckets (a pair's second entry is
+// encoded against that size); the others take the largest size (a power of two, at most 4096 entries and at most BKT_MAX
+// buckets) under which no bucket needs more than one workgroup: small dense levels of large batches get many small buckets
+// instead of few that are split.  When even the smallest size does not get there, the buckets stay large and are split.
+static uint32_t bucket_shift_for(const n2_grid_t* grid, uint32_t level, uint32_t n_points) {
+	if ((grid->tab.pair_levels >> level) & 1u) return BKT_SHIFT;
+	const uint32_t entries = grid->tab.entries[level];
+	for (uint32_t shift = BKT_SHIFT; shift >= BKT_MIN_SHIFT; --shift) {
+		const uint32_t nb = (entries + (1u << shift) - 1u) >> shift;
+		if (nb > BKT_MAX) break;
+		if ((uint64_t)n_points * 8 / nb <= 65536) return shift;  // (32768: scatter + 1.3 us on the training step, 16384: + 4.7)
+	}
+	return BKT_SHIFT;
+}
+static inline uint32_t level_buckets(const n2_grid_t* grid, uint32_t level, uint32_t n_points) {
+	const uint32_t shift = bucket_shift_for(grid, level, n_points);
+	return (grid->tab.entries[level] + (1u << shift) - 1u) >> shift;
+}
+
 static uint32_t bucket_groups(const n2_grid_t* grid, uint32_t level, uint32_t n_points, uint32_t tiles) {
-	const uint32_t nb = (grid->tab.entries[level] + BKT_ENTRIES - 1) / BKT_ENTRIES;
+	const uint32_t nb = level_buckets(grid, level, n_points);
 	const uint64_t per_bucket = (uint64_t)n_points * 8 / nb;
 	uint32_t groups = (uint32_t)((per_bucket + 65535) / 65536);
 	if (groups > N2_CMB_MAX_GROUPS) groups = N2_CMB_MAX_GROUPS;
@@ -1294,7 +1317,7 @@ static uint32_t split_images(const n2_grid_t* grid, uint32_t n_points) {
 	const uint32_t tiles = n_bin_tiles(n_points);
 	uint32_t n = 0;
 	for (uint32_t l = 0; l < grid->tab.n_levels; ++l) {
-		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES, groups = bucket_groups(grid, l, n_points, tiles);
+		const uint32_t nb = level_buckets(grid, l, n_points), groups = bucket_groups(grid, l, n_points, tiles);
 		if (groups > 1) n += nb * groups;
 	}
 	return n;
@@ -1337,8 +1360,10 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	const dim3 gd(tiles * L);
 	N2BucketPlan plan;
 	uint32_t wg = 0, images = 0, split = 0;
+	N2LevelTable tab = grid->tab;  // with this launch's bucket sizes
 	for (uint32_t l = 0; l < L; ++l) {
-		const uint32_t nb = (grid->tab.entries[l] + BKT_ENTRIES - 1) / BKT_ENTRIES;
+		tab.bucket_shift[l] = (uint8_t)bucket_shift_for(grid, l, n_points);
+		const uint32_t nb = level_buckets(grid, l, n_points);
 		const uint32_t groups = bucket_groups(grid, l, n_points, tiles);
 		plan.wg_begin[l] = wg;
 		plan.n_buckets[l] = nb;
@@ -1351,7 +1376,7 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.wg_begin[l] = wg;
 	for (uint32_t l = L; l < N2_MAX_LEVELS; ++l) { plan.n_buckets[l] = 0; plan.groups[l] = 1; plan.part_begin[l] = images; }
 	for (uint32_t l = L; l <= N2_MAX_LEVELS; ++l) plan.split_begin[l] = split;
-#define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(grid->tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
+#define LAUNCH(F, S, O) grid_bin_kernel<F, S, O><<<gd, bd, 0, s>>>(tab, 0u, n_points, tiles, d_xyz, point_stride, dim_stride, dL_dy, v, g2, \
                                                                    grid->params, dL_ddLdy, rec_vals, rec_keys, offsets, index, n_cols)
 	if (first && second && out) LAUNCH(true, true, true);
 	else if (first && second) LAUNCH(true, true, false);
@@ -1360,24 +1385,24 @@ static int launch_bucketed(n2_grid_t* grid, hipStream_t s, const float* d_xyz, u
 	else LAUNCH(true, false, false);
 #undef LAUNCH
 	N2_LAUNCH_CHECK();
-	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(grid->tab, plan, tiles, rec_vals, rec_keys, offsets, grid->grads, accumulate ? 1 : 0, partials);
+	grid_reduce_kernel<<<dim3(wg), dim3(RED_BLOCK), 0, s>>>(tab, plan, tiles, rec_vals, rec_keys, offsets, grid->grads, accumulate ? 1 : 0, partials);
 	N2_LAUNCH_CHECK();
 	if (split > 0) {
-		// the split levels are the coarsest ones (a level has at least as many buckets as the one below it)
 		N2ImageCombine cmb{};
 		cmb.images = partials;
 		cmb.grads = reinterpret_cast<_Float16*>(grid->grads);
 		cmb.bucket_entries = BKT_ENTRIES;
 		cmb.accumulate = accumulate ? 1 : 0;
-		uint32_t k = 0;
-		while (k < L && k < N2_CMB_LEVELS && plan.groups[k] > 1) {
-			cmb.split_begin[k] = plan.split_begin[k]; cmb.groups[k] = plan.groups[k]; cmb.part_begin[k] = plan.part_begin[k];
-			cmb.entries[k] = grid->tab.entries[k]; cmb.offset[k] = grid->tab.offset[k];
+		uint32_t k = 0;  // the split levels, in order
+		for (uint32_t l = 0; l < L; ++l) {
+			if (plan.groups[l] <= 1) continue;
+			N2_REQUIRE(tab.bucket_shift[l] == BKT_SHIFT, "grid scatter: level %u splits buckets of %u entries", l, 1u << tab.bucket_shift[l]);
+			cmb.split_begin[k] = plan.split_begin[l]; cmb.groups[k] = plan.groups[l]; cmb.part_begin[k] = plan.part_begin[l];
+			cmb.entries[k] = grid->tab.entries[l]; cmb.offset[k] = grid->tab.offset[l];
 			++k;
 		}
 		cmb.n_levels = k;
 		for (uint32_t l = k; l <= N2_CMB_LEVELS; ++l) cmb.split_begin[l] = split;
-		N2_REQUIRE(k > 0 && plan.split_begin[k] == split, "grid scatter: split buckets outside the coarsest %u levels", N2_CMB_LEVELS);
 		cmb.units = split * (BKT_ENTRIES / N2_CMB_ENTRIES);
 		grid_combine_kernel<<<dim3(cmb.units), dim3(256), 0, s>>>(cmb);
 		N2_LAUNCH_CHECK();

@@ -63,6 +63,9 @@ struct N2LevelTable {
 	uint32_t n_features;
 	// bit l set: level l's bucketed scatter writes one record per PAIR of x-neighbour corners (see grid_bin_kernel)
 	uint32_t pair_levels;
+	// log2 of the entries per bucket of level l's bucketed scatter (set per launch: small levels take small buckets, so
+	// that every bucket has about a workgroup's worth of records and none has to be split)
+	uint8_t bucket_shift[N2_MAX_LEVELS];
 };
 
 // What the fused field kernels need of a field's parts: the grid's level table and parameters, the weights of the two

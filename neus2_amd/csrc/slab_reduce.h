@@ -26,7 +26,7 @@ struct N2StepEpilogue {
 // (the coarsest levels of a large batch; they are levels 0 .. n_levels - 1).  Image (level, bucket, group) holds the
 // bucket's bucket_entries fp32 pairs at images + (part_begin[level] + bucket * groups[level] + group) * bucket_entries.
 // A unit adds up the images of 128 consecutive entries in the order of the groups and stores the fp16 gradients.
-constexpr uint32_t N2_CMB_LEVELS = 8, N2_CMB_SLICES = 8, N2_CMB_ENTRIES = 128, N2_CMB_MAX_GROUPS = 32;
+constexpr uint32_t N2_CMB_LEVELS = 32, N2_CMB_SLICES = 8, N2_CMB_ENTRIES = 128, N2_CMB_MAX_GROUPS = 32;
 struct N2ImageCombine {
 	const float2* images;
 	_Float16* grads;                          // the encoding's gradients: entry e of level l at grads + 2 * (offset[l] + e)
