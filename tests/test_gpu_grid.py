@@ -213,6 +213,46 @@ def test_sorted_scatter_other_table_shapes(oracle, cfg):
         assert rel_l2(got[a:b], ref[a:b]) < tol, (l, rel_l2(got[a:b], ref[a:b]), tol)
 
 
+def test_sorted_scatter_split_buckets(oracle):
+    """A small table under a large batch: every level has fewer buckets than the batch needs workgroups, so buckets are
+    split over several workgroups whose fp32 images a combine launch adds in a fixed order (both record kinds: the dense
+    levels' single records and the hashed levels' pair records).  Against the oracle, accumulate mode included, and two
+    runs give the same bits."""
+    from neus2_amd.tcnn_api import GRAD_ACCUMULATE, GRAD_OVERWRITE, GridEncoding
+    cfg = (6, 12, 4, 1.6)
+    og = oracle.Grid(*cfg)
+    gg = GridEncoding(n_levels=cfg[0], log2_hashmap_size=cfg[1], base_resolution=cfg[2], per_level_scale=cfg[3])
+    rng = np.random.default_rng(29)
+    params = q16(rng.uniform(-1, 1, og.n_params))
+    dp = dev(params, torch.float16)
+    dg = torch.zeros_like(dp)
+    gg.set_params(dp, dg)
+    n = 40 * 1024 + 77  # 8 n / 65536 = 5 workgroups per bucket
+    assert gg.reserve_scatter_workspace(n)
+    xyz = rng.random((3, n), dtype=np.float32)
+    dy = q16(rng.standard_normal((og.n_out, n)) * 0.05)
+    g2 = q16(rng.standard_normal((og.n_out, n)) * 0.01)
+    v = (rng.standard_normal((3, n)) * 1e-3).astype(np.float32)
+    ref1, _ = og.backward(params, xyz, dy, want_dx=False)
+    ref, _, _ = og.backward_backward_input(params, xyz, v, g2, grad=ref1.copy(), want_dinput=False)
+    d_xyz, d_dy, d_v, d_g2 = dev(xyz), dev(dy, torch.float16), dev(v), dev(g2, torch.float16)
+
+    def check(got, want, what):
+        for l in range(cfg[0]):
+            a, b = int(og.offset[l]) * 2, int(og.offset[l + 1]) * 2
+            assert rel_l2(got[a:b], want[a:b]) < RTOL, (what, l, rel_l2(got[a:b], want[a:b]))
+
+    dg.fill_(7.0)
+    gg.backward_fused(d_xyz, d_dy, d_v, d_g2, want_dL_ddLdy=False, mode=GRAD_OVERWRITE)
+    first = dg.clone()
+    check(host(dg), ref, "overwrite")
+    gg.backward_fused(d_xyz, d_dy, d_v, d_g2, want_dL_ddLdy=False, mode=GRAD_ACCUMULATE)
+    check(host(dg), 2 * ref, "accumulate")
+    dg.fill_(-3.0)
+    gg.backward_fused(d_xyz, d_dy, d_v, d_g2, want_dL_ddLdy=False, mode=GRAD_OVERWRITE)
+    assert torch.equal(dg, first)
+
+
 def test_errors_are_reported_not_launched():
     from neus2_amd.tcnn_api import GRAD_OVERWRITE, GridEncoding, N2Error
     gg = GridEncoding(**CFG)
