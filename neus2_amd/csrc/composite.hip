@@ -93,6 +93,16 @@ struct RayScratch {
 constexpr float T_EPS = 1e-4f;
 constexpr int CB = 256;  // 4 rays per workgroup
 
+// THE factor of fill_rollover_and_rescale (tcnn; called at src/testbed_nerf.cu:3908-3910 with n_elements = the target
+// batch size and stride = the padded output width): a wrapped copy of an output gradient is the original times
+// n_in / n_total, rows over rows, whatever the stride.  tiny-cuda-nn's source is not part of the reference tree, so this
+// reading is recalled, not checked: it is the only place in the library that holds it (the CPU oracle has the same one
+// function, orc_rollover_rescaled).  Two roundings, as written: the product first.
+__host__ __device__ __forceinline__ float rollover_rescaled(float value, uint32_t n_in, uint32_t n_total, uint32_t stride) {
+	(void)stride;
+	return value * (float)n_in / (float)n_total;
+}
+
 __global__ void __launch_bounds__(CB) composite_forward_kernel(CompParams c, uint32_t n_rays, const uint32_t* __restrict__ ray_counter,
                                                                const uint32_t* __restrict__ numsteps, const hf* __restrict__ net_out,
                                                                const float* __restrict__ coords, RayScratch* __restrict__ scratch,
@@ -342,8 +352,8 @@ __global__ void __launch_bounds__(CB) composite_backward_kernel(CompParams c, ui
 					half8 lo_f, hi_f;
 #pragma unroll
 					for (int k = 0; k < 8; ++k) {
-						lo_f[k] = (hf)((float)lo[k] * (float)n_in / (float)max_compacted);
-						hi_f[k] = (hf)((float)hi[k] * (float)n_in / (float)max_compacted);
+						lo_f[k] = (hf)rollover_rescaled((float)lo[k], n_in, max_compacted, 16u);
+						hi_f[k] = (hf)rollover_rescaled((float)hi[k], n_in, max_compacted, 16u);
 					}
 					hf* gf = dloss + (size_t)j * 16;
 					*reinterpret_cast<half8*>(gf) = lo_f;
@@ -473,7 +483,7 @@ __global__ void __launch_bounds__(256) fill_rollover_kernel(uint32_t n_total, ui
 	const size_t lim = (size_t)n_in * stride;
 	if (n_in == 0 || i < lim || i >= (size_t)n_total * stride) return;
 	T r = inout[i % lim];
-	if (RESCALE) r = (T)((float)r * (float)n_in / (float)n_total);
+	if (RESCALE) r = (T)rollover_rescaled((float)r, n_in, n_total, stride);
 	inout[i] = r;
 }
 

@@ -732,12 +732,18 @@ ORC_API void orc_composite_loss(const CompositeCfg* cfg, uint32_t n_rays, uint32
 // fill_rollover / fill_rollover_and_rescale (tcnn; call sites src/testbed_nerf.cu:3908-3916): pad a
 // compacted batch of n_in rows (stride floats each) to n_total rows by wrapping around; the
 // wrapped copies are scaled by n_in/n_total when rescale != 0.
+// THE factor of fill_rollover_and_rescale: rows over rows, whatever the stride (recalled from tiny-cuda-nn, whose source
+// is not in the reference tree: parity unpinned; the library's only copy is rollover_rescaled in composite.hip).
+static inline float orc_rollover_rescaled(float value, uint32_t n_in, uint32_t n_total, uint32_t stride) {
+	(void)stride;
+	return value * (float)n_in / (float)n_total;
+}
 ORC_API void orc_fill_rollover(uint32_t n_total, uint32_t stride, uint32_t n_in, float* inout, int rescale) {
 	if (n_in == 0 || n_in >= n_total) return;
 	const size_t lim = (size_t)n_in * stride;
 	for (size_t i = lim; i < (size_t)n_total * stride; ++i) {
 		float r = inout[i % lim];
-		if (rescale) r = r * (float)n_in / (float)n_total;
+		if (rescale) r = orc_rollover_rescaled(r, n_in, n_total, stride);
 		inout[i] = r;
 	}
 }
