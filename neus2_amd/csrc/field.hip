@@ -442,7 +442,8 @@ N2_API int n2_field_forward(n2_field_t* f, n2_stream_t stream, const float* d_co
 	return n2_field_forward_live(f, stream, d_coords, n, nullptr, d_output);
 }
 
-int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output) {
+int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output,
+                          const float* d_xyz_soa) {
 	if (int rc = check_field(f, "n2_field_forward", n)) return rc;
 	if (n == 0) return N2_OK;
 	N2_REQUIRE(d_coords != nullptr && d_output != nullptr, "n2_field_forward: null buffer");
@@ -456,7 +457,8 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 		f->pad_n.rgb_in = 0;  // the fused kernel writes sample-major, over what the row layout keeps zero
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
 		return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx,
-		                              reinterpret_cast<n2_half*>(f->dsdf_din), reinterpret_cast<n2_half*>(f->rgb_in), d_output, d_live);
+		                              reinterpret_cast<n2_half*>(f->dsdf_din), reinterpret_cast<n2_half*>(f->rgb_in), d_output, d_live, nullptr, nullptr, 0, 0,
+		                              d_xyz_soa);
 	}
 	field_pack_sdf_input_kernel<<<fgrid(n), dim3(FB), 0, s>>>(d_coords, 7, 1, n, f->sdf_in, f->xyz);
 	N2_LAUNCH_CHECK();

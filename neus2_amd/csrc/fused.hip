@@ -295,8 +295,11 @@ constexpr uint32_t FG_BLOCK = 256;
 template <bool FULL>
 __device__ __forceinline__ void gather_item(const FusedArgs& a, uint32_t level, uint32_t i, uint32_t src) {
 	const uint32_t N = a.N;
-	const float* q = FULL ? a.coords + (size_t)src * 7 : a.pos + (size_t)src * a.ps;
-	const size_t qs = FULL ? 1 : a.ds;
+	// (full field: the positions from the coordinate rows, or from three rows of their own when the caller has them: a wave
+	// then reads two lines per coordinate instead of fourteen)
+	const bool rows = FULL && a.pos == nullptr;
+	const float* q = rows ? a.coords + (size_t)src * 7 : a.pos + (size_t)src * a.ps;
+	const size_t qs = rows ? 1 : a.ds;
 	const float p[3] = {q[0], q[qs], q[2 * qs]};
 	if (FULL && level == 0) {
 #pragma unroll
@@ -676,8 +679,9 @@ static FusedArgs fused_base(const N2FusedNets& nets, uint32_t n) {
 
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
                            void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live, const uint32_t* d_list,
-                           const uint32_t* d_counts, uint32_t round, uint32_t est_samples) {
+                           const uint32_t* d_counts, uint32_t round, uint32_t est_samples, const float* d_xyz_soa) {
 	FusedArgs a = fused_base(nets, n);
+	if (d_xyz_soa) { a.pos = d_xyz_soa; a.ps = 1; a.ds = n; }
 	a.live = d_live;
 	a.list = d_list;
 	a.counts = d_counts;

@@ -96,7 +96,10 @@ bool n2_fused_supported(const N2LevelTable& tab, uint32_t sdf_hidden_layers, uin
 // d_live (or null): a device counter; only samples below min(*d_live, n) are evaluated, n stays the matrices' column count.
 int n2_fused_field_forward(const N2FusedNets& nets, hipStream_t s, const float* d_coords, uint32_t n, n2_half* sdf_in, float* xyz_rows,
                            void* slopes, n2_half* dsdf_din, n2_half* rgb_in, n2_half* d_output, const uint32_t* d_live = nullptr,
-                           const uint32_t* d_list = nullptr, const uint32_t* d_counts = nullptr, uint32_t round = 0, uint32_t est_samples = 0);
+                           const uint32_t* d_list = nullptr, const uint32_t* d_counts = nullptr, uint32_t round = 0, uint32_t est_samples = 0,
+                           const float* d_xyz_soa = nullptr);
+// d_xyz_soa (or null): the samples' positions once more as three rows of n floats ([3][n]), which the gather then reads
+// instead of the coordinate rows
 // One round of a forward pass in depth chunks (n2_composite_chunk_next): the samples begin .. begin + d_counts[round] of
 // d_coords_listed, begin = d_counts[0] + ... + d_counts[round - 1].  The output of sample c goes to row d_list[c] of d_output;
 // what the backward reads is stored at column c (n2_field_select then takes list positions).  est_samples: the caller's
@@ -105,7 +108,13 @@ int n2_field_forward_listed(n2_field_t* field, n2_stream_t stream, const float* 
                             uint32_t round, uint32_t est_samples, n2_half* d_output);
 // n2_field_forward over the samples below min(*d_live, n): the trainer's marched samples fill only part of the window it
 // evaluates (the window is the count measured some steps earlier, rounded up); what lies behind them is not computed.
-int n2_field_forward_live(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output);
+int n2_field_forward_live(n2_field_t* field, n2_stream_t stream, const float* d_coords, uint32_t n, const uint32_t* d_live, n2_half* d_output,
+                          const float* d_xyz_soa = nullptr);
+// n2_generate_training_samples that also writes the positions as three rows of max_samples floats (d_xyz_rows, or null)
+int n2_generate_training_samples_rows(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed, const n2_camera* d_cameras, uint32_t n_images,
+                                      const float* d_rgba, const float background[3], const uint8_t* d_bitfield, uint32_t max_samples,
+                                      uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices, uint32_t* d_numsteps, float* d_rgb_target,
+                                      float* d_coords, void* d_workspace, uint64_t workspace_bytes, float* d_xyz_rows);
 // NerfNetwork::sdf / density: d_out_soa (16 x n, may be null) and / or d_row0 (fp32 copy of row 0, may be null).
 // sdf_in null: one kernel that gathers sample by sample (points in lattice order, whose table lines stay cached);
 // else a level-major gather into the feature rows 3.. of sdf_in (SoA, n columns) followed by the network kernel.

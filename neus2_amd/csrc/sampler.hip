@@ -384,7 +384,8 @@ __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_emit_kernel(uint3
                                                            const uint32_t* __restrict__ counts,
                                                            const uint32_t* __restrict__ base, const uint32_t* __restrict__ slot,
                                                            uint32_t* __restrict__ ray_indices, uint32_t* __restrict__ numsteps,
-                                                           float* __restrict__ rgb_target, float* __restrict__ coords) {
+                                                           float* __restrict__ rgb_target, float* __restrict__ coords,
+                                                           float* __restrict__ xyz_soa, uint32_t soa_pitch) {
 	const uint32_t i = blockIdx.x * RAYS_PER_BLOCK + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
 	if (i >= n_rays) return;
 	const uint32_t s = slot[i];
@@ -407,10 +408,16 @@ __global__ void __launch_bounds__(64 * RAYS_PER_BLOCK) sampler_emit_kernel(uint3
 		if (bits == 0ull) continue;  // uniform: the whole wave skips the window
 		const float t = window_t(t_first[(size_t)i * WINDOWS + w], lane);
 		if ((bits >> lane) & 1ull) {
-			float* c = coords + (size_t)(first + j + (uint32_t)__popcll(bits & ((1ull << lane) - 1ull))) * 7;
+			const uint32_t at = first + j + (uint32_t)__popcll(bits & ((1ull << lane) - 1ull));
+			float* c = coords + (size_t)at * 7;
 			c[0] = __fmaf_rn(t, r.dir[0], r.o[0]);
 			c[1] = __fmaf_rn(t, r.dir[1], r.o[1]);
 			c[2] = __fmaf_rn(t, r.dir[2], r.o[2]);
+			if (xyz_soa) {  // the positions once more as three rows: what a reader of positions alone wants
+				xyz_soa[at] = c[0];
+				xyz_soa[(size_t)soa_pitch + at] = c[1];
+				xyz_soa[(size_t)2 * soa_pitch + at] = c[2];
+			}
 			c[3] = 0.0f;
 			c[4] = d0; c[5] = d1; c[6] = d2;
 		}
@@ -432,6 +439,16 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
                                         uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices,
                                         uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
                                         uint64_t workspace_bytes) {
+	return n2_generate_training_samples_rows(stream, n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background, d_bitfield, max_samples, d_ray_counter,
+	                                         d_sample_counter, d_ray_indices, d_numsteps, d_rgb_target, d_coords, d_workspace, workspace_bytes, nullptr);
+}
+
+int n2_generate_training_samples_rows(n2_stream_t stream, uint32_t n_rays, uint32_t n_rays_total, uint32_t seed,
+                                      const n2_camera* d_cameras, uint32_t n_images, const float* d_rgba,
+                                      const float background[3], const uint8_t* d_bitfield, uint32_t max_samples,
+                                      uint32_t* d_ray_counter, uint32_t* d_sample_counter, uint32_t* d_ray_indices,
+                                      uint32_t* d_numsteps, float* d_rgb_target, float* d_coords, void* d_workspace,
+                                      uint64_t workspace_bytes, float* d_xyz_rows) {
 	N2_REQUIRE(d_ray_counter && d_sample_counter, "n2_generate_training_samples: counters are null");
 	hipStream_t s = n2_stream(stream);
 	if (n_rays == 0) {
@@ -467,7 +484,8 @@ N2_API int n2_generate_training_samples(n2_stream_t stream, uint32_t n_rays, uin
 	                                                                 d_sample_counter);
 	N2_LAUNCH_CHECK();
 	sampler_emit_kernel<<<grid, block, 0, s>>>(n_rays, n_rays_total, seed, d_cameras, n_images, d_rgba, background[0], background[1],
-	                                           background[2], mask, t_first, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords);
+	                                           background[2], mask, t_first, counts, base, slot, d_ray_indices, d_numsteps, d_rgb_target, d_coords,
+	                                           d_xyz_rows, max_samples);
 	N2_LAUNCH_CHECK();
 	return N2_OK;
 }

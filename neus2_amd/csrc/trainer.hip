@@ -35,6 +35,8 @@ struct n2_trainer {
 	// per-step buffers; everything the sample generator writes exists twice
 	struct SampleSet {
 		float* coords;            // [max_samples][7]
+		float* xyz_rows;          // [3][n_inference of the generation]: the positions once more, as rows
+		bool has_rows;            // the last generation into this set wrote them
 		uint32_t* numsteps;       // [max_rays][2]
 		uint32_t* ray_indices;    // [max_rays]
 		float* rgb_target;        // [max_rays][3]
@@ -78,7 +80,7 @@ struct n2_trainer {
 };
 
 struct TrainerCarve {
-	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], mlp_out, dloss, coords_compacted, src_index, numsteps[2], ray_indices[2], rgb_target[2],
+	uint64_t master, params, grads, m1, m2, steps, ema_tmp, ema, coords[2], xyz_rows[2], mlp_out, dloss, coords_compacted, src_index, numsteps[2], ray_indices[2], rgb_target[2],
 		set_counters[2], ray_loss, counters, chunk_counts, chunk_list, chunk_column, chunk_state, chunk_coords, ws_sampler[2], ws_composite, ws_field, total;
 };
 
@@ -101,6 +103,7 @@ static TrainerCarve trainer_carve(const n2_trainer_config* cfg, const n2_field_t
 	c.ema_tmp = take(ema ? 4 * np : 0);
 	c.ema = take(ema ? 2 * np : 0);
 	for (int i = 0; i < 2; ++i) c.coords[i] = take(28 * S);
+	for (int i = 0; i < 2; ++i) c.xyz_rows[i] = take(12 * S);
 	c.mlp_out = take(32 * (S > T ? S : T));
 	c.dloss = take(32 * T);
 	c.coords_compacted = take(28 * T);
@@ -189,6 +192,7 @@ N2_API int n2_trainer_create(const n2_trainer_config* cfg, void* d_workspace, ui
 	t->training_step = 0;
 	for (int i = 0; i < 2; ++i) {
 		t->sets[i].coords = reinterpret_cast<float*>(b + c.coords[i]);
+		t->sets[i].xyz_rows = reinterpret_cast<float*>(b + c.xyz_rows[i]);
 		t->sets[i].numsteps = reinterpret_cast<uint32_t*>(b + c.numsteps[i]);
 		t->sets[i].ray_indices = reinterpret_cast<uint32_t*>(b + c.ray_indices[i]);
 		t->sets[i].rgb_target = reinterpret_cast<float*>(b + c.rgb_target[i]);
@@ -295,11 +299,16 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	// the colour rows of dL/doutput are at most 0.05 * loss_scale / n_rays: the colour net's backward lifts them out of
 	// fp16's subnormal range by an exact power of two
 	if (int rc = n2_field_set_colour_gradient_exponent(t->field, n2_colour_gradient_exponent(t->cfg.loss_scale, n_rays))) return rc;
+	// A step in depth rounds reads its positions from the rounds' lists: the generator then leaves the rows out (on a trained
+	// field it writes three times the samples, beside the forward's first round)
+	const bool want_rows = !(t->chunk_rounds >= 2 && !t->cfg.recompute_training_forward);
 	auto sample = [&](n2_trainer::SampleSet& set, hipStream_t on, uint32_t ray_base, uint32_t sd) {
+		set.has_rows = want_rows;
 		// rays -> marched samples (capacity n_inference: rays that do not fit are dropped, as when max_samples is reached)
-		return n2_generate_training_samples(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,
-		                                    t->cfg.composite.background, t->bitfield, n_inference, set.counters, set.counters + 1, set.ray_indices,
-		                                    set.numsteps, set.rgb_target, set.coords, set.ws_sampler, t->ws_sampler_bytes);
+		// (the positions also as three rows of n_inference floats, for the field's gather)
+		return n2_generate_training_samples_rows(reinterpret_cast<n2_stream_t>(on), n_rays, ray_base, sd, t->cameras, t->n_images, t->rgba,
+		                                         t->cfg.composite.background, t->bitfield, n_inference, set.counters, set.counters + 1, set.ray_indices,
+		                                         set.numsteps, set.rgb_target, set.coords, set.ws_sampler, t->ws_sampler_bytes, want_rows ? set.xyz_rows : nullptr);
 	};
 	// the following step's samples on the side stream, assuming the same ray count and the next seed
 	bool main_event_is_last_step = false;
@@ -346,6 +355,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 	cc.n_rays_norm = n_rays;
 	cc.loss_scale = t->cfg.loss_scale;
 	const bool chunked = t->chunk_rounds >= 2 && !t->cfg.recompute_training_forward;
+
 	if (chunked) {
 		// the field over the marched samples in depth chunks: only what lies in front of the rays' cuts (and at most a chunk
 		// behind them) is evaluated
@@ -366,7 +376,7 @@ N2_API int n2_trainer_step(n2_trainer_t* t, n2_stream_t stream, uint32_t n_rays,
 		}
 	} else {
 		// field over every marched sample: the window of n_inference samples, of which the generator filled set.counters[1]
-		if (int rc = n2_field_forward_live(t->field, stream, set.coords, n_inference, set.counters + 1, reinterpret_cast<n2_half*>(t->mlp_out))) return rc;
+		if (int rc = n2_field_forward_live(t->field, stream, set.coords, n_inference, set.counters + 1, reinterpret_cast<n2_half*>(t->mlp_out), set.has_rows ? set.xyz_rows : nullptr)) return rc;
 	}
 	t->last_chunked = chunked;
 	// compositing, loss, gradients w.r.t. the outputs, compaction

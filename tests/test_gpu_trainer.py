@@ -296,18 +296,23 @@ def test_depth_chunks_give_the_same_steps(oracle):
     n_rays, n_inf = a.budget.rays_per_batch, a.budget.n_inference()
     assert c["samples"] > 1.3 * c["compacted"], c   # rays do end early in this state (after a hundred to two hundred samples)
     runs = []
-    for chunks in ((0, 0), (96, 3), (16, 8), (1, 2)):
+    # the last run changes the setting between steps, while the next step's samples are already being generated (a plain
+    # step's generation also writes the positions as rows, one in rounds does not: a step takes what its samples come with)
+    for chunks in ((0, 0), (96, 3), (16, 8), (1, 2), "switched"):
         tr = make(bits)
         tr.set_parameters(master)
-        tr.set_depth_chunks(*chunks)
+        if chunks != "switched":
+            tr.set_depth_chunks(*chunks)
         seen = []
         for step in range(4):
+            if chunks == "switched":
+                tr.set_depth_chunks(*[(16, 8), (0, 0), (96, 3), (0, 0)][step])
             params16 = host(tr.params).copy()
             tr.step(n_rays=n_rays, n_inference=n_inf, seed=100 + step)
             cs = tr.read_counters()
             view = tr.last_step(cs["rays"], cs["samples"], n_inf)
             seen.append((cs, tr.grads.clone()))
-            if chunks[1]:
+            if chunks != "switched" and chunks[1]:
                 done = int(view["evaluated_counts"].sum().item())
                 assert min(cs["compacted"], T) <= done <= cs["samples"]
                 if chunks == (96, 3):
