@@ -52,6 +52,7 @@ struct n2_field {
 	void* ws_grid;
 	hf* frag_image;  // the fused forward's weight fragments
 	bool fused;  // forward passes go through the fused kernels where the configuration allows (n2_field_set_fused)
+	bool frags_ready;   // the last forward's gather launch left the weight-gradient kernels' fragments in frag_image (same weights since)
 	bool slopes_saved;  // the last forward left the encoding's Jacobian as fp16 slopes (fused forward), not as fp32 dy_dx
 };
 
@@ -325,6 +326,7 @@ N2_API int n2_field_set_params(n2_field_t* f, const n2_half* d_params, n2_half* 
 	N2_REQUIRE(reinterpret_cast<uintptr_t>(d_params) % 16 == 0 && reinterpret_cast<uintptr_t>(d_gradients) % 16 == 0,
 	           "n2_field_set_params: buffers must be 16-byte aligned");
 	f->params = reinterpret_cast<const hf*>(d_params);
+	f->frags_ready = false;
 	f->grads = reinterpret_cast<hf*>(d_gradients);
 	auto g = [&](uint32_t off) { return d_gradients ? d_gradients + off : nullptr; };
 	if (int rc = n2_mlp_set_params(f->sdf, d_params + f->off_sdf, g(f->off_sdf))) return rc;
@@ -453,6 +455,7 @@ int n2_field_forward_live(n2_field_t* f, n2_stream_t stream, const float* d_coor
 	f->sel_n = 0;
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	f->slopes_saved = f->fused && fused_ok(f);
+	f->frags_ready = f->slopes_saved;
 	if (f->slopes_saved) {
 		f->pad_n.rgb_in = 0;  // the fused kernel writes sample-major, over what the row layout keeps zero
 		N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
@@ -488,6 +491,7 @@ int n2_field_forward_listed(n2_field_t* f, n2_stream_t stream, const float* d_co
 	f->sel_n = 0;
 	if (int rc = zero_padding(s, f->sdf_in, 3 + f->enc_w, f->sdf_in_w, n, f->pad_n.sdf_in)) return rc;
 	f->slopes_saved = true;
+	if (round == 0) f->frags_ready = true;
 	f->pad_n.rgb_in = 0;
 	N2ProfScope prof(N2_PROF_FIELD_FORWARD, s);
 	return n2_fused_field_forward(fused_nets(f), s, d_coords, n, reinterpret_cast<n2_half*>(f->sdf_in), f->xyz, f->dy_dx, reinterpret_cast<n2_half*>(f->dsdf_din),
@@ -506,7 +510,17 @@ static int field_backward_passes(n2_field_t* f, n2_stream_t stream, const float*
 
 int n2_field_backward_deferred(n2_field_t* f, n2_stream_t stream, const float* d_coords, uint32_t n, const n2_half* d_dL_doutput, uint32_t ek_batch_size,
                                n2_grad_mode mode, N2SlabReduce* sums) {
+	if (f != nullptr && f->frags_ready) {
+		// the weight-gradient kernels' fragments as the forward's gather launch built them, once for all workgroups
+		const n2_half* image = reinterpret_cast<const n2_half*>(f->frag_image);
+		n2_mlp_borrow_fragment_image(f->rgb, image + N2_FUSED_FRAG_FORWARD / 2);
+		if (f->sdf_in_w == 48) n2_mlp_borrow_fragment_image(f->sdf, image + (N2_FUSED_FRAG_FORWARD + N2_FUSED_FRAG_RGB) / 2);
+	}
 	const int rc = field_backward_passes(f, stream, d_coords, n, d_dL_doutput, ek_batch_size, mode, sums);
+	if (f != nullptr) {
+		n2_mlp_borrow_fragment_image(f->rgb, nullptr);
+		n2_mlp_borrow_fragment_image(f->sdf, nullptr);
+	}
 	if (rc != N2_OK && f != nullptr) {
 		// a pass that ran before the failure left partial sums pending in its network: nobody will reduce them
 		n2_mlp_drop_pending(f->rgb);

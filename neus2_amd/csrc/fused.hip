@@ -148,11 +148,24 @@ __device__ __forceinline__ void load_fused_frags(hf* F, const hf* __restrict__ i
 	for (int idx = threadIdx.x; idx < count * 64; idx += FF_BLOCK) *reinterpret_cast<half8*>(F + (size_t)idx * 8) = *reinterpret_cast<const half8*>(image + (size_t)idx * 8);
 	__syncthreads();
 }
-// Workgroups FRAG_BLOCKS .. of a gather launch (behind those that gather) write the image.
-constexpr uint32_t FRAG_BLOCKS = (FF_COUNT * 64 + 255) / 256;
+// Workgroups FRAG_BLOCKS .. of a gather launch (behind those that gather) write the image: the network kernel's fragments,
+// then those of the backward's weight-gradient kernels (colour net: FragMap<3, 2>; SDF net with 48 inputs: FragMap<3, 1>).
+constexpr uint32_t BWD_RGB_FRAGS = FragMap<3, 2>::SEL, BWD_SDF_FRAGS = FragMap<3, 1>::SEL;
+static_assert(FF_COUNT * 1024 == N2_FUSED_FRAG_FORWARD && BWD_RGB_FRAGS * 1024 == N2_FUSED_FRAG_RGB && BWD_SDF_FRAGS * 1024 == N2_FUSED_FRAG_SDF,
+              "the image's parts as n2_common.h sizes them");
+constexpr uint32_t FRAG_BLOCKS = ((FF_COUNT + BWD_RGB_FRAGS + BWD_SDF_FRAGS) * 64 + 255) / 256;
 __device__ __forceinline__ void write_frag_image(const FusedArgs& a, uint32_t block) {
 	const uint32_t idx = block * 256u + threadIdx.x;
-	if (idx < (uint32_t)FF_COUNT * 64u) *reinterpret_cast<half8*>(a.frags + (size_t)idx * 8) = fused_frag_value(a, (int)(idx >> 6), (int)(idx & 63u));
+	half8* at = reinterpret_cast<half8*>(a.frags) + idx;
+	if (idx < (uint32_t)FF_COUNT * 64u) {
+		*at = fused_frag_value(a, (int)(idx >> 6), (int)(idx & 63u));
+	} else if (idx < (FF_COUNT + BWD_RGB_FRAGS) * 64u) {
+		const uint32_t i = idx - FF_COUNT * 64u;
+		*at = mlp_frag_value<3, 2>(a.rgb_w, (int)(i >> 6), (int)(i & 63u));
+	} else if (idx < (FF_COUNT + BWD_RGB_FRAGS + BWD_SDF_FRAGS) * 64u && a.sdf_in_w == 48u) {
+		const uint32_t i = idx - (FF_COUNT + BWD_RGB_FRAGS) * 64u;
+		*at = mlp_frag_value<3, 1>(a.sdf_w, (int)(i >> 6), (int)(i & 63u));
+	}
 }
 
 // ----------------------------------------------------------------------------

@@ -42,6 +42,7 @@ struct n2_mlp {
 	uint32_t pending_slabs;       // slabs written since the last reduction
 	n2_grad_mode pending_mode;    // mode of the first of the pending calls (later ones must accumulate)
 	int dy_exponent;              // n2_mlp_set_output_gradient_exponent
+	const hf* frag_image;         // n2_mlp_borrow_fragment_image (null: every workgroup builds its fragments from the weights)
 };
 
 // ----------------------------------------------------------------------------
@@ -536,6 +537,13 @@ N2_API int n2_mlp_set_deferred_reduction(n2_mlp_t* mlp, int enable) {
 	return N2_OK;
 }
 
+void n2_mlp_borrow_fragment_image(n2_mlp_t* mlp, const n2_half* image) { mlp->frag_image = reinterpret_cast<const hf*>(image); }
+uint32_t n2_mlp_fragment_image_bytes(uint32_t in_w, uint32_t n_hidden) {
+	if (in_w == 48 && n_hidden == 2) return (uint32_t)frag_bytes(FragMap<3, 2>::SEL);
+	if (in_w == 48 && n_hidden == 1) return (uint32_t)frag_bytes(FragMap<3, 1>::SEL);
+	return 0;
+}
+
 N2_API int n2_mlp_set_output_gradient_exponent(n2_mlp_t* mlp, int exponent) {
 	N2_REQUIRE(mlp != nullptr, "n2_mlp_set_output_gradient_exponent: mlp is null");
 	N2_REQUIRE(exponent >= -14 && exponent <= 14, "n2_mlp_set_output_gradient_exponent: exponent %d outside [-14, 14]", exponent);
@@ -630,7 +638,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 		const size_t lds = mlp_wgrad_lds<IC, NH, false>();                                                          \
 		if (int rc = allow_lds(mlp_wgrad_kernel<IC, NH, DX, false>, lds)) return rc;                                \
 		mlp_wgrad_kernel<IC, NH, DX, false><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1, (int)dy_rows, dX, \
-			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv);                            \
+			next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv, mlp->frag_image);                            \
 	} while (0)
 	// the field's colour net (48 inputs, two hidden layers): only the rows the field reads are stored
 	N2_REQUIRE(tail == nullptr || (want_dx && want_dw && dx_out_and_normal_only && mlp->in_w == 48 && mlp->n_hidden == 2 && (aos & 1) && dy_rows <= 8),
@@ -641,7 +649,7 @@ static int mlp_backward_impl(n2_mlp_t* mlp, n2_stream_t stream, const n2_half* d
 			const size_t lds = mlp_wgrad_lds<3, 2, false>();
 			if (int rc = allow_lds(mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail>, lds)) return rc;
 			mlp_wgrad_kernel<3, 2, WG_DX_OUT_AND_NORMAL, false, WgFieldPrepTail><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params, X, n, dY, aos & 1,
-				(int)dy_rows, dX, next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv, t);
+				(int)dy_rows, dX, next_slabs(mlp), nullptr, nullptr, -1, x_index, x_cols, dy_gain, dy_gain_inv, mlp->frag_image, t);
 		} else {
 			LAUNCH_W(3, 2, WG_DX_OUT_AND_NORMAL);
 		}
@@ -751,7 +759,7 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 		mlp_wgrad_kernel<3, 1, WG_DX_ENCODING, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),
-			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f);
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f, mlp->frag_image);
 		N2_LAUNCH_CHECK();
 		return reduce_partials(mlp, s, blocks, mode);
 	}
@@ -763,7 +771,7 @@ int n2_mlp_backward_and_second_order_indexed(n2_mlp_t* mlp, n2_stream_t stream, 
 		mlp_wgrad_kernel<IC, 1, WG_DX_ALL, true><<<dim3(blocks), dim3(MLP_BLOCK), lds, s>>>(mlp->params,                   \
 			reinterpret_cast<const hf*>(d_input), n, reinterpret_cast<const hf*>(d_dL_doutput), aos, MLP_OUT,              \
 			reinterpret_cast<hf*>(d_dL_dinput), next_slabs(mlp), reinterpret_cast<const hf*>(d_dL_ddLdinput),              \
-			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f);                       \
+			reinterpret_cast<const hf*>(d_second_dL_doutput), unit_row2, d_index, n_cols, 1.f, 1.f, mlp->frag_image);                       \
 		break;                                                                                                             \
 	}
 		CASE(1) CASE(2) CASE(3) CASE(4)

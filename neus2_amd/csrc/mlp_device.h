@@ -206,13 +206,14 @@ __device__ __forceinline__ half8 zero8() {
 	return z;
 }
 
+// what lane l holds of fragment f
 template <int IC, int NH>
-__device__ __forceinline__ void build_frags(hf* F, const hf* __restrict__ W, int count) {
+__device__ __forceinline__ half8 mlp_frag_value(const hf* __restrict__ W, int f, int l) {
 	using M = FragMap<IC, NH>;
 	const hf* W_hid = W + MLP_WIDTH * M::IN_W;
 	const hf* W_out = W_hid + (NH - 1) * MLP_WIDTH * MLP_WIDTH;
-	for (int idx = threadIdx.x; idx < count * 64; idx += MLP_BLOCK) {
-		const int f = idx >> 6, l = idx & 63, n = l & 31, g = l >> 5;
+	{
+		const int n = l & 31, g = l >> 5;
 		half8 v = zero8();
 		if (f < M::WH) {
 			v = wfrag_natural(W, M::IN_W, 32 * (f / IC) + n, f % IC, g);
@@ -237,8 +238,17 @@ __device__ __forceinline__ void build_frags(hf* F, const hf* __restrict__ W, int
 #pragma unroll
 			for (int e = 0; e < 8; ++e) v[e] = (8 * g + e == n) ? (hf)1 : (hf)0;
 		}
-		*reinterpret_cast<half8*>(F + (size_t)idx * 8) = v;
+		return v;
 	}
+}
+template <int IC, int NH>
+__device__ __forceinline__ void build_frags(hf* F, const hf* __restrict__ W, int count) {
+	for (int idx = threadIdx.x; idx < count * 64; idx += MLP_BLOCK) *reinterpret_cast<half8*>(F + (size_t)idx * 8) = mlp_frag_value<IC, NH>(W, idx >> 6, idx & 63);
+	__syncthreads();
+}
+// the same fragments from an image that another launch has built in global memory (count KiB)
+__device__ __forceinline__ void load_frags(hf* F, const hf* __restrict__ image, int count) {
+	for (int idx = threadIdx.x; idx < count * 64; idx += MLP_BLOCK) *reinterpret_cast<half8*>(F + (size_t)idx * 8) = *reinterpret_cast<const half8*>(image + (size_t)idx * 8);
 	__syncthreads();
 }
 

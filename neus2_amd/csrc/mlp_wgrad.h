@@ -98,7 +98,7 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
                                                                  int dy_aos, int dy_rows, hf* __restrict__ dX, float* __restrict__ partials,
                                                                  const hf* __restrict__ V, const hf* __restrict__ G2, int unit_row2,
                                                                  const uint32_t* __restrict__ x_index, uint32_t x_cols, float dy_gain, float dy_gain_inv,
-                                                                 const Tail tail = Tail()) {
+                                                                 const hf* __restrict__ frag_image, const Tail tail = Tail()) {
 	static_assert(!SECOND || NH == 1, "the second-order pass needs one hidden layer");
 	static_assert(!Tail::active || (IC == 3 && NH == 2 && WANT_DX == WG_DX_OUT_AND_NORMAL), "the field's tail goes with the colour net");
 	// dy_gain = 2^k, dy_gain_inv = 2^-k (first-order launches only).  The output gradient is multiplied by 2^k when it is
@@ -113,7 +113,9 @@ __global__ void __launch_bounds__(MLP_BLOCK, 2) mlp_wgrad_kernel(const hf* __res
 	extern __shared__ __align__(16) unsigned char smem[];
 	hf* F = reinterpret_cast<hf*>(smem);
 	unsigned char* S = smem + (size_t)M::SEL * 1024;  // staging buffer behind the fragments
-	build_frags<IC, NH>(F, W, M::SEL);
+	// (frag_image: the fragments as a launch in front of this one has left them in global memory, M::SEL KiB; null: built here)
+	if (frag_image) load_frags(F, frag_image, M::SEL);
+	else build_frags<IC, NH>(F, W, M::SEL);
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, g = lane >> 5;
 	const int mt = __builtin_amdgcn_readfirstlane(wave >> 1), nt = __builtin_amdgcn_readfirstlane(wave & 1);
 	const uint32_t s_local = 32u * wave + n;

@@ -78,9 +78,17 @@ struct N2FusedNets {
 	const n2_half* variance;
 	uint32_t sdf_in_w;
 	float sdf_bias;
-	n2_half* frag_image;  // N2_FUSED_FRAG_BYTES of scratch for the full forward's weight fragments (written by its gather launch), or null
+	// N2_FUSED_FRAG_BYTES of scratch, or null: the gather launch of a full forward leaves the weight fragments of its network
+	// kernel there (the first N2_FUSED_FRAG_FORWARD bytes) and, behind them, those of the backward's two weight-gradient
+	// kernels (colour net, then SDF net when it has 48 inputs): built once per step instead of once per workgroup
+	n2_half* frag_image;
 };
-constexpr uint64_t N2_FUSED_FRAG_BYTES = 40 * 1024;
+constexpr uint64_t N2_FUSED_FRAG_FORWARD = 40 * 1024, N2_FUSED_FRAG_RGB = 36 * 1024, N2_FUSED_FRAG_SDF = 20 * 1024;
+constexpr uint64_t N2_FUSED_FRAG_BYTES = N2_FUSED_FRAG_FORWARD + N2_FUSED_FRAG_RGB + N2_FUSED_FRAG_SDF;
+// the weight-gradient launches of `mlp` read their fragments from `image` (as mlp_frag_value lays them out; null: every
+// workgroup builds them from the weights).  Borrowed: the caller keeps it valid and matching the weights.
+void n2_mlp_borrow_fragment_image(n2_mlp_t* mlp, const n2_half* image);
+uint32_t n2_mlp_fragment_image_bytes(uint32_t in_w, uint32_t n_hidden);
 const N2LevelTable* n2_grid_table(const n2_grid_t* grid);
 const __half2* n2_grid_params(const n2_grid_t* grid);
 bool n2_grid_lattice_order(const n2_grid_t* grid);
