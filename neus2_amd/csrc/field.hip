@@ -391,6 +391,7 @@ N2_API int n2_field_set_workspace(n2_field_t* f, void* d_workspace, uint64_t n_b
 	f->var_part = reinterpret_cast<float*>(b + c.var_part);
 	f->sel_index = reinterpret_cast<uint32_t*>(b + c.sel_index);
 	f->frag_image = reinterpret_cast<hf*>(b + c.frag_image);
+	f->frags_ready = false;
 	f->last_n = 0;
 	f->sel_n = 0;
 	f->pad_n = {0, 0, 0};
