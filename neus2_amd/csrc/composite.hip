@@ -401,7 +401,7 @@ __global__ void __launch_bounds__(CHUNK_BLOCK) composite_chunk_kernel(CompParams
                                                                       ChunkRay* __restrict__ state, uint32_t* __restrict__ counts,
                                                                       uint32_t* __restrict__ counts_other, uint32_t* __restrict__ list,
                                                                       uint32_t* __restrict__ column_of, float* __restrict__ coords_listed) {
-	__shared__ uint32_t takes[CHUNK_RAYS], places[CHUNK_RAYS];
+	__shared__ uint32_t takes[CHUNK_RAYS], firsts[CHUNK_RAYS], before[CHUNK_RAYS + 1], wg_at;
 	const uint32_t l = threadIdx.x % CHUNK_LANES, slot = threadIdx.x / CHUNK_LANES;
 	const uint32_t ray = blockIdx.x * CHUNK_RAYS + slot;
 	const uint32_t live_rays = ray_counter ? min(*ray_counter, n_rays) : n_rays;
@@ -441,8 +441,8 @@ __global__ void __launch_bounds__(CHUNK_BLOCK) composite_chunk_kernel(CompParams
 		}
 	}
 	const uint32_t take = st.live ? min(n - st.done, chunk) : 0u;
-	// places in the list: the workgroup's sixteen rays in order, one atomic per workgroup for its block of places
-	if (l == 0) takes[slot] = take;
+	// places in the list: the workgroup's 64 rays in order, one atomic per workgroup for its block of places
+	if (l == 0) { takes[slot] = take; firsts[slot] = base + st.done; }
 	__syncthreads();
 	if (threadIdx.x < 64) {  // one wave scans the 64 counts
 		static_assert(CHUNK_RAYS == 64, "one count per lane");
@@ -456,18 +456,32 @@ __global__ void __launch_bounds__(CHUNK_BLOCK) composite_chunk_kernel(CompParams
 		const uint32_t total = __shfl(incl, 63);
 		uint32_t at = 0;
 		if (threadIdx.x == 0 && total) at = atomicAdd(&counts[round], total);
-		places[threadIdx.x] = __shfl(at, 0) + incl - own;
+		before[threadIdx.x] = incl - own;
+		if (threadIdx.x == 63) before[CHUNK_RAYS] = total;
+		if (threadIdx.x == 0) wg_at = at;
 	}
 	__syncthreads();
-	const uint32_t at = begin + places[slot], first = base + st.done;
-	for (uint32_t k = l; k < take; k += CHUNK_LANES) {
-		list[at + k] = first + k;
-		column_of[first + k] = at + k;
+	// The workgroup's listed samples, all threads together (a ray that lists hundreds of samples in the last round would
+	// otherwise keep its sixteen lanes busy long after the others are done): sample e of the workgroup belongs to the ray r
+	// with before[r] <= e < before[r + 1].  The coordinate rows go along: consecutive in the output over the whole workgroup.
+	const uint32_t total = before[CHUNK_RAYS], at0 = begin + wg_at;
+	auto ray_of = [&](uint32_t e) {
+		uint32_t r = 0;
+#pragma unroll
+		for (uint32_t step = CHUNK_RAYS / 2; step > 0; step >>= 1)
+			if (before[r + step] <= e) r += step;
+		return r;
+	};
+	for (uint32_t e = threadIdx.x; e < total; e += CHUNK_BLOCK) {
+		const uint32_t r = ray_of(e), id = firsts[r] + (e - before[r]);
+		list[at0 + e] = id;
+		column_of[id] = at0 + e;
 	}
-	// the coordinate rows of the listed samples: consecutive in the input (one ray's samples) and in the output
-	const float* from = coords + (size_t)first * 7;
-	float* to = coords_listed + (size_t)at * 7;
-	for (uint32_t k = l; k < take * 7u; k += CHUNK_LANES) to[k] = from[k];
+	float* to = coords_listed + (size_t)at0 * 7;
+	for (uint32_t f = threadIdx.x; f < total * 7u; f += CHUNK_BLOCK) {
+		const uint32_t e = f / 7u, r = ray_of(e);
+		to[f] = coords[(size_t)(firsts[r] + (e - before[r])) * 7 + (f - e * 7u)];
+	}
 	if (ray < live_rays && l == 0) {
 		st.prev = st.done;
 		st.done += take;
